@@ -1,0 +1,256 @@
+/*
+ * sgl_hot.h -- C ABI of libsgl_hot.so: the temporal-GNN mini-batch hot path of
+ * StarryGL for one GPU's graph partition, written for AMD gfx950 (MI355X).
+ *
+ * The four stages behind this boundary are
+ *   (1) temporal neighbour sampling over a time-sorted CSR (T-CSR),
+ *   (2) unique + compaction of sampled node ids to dense local ids,
+ *   (3) feature / TGN-memory row gather through a cache index
+ *       (HBM-resident hot rows, pinned-host cold rows),
+ *   (4) the cos(w*dt + b) time encoding.
+ *
+ * Conventions
+ *   - every pointer named in a "device" role must be dereferenceable from the
+ *     GPU (hipMalloc memory, or hipHostMalloc'ed pinned memory where stated);
+ *   - ids, timestamps and offsets are int64_t;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - every entry point returns an int32_t status (SGL_OK or a negative SGL_E*);
+ *     no C++ exception crosses the boundary, nothing calls exit();
+ *   - the library allocates no device memory: outputs and workspace belong to
+ *     the caller, `*_workspace_bytes` tells how much workspace a call needs;
+ *   - entry points are asynchronous w.r.t. the host unless stated otherwise;
+ *     two calls that share a workspace or a remap state must be ordered on one
+ *     stream.
+ *
+ * The reference interface each entry point replaces is cited as
+ * path:line relative to the StarryGL source tree.
+ */
+#ifndef SGL_HOT_H
+#define SGL_HOT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SGL_ABI_VERSION 1
+
+/* ------------------------------------------------------------------ status */
+#define SGL_OK        0
+#define SGL_EINVAL  (-1) /* null pointer, negative size, bad enum value        */
+#define SGL_ERANGE  (-2) /* node / chunk id outside [0,n), unsorted timestamps */
+#define SGL_ENOTSUP (-3) /* unknown sampling strategy, unsupported fanout      */
+#define SGL_EHIP    (-4) /* a HIP runtime call failed (see error string)       */
+#define SGL_ENOMEM  (-5) /* caller-provided workspace / capacity too small     */
+
+/* Thread-local, human readable description of the last non-OK status returned
+ * to the calling thread.  Replaces the C++ exceptions / TORCH_CHECK messages of
+ * csrc/srcs/starrygl/export.cu:237-244 and sample.cu.hpp:1001-1062. */
+const char* sgl_last_error_string(void);
+int32_t     sgl_abi_version(void);
+
+/* ------------------------------------------------------------------- T-CSR */
+/* Time-sorted CSR of one partition.  Row v occupies [row_ptr[v], row_ptr[v+1]);
+ * inside a row edges ascend in (ts, eid).  Replaces the device arrays
+ * row_ptr_/col_idx_/col_ts_/edge_id_ of `Graph` (sample.cu.hpp:960-1185). */
+typedef struct sgl_tcsr {
+    int64_t        n;       /* number of nodes                  */
+    int64_t        m;       /* number of edges                  */
+    const int64_t* row_ptr; /* [n+1] device                     */
+    const int64_t* col;     /* [m]   device: destination node   */
+    const int64_t* ts;      /* [m]   device: edge timestamp     */
+    const int64_t* eid;     /* [m]   device: edge id            */
+} sgl_tcsr;
+
+/* Build a T-CSR from a COO edge list (replaces from_edge_index / Graph::Graph,
+ * export.cu:229-250, sample.cu.hpp:985-1185).  `eid` may be NULL (= 0..m-1).
+ * Output order is the stable sort by (src, ts, eid).  Synchronous: returns
+ * SGL_ERANGE if any src/dst is outside [0,n) (sample.cu.hpp:1043-1048). */
+size_t  sgl_tcsr_build_workspace_bytes(int64_t n, int64_t m);
+int32_t sgl_tcsr_build(int64_t n, int64_t m,
+                       const int64_t* src, const int64_t* dst,
+                       const int64_t* ts, const int64_t* eid,
+                       int64_t* row_ptr, int64_t* col, int64_t* col_ts,
+                       int64_t* col_eid,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* Check an adopted (already sorted) T-CSR: row_ptr monotone with
+ * row_ptr[0]=0,row_ptr[n]=m, col in [0,n), ts ascending inside every row.
+ * Synchronous.  `workspace` needs 8 bytes. */
+int32_t sgl_tcsr_validate(const sgl_tcsr* g, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------- sampling */
+#define SGL_SAMPLE_RECENT  0 /* "recent"  : the last min(k,cnt) window edges  */
+#define SGL_SAMPLE_UNIFORM 1 /* "uniform" : k distinct window edges, uniform  */
+
+/* Largest fanout the uniform strategy accepts (one wavefront holds one slot's
+ * draws).  The recent strategy has no limit. */
+#define SGL_UNIFORM_MAX_FANOUT 64
+
+/* Arguments of Graph::sample_src_in_chunks_khop (sample.cu.hpp:1532-1534,
+ * export.cu:194-201).  Candidate window of a slot (v, t):
+ *   t_lo <= ts[e] < t_hi,  t_hi = t + (equal_root_time ? 1 : 0),
+ *   t_lo = allowed_offset < 0 ? -inf : t - allowed_offset. */
+typedef struct sgl_sample_params {
+    int32_t  type;            /* SGL_SAMPLE_*                                  */
+    int32_t  fanout;          /* k                                             */
+    int64_t  allowed_offset;  /* < 0: window is unbounded below                */
+    int32_t  equal_root_time; /* 1: edges with ts == t are candidates          */
+    int32_t  keep_root_time;  /* uniform only: neighbors_ts = root t           */
+    int32_t  replace;         /* uniform only: 1 = k iid draws (may repeat)    */
+    int32_t  hop;             /* RNG stream selector for sgl_sample_hop        */
+    uint64_t seed;            /* Philox4x32-10 key                             */
+} sgl_sample_params;
+
+/* One hop's result, caller-allocated (replaces TemporalNeighbor,
+ * sample.cu.hpp:882-915).  With S slots and E = sum_s c_s sampled edges:
+ *   root_start_ptr[0..S] = exclusive prefix of c (root_start_ptr[S] = E),
+ *   root_end_ptr[s] = root_start_ptr[s+1] for s < S, root_end_ptr[S] = E,
+ *   neighbors*, [0..E): slot s owns [root_start_ptr[s], root_end_ptr[s]),
+ *   neighbors_dt = ts[e] - t_root,
+ *   counts[0] = S, counts[1] = E, counts[2] = slots with an out-of-range
+ *   node (device scalars). */
+typedef struct sgl_hop_out {
+    int64_t  capacity_slots; /* root_*_ptr hold capacity_slots+1 entries       */
+    int64_t  capacity_edges; /* neighbors* hold capacity_edges entries;        */
+                             /* must be >= capacity_slots * fanout             */
+    int64_t* root_start_ptr;
+    int64_t* root_end_ptr;
+    int64_t* neighbors;
+    int64_t* neighbors_ts;
+    int64_t* neighbors_eid;
+    int64_t* neighbors_dt;
+    int64_t* counts;         /* device int64[3]                                */
+} sgl_hop_out;
+
+/* One sampling hop over explicit slots (slot_node[s], slot_ts[s]), s < S.
+ * S = *S_dev when S_dev != NULL (a device scalar, must be <= S_max), else
+ * S_max.  Replaces static_recent_neighbor_num + recent_sample_single_hop_kernel
+ * and static_neighbor_num + uniform_sample_single_hop_kernel plus the thrust
+ * scans between them (sample.cu.hpp:706-827, 1569-1687).
+ * A slot whose node lies outside [0,n) is sampled as empty and counted in
+ * counts[2] (the caller turns a non-zero count into SGL_ERANGE). */
+size_t  sgl_sample_hop_workspace_bytes(int64_t S_max);
+int32_t sgl_sample_hop(const sgl_tcsr* g,
+                       const int64_t* slot_node, const int64_t* slot_ts,
+                       int64_t S_max, const int64_t* S_dev,
+                       const sgl_sample_params* p, const sgl_hop_out* out,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* k-hop driver (replaces Graph::sample_src_in_chunks_khop,
+ * sample.cu.hpp:1532-1716).  Hop-0 slots are the positive roots expanded over
+ * their timestamps (root r owns root_ts[ts_ptr[r]..ts_ptr[r+1])) followed by
+ * the negative roots; they are written to slot_node0/slot_ts0
+ * ([S_pos + N_neg] each).  Hop l+1 slots are hop l's (neighbors, neighbors_ts),
+ * one slot per sampled edge, no dedup between hops.  p->hop is ignored; hop l
+ * draws from RNG stream l.  outs[l].capacity_slots must be >= the worst-case
+ * slot count of hop l ((S_pos+N_neg) * fanout^l). */
+size_t  sgl_sample_khop_workspace_bytes(int64_t S0, int32_t layers,
+                                        int32_t fanout);
+int32_t sgl_sample_khop(const sgl_tcsr* g,
+                        int64_t R, const int64_t* roots, const int64_t* ts_ptr,
+                        int64_t S_pos, const int64_t* root_ts,
+                        int64_t N_neg, const int64_t* neg_roots,
+                        const int64_t* neg_ts,
+                        int32_t layers, const sgl_sample_params* p,
+                        int64_t* slot_node0, int64_t* slot_ts0,
+                        const sgl_hop_out* outs,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------ unique / compaction */
+#define SGL_UNIQUE_SORTED  0 /* all arrays form one group: == np.unique(return_inverse) */
+#define SGL_UNIQUE_GROUPED 1 /* per array: ids new to the epoch, ascending, appended    */
+
+/* Persistent remap state over a dense id universe [0, universe): the
+ * replacement of Remapper's id_mapper/global_mask tables and epoch counter
+ * (sample.cu.hpp:1752-1763).  The caller allocates sgl_remap_state_bytes()
+ * device bytes and calls sgl_remap_init once. */
+size_t  sgl_remap_state_bytes(int64_t universe);
+int32_t sgl_remap_init(void* state, size_t state_bytes, int64_t universe,
+                       void* stream);
+
+/* Rewrite G id arrays to dense local ids and emit the local->global table
+ * (replaces Remapper::insert / remapper + mark_new_ids_kernel +
+ * update_new_ids_kernel, sample.cu.hpp:1719-1854; np.unique /
+ * _merge_and_map_nodes in prepare_sample.py:205-246).
+ *   ids[g]       device array of len_max[g] ids; the live length is
+ *                *len_dev[g] when len_dev != NULL && len_dev[g] != NULL.
+ *   local_out[g] same shape as ids[g] (may alias ids[g]).
+ *   reset        1: start a new local-id epoch (numbering restarts at 0);
+ *                0: continue the epoch of the previous call on `state`.
+ *   unique_out   local -> global; entries [U_before, U_total) are written.
+ *   U_dev        device int64[2] = {U_total, U_before}.
+ * `state` != NULL selects the dense-universe path: `universe` must be the value
+ * given to sgl_remap_init, ids outside [0, universe) map to -1.  `state` ==
+ * NULL (universe ignored) selects the hash-set path, which accepts arbitrary
+ * non-negative ids but only reset = 1.  Negative ids always map to -1. */
+size_t  sgl_unique_workspace_bytes(int64_t universe, int32_t G,
+                                   const int64_t* len_max);
+int32_t sgl_unique_compact(void* state, int64_t universe, int32_t reset,
+                           int32_t mode, int32_t G, const int64_t* const* ids,
+                           const int64_t* len_max,
+                           const int64_t* const* len_dev,
+                           int64_t* const* local_out,
+                           int64_t* unique_out, int64_t unique_capacity,
+                           int64_t* U_dev,
+                           void* workspace, size_t workspace_bytes,
+                           void* stream);
+
+/* ------------------------------------------------------------ cache gather */
+/* Two-tier row store (replaces IDMapper.to_local + DistNodeState.__getitem__,
+ * starrygl/utils/partition_book.py:106-133, starrygl/cache/NodeState.py:36-44,
+ * and tensor_gather / ShardTensor, csrc/include/starrygl/feature.cu.hpp:42-88,
+ * 236-422).  Lookup of a requested id:
+ *   key  = id & id_mask                      (id_mask = -1: use the id as is;
+ *                                             0xFFFFFFFFFFFF: DistRouteIndex.loc)
+ *   loc  = g2l ? g2l[key] : key              (-1 / out of range = not resident)
+ *   slot = hot_slot ? hot_slot[loc] : loc    (>= 0: row `slot` of `hot`,
+ *                                             < 0 : row `loc` of `cold`)
+ * A non-resident id yields an all-zero row, out_ts = 0 and bumps stats[2]. */
+typedef struct sgl_cache {
+    int64_t        rows;      /* logical (local) rows                          */
+    int64_t        row_bytes; /* multiple of 4                                 */
+    int64_t        id_mask;
+    const int64_t* g2l;       /* device [g2l_len] or NULL                      */
+    int64_t        g2l_len;
+    const int32_t* hot_slot;  /* device [rows] or NULL                         */
+    const void*    hot;       /* device (HBM) [hot_rows, row_bytes]            */
+    int64_t        hot_rows;
+    const void*    cold;      /* device-visible pinned host [rows, row_bytes]  */
+    const int64_t* ts_hot;    /* optional last-update time per hot row         */
+    const int64_t* ts_cold;   /* optional last-update time per logical row     */
+} sgl_cache;
+
+/* out[i, :] = row(ids[i]); out_ts[i] = its last-update time when out_ts and the
+ * tier's ts table are non-NULL.  N = *N_dev when N_dev != NULL (<= N_max).
+ * stats (optional device int64[3]) += {hot hits, cold hits, absent}. */
+int32_t sgl_gather(const sgl_cache* c, const int64_t* ids, int64_t N_max,
+                   const int64_t* N_dev, void* out, int64_t* out_ts,
+                   int64_t* stats, void* stream);
+
+/* Scatter rows back (replaces DistNodeState.update, NodeState.py:46-61):
+ * ids that are not resident are skipped.  Duplicate ids: the highest i wins
+ * is NOT guaranteed; callers pass unique ids (as the reference's callers do). */
+int32_t sgl_scatter_update(const sgl_cache* c, void* hot_rw, void* cold_rw,
+                           int64_t* ts_hot_rw, int64_t* ts_cold_rw,
+                           const int64_t* ids, int64_t N,
+                           const void* values, const int64_t* ts,
+                           void* stream);
+
+/* ----------------------------------------------------------- time encoding */
+#define SGL_DT_I64 0
+#define SGL_DT_F32 1
+/* out[i, j] = cos(fl32(fl32(w[j] * float(dt[i])) + b[j])), fp32, no FMA
+ * contraction (replaces TimeEncoder.forward,
+ * starrygl/nn/model/time_encoder.py:29-31). */
+int32_t sgl_time_encode(const void* dt, int32_t dt_dtype, int64_t N_max,
+                        const int64_t* N_dev, const float* w, const float* b,
+                        int32_t dim, float* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SGL_HOT_H */

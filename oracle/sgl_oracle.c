@@ -1,0 +1,575 @@
+/*
+ * sgl_oracle.c -- CPU restatement of StarryGL's temporal mini-batch hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker the HIP library is
+ * compared against and the CPU baseline the benchmark times; nothing in the
+ * shipped library links, loads or falls back to it.
+ *
+ * Every function mirrors one entry point of include/sgl_hot.h (prefix `sglo_`
+ * instead of `sgl_`), takes HOST pointers, ignores `stream` and `workspace`,
+ * and follows the reference source cited above it (paths relative to the
+ * StarryGL tree).  Where the reference disagrees with itself the rule that is
+ * implemented is written next to the citation.
+ *
+ * What pins each function (see tests/test_oracle_*.py):
+ *   window / recent      np.searchsorted + brute-force list comprehension
+ *   uniform              Philox4x32-10 known-answer vectors (Random123),
+ *                        subset invariants, chi-square over seeds
+ *   unique               np.unique(return_inverse), np.setdiff1d per group
+ *   gather / scatter     numpy fancy indexing
+ *   time encode          float64 closed form
+ *   t-csr build          np.lexsort((eid, ts, src)) + bincount/cumsum
+ *   seeds / block        brute-force python loops on tiny graphs
+ *
+ * Build:  make -C oracle      (gcc -O2 -fopenmp -ffp-contract=off)
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <stdio.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#include "../include/sgl_hot.h"
+
+static __thread char g_err[256];
+static int g_threads = 1;
+
+static int32_t fail(int32_t code, const char* msg) {
+    snprintf(g_err, sizeof g_err, "%s", msg);
+    return code;
+}
+
+const char* sglo_last_error_string(void) { return g_err; }
+int32_t     sglo_abi_version(void) { return SGL_ABI_VERSION; }
+
+/* Number of OpenMP threads the sampler loops use (1 = the scalar port).  The
+ * reference runs its sampler loops under numba.prange
+ * (prepare_sample.py:31,44,91) / at::parallel_for (graph.cpu.hpp:270,293). */
+void sglo_set_num_threads(int32_t t) { g_threads = t < 1 ? 1 : t; }
+int32_t sglo_get_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* ------------------------------------------------------------------ T-CSR */
+
+typedef struct { int64_t src, ts, eid, dst; } edge_rec;
+
+static int edge_cmp(const void* a, const void* b) {
+    const edge_rec* x = (const edge_rec*)a;
+    const edge_rec* y = (const edge_rec*)b;
+    if (x->src != y->src) return x->src < y->src ? -1 : 1;
+    if (x->ts != y->ts) return x->ts < y->ts ? -1 : 1;
+    if (x->eid != y->eid) return x->eid < y->eid ? -1 : 1;
+    return 0;
+}
+
+size_t sglo_tcsr_build_workspace_bytes(int64_t n, int64_t m) {
+    (void)n; (void)m;
+    return 0;
+}
+
+/* T-CSR build.  Reference: Graph::Graph sorts Edge records with
+ * EdgeComparator and scatters them (sample.cu.hpp:51-63, 985-1185); the CPU
+ * twin sorts with np.lexsort((ts, dst)) keyed by the row node
+ * (prepare_sample.py:192-203).  Rule implemented: rows by source node,
+ * inside a row ascending (ts, eid); row_ptr = cumsum(bincount(src)). */
+int32_t sglo_tcsr_build(int64_t n, int64_t m, const int64_t* src,
+                        const int64_t* dst, const int64_t* ts,
+                        const int64_t* eid, int64_t* row_ptr, int64_t* col,
+                        int64_t* col_ts, int64_t* col_eid, void* ws,
+                        size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (n < 0 || m < 0 || !row_ptr) return fail(SGL_EINVAL, "tcsr_build: bad sizes");
+    if (m > 0 && (!src || !dst || !ts || !col || !col_ts || !col_eid))
+        return fail(SGL_EINVAL, "tcsr_build: null array");
+    for (int64_t i = 0; i < m; ++i)
+        if (src[i] < 0 || src[i] >= n || dst[i] < 0 || dst[i] >= n)
+            return fail(SGL_ERANGE, "tcsr_build: src/dst outside [0,n)");
+    edge_rec* e = (edge_rec*)malloc((size_t)(m > 0 ? m : 1) * sizeof *e);
+    if (!e) return fail(SGL_ENOMEM, "tcsr_build: malloc");
+    for (int64_t i = 0; i < m; ++i) {
+        e[i].src = src[i]; e[i].ts = ts[i];
+        e[i].eid = eid ? eid[i] : i; e[i].dst = dst[i];
+    }
+    qsort(e, (size_t)m, sizeof *e, edge_cmp);
+    memset(row_ptr, 0, (size_t)(n + 1) * sizeof(int64_t));
+    for (int64_t i = 0; i < m; ++i) {
+        row_ptr[e[i].src + 1]++;
+        col[i] = e[i].dst; col_ts[i] = e[i].ts; col_eid[i] = e[i].eid;
+    }
+    for (int64_t v = 0; v < n; ++v) row_ptr[v + 1] += row_ptr[v];
+    free(e);
+    return SGL_OK;
+}
+
+int32_t sglo_tcsr_validate(const sgl_tcsr* g, void* ws, size_t ws_bytes,
+                           void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (!g || g->n < 0 || g->m < 0 || !g->row_ptr) return fail(SGL_EINVAL, "tcsr_validate: null");
+    if (g->row_ptr[0] != 0 || g->row_ptr[g->n] != g->m)
+        return fail(SGL_ERANGE, "tcsr_validate: row_ptr ends");
+    for (int64_t v = 0; v < g->n; ++v) {
+        int64_t a = g->row_ptr[v], b = g->row_ptr[v + 1];
+        if (b < a) return fail(SGL_ERANGE, "tcsr_validate: row_ptr not monotone");
+        for (int64_t e = a; e < b; ++e) {
+            if (g->col[e] < 0 || g->col[e] >= g->n)
+                return fail(SGL_ERANGE, "tcsr_validate: col outside [0,n)");
+            if (e > a && g->ts[e] < g->ts[e - 1])
+                return fail(SGL_ERANGE, "tcsr_validate: ts not ascending in row");
+        }
+    }
+    return SGL_OK;
+}
+
+/* --------------------------------------------------------------- sampling */
+
+/* first index in [lo,hi) whose ts >= key (np.searchsorted side='left',
+ * prepare_sample.py:50-51; std::lower_bound, graph.cpu.hpp:301). */
+static int64_t lower_bound_ts(const int64_t* ts, int64_t lo, int64_t hi, int64_t key) {
+    while (lo < hi) {
+        int64_t mid = lo + ((hi - lo) >> 1);
+        if (ts[mid] < key) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+/* Candidate window of a slot.  Reference: find_time_range
+ * (sample.cu.hpp:264-295) called with (ts - allowed_offset or 0,
+ * ts + equal_root_time) at :723-724; numba cut_idx/start_idx
+ * (prepare_sample.py:50-55).  Rule implemented: strictly before t unless
+ * equal_root_time, lower bound only when allowed_offset >= 0. */
+static void window(const sgl_tcsr* g, int64_t v, int64_t t, int64_t allowed_offset,
+                   int32_t equal_root_time, int64_t* lo_out, int64_t* hi_out) {
+    int64_t rs = g->row_ptr[v], re = g->row_ptr[v + 1];
+    int64_t t_hi = t + (equal_root_time ? 1 : 0);
+    int64_t hi = lower_bound_ts(g->ts, rs, re, t_hi);
+    int64_t lo = rs;
+    if (allowed_offset >= 0) lo = lower_bound_ts(g->ts, rs, re, t - allowed_offset);
+    if (lo > hi) lo = hi;
+    *lo_out = lo; *hi_out = hi;
+}
+
+/* Philox4x32-10 (Salmon et al., SC'11; Random123 v1.x philox.h).  Replaces
+ * curand_init(1317, threadIdx.x, 0) + curand_uniform (sample.cu.hpp:791-816)
+ * with a counter-based generator so that a draw depends only on
+ * (seed, hop, slot, draw index). */
+static void philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3];
+    uint32_t k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; ++r) {
+        uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+        uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+        uint32_t n1 = (uint32_t)p1;
+        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        uint32_t n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+void sglo_philox4x32_10(const uint32_t* ctr, const uint32_t* key, uint32_t* out) {
+    philox4x32_10(ctr, key, out);
+}
+
+/* 64 random bits of draw j of slot s in hop h: counter = (j, s_lo, s_hi, h),
+ * key = (seed_lo, seed_hi); bits = x0 | x1 << 32. */
+static uint64_t draw_bits(uint64_t seed, int32_t hop, int64_t slot, int32_t j) {
+    uint32_t ctr[4] = {(uint32_t)j, (uint32_t)((uint64_t)slot & 0xFFFFFFFFu),
+                       (uint32_t)((uint64_t)slot >> 32), (uint32_t)hop};
+    uint32_t key[2] = {(uint32_t)(seed & 0xFFFFFFFFu), (uint32_t)(seed >> 32)};
+    uint32_t x[4];
+    philox4x32_10(ctr, key, x);
+    return (uint64_t)x[0] | ((uint64_t)x[1] << 32);
+}
+
+/* floor(bits * range / 2^64): a value in [0, range). */
+static int64_t bounded(uint64_t bits, int64_t range) {
+    return (int64_t)(((unsigned __int128)bits * (uint64_t)range) >> 64);
+}
+
+uint64_t sglo_draw_bits(uint64_t seed, int32_t hop, int64_t slot, int32_t j) {
+    return draw_bits(seed, hop, slot, j);
+}
+int64_t sglo_bounded(uint64_t bits, int64_t range) { return bounded(bits, range); }
+
+/* k distinct offsets in [0,cnt), ascending (Floyd's subset sampling; the
+ * reference draws np.random.choice(cut_idx, fanout, replace=False) then
+ * sorts, prepare_sample.py:124-125). */
+static void floyd_subset(uint64_t seed, int32_t hop, int64_t slot, int64_t cnt,
+                         int32_t k, int64_t* sel) {
+    for (int32_t j = 0; j < k; ++j) {
+        int64_t i = cnt - k + j;
+        int64_t t = bounded(draw_bits(seed, hop, slot, j), i + 1);
+        int dup = 0;
+        for (int32_t q = 0; q < j; ++q) if (sel[q] == t) { dup = 1; break; }
+        sel[j] = dup ? i : t;
+    }
+    for (int32_t a = 1; a < k; ++a) { /* insertion sort, k is small */
+        int64_t x = sel[a]; int32_t b = a - 1;
+        while (b >= 0 && sel[b] > x) { sel[b + 1] = sel[b]; --b; }
+        sel[b + 1] = x;
+    }
+}
+
+size_t sglo_sample_hop_workspace_bytes(int64_t S_max) { (void)S_max; return 0; }
+
+/* One hop: count pass -> prefix sum -> fill pass, parallel over slots.
+ * Reference: _jit_sample_kernel (prepare_sample.py:43-78 count, :80-82
+ * prefix, :91-145 fill; recent :117-119, uniform :120-134);
+ * static_recent_neighbor_num / recent_sample_single_hop_kernel and
+ * static_neighbor_num / uniform_sample_single_hop_kernel
+ * (sample.cu.hpp:706-827); sample_kernel (graph.cpu.hpp:256-310). */
+int32_t sglo_sample_hop(const sgl_tcsr* g, const int64_t* slot_node,
+                        const int64_t* slot_ts, int64_t S_max,
+                        const int64_t* S_dev, const sgl_sample_params* p,
+                        const sgl_hop_out* out, void* ws, size_t ws_bytes,
+                        void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (!g || !p || !out || S_max < 0) return fail(SGL_EINVAL, "sample_hop: null/negative");
+    if (p->type != SGL_SAMPLE_RECENT && p->type != SGL_SAMPLE_UNIFORM)
+        return fail(SGL_ENOTSUP, "undefined sampling strategy");
+    if (p->fanout < 0) return fail(SGL_EINVAL, "sample_hop: fanout < 0");
+    if (p->type == SGL_SAMPLE_UNIFORM && p->fanout > SGL_UNIFORM_MAX_FANOUT)
+        return fail(SGL_ENOTSUP, "uniform fanout > SGL_UNIFORM_MAX_FANOUT");
+    int64_t S = S_dev ? *S_dev : S_max;
+    if (S > S_max || S > out->capacity_slots) return fail(SGL_ENOMEM, "sample_hop: slots > capacity");
+    if (out->capacity_edges < out->capacity_slots * (int64_t)p->fanout)
+        return fail(SGL_ENOMEM, "sample_hop: capacity_edges < capacity_slots*fanout");
+    const int32_t k = p->fanout;
+    int64_t* cnt = (int64_t*)malloc((size_t)(S + 1) * sizeof(int64_t));
+    int64_t* wlo = (int64_t*)malloc((size_t)(S + 1) * sizeof(int64_t));
+    int64_t* whi = (int64_t*)malloc((size_t)(S + 1) * sizeof(int64_t));
+    if (!cnt || !wlo || !whi) { free(cnt); free(wlo); free(whi); return fail(SGL_ENOMEM, "malloc"); }
+    int64_t bad = 0;
+    /* pass 1: count */
+#pragma omp parallel for schedule(dynamic, 256) num_threads(g_threads) reduction(+ : bad)
+    for (int64_t s = 0; s < S; ++s) {
+        int64_t v = slot_node[s];
+        if (v < 0 || v >= g->n) { cnt[s] = 0; wlo[s] = whi[s] = 0; bad++; continue; }
+        int64_t lo, hi;
+        window(g, v, slot_ts[s], p->allowed_offset, p->equal_root_time, &lo, &hi);
+        wlo[s] = lo; whi[s] = hi;
+        int64_t c = hi - lo;
+        cnt[s] = c < k ? c : k;
+    }
+    /* prefix */
+    int64_t acc = 0;
+    for (int64_t s = 0; s < S; ++s) { out->root_start_ptr[s] = acc; acc += cnt[s]; out->root_end_ptr[s] = acc; }
+    out->root_start_ptr[S] = acc; out->root_end_ptr[S] = acc;
+    /* pass 2: fill */
+#pragma omp parallel for schedule(dynamic, 256) num_threads(g_threads)
+    for (int64_t s = 0; s < S; ++s) {
+        int64_t c = cnt[s];
+        if (c == 0) continue;
+        int64_t off = out->root_start_ptr[s], t = slot_ts[s];
+        int64_t lo = wlo[s], hi = whi[s], len = hi - lo;
+        if (p->type == SGL_SAMPLE_RECENT || len <= k) {
+            int64_t b = (p->type == SGL_SAMPLE_RECENT) ? hi - c : lo;
+            for (int64_t j = 0; j < c; ++j) {
+                int64_t e = b + j;
+                out->neighbors[off + j] = g->col[e];
+                out->neighbors_ts[off + j] =
+                    (p->type == SGL_SAMPLE_UNIFORM && p->keep_root_time) ? t : g->ts[e];
+                out->neighbors_eid[off + j] = g->eid[e];
+                out->neighbors_dt[off + j] = g->ts[e] - t;
+            }
+        } else {
+            int64_t sel[SGL_UNIFORM_MAX_FANOUT];
+            if (p->replace) {
+                for (int32_t j = 0; j < k; ++j)
+                    sel[j] = bounded(draw_bits(p->seed, p->hop, s, j), len);
+            } else {
+                floyd_subset(p->seed, p->hop, s, len, k, sel);
+            }
+            for (int32_t j = 0; j < k; ++j) {
+                int64_t e = lo + sel[j];
+                out->neighbors[off + j] = g->col[e];
+                out->neighbors_ts[off + j] = p->keep_root_time ? t : g->ts[e];
+                out->neighbors_eid[off + j] = g->eid[e];
+                out->neighbors_dt[off + j] = g->ts[e] - t;
+            }
+        }
+    }
+    out->counts[0] = S; out->counts[1] = acc; out->counts[2] = bad;
+    free(cnt); free(wlo); free(whi);
+    return SGL_OK;
+}
+
+size_t sglo_sample_khop_workspace_bytes(int64_t S0, int32_t layers, int32_t fanout) {
+    (void)S0; (void)layers; (void)fanout;
+    return 0;
+}
+
+/* k-hop driver.  Reference: sample_src_in_chunks_khop
+ * (sample.cu.hpp:1532-1716): roots = concat(seeds, negatives) (:1545-1547),
+ * next hop roots = neighbors, ts = neighbors_ts, one slot each (:1692-1702). */
+int32_t sglo_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* roots,
+                         const int64_t* ts_ptr, int64_t S_pos,
+                         const int64_t* root_ts, int64_t N_neg,
+                         const int64_t* neg_roots, const int64_t* neg_ts,
+                         int32_t layers, const sgl_sample_params* p,
+                         int64_t* slot_node0, int64_t* slot_ts0,
+                         const sgl_hop_out* outs, void* ws, size_t ws_bytes,
+                         void* stream) {
+    if (!g || !p || !outs || R < 0 || S_pos < 0 || N_neg < 0 || layers < 0)
+        return fail(SGL_EINVAL, "sample_khop: null/negative");
+    for (int64_t r = 0; r < R; ++r) {
+        if (ts_ptr[r] > ts_ptr[r + 1] || ts_ptr[r] < 0 || ts_ptr[r + 1] > S_pos)
+            return fail(SGL_EINVAL, "sample_khop: ts_ptr not a prefix array over root_ts");
+        for (int64_t s = ts_ptr[r]; s < ts_ptr[r + 1]; ++s) {
+            slot_node0[s] = roots[r]; slot_ts0[s] = root_ts[s];
+        }
+    }
+    if (R > 0 && (ts_ptr[0] != 0 || ts_ptr[R] != S_pos))
+        return fail(SGL_EINVAL, "sample_khop: ts_ptr ends");
+    for (int64_t i = 0; i < N_neg; ++i) {
+        slot_node0[S_pos + i] = neg_roots[i]; slot_ts0[S_pos + i] = neg_ts[i];
+    }
+    const int64_t* sn = slot_node0; const int64_t* st = slot_ts0;
+    int64_t S = S_pos + N_neg;
+    for (int32_t l = 0; l < layers; ++l) {
+        sgl_sample_params pl = *p; pl.hop = l;
+        int32_t rc = sglo_sample_hop(g, sn, st, S, NULL, &pl, &outs[l], ws, ws_bytes, stream);
+        if (rc != SGL_OK) return rc;
+        sn = outs[l].neighbors; st = outs[l].neighbors_ts; S = outs[l].counts[1];
+    }
+    return SGL_OK;
+}
+
+/* ----------------------------------------------------- unique / compaction */
+
+/* state layout: int64 header[3] = {epoch, id_count, universe}; then
+ * int64 table[universe] holding the local id of the current epoch or -1. */
+size_t sglo_remap_state_bytes(int64_t universe) {
+    return (size_t)(universe + 3) * sizeof(int64_t);
+}
+
+int32_t sglo_remap_init(void* state, size_t bytes, int64_t universe, void* stream) {
+    (void)stream;
+    if (!state || universe < 0 || bytes < sglo_remap_state_bytes(universe))
+        return fail(SGL_EINVAL, "remap_init: state too small");
+    int64_t* h = (int64_t*)state;
+    h[0] = 1; h[1] = 0; h[2] = universe;
+    for (int64_t i = 0; i < universe; ++i) h[3 + i] = -1;
+    return SGL_OK;
+}
+
+static int i64_cmp(const void* a, const void* b) {
+    int64_t x = *(const int64_t*)a, y = *(const int64_t*)b;
+    return x < y ? -1 : (x > y ? 1 : 0);
+}
+
+typedef struct { int64_t id, local; } seen_rec;
+static int seen_cmp(const void* a, const void* b) {
+    return i64_cmp(&((const seen_rec*)a)->id, &((const seen_rec*)b)->id);
+}
+static int64_t seen_find(const seen_rec* s, int64_t n, int64_t id) {
+    int64_t lo = 0, hi = n;
+    while (lo < hi) { int64_t mid = (lo + hi) >> 1; if (s[mid].id < id) lo = mid + 1; else hi = mid; }
+    return (lo < n && s[lo].id == id) ? s[lo].local : -1;
+}
+
+size_t sglo_unique_workspace_bytes(int64_t universe, int32_t G, const int64_t* len_max) {
+    (void)universe; (void)G; (void)len_max;
+    return 0;
+}
+
+/* unique + compaction.  Reference: Remapper::insert -> remapper per array:
+ * mark ids already mapped in this epoch, copy_if the rest, sort, unique,
+ * number consecutively from id_counts, scatter into id_mapper, patch
+ * (sample.cu.hpp:1764-1852); sorted mode == np.unique(return_inverse=True)
+ * (prepare_sample.py:205-213).  Rule implemented for the epoch flag: reset=1
+ * restarts numbering, reset=0 continues it (the comment at
+ * sample.cu.hpp:1874, and graph.py:291).  Ids that are negative, or outside
+ * the state's universe, map to -1 and are never numbered. */
+int32_t sglo_unique_compact(void* state, int64_t universe_arg, int32_t reset, int32_t mode, int32_t G,
+                            const int64_t* const* ids, const int64_t* len_max,
+                            const int64_t* const* len_dev,
+                            int64_t* const* local_out, int64_t* unique_out,
+                            int64_t unique_capacity, int64_t* U_dev, void* ws,
+                            size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (G < 0 || (G > 0 && (!ids || !len_max || !local_out)) || !U_dev)
+        return fail(SGL_EINVAL, "unique_compact: null");
+    if (mode != SGL_UNIQUE_SORTED && mode != SGL_UNIQUE_GROUPED)
+        return fail(SGL_EINVAL, "unique_compact: bad mode");
+    if (!state && !reset) return fail(SGL_ENOTSUP, "unique_compact: hash path needs reset=1");
+    int64_t* hdr = (int64_t*)state;
+    int64_t* table = state ? hdr + 3 : NULL;
+    const int64_t universe = state ? hdr[2] : INT64_MAX;
+    if (state && universe_arg != hdr[2]) return fail(SGL_EINVAL, "unique_compact: universe differs from remap_init");
+    int64_t total = 0;
+    for (int32_t g = 0; g < G; ++g) {
+        int64_t L = (len_dev && len_dev[g]) ? *len_dev[g] : len_max[g];
+        if (L < 0 || L > len_max[g]) return fail(SGL_EINVAL, "unique_compact: bad length");
+        total += L;
+    }
+    int64_t id_count = 0;
+    if (state) {
+        if (reset) {
+            hdr[0] += 1; hdr[1] = 0;
+            for (int64_t i = 0; i < universe; ++i) table[i] = -1;
+        }
+        id_count = hdr[1];
+    }
+    const int64_t U_before = id_count;
+    /* `seen` = ids numbered by this call, kept sorted by id. */
+    seen_rec* seen = (seen_rec*)malloc((size_t)(total + 1) * sizeof *seen);
+    int64_t n_seen = 0;
+    int64_t* tmp = (int64_t*)malloc((size_t)(total + 1) * sizeof(int64_t));
+    if (!seen || !tmp) { free(seen); free(tmp); return fail(SGL_ENOMEM, "malloc"); }
+    const int32_t n_groups = (mode == SGL_UNIQUE_SORTED) ? 1 : G;
+    for (int32_t grp = 0; grp < n_groups; ++grp) {
+        int64_t nt = 0;
+        for (int32_t g = 0; g < G; ++g) {
+            if (mode == SGL_UNIQUE_GROUPED && g != grp) continue;
+            int64_t L = (len_dev && len_dev[g]) ? *len_dev[g] : len_max[g];
+            for (int64_t i = 0; i < L; ++i) {
+                int64_t id = ids[g][i];
+                if (id < 0 || id >= universe) continue;
+                tmp[nt++] = id;
+            }
+        }
+        qsort(tmp, (size_t)nt, sizeof(int64_t), i64_cmp);
+        const int64_t n_prev = n_seen;
+        for (int64_t i = 0; i < nt; ++i) {
+            if (i > 0 && tmp[i] == tmp[i - 1]) continue;
+            int64_t id = tmp[i];
+            if (state && table[id] >= 0) continue;            /* earlier call, same epoch */
+            if (seen_find(seen, n_prev, id) >= 0) continue;   /* earlier group, this call */
+            if (id_count >= unique_capacity) { free(seen); free(tmp); return fail(SGL_ENOMEM, "unique_out too small"); }
+            seen[n_seen].id = id; seen[n_seen].local = id_count; n_seen++;
+            unique_out[id_count] = id;
+            id_count++;
+        }
+        qsort(seen, (size_t)n_seen, sizeof *seen, seen_cmp);
+    }
+    for (int32_t g = 0; g < G; ++g) {
+        int64_t L = (len_dev && len_dev[g]) ? *len_dev[g] : len_max[g];
+        for (int64_t i = 0; i < L; ++i) {
+            int64_t id = ids[g][i];
+            int64_t loc = -1;
+            if (id >= 0 && id < universe) {
+                loc = seen_find(seen, n_seen, id);
+                if (loc < 0 && state) loc = table[id];
+            }
+            local_out[g][i] = loc;
+        }
+    }
+    if (state) {
+        for (int64_t i = 0; i < n_seen; ++i) table[seen[i].id] = seen[i].local;
+        hdr[1] = id_count;
+    }
+    U_dev[0] = id_count; U_dev[1] = U_before;
+    free(seen); free(tmp);
+    return SGL_OK;
+}
+
+/* ------------------------------------------------------------ cache gather */
+
+static int64_t cache_loc(const sgl_cache* c, int64_t id) {
+    int64_t key = id & c->id_mask;
+    if (id < 0) return -1;
+    if (c->g2l) {
+        if (key < 0 || key >= c->g2l_len) return -1;
+        key = c->g2l[key];
+    }
+    if (key < 0 || key >= c->rows) return -1;
+    return key;
+}
+
+/* Reference: IDMapper.to_local (partition_book.py:106-133) then
+ * data[loc], ts[loc] (NodeState.py:36-44); tensor_gather row copy
+ * (feature.cu.hpp:42-88); DistRouteIndex.loc = id & 0xFFFFFFFFFFFF
+ * (partition_book.py:14-31). */
+int32_t sglo_gather(const sgl_cache* c, const int64_t* ids, int64_t N_max,
+                    const int64_t* N_dev, void* out, int64_t* out_ts,
+                    int64_t* stats, void* stream) {
+    (void)stream;
+    if (!c || N_max < 0 || (N_max > 0 && (!ids || !out))) return fail(SGL_EINVAL, "gather: null");
+    if (c->row_bytes <= 0 || c->row_bytes % 4) return fail(SGL_EINVAL, "gather: row_bytes must be a positive multiple of 4");
+    int64_t N = N_dev ? *N_dev : N_max;
+    if (N > N_max) return fail(SGL_EINVAL, "gather: N > N_max");
+    int64_t hit = 0, cold = 0, absent = 0;
+    for (int64_t i = 0; i < N; ++i) {
+        char* dst = (char*)out + i * c->row_bytes;
+        int64_t loc = cache_loc(c, ids[i]);
+        if (loc < 0) {
+            memset(dst, 0, (size_t)c->row_bytes);
+            if (out_ts) out_ts[i] = 0;
+            absent++;
+            continue;
+        }
+        int64_t slot = c->hot_slot ? (int64_t)c->hot_slot[loc] : loc;
+        if (slot >= 0) {
+            memcpy(dst, (const char*)c->hot + slot * c->row_bytes, (size_t)c->row_bytes);
+            if (out_ts) out_ts[i] = c->ts_hot ? c->ts_hot[slot] : 0;
+            hit++;
+        } else {
+            memcpy(dst, (const char*)c->cold + loc * c->row_bytes, (size_t)c->row_bytes);
+            if (out_ts) out_ts[i] = c->ts_cold ? c->ts_cold[loc] : 0;
+            cold++;
+        }
+    }
+    if (stats) { stats[0] += hit; stats[1] += cold; stats[2] += absent; }
+    return SGL_OK;
+}
+
+/* Reference: DistNodeState.update (NodeState.py:46-61): loc = to_local(gids),
+ * rows with loc >= 0 are overwritten, ts likewise. */
+int32_t sglo_scatter_update(const sgl_cache* c, void* hot_rw, void* cold_rw,
+                            int64_t* ts_hot_rw, int64_t* ts_cold_rw,
+                            const int64_t* ids, int64_t N, const void* values,
+                            const int64_t* ts, void* stream) {
+    (void)stream;
+    if (!c || N < 0 || (N > 0 && (!ids || !values))) return fail(SGL_EINVAL, "scatter_update: null");
+    for (int64_t i = 0; i < N; ++i) {
+        int64_t loc = cache_loc(c, ids[i]);
+        if (loc < 0) continue;
+        int64_t slot = c->hot_slot ? (int64_t)c->hot_slot[loc] : loc;
+        const char* srcp = (const char*)values + i * c->row_bytes;
+        if (slot >= 0) {
+            memcpy((char*)hot_rw + slot * c->row_bytes, srcp, (size_t)c->row_bytes);
+            if (ts && ts_hot_rw) ts_hot_rw[slot] = ts[i];
+        } else {
+            memcpy((char*)cold_rw + loc * c->row_bytes, srcp, (size_t)c->row_bytes);
+            if (ts && ts_cold_rw) ts_cold_rw[loc] = ts[i];
+        }
+    }
+    return SGL_OK;
+}
+
+/* ----------------------------------------------------------- time encoding */
+
+/* Reference: TimeEncoder.forward = cos(Linear(1,dim)(t.float()))
+ * (time_encoder.py:29-31); Linear computes x*W^T + b.  Rule implemented:
+ * x = (float)dt (round to nearest even), a = fl32(fl32(w*x) + b) with a
+ * separately rounded multiply and add, y = (float)cos((double)a). */
+int32_t sglo_time_encode(const void* dt, int32_t dt_dtype, int64_t N_max,
+                         const int64_t* N_dev, const float* w, const float* b,
+                         int32_t dim, float* out, void* stream) {
+    (void)stream;
+    if (N_max < 0 || dim <= 0 || !w || !b || (N_max > 0 && (!dt || !out)))
+        return fail(SGL_EINVAL, "time_encode: null");
+    if (dt_dtype != SGL_DT_I64 && dt_dtype != SGL_DT_F32) return fail(SGL_EINVAL, "time_encode: dtype");
+    int64_t N = N_dev ? *N_dev : N_max;
+    for (int64_t i = 0; i < N; ++i) {
+        volatile float x = dt_dtype == SGL_DT_I64 ? (float)((const int64_t*)dt)[i]
+                                                  : ((const float*)dt)[i];
+        for (int32_t j = 0; j < dim; ++j) {
+            volatile float prod = w[j] * x;
+            volatile float a = prod + b[j];
+            out[i * (int64_t)dim + j] = (float)cos((double)a);
+        }
+    }
+    return SGL_OK;
+}

@@ -1,0 +1,82 @@
+// Shared host/device helpers of libsgl_hot.so (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/sgl_hot.h"
+
+namespace sgl {
+
+constexpr int WAVE = 64;
+
+// ---- status plumbing (thread-local error string, no exceptions) -------------
+char* err_buf();
+constexpr size_t ERR_BUF = 512;
+
+int32_t fail(int32_t code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define SGL_HIP_TRY(expr)                                                              \
+    do {                                                                               \
+        hipError_t e_ = (expr);                                                        \
+        if (e_ != hipSuccess)                                                          \
+            return ::sgl::fail(SGL_EHIP, "%s: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                               __FILE__, __LINE__);                                    \
+    } while (0)
+
+// Launch check: a bad launch configuration is reported by hipGetLastError.
+#define SGL_LAUNCH_CHECK() SGL_HIP_TRY(hipGetLastError())
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+template <typename T>
+__host__ __device__ constexpr T ceil_div(T a, T b) { return (a + b - 1) / b; }
+
+inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
+
+// Bump allocator over a caller-provided workspace.
+struct Arena {
+    char*  base;
+    size_t size, used;
+    Arena(void* p, size_t n) : base(static_cast<char*>(p)), size(n), used(0) {}
+    template <typename T>
+    T* take(size_t count) {
+        size_t off = align_up(used);
+        used = off + count * sizeof(T);
+        return reinterpret_cast<T*>(base + off);
+    }
+    bool ok() const { return base != nullptr && used <= size; }
+};
+
+// ---- device helpers ---------------------------------------------------------
+#if defined(__HIPCC__)
+
+// Ballot restricted to the G-lane group that starts at bit `gshift` of the wave.
+template <int G>
+__device__ __forceinline__ uint64_t group_ballot(bool pred, int gshift) {
+    uint64_t b = __ballot(pred);
+    if constexpr (G == 64) {
+        (void)gshift;
+        return b;
+    } else {
+        return (b >> gshift) & ((1ull << G) - 1ull);
+    }
+}
+
+__device__ __forceinline__ int64_t shfl_i64(int64_t v, int src_lane) {
+    int lo = __shfl(static_cast<int>(v & 0xFFFFFFFFll), src_lane);
+    int hi = __shfl(static_cast<int>(v >> 32), src_lane);
+    return (static_cast<int64_t>(hi) << 32) | static_cast<uint32_t>(lo);
+}
+
+// Live element count of a launch: *n_dev clamped to [0, n_max] when given.
+__device__ __forceinline__ int64_t live_count(const int64_t* n_dev, int64_t n_max) {
+    if (n_dev == nullptr) return n_max;
+    int64_t n = *n_dev;
+    return n < 0 ? 0 : (n > n_max ? n_max : n);
+}
+
+#endif  // __HIPCC__
+
+}  // namespace sgl

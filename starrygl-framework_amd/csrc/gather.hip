@@ -1,0 +1,247 @@
+// Two-tier row gather / scatter through the cache index for gfx950.
+//
+// A block owns RPB consecutive output rows.  Phase 1: one thread per row walks
+// the lookup chain id -> key -> local row -> hot slot once and parks the row's
+// source address in LDS.  Phase 2: all 256 threads stream the block's
+// RPB * row_bytes output bytes as flat, fully coalesced 16-byte chunks (8- or
+// 4-byte chunks when the row size or a base address is not 16-byte aligned),
+// several independent loads in flight per lane.  Hot rows come from HBM, cold
+// rows are read in place from device-visible pinned host memory.
+//
+// Replaces IDMapper.to_local + DistNodeState.__getitem__/update
+// (starrygl/utils/partition_book.py:106-133, starrygl/cache/NodeState.py:36-61)
+// and tensor_gather (csrc/include/starrygl/feature.cu.hpp:42-88).
+#include "common.hpp"
+
+namespace sgl {
+namespace {
+
+constexpr int BLOCK = 256;
+constexpr int UNROLL = 4;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct GatherArgs {
+    sgl_cache c;
+    const int64_t* ids;
+    int64_t N_max;
+    const int64_t* N_dev;
+    char* out;
+    int64_t* out_ts;
+    int64_t* stats;
+    int32_t rpb;  // rows per block
+    int32_t cpr;  // chunks per row
+};
+
+// id -> (source row address, last-update time); nullptr when not resident.
+// tier: 0 hot, 1 cold, 2 absent.
+__device__ __forceinline__ const char* resolve(const sgl_cache& c, int64_t id, int64_t* ts_out,
+                                               int* tier) {
+    *ts_out = 0;
+    *tier = 2;
+    if (id < 0) return nullptr;
+    int64_t key = id & c.id_mask;
+    if (c.g2l != nullptr) {
+        if (key < 0 || key >= c.g2l_len) return nullptr;
+        key = c.g2l[key];
+    }
+    if (key < 0 || key >= c.rows) return nullptr;
+    const int64_t slot = c.hot_slot != nullptr ? (int64_t)c.hot_slot[key] : key;
+    if (slot >= 0) {
+        *tier = 0;
+        if (c.ts_hot != nullptr) *ts_out = c.ts_hot[slot];
+        return static_cast<const char*>(c.hot) + slot * c.row_bytes;
+    }
+    *tier = 1;
+    if (c.ts_cold != nullptr) *ts_out = c.ts_cold[key];
+    return static_cast<const char*>(c.cold) + key * c.row_bytes;
+}
+
+template <typename V>
+__global__ __launch_bounds__(BLOCK) void gather_kernel(GatherArgs a) {
+    extern __shared__ const char* s_src[];  // [rpb]
+    __shared__ int32_t s_tier[3];
+    const int64_t N = live_count(a.N_dev, a.N_max);
+    const int64_t row0 = (int64_t)blockIdx.x * a.rpb;
+    if (row0 >= N) return;
+    const int32_t rows = (int32_t)((N - row0) < a.rpb ? (N - row0) : a.rpb);
+    if (threadIdx.x < 3) s_tier[threadIdx.x] = 0;
+    __syncthreads();
+    for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
+        int64_t ts;
+        int tier;
+        s_src[r] = resolve(a.c, a.ids[row0 + r], &ts, &tier);
+        if (a.out_ts != nullptr) a.out_ts[row0 + r] = ts;
+        if (a.stats != nullptr) atomicAdd(&s_tier[tier], 1);
+    }
+    __syncthreads();
+    const int32_t cpr = a.cpr;
+    const int32_t total = rows * cpr;
+    V* __restrict__ dst = reinterpret_cast<V*>(a.out + row0 * a.c.row_bytes);
+    for (int32_t base = 0; base < total; base += BLOCK * UNROLL) {
+        V val[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int32_t lc = base + u * BLOCK + threadIdx.x;
+            V v = {};
+            if (lc < total) {
+                const int32_t r = lc / cpr;
+                const int32_t part = lc - r * cpr;
+                const V* src = reinterpret_cast<const V*>(s_src[r]);
+                if (src != nullptr) v = src[part];
+            }
+            val[u] = v;
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int32_t lc = base + u * BLOCK + threadIdx.x;
+            if (lc < total) dst[lc] = val[u];
+        }
+    }
+    if (a.stats != nullptr && threadIdx.x < 3 && s_tier[threadIdx.x] != 0)
+        atomicAdd(reinterpret_cast<unsigned long long*>(a.stats + threadIdx.x),
+                  (unsigned long long)s_tier[threadIdx.x]);
+}
+
+struct ScatterArgs {
+    sgl_cache c;
+    char* hot_rw;
+    char* cold_rw;
+    int64_t* ts_hot_rw;
+    int64_t* ts_cold_rw;
+    const int64_t* ids;
+    int64_t N;
+    const char* values;
+    const int64_t* ts;
+    int32_t rpb, cpr;
+};
+
+template <typename V>
+__global__ __launch_bounds__(BLOCK) void scatter_kernel(ScatterArgs a) {
+    extern __shared__ char* s_dst[];
+    const int64_t row0 = (int64_t)blockIdx.x * a.rpb;
+    if (row0 >= a.N) return;
+    const int32_t rows = (int32_t)((a.N - row0) < a.rpb ? (a.N - row0) : a.rpb);
+    for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
+        int64_t ts_unused;
+        int tier;
+        const char* p = resolve(a.c, a.ids[row0 + r], &ts_unused, &tier);
+        char* d = nullptr;
+        if (tier == 0) {
+            const int64_t slot = (p - static_cast<const char*>(a.c.hot)) / a.c.row_bytes;
+            d = a.hot_rw + slot * a.c.row_bytes;
+            if (a.ts != nullptr && a.ts_hot_rw != nullptr) a.ts_hot_rw[slot] = a.ts[row0 + r];
+        } else if (tier == 1) {
+            const int64_t loc = (p - static_cast<const char*>(a.c.cold)) / a.c.row_bytes;
+            d = a.cold_rw + loc * a.c.row_bytes;
+            if (a.ts != nullptr && a.ts_cold_rw != nullptr) a.ts_cold_rw[loc] = a.ts[row0 + r];
+        }
+        s_dst[r] = d;
+    }
+    __syncthreads();
+    const int32_t cpr = a.cpr;
+    const int32_t total = rows * cpr;
+    const V* __restrict__ src = reinterpret_cast<const V*>(a.values + row0 * a.c.row_bytes);
+    for (int32_t lc = threadIdx.x; lc < total; lc += BLOCK) {
+        const int32_t r = lc / cpr;
+        const int32_t part = lc - r * cpr;
+        V* d = reinterpret_cast<V*>(s_dst[r]);
+        if (d != nullptr) d[part] = src[lc];
+    }
+}
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+int32_t check_cache(const sgl_cache* c) {
+    if (!c) return fail(SGL_EINVAL, "cache is NULL");
+    if (c->rows < 0 || c->hot_rows < 0 || c->g2l_len < 0) return fail(SGL_EINVAL, "cache: negative size");
+    if (c->row_bytes <= 0 || c->row_bytes % 4 != 0)
+        return fail(SGL_EINVAL, "cache: row_bytes %lld must be a positive multiple of 4", (long long)c->row_bytes);
+    if (c->row_bytes > (1 << 20)) return fail(SGL_ENOTSUP, "cache: row_bytes > 1 MiB");
+    if (c->hot_slot == nullptr && c->hot == nullptr && c->rows > 0)
+        return fail(SGL_EINVAL, "cache: hot table is NULL while hot_slot is NULL");
+    if (c->hot_slot == nullptr && c->rows > c->hot_rows)
+        return fail(SGL_EINVAL, "cache: without hot_slot every logical row must be a hot row");
+    if (c->hot_slot != nullptr && c->cold == nullptr && c->rows > 0)
+        return fail(SGL_EINVAL, "cache: hot_slot given but cold table is NULL");
+    return SGL_OK;
+}
+
+// widest chunk every involved address / the row size allows
+int pick_vec(int64_t row_bytes, std::initializer_list<const void*> ptrs) {
+    int v = 16;
+    if (row_bytes % 16) v = (row_bytes % 8) ? 4 : 8;
+    for (const void* p : ptrs) {
+        if (!p) continue;
+        while (v > 4 && !aligned(p, v)) v >>= 1;
+    }
+    return v;
+}
+
+}  // namespace
+}  // namespace sgl
+
+using namespace sgl;
+
+extern "C" int32_t sgl_gather(const sgl_cache* c, const int64_t* ids, int64_t N_max,
+                              const int64_t* N_dev, void* out, int64_t* out_ts, int64_t* stats,
+                              void* stream) {
+    int32_t rc;
+    if ((rc = check_cache(c)) != SGL_OK) return rc;
+    if (N_max < 0) return fail(SGL_EINVAL, "gather: N_max < 0");
+    if (N_max == 0) return SGL_OK;
+    if (!ids || !out) return fail(SGL_EINVAL, "gather: ids/out is NULL");
+    const int vec = pick_vec(c->row_bytes, {c->hot, c->cold, out});
+    GatherArgs a;
+    a.c = *c; a.ids = ids; a.N_max = N_max; a.N_dev = N_dev;
+    a.out = static_cast<char*>(out); a.out_ts = out_ts; a.stats = stats;
+    a.cpr = (int32_t)(c->row_bytes / vec);
+    // about BLOCK*UNROLL chunks per block, at least one row, at most 1024 rows
+    int64_t rpb = (int64_t)BLOCK * UNROLL / a.cpr;
+    rpb = rpb < 1 ? 1 : (rpb > 1024 ? 1024 : rpb);
+    a.rpb = (int32_t)rpb;
+    const int64_t blocks = ceil_div<int64_t>(N_max, rpb);
+    if (blocks > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "gather: too many rows for one launch");
+    const size_t shmem = (size_t)rpb * sizeof(char*);
+    hipStream_t st = as_stream(stream);
+    switch (vec) {
+        case 16: hipLaunchKernelGGL(gather_kernel<u32x4>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
+        case 8: hipLaunchKernelGGL(gather_kernel<u32x2>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
+        default: hipLaunchKernelGGL(gather_kernel<uint32_t>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
+    }
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}
+
+extern "C" int32_t sgl_scatter_update(const sgl_cache* c, void* hot_rw, void* cold_rw,
+                                      int64_t* ts_hot_rw, int64_t* ts_cold_rw, const int64_t* ids,
+                                      int64_t N, const void* values, const int64_t* ts, void* stream) {
+    int32_t rc;
+    if ((rc = check_cache(c)) != SGL_OK) return rc;
+    if (N < 0) return fail(SGL_EINVAL, "scatter_update: N < 0");
+    if (N == 0) return SGL_OK;
+    if (!ids || !values) return fail(SGL_EINVAL, "scatter_update: ids/values is NULL");
+    if (c->hot != nullptr && hot_rw == nullptr) return fail(SGL_EINVAL, "scatter_update: hot_rw is NULL");
+    if (c->hot_slot != nullptr && cold_rw == nullptr) return fail(SGL_EINVAL, "scatter_update: cold_rw is NULL");
+    const int vec = pick_vec(c->row_bytes, {hot_rw, cold_rw, values});
+    ScatterArgs a;
+    a.c = *c; a.hot_rw = static_cast<char*>(hot_rw); a.cold_rw = static_cast<char*>(cold_rw);
+    a.ts_hot_rw = ts_hot_rw; a.ts_cold_rw = ts_cold_rw; a.ids = ids; a.N = N;
+    a.values = static_cast<const char*>(values); a.ts = ts;
+    a.cpr = (int32_t)(c->row_bytes / vec);
+    int64_t rpb = (int64_t)BLOCK * UNROLL / a.cpr;
+    rpb = rpb < 1 ? 1 : (rpb > 1024 ? 1024 : rpb);
+    a.rpb = (int32_t)rpb;
+    const int64_t blocks = ceil_div<int64_t>(N, rpb);
+    if (blocks > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "scatter_update: too many rows for one launch");
+    const size_t shmem = (size_t)rpb * sizeof(char*);
+    hipStream_t st = as_stream(stream);
+    switch (vec) {
+        case 16: hipLaunchKernelGGL(scatter_kernel<u32x4>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
+        case 8: hipLaunchKernelGGL(scatter_kernel<u32x2>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
+        default: hipLaunchKernelGGL(scatter_kernel<uint32_t>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
+    }
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}

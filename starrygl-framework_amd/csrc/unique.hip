@@ -1,0 +1,334 @@
+// Unique + compaction of sampled node ids to dense local ids for gfx950.
+//
+// Dense-universe path (ids in [0, universe), `state` given):
+//   the persistent state holds a 64-bit table entry per id
+//   (epoch << 32 | local id) and a bitmap of universe bits.  Per group
+//     mark   : ids whose table entry is not of the current epoch set their bit
+//              (atomicOr), duplicates collapse for free;
+//     reduce : per-tile popcount sums;   scan: one block scans the tile sums;
+//     assign : every set bit gets local id = base + rank of the bit, which is
+//              the ascending-id order the reference obtains by sort + unique;
+//              the entry, the local->global list and the cleared word are
+//              written in the same pass;
+//   then one lookup launch rewrites every input array through the table.
+//   No sort, no hash probing; the result is deterministic.
+//
+// Replaces Remapper::remapper / insert, mark_new_ids_kernel and
+// update_new_ids_kernel (csrc/include/starrygl/sample.cu.hpp:1719-1854).
+#include "common.hpp"
+
+namespace sgl {
+
+// hash-set path, defined in unique_hash.hip
+size_t hash_unique_workspace_bytes(int32_t G, const int64_t* len_max);
+int32_t hash_unique_compact(int32_t mode, int32_t G, const int64_t* const* ids, const int64_t* len_max,
+                            const int64_t* const* len_dev, int64_t* const* local_out,
+                            int64_t* unique_out, int64_t unique_capacity, int64_t* U_dev, void* ws,
+                            size_t ws_bytes, hipStream_t st);
+
+namespace {
+
+constexpr int BLOCK = 256;
+constexpr int MAXG = 8;
+constexpr int WPT = 8;                 // bitmap words per thread in reduce/assign
+constexpr int TILE = BLOCK * WPT;      // words per block
+constexpr int SCAN_BLOCK = 1024;
+constexpr size_t HEADER_BYTES = 256;
+
+struct Header {
+    uint64_t epoch;     // current epoch (low 32 bits are stamped into the table)
+    int64_t id_count;   // local ids handed out in this epoch
+    int64_t base;       // first local id of the group being numbered
+};
+
+struct State {
+    Header* hdr;
+    uint64_t* table;
+    uint64_t* bitmap;
+    int64_t universe, words;
+};
+
+State carve(void* state, int64_t universe) {
+    State s;
+    char* p = static_cast<char*>(state);
+    s.universe = universe;
+    s.words = ceil_div<int64_t>(universe, 64);
+    s.hdr = reinterpret_cast<Header*>(p);
+    s.table = reinterpret_cast<uint64_t*>(p + HEADER_BYTES);
+    s.bitmap = s.table + universe;
+    return s;
+}
+
+struct Arrays {
+    int32_t G;
+    const int64_t* ids[MAXG];
+    int64_t* out[MAXG];
+    const int64_t* len_dev[MAXG];
+    int64_t len_max[MAXG];
+    int64_t start[MAXG + 1];  // flat index space over len_max
+};
+
+__device__ __forceinline__ bool locate(const Arrays& a, int64_t t, int* g_out, int64_t* i_out) {
+    if (t >= a.start[a.G]) return false;
+    int g = 0;
+#pragma unroll
+    for (int q = 1; q < MAXG; ++q)
+        if (q < a.G && t >= a.start[q]) g = q;
+    const int64_t i = t - a.start[g];
+    if (i >= live_count(a.len_dev[g], a.len_max[g])) return false;
+    *g_out = g;
+    *i_out = i;
+    return true;
+}
+
+__global__ void init_state_kernel(State s) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = t; i < s.universe; i += stride) s.table[i] = 0;
+    for (int64_t i = t; i < s.words; i += stride) s.bitmap[i] = 0;
+    if (t == 0) {
+        s.hdr->epoch = 1;
+        s.hdr->id_count = 0;
+        s.hdr->base = 0;
+    }
+}
+
+__global__ void begin_kernel(State s, int reset, int64_t* U_dev) {
+    if (reset) {
+        uint64_t e = s.hdr->epoch + 1;
+        if ((e & 0xFFFFFFFFull) == 0) e += 1;  // stamp 0 means "never mapped"
+        s.hdr->epoch = e;
+        s.hdr->id_count = 0;
+    }
+    U_dev[1] = s.hdr->id_count;
+}
+
+__global__ __launch_bounds__(BLOCK) void mark_kernel(State s, Arrays a) {
+    const int64_t t = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    int g;
+    int64_t i;
+    if (!locate(a, t, &g, &i)) return;
+    const int64_t id = a.ids[g][i];
+    if (id < 0 || id >= s.universe) return;
+    const uint32_t stamp = (uint32_t)(s.hdr->epoch & 0xFFFFFFFFull);
+    if ((uint32_t)(s.table[id] >> 32) == stamp) return;  // numbered earlier in this epoch
+    const uint64_t bit = 1ull << (id & 63);
+    // skip the atomic when the bit is already visible
+    if ((__atomic_load_n(&s.bitmap[id >> 6], __ATOMIC_RELAXED) & bit) == 0)
+        atomicOr(reinterpret_cast<unsigned long long*>(&s.bitmap[id >> 6]), (unsigned long long)bit);
+}
+
+__global__ __launch_bounds__(BLOCK) void reduce_kernel(State s, int64_t* tile_sum) {
+    __shared__ int32_t s_w[BLOCK / WAVE];
+    const int64_t w0 = (int64_t)blockIdx.x * TILE + (int64_t)threadIdx.x * WPT;
+    int32_t c = 0;
+#pragma unroll
+    for (int q = 0; q < WPT; ++q)
+        if (w0 + q < s.words) c += __popcll(s.bitmap[w0 + q]);
+    // wave reduction, then 4 partials
+    for (int d = WAVE / 2; d > 0; d >>= 1) c += __shfl_down(c, d);
+    if (threadIdx.x % WAVE == 0) s_w[threadIdx.x / WAVE] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int64_t sum = 0;
+        for (int q = 0; q < BLOCK / WAVE; ++q) sum += s_w[q];
+        tile_sum[blockIdx.x] = sum;
+    }
+}
+
+// exclusive scan of `nt` tile sums in place; advances id_count
+__global__ __launch_bounds__(SCAN_BLOCK) void scan_tiles_kernel(State s, int64_t* tile_sum, int64_t nt) {
+    __shared__ int64_t s_part[SCAN_BLOCK];
+    const int64_t per = ceil_div<int64_t>(nt, SCAN_BLOCK);
+    const int64_t b0 = (int64_t)threadIdx.x * per;
+    const int64_t b1 = b0 + per < nt ? b0 + per : nt;
+    int64_t sum = 0;
+    for (int64_t b = b0; b < b1; ++b) sum += tile_sum[b];
+    s_part[threadIdx.x] = sum;
+    __syncthreads();
+    for (int d = 1; d < SCAN_BLOCK; d <<= 1) {
+        int64_t x = 0;
+        if ((int)threadIdx.x >= d) x = s_part[threadIdx.x - d];
+        __syncthreads();
+        s_part[threadIdx.x] += x;
+        __syncthreads();
+    }
+    int64_t run = s_part[threadIdx.x] - sum;
+    for (int64_t b = b0; b < b1; ++b) {
+        const int64_t x = tile_sum[b];
+        tile_sum[b] = run;
+        run += x;
+    }
+    if (threadIdx.x == SCAN_BLOCK - 1) {
+        s.hdr->base = s.hdr->id_count;
+        s.hdr->id_count += s_part[SCAN_BLOCK - 1];
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* tile_off,
+                                                       int64_t* unique_out, int64_t unique_capacity) {
+    __shared__ int32_t s_wave[BLOCK / WAVE];
+    const int64_t w0 = (int64_t)blockIdx.x * TILE + (int64_t)threadIdx.x * WPT;
+    uint64_t word[WPT];
+    int32_t c = 0;
+#pragma unroll
+    for (int q = 0; q < WPT; ++q) {
+        word[q] = (w0 + q < s.words) ? s.bitmap[w0 + q] : 0ull;
+        c += __popcll(word[q]);
+    }
+    // exclusive prefix of c inside the block: wave scan + 4 wave totals
+    int32_t inc = c;
+    const int lane = threadIdx.x % WAVE;
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const int32_t x = __shfl_up(inc, d);
+        if (lane >= d) inc += x;
+    }
+    if (lane == WAVE - 1) s_wave[threadIdx.x / WAVE] = inc;
+    __syncthreads();
+    int32_t wave_off = 0;
+    for (int q = 0; q < (int)(threadIdx.x / WAVE); ++q) wave_off += s_wave[q];
+    if (c == 0) return;
+    int64_t local = s.hdr->base + tile_off[blockIdx.x] + wave_off + (inc - c);
+    const uint64_t stamp = (s.hdr->epoch & 0xFFFFFFFFull) << 32;
+#pragma unroll
+    for (int q = 0; q < WPT; ++q) {
+        uint64_t w = word[q];
+        if (w == 0) continue;
+        const int64_t id0 = (w0 + q) * 64;
+        while (w) {
+            const int bit = __ffsll((unsigned long long)w) - 1;
+            w &= w - 1;
+            const int64_t id = id0 + bit;
+            s.table[id] = stamp | (uint64_t)(uint32_t)local;
+            if (local < unique_capacity) unique_out[local] = id;
+            ++local;
+        }
+        s.bitmap[w0 + q] = 0;
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a) {
+    const int64_t t = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    int g;
+    int64_t i;
+    if (!locate(a, t, &g, &i)) return;
+    const int64_t id = a.ids[g][i];
+    int64_t local = -1;
+    if (id >= 0 && id < s.universe) {
+        const uint64_t e = s.table[id];
+        if ((uint32_t)(e >> 32) == (uint32_t)(s.hdr->epoch & 0xFFFFFFFFull)) local = (int64_t)(e & 0xFFFFFFFFull);
+    }
+    a.out[g][i] = local;
+}
+
+__global__ void end_kernel(State s, int64_t* U_dev) { U_dev[0] = s.hdr->id_count; }
+
+size_t dense_workspace_bytes(int64_t universe) {
+    const int64_t words = ceil_div<int64_t>(universe, 64);
+    return align_up((size_t)(ceil_div<int64_t>(words, TILE) + 1) * 8) + 256;
+}
+
+}  // namespace
+}  // namespace sgl
+
+using namespace sgl;
+
+extern "C" size_t sgl_remap_state_bytes(int64_t universe) {
+    if (universe < 0) return 0;
+    return HEADER_BYTES + (size_t)universe * 8 + (size_t)ceil_div<int64_t>(universe, 64) * 8 + 8;
+}
+
+extern "C" int32_t sgl_remap_init(void* state, size_t state_bytes, int64_t universe, void* stream) {
+    if (!state || universe < 0) return fail(SGL_EINVAL, "remap_init: state is NULL or universe < 0");
+    if (universe > 0xFFFFFFFFll) return fail(SGL_ENOTSUP, "remap_init: universe > 2^32");
+    if (state_bytes < sgl_remap_state_bytes(universe))
+        return fail(SGL_ENOMEM, "remap_init: state %zu < %zu bytes", state_bytes, sgl_remap_state_bytes(universe));
+    if (reinterpret_cast<uintptr_t>(state) % 8) return fail(SGL_EINVAL, "remap_init: state must be 8-byte aligned");
+    State s = carve(state, universe);
+    int64_t blocks = ceil_div<int64_t>(universe > 0 ? universe : 1, 256);
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(init_state_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), s);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}
+
+extern "C" size_t sgl_unique_workspace_bytes(int64_t universe, int32_t G, const int64_t* len_max) {
+    if (universe > 0) return dense_workspace_bytes(universe);
+    return hash_unique_workspace_bytes(G, len_max);
+}
+
+extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t reset, int32_t mode,
+                                      int32_t G, const int64_t* const* ids, const int64_t* len_max,
+                                      const int64_t* const* len_dev, int64_t* const* local_out,
+                                      int64_t* unique_out, int64_t unique_capacity, int64_t* U_dev,
+                                      void* ws, size_t ws_bytes, void* stream) {
+    if (G < 0 || (G > 0 && (!ids || !len_max || !local_out)) || !U_dev)
+        return fail(SGL_EINVAL, "unique_compact: NULL argument");
+    if (mode != SGL_UNIQUE_SORTED && mode != SGL_UNIQUE_GROUPED) return fail(SGL_EINVAL, "unique_compact: bad mode");
+    if (G > MAXG) return fail(SGL_ENOTSUP, "unique_compact: more than %d arrays", MAXG);
+    if (unique_capacity < 0 || (unique_capacity > 0 && !unique_out))
+        return fail(SGL_EINVAL, "unique_compact: unique_out is NULL");
+    for (int32_t g = 0; g < G; ++g) {
+        if (len_max[g] < 0) return fail(SGL_EINVAL, "unique_compact: negative length");
+        if (len_max[g] > 0 && (!ids[g] || !local_out[g])) return fail(SGL_EINVAL, "unique_compact: array %d is NULL", g);
+    }
+    hipStream_t st = as_stream(stream);
+    if (!state) {
+        if (!reset) return fail(SGL_ENOTSUP, "unique_compact: hash path needs reset=1");
+        return hash_unique_compact(mode, G, ids, len_max, len_dev, local_out, unique_out, unique_capacity,
+                                   U_dev, ws, ws_bytes, st);
+    }
+    if (universe < 0 || universe > 0xFFFFFFFFll) return fail(SGL_EINVAL, "unique_compact: bad universe");
+    if (!ws || ws_bytes < dense_workspace_bytes(universe))
+        return fail(SGL_ENOMEM, "unique_compact: workspace %zu < %zu bytes", ws_bytes, dense_workspace_bytes(universe));
+    State s = carve(state, universe);
+    Arena ar(ws, ws_bytes);
+    const int64_t nt = ceil_div<int64_t>(s.words, TILE);
+    int64_t* tile_sum = ar.take<int64_t>(nt + 1);
+
+    Arrays all;
+    all.G = G;
+    all.start[0] = 0;
+    for (int g = 0; g < MAXG; ++g) {
+        const bool live = g < G;
+        all.ids[g] = live ? ids[g] : nullptr;
+        all.out[g] = live ? local_out[g] : nullptr;
+        all.len_dev[g] = (live && len_dev) ? len_dev[g] : nullptr;
+        all.len_max[g] = live ? len_max[g] : 0;
+        all.start[g + 1] = all.start[g] + all.len_max[g];
+    }
+    const int64_t total = all.start[MAXG];
+    if (ceil_div<int64_t>(total, BLOCK) > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "unique_compact: too many ids");
+
+    hipLaunchKernelGGL(begin_kernel, dim3(1), dim3(1), 0, st, s, reset, U_dev);
+    SGL_LAUNCH_CHECK();
+    const int n_groups = (mode == SGL_UNIQUE_SORTED) ? (G > 0 ? 1 : 0) : G;
+    for (int grp = 0; grp < n_groups; ++grp) {
+        Arrays sub = all;
+        if (mode == SGL_UNIQUE_GROUPED) {  // only array `grp`
+            sub.G = 1;
+            sub.ids[0] = all.ids[grp]; sub.out[0] = all.out[grp];
+            sub.len_dev[0] = all.len_dev[grp]; sub.len_max[0] = all.len_max[grp];
+            sub.start[0] = 0;
+            for (int g = 1; g <= MAXG; ++g) sub.start[g] = sub.len_max[0];
+        }
+        const int64_t sub_total = sub.start[sub.G];
+        if (sub_total == 0 || universe == 0) continue;
+        hipLaunchKernelGGL(mark_kernel, dim3((unsigned)ceil_div<int64_t>(sub_total, BLOCK)), dim3(BLOCK), 0, st, s, sub);
+        SGL_LAUNCH_CHECK();
+        hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
+        SGL_LAUNCH_CHECK();
+        hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, s, tile_sum, nt);
+        SGL_LAUNCH_CHECK();
+        hipLaunchKernelGGL(assign_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, unique_out,
+                           unique_capacity);
+        SGL_LAUNCH_CHECK();
+    }
+    if (total > 0) {
+        hipLaunchKernelGGL(lookup_kernel, dim3((unsigned)ceil_div<int64_t>(total, BLOCK)), dim3(BLOCK), 0, st, s, all);
+        SGL_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(end_kernel, dim3(1), dim3(1), 0, st, s, U_dev);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}

@@ -1,0 +1,104 @@
+"""ctypes view of include/sgl_hot.h: structs, constants and prototypes.
+
+`bind(cdll, prefix)` attaches argument/return types to every entry point the
+header declares.  The product library exports them as ``sgl_*``.
+"""
+import ctypes as C
+
+ABI_VERSION = 1
+
+SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
+SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
+UNIFORM_MAX_FANOUT = 64
+UNIQUE_SORTED, UNIQUE_GROUPED = 0, 1
+DT_I64, DT_F32 = 0, 1
+
+SAMPLE_TYPES = {"recent": SAMPLE_RECENT, "uniform": SAMPLE_UNIFORM}
+
+i32, i64, u64, vp, sz = C.c_int32, C.c_int64, C.c_uint64, C.c_void_p, C.c_size_t
+
+
+class TCSR(C.Structure):
+    _fields_ = [("n", i64), ("m", i64), ("row_ptr", vp), ("col", vp), ("ts", vp), ("eid", vp)]
+
+
+class SampleParams(C.Structure):
+    _fields_ = [("type", i32), ("fanout", i32), ("allowed_offset", i64),
+                ("equal_root_time", i32), ("keep_root_time", i32),
+                ("replace", i32), ("hop", i32), ("seed", u64)]
+
+
+class HopOut(C.Structure):
+    _fields_ = [("capacity_slots", i64), ("capacity_edges", i64),
+                ("root_start_ptr", vp), ("root_end_ptr", vp),
+                ("neighbors", vp), ("neighbors_ts", vp),
+                ("neighbors_eid", vp), ("neighbors_dt", vp), ("counts", vp)]
+
+
+class Cache(C.Structure):
+    _fields_ = [("rows", i64), ("row_bytes", i64), ("id_mask", i64),
+                ("g2l", vp), ("g2l_len", i64), ("hot_slot", vp),
+                ("hot", vp), ("hot_rows", i64), ("cold", vp),
+                ("ts_hot", vp), ("ts_cold", vp)]
+
+
+P = C.POINTER
+
+# name -> (restype, argtypes); the order follows include/sgl_hot.h
+PROTOTYPES = {
+    "last_error_string": (C.c_char_p, []),
+    "abi_version": (i32, []),
+    "tcsr_build_workspace_bytes": (sz, [i64, i64]),
+    "tcsr_build": (i32, [i64, i64, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]),
+    "tcsr_validate": (i32, [P(TCSR), vp, sz, vp]),
+    "sample_hop_workspace_bytes": (sz, [i64]),
+    "sample_hop": (i32, [P(TCSR), vp, vp, i64, vp, P(SampleParams), P(HopOut), vp, sz, vp]),
+    "sample_khop_workspace_bytes": (sz, [i64, i32, i32]),
+    "sample_khop": (i32, [P(TCSR), i64, vp, vp, i64, vp, i64, vp, vp, i32,
+                          P(SampleParams), vp, vp, P(HopOut), vp, sz, vp]),
+    "remap_state_bytes": (sz, [i64]),
+    "remap_init": (i32, [vp, sz, i64, vp]),
+    "unique_workspace_bytes": (sz, [i64, i32, P(i64)]),
+    "unique_compact": (i32, [vp, i64, i32, i32, i32, P(vp), P(i64), P(vp), P(vp),
+                             vp, i64, vp, vp, sz, vp]),
+    "gather": (i32, [P(Cache), vp, i64, vp, vp, vp, vp, vp]),
+    "scatter_update": (i32, [P(Cache), vp, vp, vp, vp, vp, i64, vp, vp, vp]),
+    "time_encode": (i32, [vp, i32, i64, vp, vp, vp, i32, vp, vp]),
+}
+
+
+class BoundLib:
+    """Entry points of one shared library, addressed without their prefix."""
+
+    def __init__(self, cdll, prefix):
+        self._cdll, self._prefix = cdll, prefix
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(cdll, prefix + name)  # AttributeError if a symbol is missing
+            fn.restype, fn.argtypes = res, args
+            setattr(self, name, fn)
+
+    def error(self):
+        msg = self.last_error_string()
+        return msg.decode() if msg else ""
+
+
+def bind(cdll, prefix="sgl_"):
+    return BoundLib(cdll, prefix)
+
+
+class SglError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"sgl status {code}: {msg}")
+        self.code = code
+
+
+_EXC = {SGL_EINVAL: ValueError, SGL_ERANGE: IndexError, SGL_ENOTSUP: RuntimeError,
+        SGL_EHIP: RuntimeError, SGL_ENOMEM: MemoryError}
+
+
+def check(lib, rc):
+    """Map a status code to the exception the reference raised for the same
+    condition (RuntimeError from C++ exceptions / TORCH_CHECK, export.cu:237-244)."""
+    if rc == SGL_OK:
+        return
+    raise _EXC.get(rc, SglError)(f"sgl status {rc}: {lib.error()}")

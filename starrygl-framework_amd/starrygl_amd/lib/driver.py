@@ -1,0 +1,267 @@
+"""Array-level driver of the C ABI in include/sgl_hot.h.
+
+`HotPath(lib, backend)` marshals arrays into the structs of the ABI, sizes the
+outputs and the workspace, and narrows ragged results.  The backend decides
+where arrays live: `TorchBackend` (device tensors, current HIP stream) is what
+the package uses; anything else that offers the same five methods can drive a
+library with the same ABI on host memory.
+"""
+import ctypes as C
+
+from . import _abi
+from ._abi import (TCSR, Cache, HopOut, SampleParams, check, i64, vp)
+
+
+class TorchBackend:
+    """Device memory and stream plumbing through PyTorch-ROCm."""
+
+    def __init__(self, device):
+        import torch
+        self.torch = torch
+        self.device = torch.device(device)
+        self._dt = {"i64": torch.int64, "i32": torch.int32, "f32": torch.float32,
+                    "u8": torch.uint8, "bf16": torch.bfloat16, "f16": torch.float16}
+
+    def empty(self, shape, dtype="i64"):
+        return self.torch.empty(shape, dtype=self._dt[dtype], device=self.device)
+
+    def zeros(self, shape, dtype="i64"):
+        return self.torch.zeros(shape, dtype=self._dt[dtype], device=self.device)
+
+    def asarray(self, a, dtype="i64"):
+        t = self.torch.as_tensor(a, dtype=self._dt[dtype])
+        return t.to(self.device).contiguous()
+
+    def ptr(self, a):
+        return None if a is None else a.data_ptr()
+
+    def stream(self):
+        if self.device.type != "cuda":
+            return None
+        return self.torch.cuda.current_stream(self.device).cuda_stream
+
+    def tolist(self, a):
+        return a.cpu().tolist()
+
+    def nbytes(self, a):
+        return a.numel() * a.element_size()
+
+    def check(self, a, dtype, name):
+        if a.dtype != self._dt[dtype]:
+            raise TypeError(f"{name} must be {dtype}, got {a.dtype}")
+        if a.device != self.device and not (a.device.type == "cpu" and a.is_pinned()):
+            raise ValueError(f"{name} must live on {self.device}, got {a.device}")
+        if not a.is_contiguous():
+            raise ValueError(f"{name} must be contiguous")
+        return a
+
+
+class TCSRArrays:
+    """Owner of the four T-CSR arrays plus the ABI view of them."""
+
+    def __init__(self, backend, n, row_ptr, col, ts, eid):
+        self.n, self.m = int(n), int(col.shape[0])
+        self.row_ptr, self.col, self.ts, self.eid = row_ptr, col, ts, eid
+        self.view = TCSR(self.n, self.m, backend.ptr(row_ptr), backend.ptr(col),
+                         backend.ptr(ts), backend.ptr(eid))
+
+
+class HopResult:
+    """One hop's ragged output.  Arrays are over-allocated to the worst case;
+    `finalize(S, E)` narrows them once the device counts are known."""
+
+    FIELDS = ("neighbors", "neighbors_ts", "neighbors_eid", "neighbors_dt")
+
+    def __init__(self, backend, cap_slots, cap_edges, counts=None):
+        self.cap_slots, self.cap_edges = cap_slots, cap_edges
+        self.root_start_ptr = backend.empty(cap_slots + 1)
+        self.root_end_ptr = backend.empty(cap_slots + 1)
+        for f in self.FIELDS:
+            setattr(self, f, backend.empty(cap_edges))
+        self.counts = backend.zeros(3) if counts is None else counts
+        self.struct = HopOut(cap_slots, cap_edges, backend.ptr(self.root_start_ptr),
+                             backend.ptr(self.root_end_ptr), backend.ptr(self.neighbors),
+                             backend.ptr(self.neighbors_ts), backend.ptr(self.neighbors_eid),
+                             backend.ptr(self.neighbors_dt), backend.ptr(self.counts))
+        self.S = self.E = None
+
+    def finalize(self, S, E, bad=0):
+        if bad:
+            raise IndexError(f"sgl status {_abi.SGL_ERANGE}: {bad} sampling slots name a node outside [0,n)")
+        self.S, self.E = int(S), int(E)
+        self.root_start_ptr = self.root_start_ptr[: self.S + 1]
+        self.root_end_ptr = self.root_end_ptr[: self.S + 1]
+        for f in self.FIELDS:
+            setattr(self, f, getattr(self, f)[: self.E])
+        return self
+
+
+class HotPath:
+    def __init__(self, lib, backend):
+        self.lib, self.be = lib, backend
+        if lib.abi_version() != _abi.ABI_VERSION:
+            raise RuntimeError("sgl ABI version mismatch")
+        self._ws = None
+
+    # ------------------------------------------------------------ helpers
+    def _workspace(self, nbytes):
+        nbytes = max(int(nbytes), 256)
+        if self._ws is None or self.be.nbytes(self._ws) < nbytes:
+            self._ws = self.be.empty(nbytes, "u8")
+        return self._ws, self.be.nbytes(self._ws)
+
+    def _ck(self, rc):
+        check(self.lib, rc)
+
+    # -------------------------------------------------------------- T-CSR
+    def tcsr_build(self, n, src, dst, ts, eid=None):
+        be, m = self.be, int(src.shape[0])
+        row_ptr, col, cts, ceid = be.empty(n + 1), be.empty(m), be.empty(m), be.empty(m)
+        ws, wsb = self._workspace(self.lib.tcsr_build_workspace_bytes(n, m))
+        self._ck(self.lib.tcsr_build(n, m, be.ptr(src), be.ptr(dst), be.ptr(ts), be.ptr(eid),
+                                     be.ptr(row_ptr), be.ptr(col), be.ptr(cts), be.ptr(ceid),
+                                     be.ptr(ws), wsb, be.stream()))
+        return TCSRArrays(be, n, row_ptr, col, cts, ceid)
+
+    def tcsr_from_sorted(self, n, row_ptr, col, ts, eid, validate=True):
+        g = TCSRArrays(self.be, n, row_ptr, col, ts, eid)
+        if validate:
+            ws, wsb = self._workspace(256)
+            self._ck(self.lib.tcsr_validate(C.byref(g.view), self.be.ptr(ws), wsb, self.be.stream()))
+        return g
+
+    # ----------------------------------------------------------- sampling
+    @staticmethod
+    def params(sample_type, fanout, allowed_offset=-1, equal_root_time=False,
+               keep_root_time=False, replace=False, hop=0, seed=0):
+        if isinstance(sample_type, str):
+            if sample_type not in _abi.SAMPLE_TYPES:
+                # same message as sample.cu.hpp:1688-1690
+                raise RuntimeError("undefined sampling strategy")
+            sample_type = _abi.SAMPLE_TYPES[sample_type]
+        return SampleParams(int(sample_type), int(fanout), int(allowed_offset),
+                            int(bool(equal_root_time)), int(bool(keep_root_time)),
+                            int(bool(replace)), int(hop), int(seed) & (2**64 - 1))
+
+    def sample_hop(self, g, slot_node, slot_ts, p, S_dev=None, finalize=True):
+        be, S = self.be, int(slot_node.shape[0])
+        out = HopResult(be, S, S * p.fanout)
+        ws, wsb = self._workspace(self.lib.sample_hop_workspace_bytes(S))
+        self._ck(self.lib.sample_hop(C.byref(g.view), be.ptr(slot_node), be.ptr(slot_ts), S,
+                                     be.ptr(S_dev), C.byref(p), C.byref(out.struct),
+                                     be.ptr(ws), wsb, be.stream()))
+        if finalize:
+            out.finalize(*be.tolist(out.counts))
+        return out
+
+    def sample_khop(self, g, roots, ts_ptr, root_ts, neg_roots, neg_ts, layers, p,
+                    finalize=True):
+        be = self.be
+        R, S_pos, N_neg = int(roots.shape[0]), int(root_ts.shape[0]), int(neg_roots.shape[0])
+        S0 = S_pos + N_neg
+        slot_node0, slot_ts0 = be.empty(S0), be.empty(S0)
+        outs, cap = [], S0
+        counts = be.zeros(3 * max(layers, 1))
+        for l in range(layers):
+            outs.append(HopResult(be, cap, cap * p.fanout, counts[3 * l: 3 * l + 3]))
+            cap *= p.fanout
+        arr = (HopOut * max(layers, 1))(*[o.struct for o in outs])
+        ws, wsb = self._workspace(self.lib.sample_khop_workspace_bytes(S0, layers, p.fanout))
+        self._ck(self.lib.sample_khop(C.byref(g.view), R, be.ptr(roots), be.ptr(ts_ptr), S_pos,
+                                      be.ptr(root_ts), N_neg, be.ptr(neg_roots), be.ptr(neg_ts),
+                                      layers, C.byref(p), be.ptr(slot_node0), be.ptr(slot_ts0),
+                                      arr, be.ptr(ws), wsb, be.stream()))
+        res = KHopResult(self, slot_node0, slot_ts0, outs, counts)
+        return res.finalize() if finalize else res
+
+    # ------------------------------------------------------------- unique
+    def remap_state(self, universe):
+        nbytes = self.lib.remap_state_bytes(universe)
+        st = self.be.empty(max(nbytes, 8), "u8")
+        self._ck(self.lib.remap_init(self.be.ptr(st), nbytes, universe, self.be.stream()))
+        return RemapState(st, universe)
+
+    def unique_compact(self, arrays, mode=_abi.UNIQUE_SORTED, state=None, reset=True,
+                       lens_dev=None, out_arrays=None, finalize=True):
+        be, G = self.be, len(arrays)
+        len_max = (i64 * max(G, 1))(*[int(a.shape[0]) for a in arrays])
+        total = sum(len_max[:G])
+        ids = (vp * max(G, 1))(*[be.ptr(a) for a in arrays])
+        if out_arrays is None:
+            out_arrays = [be.empty(int(a.shape[0])) for a in arrays]
+        outs = (vp * max(G, 1))(*[be.ptr(a) for a in out_arrays])
+        ldev = None
+        if lens_dev is not None:
+            ldev = (vp * max(G, 1))(*[be.ptr(a) for a in lens_dev])
+        cap = total if state is None else min(total + state.count_bound, state.universe)
+        if state is not None and reset:
+            cap = min(total, state.universe)
+        unique = be.empty(max(cap, 1))
+        U = be.zeros(2)
+        universe = 0 if state is None else state.universe
+        ws, wsb = self._workspace(self.lib.unique_workspace_bytes(universe, G, len_max))
+        self._ck(self.lib.unique_compact(None if state is None else be.ptr(state.buf), universe,
+                                         int(bool(reset)), int(mode), G, ids, len_max, ldev, outs,
+                                         be.ptr(unique), cap, be.ptr(U), be.ptr(ws), wsb,
+                                         be.stream()))
+        if state is not None:
+            state.count_bound = cap
+        if not finalize:
+            return out_arrays, unique, U
+        u_total, u_before = be.tolist(U)
+        return out_arrays, unique[:u_total], (u_total, u_before)
+
+    # ------------------------------------------------------------- gather
+    def cache(self, row_bytes, hot, rows=None, cold=None, hot_slot=None, g2l=None,
+              id_mask=-1, ts_hot=None, ts_cold=None):
+        be = self.be
+        hot_rows = 0 if hot is None else int(hot.shape[0])
+        if rows is None:
+            rows = int(cold.shape[0]) if cold is not None else hot_rows
+        c = Cache(int(rows), int(row_bytes), int(id_mask), be.ptr(g2l),
+                  0 if g2l is None else int(g2l.shape[0]), be.ptr(hot_slot), be.ptr(hot),
+                  hot_rows, be.ptr(cold), be.ptr(ts_hot), be.ptr(ts_cold))
+        c._keep = (hot, cold, hot_slot, g2l, ts_hot, ts_cold)  # keep the arrays alive
+        return c
+
+    def gather(self, cache, ids, out, out_ts=None, stats=None, N_dev=None):
+        be = self.be
+        self._ck(self.lib.gather(C.byref(cache), be.ptr(ids), int(ids.shape[0]), be.ptr(N_dev),
+                                 be.ptr(out), be.ptr(out_ts), be.ptr(stats), be.stream()))
+        return out
+
+    def scatter_update(self, cache, hot_rw, cold_rw, ts_hot_rw, ts_cold_rw, ids, values, ts=None):
+        be = self.be
+        self._ck(self.lib.scatter_update(C.byref(cache), be.ptr(hot_rw), be.ptr(cold_rw),
+                                         be.ptr(ts_hot_rw), be.ptr(ts_cold_rw), be.ptr(ids),
+                                         int(ids.shape[0]), be.ptr(values), be.ptr(ts),
+                                         be.stream()))
+
+    # -------------------------------------------------------- time encode
+    def time_encode(self, dt, w, b, dt_dtype=_abi.DT_I64, out=None, N_dev=None):
+        be, N, dim = self.be, int(dt.shape[0]), int(w.shape[0])
+        if out is None:
+            out = be.empty((N, dim), "f32")
+        self._ck(self.lib.time_encode(be.ptr(dt), dt_dtype, N, be.ptr(N_dev), be.ptr(w),
+                                      be.ptr(b), dim, be.ptr(out), be.stream()))
+        return out
+
+
+class RemapState:
+    def __init__(self, buf, universe):
+        self.buf, self.universe, self.count_bound = buf, int(universe), 0
+
+
+class KHopResult:
+    def __init__(self, hp, slot_node0, slot_ts0, hops, counts):
+        self.hp, self.slot_node0, self.slot_ts0, self.hops = hp, slot_node0, slot_ts0, hops
+        self.counts, self.final = counts, False
+
+    def finalize(self):
+        """Read the per-hop device counts (one synchronising copy) and narrow."""
+        if not self.final:
+            c = self.hp.be.tolist(self.counts)
+            for l, h in enumerate(self.hops):
+                h.finalize(*c[3 * l: 3 * l + 3])
+            self.final = True
+        return self

@@ -1,0 +1,88 @@
+"""Synthetic power-law temporal graphs and request streams (numpy, seeded).
+
+These generate the workloads the benchmark and the tests run on; every array
+is int64 unless stated.  Nothing here touches the GPU.
+"""
+import numpy as np
+
+
+def zipf_degrees(n, m, a):
+    """Degree sequence deg[r] ~ (r+1)^-a over ranks r, scaled to sum exactly m."""
+    w = np.arange(1, n + 1, dtype=np.float64) ** (-a)
+    w /= w.sum()
+    deg = np.floor(w * m).astype(np.int64)
+    rest = int(m - deg.sum())
+    if rest > 0:  # hand the remainder to the top ranks, one edge each (wrapping)
+        idx = np.arange(rest) % n
+        np.add.at(deg, idx, 1)
+    return deg
+
+
+def graph_by_degree(n, m, a, t_max, seed, perm=True):
+    """Out-degree follows Zipf(a) by rank; destinations uniform; timestamps
+    uniform in [0, t_max), ascending inside every source row; eid = position
+    in that (src, ts) order.  Returns (src, dst, ts, eid, row_ptr): the edge
+    list is already in T-CSR order."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    deg_rank = zipf_degrees(n, m, a)
+    ids = rng.permutation(n).astype(np.int64) if perm else np.arange(n, dtype=np.int64)
+    deg = np.zeros(n, dtype=np.int64)
+    deg[ids] = deg_rank
+    row_ptr = np.zeros(n + 1, dtype=np.int64)
+    np.cumsum(deg, out=row_ptr[1:])
+    src = np.repeat(np.arange(n, dtype=np.int64), deg)
+    dst = rng.integers(0, n, size=m, dtype=np.int64)
+    ts = rng.integers(0, t_max, size=m, dtype=np.int64)
+    # sort timestamps inside each row: one global sort of (src, ts) keys
+    bits = max(int(t_max - 1).bit_length(), 1)
+    if bits + max(int(n - 1).bit_length(), 1) <= 62:
+        key = (src << bits) | ts
+        key.sort()
+        ts = key & ((1 << bits) - 1)
+    else:
+        order = np.lexsort((ts, src))
+        ts = ts[order]
+    eid = np.arange(m, dtype=np.int64)
+    return src, dst, ts, eid, row_ptr
+
+
+def graph_stream(n, m, a, t_max, seed):
+    """Edge stream in arrival order: sources iid Zipf(a) over a fixed rank->id
+    permutation, destinations uniform, timestamps ascending uniform draws from
+    [0, t_max); eid = arrival index."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    w = np.arange(1, n + 1, dtype=np.float64) ** (-a)
+    w /= w.sum()
+    ids = rng.permutation(n).astype(np.int64)
+    src = ids[rng.choice(n, size=m, p=w)]
+    dst = rng.integers(0, n, size=m, dtype=np.int64)
+    ts = np.sort(rng.integers(0, t_max, size=m, dtype=np.int64))
+    eid = np.arange(m, dtype=np.int64)
+    return src, dst, ts, eid
+
+
+def link_batch(src, dst, ts, lo, hi, n, n_neg, rng):
+    """Roots of one link-prediction batch over events [lo, hi): sources, then
+    destinations (positives), plus n_neg uniform negative destinations that
+    reuse the event timestamps.  Every positive root has one timestamp."""
+    roots = np.concatenate([src[lo:hi], dst[lo:hi]])
+    root_ts = np.concatenate([ts[lo:hi], ts[lo:hi]])
+    ts_ptr = np.arange(roots.shape[0] + 1, dtype=np.int64)
+    neg = rng.integers(0, n, size=n_neg, dtype=np.int64)
+    neg_ts = np.resize(ts[lo:hi], n_neg).astype(np.int64) if n_neg else np.zeros(0, np.int64)
+    return roots, ts_ptr, root_ts, neg, neg_ts
+
+
+def zipf_requests(rows, count, a, seed):
+    """`count` row ids drawn Zipf(a) by access rank; rank r maps to row id r, so
+    the hottest rows are the lowest ids (callers permute if they need to)."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    # inverse-CDF sampling on the continuous approximation of the rank law,
+    # then clipped: exact enough for a request stream and O(count) in memory
+    u = rng.random(count)
+    if abs(a - 1.0) < 1e-9:
+        r = np.exp(u * np.log(rows + 1.0))
+    else:
+        b = 1.0 - a
+        r = (1.0 + u * ((rows + 1.0) ** b - 1.0)) ** (1.0 / b)
+    return np.clip(np.floor(r).astype(np.int64) - 1, 0, rows - 1)

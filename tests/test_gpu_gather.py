@@ -1,0 +1,135 @@
+"""GPU parity: two-tier cache gather / scatter-update through the C ABI vs the
+CPU oracle and numpy fancy indexing, byte-exact."""
+import numpy as np
+import pytest
+import torch
+
+from util import np_of, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _tables(rows, dim, dtype, hot_frac, seed):
+    rng = np.random.default_rng(seed)
+    if dtype == np.uint16:  # bf16 payload: any bit pattern is a valid row
+        full = rng.integers(0, 2**16, (rows, dim), dtype=np.uint16)
+    else:
+        full = rng.standard_normal((rows, dim)).astype(dtype)
+    hot_rows = int(rows * hot_frac)
+    hot_ids = rng.permutation(rows)[:hot_rows]
+    hot_slot = np.full(rows, -1, dtype=np.int32)
+    hot_slot[hot_ids] = np.arange(hot_rows, dtype=np.int32)
+    hot = full[hot_ids].copy()
+    cold = full.copy()
+    cold[hot_ids] = 0  # a hot row must never be served from the cold tier
+    return full, hot, cold, hot_slot
+
+
+def _dev_cache(hot_path, full, hot, cold, hot_slot, **kw):
+    t_hot = torch.from_numpy(hot).to(hot_path.be.device)
+    t_cold = torch.from_numpy(cold).pin_memory()
+    t_slot = to_dev(hot_path, hot_slot, "i32")
+    rb = full.shape[1] * full.dtype.itemsize
+    return hot_path.cache(rb, t_hot, rows=full.shape[0], cold=t_cold, hot_slot=t_slot, **kw), (t_hot, t_cold)
+
+
+@pytest.mark.parametrize("dim,dtype", [(128, np.uint16), (100, np.float32), (172, np.float32), (1, np.float32),
+                                       (3, np.float32), (6, np.float32), (1000, np.float32)])
+def test_gather_matches_numpy(oracle, hot, dim, dtype):
+    rows, N = 20_000, 50_000
+    full, h, c, slot = _tables(rows, dim, dtype, 0.1, dim)
+    ids = np.random.default_rng(1).integers(0, rows, N).astype(np.int64)
+    cache, keep = _dev_cache(hot, full, h, c, slot)
+    out = torch.empty((N, dim), dtype=torch.from_numpy(full[:1]).dtype, device=hot.be.device)
+    stats = hot.be.zeros(3)
+    hot.gather(cache, to_dev(hot, ids), out, stats=stats)
+    assert np.array_equal(np_of(out).view(np.uint8), full[ids].view(np.uint8))
+    n_hot = int((slot[ids] >= 0).sum())
+    assert np_of(stats).tolist() == [n_hot, N - n_hot, 0]
+    # the oracle agrees with numpy on the same tables
+    oc = oracle.cache(full.shape[1] * full.dtype.itemsize, h, rows=rows, cold=c, hot_slot=slot)
+    o_out = np.empty((N, dim), dtype=full.dtype)
+    oracle.gather(oc, ids, o_out)
+    assert np.array_equal(o_out.view(np.uint8), full[ids].view(np.uint8))
+
+
+def test_gather_g2l_mask_ts_and_absent(oracle, hot):
+    """global id -> local row through a dense map, DistRouteIndex low-48-bit
+    mask, last-update timestamps from both tiers, absent ids -> zero rows."""
+    rows, dim, G = 5000, 100, 12_000
+    full, h, c, slot = _tables(rows, dim, np.float32, 0.3, 2)
+    rng = np.random.default_rng(3)
+    loc_ids = rng.permutation(G)[:rows].astype(np.int64)       # global id of each local row
+    g2l = np.full(G + 1, -1, dtype=np.int64)
+    g2l[loc_ids] = np.arange(rows)
+    ts_full = rng.integers(0, 10**9, rows).astype(np.int64)
+    hot_rows = h.shape[0]
+    ts_hot = np.zeros(hot_rows, dtype=np.int64)
+    ts_hot[slot[slot >= 0]] = ts_full[slot >= 0]
+    gids = rng.integers(0, G, 30_000).astype(np.int64)
+    gids[::97] = -5
+    gids[::101] = G + 3
+    part = rng.integers(0, 2**14, gids.shape[0]).astype(np.int64)
+    enc = np.where(gids >= 0, gids | (part << 48) | (1 << 62), gids)   # DistRouteIndex encoding
+    kw = dict(id_mask=0xFFFFFFFFFFFF)
+    cache, keep = _dev_cache(hot, full, h, c, slot, g2l=to_dev(hot, g2l), ts_hot=to_dev(hot, ts_hot),
+                             ts_cold=torch.from_numpy(ts_full).pin_memory(), **kw)
+    out = torch.empty((gids.shape[0], dim), dtype=torch.float32, device=hot.be.device)
+    out_ts = hot.be.empty(gids.shape[0])
+    stats = hot.be.zeros(3)
+    hot.gather(cache, to_dev(hot, enc), out, out_ts=out_ts, stats=stats)
+    oc = oracle.cache(dim * 4, h, rows=rows, cold=c, hot_slot=slot, g2l=g2l, ts_hot=ts_hot, ts_cold=ts_full, **kw)
+    o_out, o_ts, o_stats = np.empty((gids.shape[0], dim), np.float32), np.empty(gids.shape[0], np.int64), np.zeros(3, np.int64)
+    oracle.gather(oc, enc, o_out, out_ts=o_ts, stats=o_stats)
+    assert np.array_equal(np_of(out).view(np.uint32), o_out.view(np.uint32))
+    assert np.array_equal(np_of(out_ts), o_ts)
+    assert np_of(stats).tolist() == o_stats.tolist()
+    # numpy closed form
+    ok = (gids >= 0) & (gids < G + 1)
+    loc = np.where(ok, g2l[np.clip(gids, 0, G)], -1)
+    want = np.where((loc >= 0)[:, None], full[np.clip(loc, 0, rows - 1)], 0).astype(np.float32)
+    assert np.array_equal(o_out.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(o_ts, np.where(loc >= 0, ts_full[np.clip(loc, 0, rows - 1)], 0))
+    assert o_stats[2] == int((loc < 0).sum())
+
+
+def test_all_hot_table_without_index(hot):
+    rows, dim = 3000, 172
+    full = np.random.default_rng(0).standard_normal((rows, dim)).astype(np.float32)
+    ids = np.random.default_rng(1).integers(0, rows, 10_000).astype(np.int64)
+    t = torch.from_numpy(full).to(hot.be.device)
+    cache = hot.cache(dim * 4, t)
+    out = torch.empty((ids.shape[0], dim), dtype=torch.float32, device=hot.be.device)
+    hot.gather(cache, to_dev(hot, ids), out)
+    assert np.array_equal(np_of(out), full[ids])
+    # a live count on the device shortens the gather
+    out.zero_()
+    n_dev = to_dev(hot, np.array([123], dtype=np.int64))
+    hot.gather(cache, to_dev(hot, ids), out, N_dev=n_dev)
+    assert np.array_equal(np_of(out)[:123], full[ids[:123]]) and not np_of(out)[123:].any()
+
+
+def test_scatter_update_roundtrip(oracle, hot):
+    rows, dim = 4000, 100
+    full, h, c, slot = _tables(rows, dim, np.float32, 0.25, 7)
+    cache, (t_hot, t_cold) = _dev_cache(hot, full, h, c, slot)
+    rng = np.random.default_rng(8)
+    ids = rng.permutation(rows)[:1500].astype(np.int64)
+    ids_bad = ids.copy()
+    ids_bad[::50] = -1
+    vals = rng.standard_normal((1500, dim)).astype(np.float32)
+    ts = rng.integers(0, 10**6, 1500).astype(np.int64)
+    ts_hot = hot.be.zeros(h.shape[0])
+    ts_cold = torch.zeros(rows, dtype=torch.int64).pin_memory()
+    hot.scatter_update(cache, t_hot, t_cold, ts_hot, ts_cold, to_dev(hot, ids_bad), to_dev(hot, vals, "f32"), to_dev(hot, ts))
+    torch.cuda.synchronize()
+    oh, oc_, oth, otc = h.copy(), c.copy(), np.zeros(h.shape[0], np.int64), np.zeros(rows, np.int64)
+    ocache = oracle.cache(dim * 4, oh, rows=rows, cold=oc_, hot_slot=slot)
+    oracle.scatter_update(ocache, oh, oc_, oth, otc, ids_bad, vals, ts)
+    assert np.array_equal(np_of(t_hot), oh) and np.array_equal(t_cold.numpy(), oc_)
+    assert np.array_equal(np_of(ts_hot), oth) and np.array_equal(ts_cold.numpy(), otc)
+    # and the gather reads the updated rows back
+    out = torch.empty((1500, dim), dtype=torch.float32, device=hot.be.device)
+    hot.gather(cache, to_dev(hot, ids), out)
+    keep = ids_bad >= 0
+    assert np.array_equal(np_of(out)[keep], vals[keep])

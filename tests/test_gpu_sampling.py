@@ -1,0 +1,121 @@
+"""GPU parity: temporal sampling through the C ABI vs the CPU oracle, bit-exact
+(recent AND uniform: both sides draw from the same counter-based generator)."""
+import numpy as np
+import pytest
+
+from starrygl_amd.utils import synth
+from util import assert_hop_equal, host_graph, mirror_graph, np_of, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph(oracle, hot, n, m, a, t_max, seed, hub=None):
+    src, dst, ts, eid = synth.graph_stream(n, m, a, t_max, seed)
+    if hub is not None:  # one very long row to exercise the multi-step search
+        src[: hub] = 3
+    g = host_graph(oracle, n, src, dst, ts, eid)
+    return (src, dst, ts, eid), g, mirror_graph(hot, g)
+
+
+def _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, neg, neg_ts, layers, **kw):
+    p = oracle.params(**kw)
+    want = oracle.sample_khop(g, roots, ts_ptr, root_ts, neg, neg_ts, layers, p)
+    got = hot.sample_khop(dg, to_dev(hot, roots), to_dev(hot, ts_ptr), to_dev(hot, root_ts),
+                          to_dev(hot, neg), to_dev(hot, neg_ts), layers, hot.params(**kw))
+    assert np.array_equal(np_of(got.slot_node0), want.slot_node0)
+    assert np.array_equal(np_of(got.slot_ts0), want.slot_ts0)
+    for l in range(layers):
+        assert_hop_equal(got.hops[l], want.hops[l], tag=f"hop{l} {kw}")
+    return got, want
+
+
+@pytest.mark.parametrize("sample_type", ["recent", "uniform"])
+@pytest.mark.parametrize("layers,fanout", [(1, 10), (2, 10), (2, 5), (1, 20), (1, 1)])
+def test_khop_parity_plumbing_graph(oracle, hot, sample_type, layers, fanout):
+    """configs[0]: 10k nodes / 160k edges, batches of 600 edges + 600 negatives."""
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 10_000, 160_000, 1.2, 2_600_000, 20240)
+    rng = np.random.default_rng(1)
+    for lo in (0, 80_000, 159_400):
+        b = synth.link_batch(src, dst, ts, lo, lo + 600, g.n, 600, rng)
+        _run_both(oracle, hot, g, dg, *b, layers, sample_type=sample_type, fanout=fanout, seed=7 + lo)
+
+
+@pytest.mark.parametrize("sample_type", ["recent", "uniform"])
+def test_window_flags(oracle, hot, sample_type):
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 2_000, 60_000, 1.1, 50_000, 3)
+    rng = np.random.default_rng(2)
+    b = synth.link_batch(src, dst, ts, 30_000, 30_500, g.n, 300, rng)
+    for kw in (dict(allowed_offset=0), dict(allowed_offset=500), dict(allowed_offset=10**9),
+               dict(equal_root_time=True), dict(equal_root_time=True, allowed_offset=100),
+               dict(keep_root_time=True), dict(replace=True), dict(replace=True, keep_root_time=True)):
+        _run_both(oracle, hot, g, dg, *b, 2, sample_type=sample_type, fanout=7, seed=11, **kw)
+
+
+@pytest.mark.parametrize("sample_type", ["recent", "uniform"])
+@pytest.mark.parametrize("fanout", [3, 16, 17, 32, 33, 64])
+def test_long_rows_and_wide_fanout(oracle, hot, sample_type, fanout):
+    """a 120k-edge row (5 search steps with 16 lanes) and every group width."""
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 500, 150_000, 1.05, 10**12, 5, hub=120_000)
+    rng = np.random.default_rng(3)
+    roots = np.concatenate([np.full(200, 3), rng.integers(0, g.n, 300)]).astype(np.int64)
+    root_ts = rng.integers(0, 10**12, roots.shape[0]).astype(np.int64)
+    ts_ptr = np.arange(roots.shape[0] + 1, dtype=np.int64)
+    e = np.zeros(0, np.int64)
+    _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, e, e, 1, sample_type=sample_type, fanout=fanout, seed=99)
+
+
+def test_multi_timestamp_roots_and_empty_inputs(oracle, hot):
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 300, 5_000, 1.1, 10_000, 8)
+    roots = np.array([5, 7, 7, 250, 0], dtype=np.int64)
+    ts_ptr = np.array([0, 3, 3, 4, 9, 10], dtype=np.int64)  # root 1 has no timestamp
+    root_ts = np.array([100, 5000, 9999, 7000, 1, 2, 3, 4, 9000, 10_000], dtype=np.int64)
+    neg = np.array([299, 0], dtype=np.int64)
+    neg_ts = np.array([10_001, 0], dtype=np.int64)
+    for st in ("recent", "uniform"):
+        _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, neg, neg_ts, 2, sample_type=st, fanout=4, seed=1)
+    e = np.zeros(0, np.int64)
+    got, _ = _run_both(oracle, hot, g, dg, e, np.zeros(1, np.int64), e, e, e, 2, sample_type="recent", fanout=4)
+    assert got.hops[0].E == 0 and got.hops[1].S == 0
+    # only negatives
+    _run_both(oracle, hot, g, dg, e, np.zeros(1, np.int64), e, neg, neg_ts, 1, sample_type="uniform", fanout=4)
+
+
+def test_isolated_nodes_and_time_zero(oracle, hot):
+    """nodes without edges and roots at t <= every timestamp sample nothing."""
+    n = 50
+    src = np.array([1, 1, 1, 2], dtype=np.int64)
+    dst = np.array([2, 3, 4, 1], dtype=np.int64)
+    ts = np.array([10, 10, 20, 5], dtype=np.int64)
+    g = host_graph(oracle, n, src, dst, ts)
+    dg = mirror_graph(hot, g)
+    roots = np.array([0, 1, 1, 1, 2, 49], dtype=np.int64)
+    root_ts = np.array([100, 10, 11, 21, 5, 100], dtype=np.int64)
+    ts_ptr = np.arange(7, dtype=np.int64)
+    e = np.zeros(0, np.int64)
+    got, want = _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, e, e, 1, sample_type="recent", fanout=2)
+    assert np_of(got.hops[0].root_end_ptr).tolist()[:-1] == [0, 0, 2, 4, 4, 4]
+    assert np_of(got.hops[0].neighbors).tolist() == [2, 3, 3, 4]  # ties keep storage (eid) order
+
+
+def test_out_of_range_root_is_reported(oracle, hot):
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 100, 1_000, 1.1, 1000, 4)
+    roots = np.array([5, 100, -1, 7], dtype=np.int64)
+    ts_ptr = np.arange(5, dtype=np.int64)
+    root_ts = np.full(4, 900, dtype=np.int64)
+    e = to_dev(hot, np.zeros(0, np.int64))
+    res = hot.sample_khop(dg, to_dev(hot, roots), to_dev(hot, ts_ptr), to_dev(hot, root_ts), e, e, 1,
+                          hot.params("recent", 3), finalize=False)
+    assert np_of(res.counts).tolist()[2] == 2
+    with pytest.raises(IndexError):
+        res.finalize()
+
+
+def test_error_codes(hot):
+    with pytest.raises(RuntimeError, match="undefined sampling strategy"):
+        hot.params("nearest", 3)
+    import ctypes as C
+    from starrygl_amd.lib import _abi
+    p = hot.params("recent", 3)
+    p.type = 9
+    assert hot.lib.sample_khop(None, 0, None, None, 0, None, 0, None, None, 1, C.byref(p), None, None, None,
+                               None, 0, None) == _abi.SGL_EINVAL

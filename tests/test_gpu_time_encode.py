@@ -1,0 +1,45 @@
+"""GPU parity: cos(w*dt+b) through the C ABI vs the CPU oracle.
+Tolerance (stated by the task): |y - y_ref| <= 1e-6 * max(1, |y_ref|) with
+y_ref = float32(cos(float64(a))), a = fl32(fl32(w*x) + b)."""
+import numpy as np
+import pytest
+
+from starrygl_amd.lib import _abi
+from util import np_of, to_dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-6
+
+
+def _w(dim):
+    return (1.0 / 10 ** np.linspace(0, 9, dim, dtype=np.float32)).astype(np.float32)
+
+
+@pytest.mark.parametrize("dim", [100, 16, 7, 1, 172])
+@pytest.mark.parametrize("bias", [False, True])
+def test_time_encode_i64(oracle, hot, dim, bias):
+    rng = np.random.default_rng(dim)
+    dt = np.concatenate([np.zeros(3, np.int64), -rng.integers(0, 2_600_000, 4000), rng.integers(0, 2**40, 2000),
+                         np.array([1, -1, 2**31, -(2**40)])]).astype(np.int64)
+    w = _w(dim)
+    b = (rng.standard_normal(dim).astype(np.float32) if bias else np.zeros(dim, np.float32))
+    want = oracle.time_encode(dt, w, b)
+    got = np_of(hot.time_encode(to_dev(hot, dt), to_dev(hot, w, "f32"), to_dev(hot, b, "f32")))
+    err = np.abs(got.astype(np.float64) - want) / np.maximum(1.0, np.abs(want))
+    assert err.max() <= TOL, f"max err {err.max()} at {np.unravel_index(err.argmax(), err.shape)}"
+    # closed form in float64 on the separately rounded argument
+    a = (w[None, :] * dt.astype(np.float32)[:, None]).astype(np.float32) + b[None, :]
+    assert np.array_equal(want, np.cos(a.astype(np.float64)).astype(np.float32))
+
+
+def test_time_encode_f32_input_and_device_count(oracle, hot):
+    rng = np.random.default_rng(1)
+    dt = (rng.random(5000) * 1e6).astype(np.float32)
+    w, b = _w(100), np.zeros(100, np.float32)
+    want = oracle.time_encode(dt, w, b, dt_dtype=_abi.DT_F32)
+    n_dev = to_dev(hot, np.array([777], dtype=np.int64))
+    out = hot.be.zeros((5000, 100), "f32")
+    hot.time_encode(to_dev(hot, dt, "f32"), to_dev(hot, w, "f32"), to_dev(hot, b, "f32"), dt_dtype=_abi.DT_F32,
+                    out=out, N_dev=n_dev)
+    got = np_of(out)
+    assert np.abs(got[:777] - want[:777]).max() <= TOL and not got[777:].any()

@@ -1,0 +1,286 @@
+"""Pins the CPU oracle (oracle/sgl_oracle.c) without any GPU: library routines
+(np.searchsorted, np.unique, np.lexsort, fancy indexing), brute force on small
+graphs, Random123's published Philox4x32-10 vectors, closed forms, chi-square."""
+import numpy as np
+import pytest
+from scipy import stats as sps
+
+from starrygl_amd.lib import _abi
+from starrygl_amd.utils import synth
+from util import host_graph
+
+E = np.zeros(0, np.int64)
+
+
+# ------------------------------------------------------------------ T-CSR
+def test_tcsr_build_is_lexsort(oracle):
+    rng = np.random.default_rng(0)
+    n, m = 200, 5000
+    src, dst = rng.integers(0, n, m), rng.integers(0, n, m)
+    ts = rng.integers(0, 50, m)            # many ties
+    eid = rng.permutation(m)
+    g = host_graph(oracle, n, src, dst, ts, eid)
+    o = np.lexsort((eid, ts, src))
+    assert np.array_equal(g.col, dst[o]) and np.array_equal(g.ts, ts[o]) and np.array_equal(g.eid, eid[o])
+    assert np.array_equal(g.row_ptr, np.concatenate([[0], np.cumsum(np.bincount(src, minlength=n))]))
+    # eid defaults to arange
+    g2 = host_graph(oracle, n, src, dst, ts)
+    o2 = np.lexsort((np.arange(m), ts, src))
+    assert np.array_equal(g2.eid, o2)
+
+
+def test_tcsr_build_rejects_out_of_range(oracle):
+    with pytest.raises(IndexError):
+        host_graph(oracle, 5, np.array([0, 5]), np.array([1, 1]), np.array([0, 1]))
+    with pytest.raises(IndexError):
+        host_graph(oracle, 5, np.array([0, 1]), np.array([1, -1]), np.array([0, 1]))
+
+
+def test_tcsr_validate(oracle):
+    g = host_graph(oracle, 4, np.array([0, 0, 2]), np.array([1, 2, 3]), np.array([5, 6, 1]))
+    oracle.tcsr_from_sorted(4, g.row_ptr, g.col, g.ts, g.eid)
+    bad_ts = g.ts.copy(); bad_ts[:2] = [6, 5]
+    with pytest.raises(IndexError):
+        oracle.tcsr_from_sorted(4, g.row_ptr, g.col, bad_ts, g.eid)
+    bad_col = g.col.copy(); bad_col[0] = 4
+    with pytest.raises(IndexError):
+        oracle.tcsr_from_sorted(4, g.row_ptr, bad_col, g.ts, g.eid)
+
+
+# ---------------------------------------------------------------- sampling
+def _brute(g, v, t, k, allowed_offset=-1, equal=False):
+    a, b = g.row_ptr[v], g.row_ptr[v + 1]
+    t_hi = t + (1 if equal else 0)
+    return [e for e in range(a, b) if g.ts[e] < t_hi and (allowed_offset < 0 or g.ts[e] >= t - allowed_offset)]
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(allowed_offset=0), dict(allowed_offset=40), dict(equal_root_time=True),
+                                dict(equal_root_time=True, allowed_offset=3)])
+def test_recent_matches_brute_force(oracle, kw):
+    rng = np.random.default_rng(1)
+    n, m = 60, 3000
+    g = host_graph(oracle, n, rng.integers(0, n, m), rng.integers(0, n, m), rng.integers(0, 200, m))
+    slots = rng.integers(0, n, 400).astype(np.int64)
+    t = rng.integers(-5, 210, 400).astype(np.int64)
+    k = 6
+    h = oracle.sample_hop(g, slots, t, oracle.params("recent", k, **kw))
+    assert h.S == 400 and h.root_start_ptr[0] == 0 and h.root_start_ptr[-1] == h.E == h.root_end_ptr[-1]
+    assert np.array_equal(h.root_end_ptr[:-1], h.root_start_ptr[1:])
+    for s in range(400):
+        cand = _brute(g, slots[s], t[s], k, kw.get("allowed_offset", -1), kw.get("equal_root_time", False))[-k:]
+        lo, hi = h.root_start_ptr[s], h.root_end_ptr[s]
+        assert h.neighbors_eid[lo:hi].tolist() == g.eid[cand].tolist()
+        assert h.neighbors[lo:hi].tolist() == g.col[cand].tolist()
+        assert h.neighbors_ts[lo:hi].tolist() == g.ts[cand].tolist()
+        assert h.neighbors_dt[lo:hi].tolist() == (g.ts[cand] - t[s]).tolist()
+    # window ends == np.searchsorted(side='left') on the row slice
+    for s in range(0, 400, 7):
+        a, b = g.row_ptr[slots[s]], g.row_ptr[slots[s] + 1]
+        cut = np.searchsorted(g.ts[a:b], t[s] + (1 if kw.get("equal_root_time") else 0), side="left")
+        full = oracle.sample_hop(g, slots[s:s + 1], t[s:s + 1], oracle.params("recent", 10**6, **kw))
+        if kw.get("allowed_offset", -1) < 0:
+            assert full.E == cut
+
+
+PHILOX_KAT = [  # Random123 kat_vectors, philox4x32 with 10 rounds: ctr, key, expected
+    ([0, 0, 0, 0], [0, 0], [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+    ([0xffffffff] * 4, [0xffffffff] * 2, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+    ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+     [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]),
+]
+
+
+def test_philox_known_answers(oracle_cdll):
+    for ctr, key, want in PHILOX_KAT:
+        c, k, o = np.array(ctr, np.uint32), np.array(key, np.uint32), np.zeros(4, np.uint32)
+        oracle_cdll.sglo_philox4x32_10(c.ctypes.data, k.ctypes.data, o.ctypes.data)
+        assert o.tolist() == want
+
+
+def test_draw_bits_layout_and_bounded(oracle_cdll):
+    # counter = (draw, slot_lo, slot_hi, hop), key = (seed_lo, seed_hi), bits = x0 | x1 << 32
+    c = np.array([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], np.uint32)
+    bits = oracle_cdll.sglo_draw_bits(0x299f31d0a4093822, 0x03707344, (0x13198a2e << 32) | 0x85a308d3, 0x243f6a88)
+    assert bits == (0x94fdcceb << 32) | 0xd16cfe09
+    for b, r in [(0, 10), (2**64 - 1, 10), (2**63, 10), (2**63, 7), (12345678901234567, 10**12)]:
+        assert oracle_cdll.sglo_bounded(b, r) == (b * r) >> 64
+
+
+@pytest.mark.parametrize("replace", [False, True])
+def test_uniform_invariants(oracle, replace):
+    rng = np.random.default_rng(2)
+    n, m, k = 40, 4000, 8
+    g = host_graph(oracle, n, rng.integers(0, n, m), rng.integers(0, n, m), rng.integers(0, 500, m))
+    slots, t = rng.integers(0, n, 300).astype(np.int64), rng.integers(0, 520, 300).astype(np.int64)
+    pos_of = {int(e): i for i, e in enumerate(g.eid)}
+    for keep in (False, True):
+        h = oracle.sample_hop(g, slots, t, oracle.params("uniform", k, replace=replace, keep_root_time=keep, seed=3))
+        for s in range(300):
+            cand = _brute(g, slots[s], t[s], k)
+            lo, hi = h.root_start_ptr[s], h.root_end_ptr[s]
+            assert hi - lo == min(k, len(cand))
+            pos = [pos_of[int(e)] for e in h.neighbors_eid[lo:hi]]
+            assert set(pos) <= set(cand)
+            if len(cand) <= k:
+                assert pos == cand
+            elif not replace:
+                assert len(set(pos)) == k and pos == sorted(pos)
+            assert h.neighbors[lo:hi].tolist() == g.col[pos].tolist()          # eid <-> dst mapping
+            assert (g.ts[pos] < t[s]).all()
+            assert h.neighbors_dt[lo:hi].tolist() == (g.ts[pos] - t[s]).tolist()
+            assert h.neighbors_ts[lo:hi].tolist() == ([t[s]] * len(pos) if keep else g.ts[pos].tolist())
+
+
+@pytest.mark.parametrize("replace", [False, True])
+def test_uniform_chi_square(oracle, replace):
+    """every candidate position of a row is picked with probability k/cnt."""
+    cnt, k, trials = 37, 10, 20_000
+    g = host_graph(oracle, 2, np.zeros(cnt, np.int64), np.ones(cnt, np.int64), np.arange(cnt))
+    slots, t = np.zeros(trials, np.int64), np.full(trials, cnt + 5, np.int64)
+    freq = np.zeros(cnt)
+    h = oracle.sample_hop(g, slots, t, oracle.params("uniform", k, replace=replace, seed=12345))
+    np.add.at(freq, h.neighbors_eid, 1)
+    assert h.E == trials * k
+    chi2 = ((freq - trials * k / cnt) ** 2 / (trials * k / cnt)).sum()
+    # without replacement the per-position counts are negatively correlated, which only lowers chi2
+    assert chi2 < sps.chi2.ppf(0.999, cnt - 1), chi2
+    # different seeds and hops give different draws
+    h2 = oracle.sample_hop(g, slots[:50], t[:50], oracle.params("uniform", k, replace=replace, seed=12346))
+    h3 = oracle.sample_hop(g, slots[:50], t[:50], oracle.params("uniform", k, replace=replace, seed=12345, hop=1))
+    assert not np.array_equal(h2.neighbors_eid, h.neighbors_eid[:500])
+    assert not np.array_equal(h3.neighbors_eid, h.neighbors_eid[:500])
+
+
+def test_khop_is_composition_of_hops(oracle):
+    src, dst, ts, eid = synth.graph_stream(500, 20_000, 1.1, 10_000, 4)
+    g = host_graph(oracle, 500, src, dst, ts, eid)
+    rng = np.random.default_rng(0)
+    roots, ts_ptr, root_ts, neg, neg_ts = synth.link_batch(src, dst, ts, 10_000, 10_100, 500, 100, rng)
+    for st in ("recent", "uniform"):
+        p = oracle.params(st, 5, seed=8)
+        res = oracle.sample_khop(g, roots, ts_ptr, root_ts, neg, neg_ts, 3, p)
+        assert np.array_equal(res.slot_node0, np.concatenate([roots, neg]))
+        assert np.array_equal(res.slot_ts0, np.concatenate([root_ts, neg_ts]))
+        sn, stt = res.slot_node0, res.slot_ts0
+        for l in range(3):
+            h = oracle.sample_hop(g, sn, stt, oracle.params(st, 5, seed=8, hop=l))
+            for f in ("root_start_ptr", "root_end_ptr", "neighbors", "neighbors_ts", "neighbors_eid", "neighbors_dt"):
+                assert np.array_equal(getattr(h, f), getattr(res.hops[l], f))
+            sn, stt = h.neighbors, h.neighbors_ts
+
+
+def test_khop_multi_timestamp_roots(oracle):
+    g = host_graph(oracle, 4, np.array([0, 0, 0, 1]), np.array([1, 2, 3, 0]), np.array([1, 2, 3, 1]))
+    res = oracle.sample_khop(g, np.array([0, 1, 2]), np.array([0, 2, 2, 3]), np.array([3, 10, 5]), np.array([1]),
+                             np.array([2]), 1, oracle.params("recent", 2))
+    assert res.slot_node0.tolist() == [0, 0, 2, 1] and res.slot_ts0.tolist() == [3, 10, 5, 2]
+    assert res.hops[0].neighbors.tolist() == [1, 2, 2, 3, 0]
+    with pytest.raises(ValueError):
+        oracle.sample_khop(g, np.array([0]), np.array([0, 5]), np.array([3]), E, E, 1, oracle.params("recent", 2))
+
+
+def test_sampling_errors(oracle):
+    g = host_graph(oracle, 3, np.array([0]), np.array([1]), np.array([1]))
+    p = oracle.params("recent", 2)
+    p.type = 5
+    with pytest.raises(RuntimeError, match="undefined sampling strategy"):
+        oracle.sample_hop(g, np.array([0]), np.array([5]), p)
+    with pytest.raises(RuntimeError):
+        oracle.sample_hop(g, np.array([0]), np.array([5]), oracle.params("uniform", 65))
+    with pytest.raises(IndexError):
+        oracle.sample_hop(g, np.array([3]), np.array([5]), oracle.params("recent", 2))
+
+
+# ------------------------------------------------------------------ unique
+@pytest.mark.parametrize("with_state", [True, False])
+def test_unique_sorted_is_np_unique(oracle, with_state):
+    rng = np.random.default_rng(3)
+    arrs = [rng.integers(0, 3000, s).astype(np.int64) for s in (10, 2000, 0, 7000)]
+    st = oracle.remap_state(3000) if with_state else None
+    loc, uniq, (tot, before) = oracle.unique_compact(arrs, _abi.UNIQUE_SORTED, st, True)
+    u, inv = np.unique(np.concatenate(arrs), return_inverse=True)
+    assert before == 0 and tot == u.shape[0] and np.array_equal(uniq, u)
+    assert np.array_equal(np.concatenate(loc), inv)
+
+
+@pytest.mark.parametrize("with_state", [True, False])
+def test_unique_grouped_is_setdiff(oracle, with_state):
+    rng = np.random.default_rng(4)
+    arrs = [rng.integers(0, 2000, s).astype(np.int64) for s in (100, 1000, 5000)]
+    st = oracle.remap_state(2000) if with_state else None
+    loc, uniq, (tot, _) = oracle.unique_compact(arrs, _abi.UNIQUE_GROUPED, st, True)
+    seen, want = np.zeros(0, np.int64), []
+    for x in arrs:
+        new = np.setdiff1d(np.unique(x), seen)
+        want.append(new)
+        seen = np.concatenate([seen, new])
+    assert np.array_equal(uniq, np.concatenate(want))
+    for x, l in zip(arrs, loc):
+        assert np.array_equal(uniq[l], x)
+
+
+def test_unique_epochs(oracle):
+    st = oracle.remap_state(100)
+    a = np.array([5, 3, 5, 9], np.int64)
+    l1, u1, c1 = oracle.unique_compact([a], _abi.UNIQUE_SORTED, st, True)
+    assert l1[0].tolist() == [1, 0, 1, 2] and u1.tolist() == [3, 5, 9] and c1 == (3, 0)
+    b = np.array([9, 1, 50, 3], np.int64)
+    l2, u2, c2 = oracle.unique_compact([b], _abi.UNIQUE_SORTED, st, False)   # 'f': continue numbering
+    assert l2[0].tolist() == [2, 3, 4, 0] and u2[3:5].tolist() == [1, 50] and c2 == (5, 3)
+    l3, u3, c3 = oracle.unique_compact([b], _abi.UNIQUE_SORTED, st, True)    # 'r': restart
+    assert l3[0].tolist() == [2, 0, 3, 1] and u3.tolist() == [1, 3, 9, 50] and c3 == (4, 0)
+    with pytest.raises(RuntimeError):
+        oracle.unique_compact([b], _abi.UNIQUE_SORTED, None, False)
+
+
+# ------------------------------------------------------------------ gather
+def test_gather_and_scatter_are_fancy_indexing(oracle):
+    rng = np.random.default_rng(5)
+    rows, dim = 500, 12
+    full = rng.standard_normal((rows, dim)).astype(np.float32)
+    hot_ids = rng.permutation(rows)[:100]
+    slot = np.full(rows, -1, np.int32); slot[hot_ids] = np.arange(100, dtype=np.int32)
+    hot, cold = full[hot_ids].copy(), full.copy(); cold[hot_ids] = np.nan
+    ids = rng.integers(0, rows, 3000).astype(np.int64); ids[5] = -1; ids[6] = rows
+    c = oracle.cache(dim * 4, hot, rows=rows, cold=cold, hot_slot=slot)
+    out, stats = np.empty((3000, dim), np.float32), np.zeros(3, np.int64)
+    oracle.gather(c, ids, out, stats=stats)
+    ok = (ids >= 0) & (ids < rows)
+    assert np.array_equal(out[ok], full[ids[ok]]) and not out[~ok].any()
+    assert stats.tolist() == [int((slot[ids[ok]] >= 0).sum()), int((slot[ids[ok]] < 0).sum()), 2]
+    # scatter then gather
+    upd = rng.permutation(rows)[:200].astype(np.int64)
+    vals = rng.standard_normal((200, dim)).astype(np.float32)
+    oracle.scatter_update(c, hot, cold, None, None, upd, vals)
+    full[upd] = vals
+    oracle.gather(c, ids, out)
+    assert np.array_equal(out[ok], full[ids[ok]])
+
+
+def test_dist_route_index_mask(oracle):
+    full = np.arange(40, dtype=np.float32).reshape(10, 4)
+    c = oracle.cache(16, full, id_mask=0xFFFFFFFFFFFF)
+    ids = np.array([3 | (7 << 48), 9 | (1 << 62) | (100 << 48), 2], np.int64)
+    out = np.empty((3, 4), np.float32)
+    oracle.gather(c, ids, out)
+    assert np.array_equal(out, full[[3, 9, 2]])
+
+
+# ------------------------------------------------------------- time encode
+def test_time_encode_closed_form(oracle):
+    rng = np.random.default_rng(6)
+    dim = 100
+    w = (1.0 / 10 ** np.linspace(0, 9, dim, dtype=np.float32)).astype(np.float32)
+    b = rng.standard_normal(dim).astype(np.float32)
+    dt = np.concatenate([[0, 1, -1, 2**40, -(2**40) + 1], rng.integers(-2_600_000, 2_600_000, 500)]).astype(np.int64)
+    y = oracle.time_encode(dt, w, b)
+    x = dt.astype(np.float32)
+    a = (w[None, :] * x[:, None]).astype(np.float32) + b[None, :]
+    assert a.dtype == np.float32
+    assert np.array_equal(y, np.cos(a.astype(np.float64)).astype(np.float32))
+    # b = 0, dt = 0 -> exactly 1; cos is even in dt when b = 0
+    y0 = oracle.time_encode(np.array([0, 5, -5], np.int64), w, np.zeros(dim, np.float32))
+    assert (y0[0] == 1).all() and np.array_equal(y0[1], y0[2])
+    # a fused multiply-add would give different bits somewhere on this input
+    fused = np.cos((w[None, :].astype(np.float64) * x[:, None].astype(np.float64) + b[None, :]).astype(np.float32).astype(np.float64)).astype(np.float32)
+    assert not np.array_equal(fused, y)
