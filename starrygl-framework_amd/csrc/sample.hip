@@ -342,8 +342,8 @@ int pick_group(const sgl_sample_params* p) {
 }
 
 size_t hop_workspace_bytes(int64_t S_max) {
-    // sized for the densest block grid: 16-lane groups, 16 slots per block
-    const int64_t blocks = ceil_div<int64_t>(S_max > 0 ? S_max : 1, BLOCK / 16);
+    // sized for the largest block grid: 64-lane groups, 4 slots per block
+    const int64_t blocks = ceil_div<int64_t>(S_max > 0 ? S_max : 1, BLOCK / 64);
     size_t b = 0;
     b += align_up((size_t)(S_max + 1) * 8) * 2;
     b += align_up((size_t)blocks * 8);
@@ -416,11 +416,11 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
     a.type = p->type; a.k = p->fanout; a.allowed_offset = p->allowed_offset;
     a.equal_root_time = p->equal_root_time; a.keep_root_time = p->keep_root_time;
     a.replace = p->replace; a.hop = p->hop; a.seed = p->seed;
-    const int64_t blocks16 = ceil_div<int64_t>(S_max > 0 ? S_max : 1, BLOCK / 16);
+    const int64_t max_blocks = ceil_div<int64_t>(S_max > 0 ? S_max : 1, BLOCK / 64);
     a.w_start = ar.take<int64_t>(S_max + 1);
     a.w_len = ar.take<int64_t>(S_max + 1);
-    a.block_sum = ar.take<int64_t>(blocks16);
-    a.block_bad = ar.take<int32_t>(blocks16);
+    a.block_sum = ar.take<int64_t>(max_blocks);
+    a.block_bad = ar.take<int32_t>(max_blocks);
     if (!ar.ok()) return fail(SGL_ENOMEM, "sample: workspace too small");
     a.root_start_ptr = out->root_start_ptr; a.root_end_ptr = out->root_end_ptr;
     a.nbr = out->neighbors; a.nbr_ts = out->neighbors_ts; a.nbr_eid = out->neighbors_eid;
