@@ -5,11 +5,12 @@
 //   (epoch << 32 | local id) and a bitmap of universe bits.  Per group
 //     mark   : ids whose table entry is not of the current epoch set their bit
 //              (atomicOr), duplicates collapse for free;
-//     reduce : per-tile popcount sums;   scan: one block scans the tile sums;
+//     reduce : per-tile popcount sums;
 //     assign : every set bit gets local id = base + rank of the bit, which is
 //              the ascending-id order the reference obtains by sort + unique;
 //              the entry, the local->global list and the cleared word are
 //              written in the same pass;
+//     commit : the call's epoch and id count become the committed ones;
 //   then one lookup launch rewrites every input array through the table.
 //   No sort, no hash probing; the result is deterministic.
 //
@@ -30,15 +31,14 @@ namespace {
 
 constexpr int BLOCK = 256;
 constexpr int MAXG = 8;
-constexpr int WPT = 8;                 // bitmap words per thread in reduce/assign
-constexpr int TILE = BLOCK * WPT;      // words per block
+constexpr int TILE = BLOCK;            // bitmap words per block in reduce/assign (one per thread)
 constexpr int SCAN_BLOCK = 1024;
+constexpr int FUSED_SCAN_MAX = 4096;   // up to this many tiles assign sums the preceding tiles itself
 constexpr size_t HEADER_BYTES = 256;
 
 struct Header {
-    uint64_t epoch;     // current epoch (low 32 bits are stamped into the table)
-    int64_t id_count;   // local ids handed out in this epoch
-    int64_t base;       // first local id of the group being numbered
+    uint64_t epoch;     // committed epoch (low 32 bits are stamped into the table)
+    int64_t id_count;   // committed number of local ids handed out in this epoch
 };
 
 struct State {
@@ -58,6 +58,21 @@ State carve(void* state, int64_t universe) {
     s.bitmap = s.table + universe;
     return s;
 }
+
+// Epoch stamp / first local id a call works with.  The header is only written
+// by commit_kernel, so every kernel of a call derives the same values from it.
+__device__ __forceinline__ uint64_t eff_epoch(const State& s, int reset) {
+    uint64_t e = s.hdr->epoch;
+    if (reset) {
+        e += 1;
+        if ((e & 0xFFFFFFFFull) == 0) e += 1;  // stamp 0 means "never mapped"
+    }
+    return e;
+}
+__device__ __forceinline__ uint32_t eff_stamp(const State& s, int reset) {
+    return (uint32_t)(eff_epoch(s, reset) & 0xFFFFFFFFull);
+}
+__device__ __forceinline__ int64_t eff_base(const State& s, int reset) { return reset ? 0 : s.hdr->id_count; }
 
 struct Arrays {
     int32_t G;
@@ -89,43 +104,28 @@ __global__ void init_state_kernel(State s) {
     if (t == 0) {
         s.hdr->epoch = 1;
         s.hdr->id_count = 0;
-        s.hdr->base = 0;
     }
 }
 
-__global__ void begin_kernel(State s, int reset, int64_t* U_dev) {
-    if (reset) {
-        uint64_t e = s.hdr->epoch + 1;
-        if ((e & 0xFFFFFFFFull) == 0) e += 1;  // stamp 0 means "never mapped"
-        s.hdr->epoch = e;
-        s.hdr->id_count = 0;
-    }
-    U_dev[1] = s.hdr->id_count;
-}
-
-__global__ __launch_bounds__(BLOCK) void mark_kernel(State s, Arrays a) {
+// Sets the bitmap bit of every id that has no local id in this epoch yet: one
+// id per thread and an unconditional fire-and-forget atomicOr.  (Measured on
+// MI355X: testing the bit first, or folding the block's ids through an LDS
+// hash set first, both lengthen the dependent chain and run 2-3x slower.)
+__global__ __launch_bounds__(BLOCK) void mark_kernel(State s, Arrays a, int reset) {
     const int64_t t = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
     int g;
     int64_t i;
     if (!locate(a, t, &g, &i)) return;
     const int64_t id = a.ids[g][i];
     if (id < 0 || id >= s.universe) return;
-    const uint32_t stamp = (uint32_t)(s.hdr->epoch & 0xFFFFFFFFull);
-    if ((uint32_t)(s.table[id] >> 32) == stamp) return;  // numbered earlier in this epoch
-    const uint64_t bit = 1ull << (id & 63);
-    // skip the atomic when the bit is already visible
-    if ((__atomic_load_n(&s.bitmap[id >> 6], __ATOMIC_RELAXED) & bit) == 0)
-        atomicOr(reinterpret_cast<unsigned long long*>(&s.bitmap[id >> 6]), (unsigned long long)bit);
+    if ((uint32_t)(s.table[id] >> 32) == eff_stamp(s, reset)) return;  // numbered earlier in this epoch
+    atomicOr(reinterpret_cast<unsigned long long*>(&s.bitmap[id >> 6]), 1ull << (id & 63));
 }
 
 __global__ __launch_bounds__(BLOCK) void reduce_kernel(State s, int64_t* tile_sum) {
     __shared__ int32_t s_w[BLOCK / WAVE];
-    const int64_t w0 = (int64_t)blockIdx.x * TILE + (int64_t)threadIdx.x * WPT;
-    int32_t c = 0;
-#pragma unroll
-    for (int q = 0; q < WPT; ++q)
-        if (w0 + q < s.words) c += __popcll(s.bitmap[w0 + q]);
-    // wave reduction, then 4 partials
+    const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
+    int32_t c = (w < s.words) ? __popcll(s.bitmap[w]) : 0;
     for (int d = WAVE / 2; d > 0; d >>= 1) c += __shfl_down(c, d);
     if (threadIdx.x % WAVE == 0) s_w[threadIdx.x / WAVE] = c;
     __syncthreads();
@@ -136,8 +136,8 @@ __global__ __launch_bounds__(BLOCK) void reduce_kernel(State s, int64_t* tile_su
     }
 }
 
-// exclusive scan of `nt` tile sums in place; advances id_count
-__global__ __launch_bounds__(SCAN_BLOCK) void scan_tiles_kernel(State s, int64_t* tile_sum, int64_t nt) {
+// exclusive scan of `nt` tile sums in place (only used beyond FUSED_SCAN_MAX tiles)
+__global__ __launch_bounds__(SCAN_BLOCK) void scan_tiles_kernel(int64_t* tile_sum, int64_t nt) {
     __shared__ int64_t s_part[SCAN_BLOCK];
     const int64_t per = ceil_div<int64_t>(nt, SCAN_BLOCK);
     const int64_t b0 = (int64_t)threadIdx.x * per;
@@ -159,52 +159,72 @@ __global__ __launch_bounds__(SCAN_BLOCK) void scan_tiles_kernel(State s, int64_t
         tile_sum[b] = run;
         run += x;
     }
-    if (threadIdx.x == SCAN_BLOCK - 1) {
-        s.hdr->base = s.hdr->id_count;
-        s.hdr->id_count += s_part[SCAN_BLOCK - 1];
-    }
+    if (threadIdx.x == SCAN_BLOCK - 1) tile_sum[nt] = s_part[SCAN_BLOCK - 1];  // grand total
 }
 
-__global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* tile_off,
-                                                       int64_t* unique_out, int64_t unique_capacity) {
+// Numbers the set bits in ascending id order.  `scanned`: tile_sum already holds
+// exclusive offsets (+ total at [nt]); otherwise it holds raw sums and the block
+// adds up the tiles before it.
+__global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* tile_sum, int64_t nt,
+                                                       int scanned, int reset, int64_t* unique_out,
+                                                       int64_t unique_capacity, int64_t* U_dev) {
+    __shared__ int64_t s_red[BLOCK / WAVE];
     __shared__ int32_t s_wave[BLOCK / WAVE];
-    const int64_t w0 = (int64_t)blockIdx.x * TILE + (int64_t)threadIdx.x * WPT;
-    uint64_t word[WPT];
-    int32_t c = 0;
-#pragma unroll
-    for (int q = 0; q < WPT; ++q) {
-        word[q] = (w0 + q < s.words) ? s.bitmap[w0 + q] : 0ull;
-        c += __popcll(word[q]);
+    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    int64_t tile_off = 0;
+    if (scanned) {
+        tile_off = tile_sum[blockIdx.x];
+    } else {
+        int64_t part = 0;
+        for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += BLOCK) part += tile_sum[b];
+        for (int d = WAVE / 2; d > 0; d >>= 1) part += shfl_i64(part, lane ^ d);  // butterfly: all lanes hold the wave sum
+        if (lane == 0) s_red[wid] = part;
+        __syncthreads();
+        for (int q = 0; q < BLOCK / WAVE; ++q) tile_off += s_red[q];
     }
-    // exclusive prefix of c inside the block: wave scan + 4 wave totals
+    const int64_t base = eff_base(s, reset);
+    const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
+    uint64_t word = (w < s.words) ? s.bitmap[w] : 0ull;
+    const int32_t c = __popcll(word);
     int32_t inc = c;
-    const int lane = threadIdx.x % WAVE;
     for (int d = 1; d < WAVE; d <<= 1) {
         const int32_t x = __shfl_up(inc, d);
         if (lane >= d) inc += x;
     }
-    if (lane == WAVE - 1) s_wave[threadIdx.x / WAVE] = inc;
+    if (lane == WAVE - 1) s_wave[wid] = inc;
     __syncthreads();
-    int32_t wave_off = 0;
-    for (int q = 0; q < (int)(threadIdx.x / WAVE); ++q) wave_off += s_wave[q];
-    if (c == 0) return;
-    int64_t local = s.hdr->base + tile_off[blockIdx.x] + wave_off + (inc - c);
-    const uint64_t stamp = (s.hdr->epoch & 0xFFFFFFFFull) << 32;
-#pragma unroll
-    for (int q = 0; q < WPT; ++q) {
-        uint64_t w = word[q];
-        if (w == 0) continue;
-        const int64_t id0 = (w0 + q) * 64;
-        while (w) {
-            const int bit = __ffsll((unsigned long long)w) - 1;
-            w &= w - 1;
-            const int64_t id = id0 + bit;
-            s.table[id] = stamp | (uint64_t)(uint32_t)local;
-            if (local < unique_capacity) unique_out[local] = id;
-            ++local;
-        }
-        s.bitmap[w0 + q] = 0;
+    int32_t wave_off = 0, block_total = 0;
+    for (int q = 0; q < BLOCK / WAVE; ++q) {
+        if (q < wid) wave_off += s_wave[q];
+        block_total += s_wave[q];
     }
+    if (blockIdx.x == nt - 1 && threadIdx.x == 0) {  // publish the counts of this call
+        U_dev[0] = base + tile_off + block_total;
+    }
+    if (c == 0) return;
+    int64_t local = base + tile_off + wave_off + (inc - c);
+    const uint64_t stamp = (uint64_t)eff_stamp(s, reset) << 32;
+    const int64_t id0 = w * 64;
+    while (word) {
+        const int bit = __ffsll((unsigned long long)word) - 1;
+        word &= word - 1;
+        const int64_t id = id0 + bit;
+        s.table[id] = stamp | (uint64_t)(uint32_t)local;
+        if (local < unique_capacity) unique_out[local] = id;
+        ++local;
+    }
+    s.bitmap[w] = 0;
+}
+
+// Makes the call's epoch and id count the committed ones.  `first`: U_dev[1]
+// (ids numbered before this call) is recorded.  `has_new` == 0: no assign ran.
+__global__ void commit_kernel(State s, int reset, int first, int has_new, int64_t* U_dev) {
+    const int64_t base = eff_base(s, reset);
+    const uint64_t epoch = eff_epoch(s, reset);
+    if (first) U_dev[1] = base;
+    if (!has_new) U_dev[0] = base;
+    s.hdr->epoch = epoch;
+    s.hdr->id_count = U_dev[0];
 }
 
 __global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a) {
@@ -221,11 +241,9 @@ __global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a) {
     a.out[g][i] = local;
 }
 
-__global__ void end_kernel(State s, int64_t* U_dev) { U_dev[0] = s.hdr->id_count; }
-
 size_t dense_workspace_bytes(int64_t universe) {
     const int64_t words = ceil_div<int64_t>(universe, 64);
-    return align_up((size_t)(ceil_div<int64_t>(words, TILE) + 1) * 8) + 256;
+    return align_up((size_t)(ceil_div<int64_t>(words, TILE) + 2) * 8) + 256;
 }
 
 }  // namespace
@@ -283,8 +301,7 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
         return fail(SGL_ENOMEM, "unique_compact: workspace %zu < %zu bytes", ws_bytes, dense_workspace_bytes(universe));
     State s = carve(state, universe);
     Arena ar(ws, ws_bytes);
-    const int64_t nt = ceil_div<int64_t>(s.words, TILE);
-    int64_t* tile_sum = ar.take<int64_t>(nt + 1);
+    const int64_t nt = ceil_div<int64_t>(s.words > 0 ? s.words : 1, TILE);
 
     Arrays all;
     all.G = G;
@@ -300,9 +317,10 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
     const int64_t total = all.start[MAXG];
     if (ceil_div<int64_t>(total, BLOCK) > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "unique_compact: too many ids");
 
-    hipLaunchKernelGGL(begin_kernel, dim3(1), dim3(1), 0, st, s, reset, U_dev);
-    SGL_LAUNCH_CHECK();
+    int64_t* tile_sum = ar.take<int64_t>(nt + 2);
+    if (!ar.ok()) return fail(SGL_ENOMEM, "unique_compact: workspace too small");
     const int n_groups = (mode == SGL_UNIQUE_SORTED) ? (G > 0 ? 1 : 0) : G;
+    int first = 1, rst = reset ? 1 : 0;
     for (int grp = 0; grp < n_groups; ++grp) {
         Arrays sub = all;
         if (mode == SGL_UNIQUE_GROUPED) {  // only array `grp`
@@ -314,21 +332,31 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
         }
         const int64_t sub_total = sub.start[sub.G];
         if (sub_total == 0 || universe == 0) continue;
-        hipLaunchKernelGGL(mark_kernel, dim3((unsigned)ceil_div<int64_t>(sub_total, BLOCK)), dim3(BLOCK), 0, st, s, sub);
+        hipLaunchKernelGGL(mark_kernel, dim3((unsigned)ceil_div<int64_t>(sub_total, BLOCK)), dim3(BLOCK), 0, st,
+                           s, sub, rst);
         SGL_LAUNCH_CHECK();
         hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
         SGL_LAUNCH_CHECK();
-        hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, s, tile_sum, nt);
+        const int scanned = nt > FUSED_SCAN_MAX ? 1 : 0;
+        if (scanned) {
+            hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, tile_sum, nt);
+            SGL_LAUNCH_CHECK();
+        }
+        hipLaunchKernelGGL(assign_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, scanned, rst,
+                           unique_out, unique_capacity, U_dev);
         SGL_LAUNCH_CHECK();
-        hipLaunchKernelGGL(assign_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, unique_out,
-                           unique_capacity);
+        hipLaunchKernelGGL(commit_kernel, dim3(1), dim3(1), 0, st, s, rst, first, 1, U_dev);
+        SGL_LAUNCH_CHECK();
+        first = 0;
+        rst = 0;  // the epoch has been opened; later groups continue it
+    }
+    if (first) {  // nothing was numbered: still open the epoch / report the counts
+        hipLaunchKernelGGL(commit_kernel, dim3(1), dim3(1), 0, st, s, rst, 1, 0, U_dev);
         SGL_LAUNCH_CHECK();
     }
     if (total > 0) {
         hipLaunchKernelGGL(lookup_kernel, dim3((unsigned)ceil_div<int64_t>(total, BLOCK)), dim3(BLOCK), 0, st, s, all);
         SGL_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(end_kernel, dim3(1), dim3(1), 0, st, s, U_dev);
-    SGL_LAUNCH_CHECK();
     return SGL_OK;
 }

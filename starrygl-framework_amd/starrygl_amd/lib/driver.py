@@ -154,24 +154,37 @@ class HotPath:
             out.finalize(*be.tolist(out.counts))
         return out
 
-    def sample_khop(self, g, roots, ts_ptr, root_ts, neg_roots, neg_ts, layers, p,
-                    finalize=True):
+    def khop_buffers(self, S0, layers, fanout):
+        """Worst-case output buffers of a k-hop call; reusable across calls."""
         be = self.be
-        R, S_pos, N_neg = int(roots.shape[0]), int(root_ts.shape[0]), int(neg_roots.shape[0])
-        S0 = S_pos + N_neg
         slot_node0, slot_ts0 = be.empty(S0), be.empty(S0)
         outs, cap = [], S0
         counts = be.zeros(3 * max(layers, 1))
         for l in range(layers):
-            outs.append(HopResult(be, cap, cap * p.fanout, counts[3 * l: 3 * l + 3]))
-            cap *= p.fanout
-        arr = (HopOut * max(layers, 1))(*[o.struct for o in outs])
-        ws, wsb = self._workspace(self.lib.sample_khop_workspace_bytes(S0, layers, p.fanout))
+            outs.append(HopResult(be, cap, cap * fanout, counts[3 * l: 3 * l + 3]))
+            cap *= fanout
+        res = KHopResult(self, slot_node0, slot_ts0, outs, counts)
+        res.S0, res.fanout = S0, fanout
+        res.structs = (HopOut * max(layers, 1))(*[o.struct for o in outs])
+        # a private workspace: calls on different buffers may overlap on different streams
+        res.ws_bytes = int(self.lib.sample_khop_workspace_bytes(S0, layers, fanout))
+        res.ws = be.empty(max(res.ws_bytes, 256), "u8")
+        return res
+
+    def sample_khop(self, g, roots, ts_ptr, root_ts, neg_roots, neg_ts, layers, p,
+                    finalize=True, out=None):
+        be = self.be
+        R, S_pos, N_neg = int(roots.shape[0]), int(root_ts.shape[0]), int(neg_roots.shape[0])
+        S0 = S_pos + N_neg
+        res = out if out is not None else self.khop_buffers(S0, layers, p.fanout)
+        if res.S0 < S0 or len(res.hops) != layers or res.fanout < p.fanout:
+            raise MemoryError("khop buffers are smaller than this call needs")
+        ws, wsb = res.ws, be.nbytes(res.ws)
         self._ck(self.lib.sample_khop(C.byref(g.view), R, be.ptr(roots), be.ptr(ts_ptr), S_pos,
                                       be.ptr(root_ts), N_neg, be.ptr(neg_roots), be.ptr(neg_ts),
-                                      layers, C.byref(p), be.ptr(slot_node0), be.ptr(slot_ts0),
-                                      arr, be.ptr(ws), wsb, be.stream()))
-        res = KHopResult(self, slot_node0, slot_ts0, outs, counts)
+                                      layers, C.byref(p), be.ptr(res.slot_node0), be.ptr(res.slot_ts0),
+                                      res.structs, be.ptr(ws), wsb, be.stream()))
+        res.S0_live = S0
         return res.finalize() if finalize else res
 
     # ------------------------------------------------------------- unique
@@ -182,7 +195,7 @@ class HotPath:
         return RemapState(st, universe)
 
     def unique_compact(self, arrays, mode=_abi.UNIQUE_SORTED, state=None, reset=True,
-                       lens_dev=None, out_arrays=None, finalize=True):
+                       lens_dev=None, out_arrays=None, finalize=True, unique_out=None, U_out=None):
         be, G = self.be, len(arrays)
         len_max = (i64 * max(G, 1))(*[int(a.shape[0]) for a in arrays])
         total = sum(len_max[:G])
@@ -196,8 +209,11 @@ class HotPath:
         cap = total if state is None else min(total + state.count_bound, state.universe)
         if state is not None and reset:
             cap = min(total, state.universe)
-        unique = be.empty(max(cap, 1))
-        U = be.zeros(2)
+        if unique_out is not None:
+            unique, cap = unique_out, int(unique_out.shape[0])
+        else:
+            unique = be.empty(max(cap, 1))
+        U = be.zeros(2) if U_out is None else U_out
         universe = 0 if state is None else state.universe
         ws, wsb = self._workspace(self.lib.unique_workspace_bytes(universe, G, len_max))
         self._ck(self.lib.unique_compact(None if state is None else be.ptr(state.buf), universe,
@@ -263,5 +279,8 @@ class KHopResult:
             c = self.hp.be.tolist(self.counts)
             for l, h in enumerate(self.hops):
                 h.finalize(*c[3 * l: 3 * l + 3])
+            S0 = getattr(self, "S0_live", None)
+            if S0 is not None:
+                self.slot_node0, self.slot_ts0 = self.slot_node0[:S0], self.slot_ts0[:S0]
             self.final = True
         return self
