@@ -90,3 +90,34 @@ def test_device_side_lengths(oracle, hot):
     u, inv = np.unique(full[0][:1234], return_inverse=True)
     assert th == u.shape[0] and np.array_equal(np_of(uh), u)
     assert np.array_equal(np_of(lh[0])[:1234], inv)
+
+
+# ------------------------------------------------------------- hash-set path
+@pytest.mark.parametrize("mode", [_abi.UNIQUE_SORTED, _abi.UNIQUE_GROUPED])
+@pytest.mark.parametrize("span,sizes", [(1000, (50, 500, 5000)), (2**40, (12_000, 120_000, 400_000)),
+                                        (2**62, (3000, 0, 7)), (3, (4096,)), (10**7, (1_000_000,))])
+def test_hash_path_matches_oracle_and_numpy(oracle, hot, mode, span, sizes):
+    """no remap state: arbitrary non-negative 63-bit ids, negative ids map to -1."""
+    rng = np.random.default_rng(len(sizes) + span % 97)
+    pool = rng.integers(0, span, max(sum(sizes) // 3, 1))            # ~3x duplication
+    arrs = [pool[rng.integers(0, pool.shape[0], s)].astype(np.int64) for s in sizes]
+    if arrs[0].shape[0] > 10:
+        arrs[0][::7] = -3
+    lo, uo, (to_, _) = oracle.unique_compact([a.copy() for a in arrs], mode, None, True)
+    lh, uh, (th, bh) = hot.unique_compact([to_dev(hot, a) for a in arrs], mode, None, True)
+    assert (th, bh) == (to_, 0)
+    assert np.array_equal(np_of(uh), uo)
+    for a, b in zip(lh, lo):
+        assert np.array_equal(np_of(a), b)
+    if mode == _abi.UNIQUE_SORTED:
+        cat = np.concatenate(arrs)
+        u = np.unique(cat[cat >= 0])
+        assert np.array_equal(uo, u)
+    for a, l in zip(arrs, lo):
+        assert np.array_equal(uo[l[a >= 0]], a[a >= 0]) and (l[a < 0] == -1).all()
+
+
+def test_hash_path_rejects_follow(hot):
+    a = to_dev(hot, np.arange(10, dtype=np.int64))
+    with pytest.raises(RuntimeError):
+        hot.unique_compact([a], _abi.UNIQUE_SORTED, None, False)
