@@ -240,6 +240,64 @@ int32_t sgl_scatter_update(const sgl_cache* c, void* hot_rw, void* cold_rw,
                            const void* values, const int64_t* ts,
                            void* stream);
 
+/* ------------------------------------------------------- chunks and seeds */
+/* Nodes grouped by chunk: chunk c owns chunk_nodes[chunk_ptr[c] ..
+ * chunk_ptr[c+1]), node ids ascending (replaces chunk_ptr_/row_idx_ of `Graph`,
+ * sample.cu.hpp:1053-1065, 1135-1146).  Synchronous; SGL_ERANGE when a node's
+ * chunk id is outside [0, num_chunks) (sample.cu.hpp:1059-1062). */
+size_t  sgl_chunk_index_workspace_bytes(int64_t n);
+int32_t sgl_chunk_index_build(int64_t n, int64_t num_chunks,
+                              const int64_t* node_chunk, int64_t* chunk_ptr,
+                              int64_t* chunk_nodes, void* workspace,
+                              size_t workspace_bytes, void* stream);
+
+/* Seed (root) extraction: every node of the selected chunks that has at least
+ * one out-edge with t_begin <= ts < t_end becomes a root, in the order of
+ * `chunks` and by ascending node id inside a chunk.  Per root: its distinct
+ * event timestamps inside the window (ts, delimited by ts_ptr) and per
+ * timestamp the ids of the events at that (node, timestamp) (q_eid, delimited
+ * by q_ptr).  Replaces Graph::get_seeds_in_chunks with filter_seeds_kernel /
+ * collect_seeds_kernel (sample.cu.hpp:517-705, 1303-1449).
+ * cand_off is the exclusive prefix of the selected chunks' sizes
+ * (cand_off[num_chunks] = n_cand).  Two calls sharing one workspace:
+ *   sgl_seeds_count -> totals[0..2] = {R roots, S timestamps, Q events};
+ *   (caller allocates roots[R], ts_ptr[R+1], ts[S], q_ptr[S+1], q_eid[Q])
+ *   sgl_seeds_fill. */
+typedef struct sgl_seed_query {
+    const int64_t* chunk_ptr;   /* device [total chunks + 1]          */
+    const int64_t* chunk_nodes; /* device [n]                          */
+    int64_t        num_chunks;  /* selected chunks                     */
+    const int64_t* chunks;      /* device [num_chunks] chunk ids       */
+    const int64_t* cand_off;    /* device [num_chunks + 1]             */
+    int64_t        n_cand;
+    int64_t        t_begin, t_end;
+} sgl_seed_query;
+
+size_t  sgl_seeds_workspace_bytes(int64_t n_cand);
+int32_t sgl_seeds_count(const sgl_tcsr* g, const sgl_seed_query* q,
+                        int64_t* totals, void* workspace,
+                        size_t workspace_bytes, void* stream);
+int32_t sgl_seeds_fill(const sgl_tcsr* g, const sgl_seed_query* q,
+                       const int64_t* totals,
+                       int64_t* roots, int64_t* ts_ptr, int64_t* ts,
+                       int64_t* q_ptr, int64_t* q_eid, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/* --------------------------------------------------------- block building */
+/* Message-flow block of one layer in CSC form (replaces the tensor algebra of
+ * AsyncBlock.to_block, starrygl/graph/graph.py:153-271, and
+ * _build_csc_from_pairs, prepare_sample.py:215-229).  The layer has S slots
+ * (= its destination nodes dst_offset .. dst_offset+S-1 of num_dst) and E
+ * sampled edges; source node of edge e is src_offset + e.
+ *   indptr[0 .. num_dst]   : 0 for dst < dst_offset, root_start_ptr beyond
+ *   indices[e]             : src_offset + e
+ *   edge_dst[e] (optional) : dst_offset + slot of e   (COO destination)
+ * S, E are read from counts[0], counts[1] of the hop (device). */
+int32_t sgl_block_build(const int64_t* root_start_ptr, const int64_t* counts,
+                        int64_t S_max, int64_t E_max, int64_t dst_offset,
+                        int64_t src_offset, int64_t* indptr, int64_t* indices,
+                        int64_t* edge_dst, void* stream);
+
 /* ----------------------------------------------------------- time encoding */
 #define SGL_DT_I64 0
 #define SGL_DT_F32 1

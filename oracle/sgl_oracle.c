@@ -573,3 +573,110 @@ int32_t sglo_time_encode(const void* dt, int32_t dt_dtype, int64_t N_max,
     }
     return SGL_OK;
 }
+
+/* ------------------------------------------------------- chunks and seeds */
+
+size_t sglo_chunk_index_workspace_bytes(int64_t n) { (void)n; return 0; }
+
+/* Reference: Graph::Graph computes each edge's source chunk from
+ * row_chunk_mapper, sorts by it first and derives chunk_ptr_/row_idx_
+ * (sample.cu.hpp:1053-1065, 1135-1146).  Rule implemented: nodes grouped by
+ * chunk id, ascending node id inside a chunk (a counting sort). */
+int32_t sglo_chunk_index_build(int64_t n, int64_t num_chunks, const int64_t* node_chunk,
+                               int64_t* chunk_ptr, int64_t* chunk_nodes, void* ws,
+                               size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (n < 0 || num_chunks < 0 || !chunk_ptr) return fail(SGL_EINVAL, "chunk_index_build: bad sizes");
+    for (int64_t v = 0; v < n; ++v)
+        if (node_chunk[v] < 0 || node_chunk[v] >= num_chunks)
+            return fail(SGL_ERANGE, "chunk_index_build: chunk id outside [0, num_chunks)");
+    for (int64_t c = 0; c <= num_chunks; ++c) chunk_ptr[c] = 0;
+    for (int64_t v = 0; v < n; ++v) chunk_ptr[node_chunk[v] + 1]++;
+    for (int64_t c = 0; c < num_chunks; ++c) chunk_ptr[c + 1] += chunk_ptr[c];
+    int64_t* fill = (int64_t*)malloc((size_t)(num_chunks + 1) * sizeof(int64_t));
+    if (!fill) return fail(SGL_ENOMEM, "malloc");
+    memcpy(fill, chunk_ptr, (size_t)(num_chunks + 1) * sizeof(int64_t));
+    for (int64_t v = 0; v < n; ++v) chunk_nodes[fill[node_chunk[v]]++] = v;
+    free(fill);
+    return SGL_OK;
+}
+
+size_t sglo_seeds_workspace_bytes(int64_t n_cand) { (void)n_cand; return 0; }
+
+/* Walks the candidates in output order and either counts (roots == NULL) or
+ * writes.  Reference: filter_seeds_kernel / collect_seeds_kernel
+ * (sample.cu.hpp:517-705): a node of a selected chunk is a root when
+ * find_time_range gives a non-empty edge range; its timestamps are the
+ * distinct ts of that range ("prefix_different_timestamp", :944-952,
+ * 1147-1162), q_ptr/q_eid list the events per (node, timestamp).  Rule
+ * implemented for the window: t_begin <= ts < t_end (the early-exit tests of
+ * find_time_range, :273, 279). */
+static int32_t seeds_walk(const sgl_tcsr* g, const sgl_seed_query* q, int64_t* totals,
+                          int64_t* roots, int64_t* ts_ptr, int64_t* ts, int64_t* q_ptr, int64_t* q_eid) {
+    int64_t R = 0, S = 0, Q = 0;
+    for (int64_t p = 0; p < q->num_chunks; ++p) {
+        const int64_t c = q->chunks[p];
+        const int64_t a = q->chunk_ptr[c], b = q->chunk_ptr[c + 1];
+        if (q->cand_off[p + 1] - q->cand_off[p] != b - a)
+            return fail(SGL_EINVAL, "seeds: cand_off is not the prefix of the selected chunk sizes");
+        for (int64_t x = a; x < b; ++x) {
+            const int64_t v = q->chunk_nodes[x];
+            const int64_t rs = g->row_ptr[v], re = g->row_ptr[v + 1];
+            const int64_t lo = lower_bound_ts(g->ts, rs, re, q->t_begin);
+            const int64_t hi = lower_bound_ts(g->ts, lo, re, q->t_end);
+            if (hi <= lo) continue;
+            if (roots) { roots[R] = v; ts_ptr[R] = S; }
+            for (int64_t e = lo; e < hi; ++e) {
+                if (e == lo || g->ts[e] != g->ts[e - 1]) {
+                    if (roots) { ts[S] = g->ts[e]; q_ptr[S] = Q; }
+                    ++S;
+                }
+                if (roots) q_eid[Q] = g->eid[e];
+                ++Q;
+            }
+            ++R;
+        }
+    }
+    if (roots) { ts_ptr[R] = S; q_ptr[S] = Q; }
+    if (totals) { totals[0] = R; totals[1] = S; totals[2] = Q; }
+    return SGL_OK;
+}
+
+int32_t sglo_seeds_count(const sgl_tcsr* g, const sgl_seed_query* q, int64_t* totals, void* ws,
+                         size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (!g || !q || !totals) return fail(SGL_EINVAL, "seeds_count: null");
+    return seeds_walk(g, q, totals, NULL, NULL, NULL, NULL, NULL);
+}
+
+int32_t sglo_seeds_fill(const sgl_tcsr* g, const sgl_seed_query* q, const int64_t* totals,
+                        int64_t* roots, int64_t* ts_ptr, int64_t* ts, int64_t* q_ptr, int64_t* q_eid,
+                        void* ws, size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream; (void)totals;
+    if (!g || !q || !ts_ptr || !q_ptr) return fail(SGL_EINVAL, "seeds_fill: null");
+    int64_t dummy;
+    if (!roots) roots = &dummy; /* R == 0 */
+    return seeds_walk(g, q, NULL, roots, ts_ptr, ts, q_ptr, q_eid);
+}
+
+/* --------------------------------------------------------- block building */
+
+/* Reference: AsyncBlock.to_block builds ('csc', (indptr, indices, [])) with
+ * indices = arange(E) + number of self-loop sources (graph.py:186-197,
+ * 228-241); _build_csc_from_pairs builds indptr by bincount + cumsum
+ * (prepare_sample.py:220-227). */
+int32_t sglo_block_build(const int64_t* root_start_ptr, const int64_t* counts, int64_t S_max,
+                         int64_t E_max, int64_t dst_offset, int64_t src_offset, int64_t* indptr,
+                         int64_t* indices, int64_t* edge_dst, void* stream) {
+    (void)stream;
+    if (!root_start_ptr || !counts || !indptr) return fail(SGL_EINVAL, "block_build: null");
+    int64_t S = counts[0] < S_max ? counts[0] : S_max, E = counts[1] < E_max ? counts[1] : E_max;
+    for (int64_t d = 0; d < dst_offset; ++d) indptr[d] = 0;
+    for (int64_t s = 0; s <= S; ++s) indptr[dst_offset + s] = root_start_ptr[s];
+    for (int64_t s = 0; s < S; ++s)
+        for (int64_t e = root_start_ptr[s]; e < root_start_ptr[s + 1] && e < E; ++e) {
+            indices[e] = src_offset + e;
+            if (edge_dst) edge_dst[e] = dst_offset + s;
+        }
+    return SGL_OK;
+}

@@ -246,3 +246,63 @@ extern "C" int32_t sgl_tcsr_build(int64_t n, int64_t m, const int64_t* src, cons
     SGL_HIP_TRY(hipStreamSynchronize(st));
     return SGL_OK;
 }
+
+namespace sgl {
+namespace {
+__global__ void chunk_range_kernel(const int64_t* __restrict__ node_chunk, int64_t n, int64_t num_chunks, int32_t* flag) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n && (node_chunk[i] < 0 || node_chunk[i] >= num_chunks)) atomicOr(flag, 1);
+}
+}  // namespace
+}  // namespace sgl
+
+extern "C" size_t sgl_chunk_index_workspace_bytes(int64_t n) {
+    if (n < 0) n = 0;
+    return 3 * align_up((size_t)(n + 1) * 8) + radix_sort_workspace_bytes(n) + 2048;
+}
+
+extern "C" int32_t sgl_chunk_index_build(int64_t n, int64_t num_chunks, const int64_t* node_chunk,
+                                         int64_t* chunk_ptr, int64_t* chunk_nodes, void* ws, size_t ws_bytes,
+                                         void* stream) {
+    if (n < 0 || num_chunks < 0 || !chunk_ptr) return fail(SGL_EINVAL, "chunk_index_build: negative size or NULL chunk_ptr");
+    if (n > 0 && (!node_chunk || !chunk_nodes)) return fail(SGL_EINVAL, "chunk_index_build: NULL array");
+    if (!ws || ws_bytes < sgl_chunk_index_workspace_bytes(n)) return fail(SGL_ENOMEM, "chunk_index_build: workspace too small");
+    if (ceil_div<int64_t>((n > num_chunks ? n : num_chunks) + 1, BLOCK) > 0x7FFFFFFFll)
+        return fail(SGL_ENOTSUP, "chunk_index_build: too many nodes");
+    hipStream_t st = as_stream(stream);
+    Arena ar(ws, ws_bytes);
+    int32_t* flag = ar.take<int32_t>(2);
+    uint64_t* key_a = ar.take<uint64_t>(n + 1);
+    uint64_t* key_b = ar.take<uint64_t>(n + 1);
+    int64_t* val_b = ar.take<int64_t>(n + 1);
+    const size_t rws_bytes = radix_sort_workspace_bytes(n);
+    void* rws = ar.take<char>(rws_bytes);
+    if (!ar.ok()) return fail(SGL_ENOMEM, "chunk_index_build: workspace too small");
+    const unsigned nb = (unsigned)ceil_div<int64_t>(n > 0 ? n : 1, BLOCK);
+    SGL_HIP_TRY(hipMemsetAsync(flag, 0, 8, st));
+    const uint64_t* skey = key_a;
+    if (n > 0) {
+        hipLaunchKernelGGL(chunk_range_kernel, dim3(nb), dim3(BLOCK), 0, st, node_chunk, n, num_chunks, flag);
+        SGL_LAUNCH_CHECK();
+        int32_t h = 0;
+        SGL_HIP_TRY(hipMemcpyAsync(&h, flag, 4, hipMemcpyDeviceToHost, st));
+        SGL_HIP_TRY(hipStreamSynchronize(st));
+        if (h) return fail(SGL_ERANGE, "chunk_index_build: chunk id outside [0, num_chunks)");
+        hipLaunchKernelGGL(iota_kernel, dim3(nb), dim3(BLOCK), 0, st, chunk_nodes, n);
+        SGL_LAUNCH_CHECK();
+        hipLaunchKernelGGL(gather_key_kernel, dim3(nb), dim3(BLOCK), 0, st, node_chunk, chunk_nodes, (int64_t)0, n, key_a);
+        SGL_LAUNCH_CHECK();
+        int in_b = 0;
+        int32_t rc = radix_sort_pairs(key_a, chunk_nodes, key_b, val_b, n, nullptr, 0,
+                                      bits_of((uint64_t)(num_chunks > 0 ? num_chunks - 1 : 0)), &in_b, rws, rws_bytes, st);
+        if (rc != SGL_OK) return rc;
+        if (in_b) {
+            SGL_HIP_TRY(hipMemcpyAsync(chunk_nodes, val_b, (size_t)n * 8, hipMemcpyDeviceToDevice, st));
+            skey = key_b;
+        }
+    }
+    hipLaunchKernelGGL(row_ptr_kernel, dim3((unsigned)ceil_div<int64_t>(n + 1, BLOCK)), dim3(BLOCK), 0, st, skey, num_chunks, n, chunk_ptr);
+    SGL_LAUNCH_CHECK();
+    SGL_HIP_TRY(hipStreamSynchronize(st));
+    return SGL_OK;
+}

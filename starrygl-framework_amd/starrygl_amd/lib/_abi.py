@@ -42,6 +42,11 @@ class Cache(C.Structure):
                 ("ts_hot", vp), ("ts_cold", vp)]
 
 
+class SeedQuery(C.Structure):
+    _fields_ = [("chunk_ptr", vp), ("chunk_nodes", vp), ("num_chunks", i64), ("chunks", vp),
+                ("cand_off", vp), ("n_cand", i64), ("t_begin", i64), ("t_end", i64)]
+
+
 P = C.POINTER
 
 # name -> (restype, argtypes); the order follows include/sgl_hot.h
@@ -63,6 +68,12 @@ PROTOTYPES = {
                              vp, i64, vp, vp, sz, vp]),
     "gather": (i32, [P(Cache), vp, i64, vp, vp, vp, vp, vp]),
     "scatter_update": (i32, [P(Cache), vp, vp, vp, vp, vp, i64, vp, vp, vp]),
+    "chunk_index_workspace_bytes": (sz, [i64]),
+    "chunk_index_build": (i32, [i64, i64, vp, vp, vp, vp, sz, vp]),
+    "seeds_workspace_bytes": (sz, [i64]),
+    "seeds_count": (i32, [P(TCSR), P(SeedQuery), vp, vp, sz, vp]),
+    "seeds_fill": (i32, [P(TCSR), P(SeedQuery), vp, vp, vp, vp, vp, vp, vp, sz, vp]),
+    "block_build": (i32, [vp, vp, i64, i64, i64, i64, vp, vp, vp, vp]),
     "time_encode": (i32, [vp, i32, i64, vp, vp, vp, i32, vp, vp]),
 }
 

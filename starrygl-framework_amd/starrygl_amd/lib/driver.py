@@ -9,7 +9,7 @@ library with the same ABI on host memory.
 import ctypes as C
 
 from . import _abi
-from ._abi import (TCSR, Cache, HopOut, SampleParams, check, i64, vp)
+from ._abi import (TCSR, Cache, HopOut, SampleParams, SeedQuery, check, i64, vp)
 
 
 class TorchBackend:
@@ -252,6 +252,40 @@ class HotPath:
                                          be.ptr(ts_hot_rw), be.ptr(ts_cold_rw), be.ptr(ids),
                                          int(ids.shape[0]), be.ptr(values), be.ptr(ts),
                                          be.stream()))
+
+    # ------------------------------------------------------ chunks / seeds
+    def chunk_index(self, n, num_chunks, node_chunk):
+        """-> (chunk_ptr[num_chunks+1], chunk_nodes[n]) on the backend's device."""
+        be = self.be
+        chunk_ptr, chunk_nodes = be.empty(num_chunks + 1), be.empty(max(n, 1))
+        ws, wsb = self._workspace(self.lib.chunk_index_workspace_bytes(n))
+        self._ck(self.lib.chunk_index_build(n, num_chunks, be.ptr(node_chunk), be.ptr(chunk_ptr),
+                                            be.ptr(chunk_nodes), be.ptr(ws), wsb, be.stream()))
+        return chunk_ptr, chunk_nodes[:n]
+
+    def seeds(self, g, chunk_ptr, chunk_nodes, chunks, cand_off, n_cand, t_begin, t_end):
+        """-> (roots, ts_ptr, ts, q_ptr, q_eid).  `cand_off` is the exclusive prefix
+        of the selected chunks' sizes, `n_cand` its last entry (host int)."""
+        be = self.be
+        q = SeedQuery(be.ptr(chunk_ptr), be.ptr(chunk_nodes), int(chunks.shape[0]), be.ptr(chunks),
+                      be.ptr(cand_off), int(n_cand), int(t_begin), int(t_end))
+        totals = be.zeros(3)
+        ws, wsb = self._workspace(self.lib.seeds_workspace_bytes(n_cand))
+        self._ck(self.lib.seeds_count(C.byref(g.view), C.byref(q), be.ptr(totals), be.ptr(ws), wsb, be.stream()))
+        R, S, Q = be.tolist(totals)
+        roots, ts_ptr, ts, q_ptr, q_eid = be.empty(R), be.empty(R + 1), be.empty(S), be.empty(S + 1), be.empty(Q)
+        self._ck(self.lib.seeds_fill(C.byref(g.view), C.byref(q), be.ptr(totals), be.ptr(roots), be.ptr(ts_ptr),
+                                     be.ptr(ts), be.ptr(q_ptr), be.ptr(q_eid), be.ptr(ws), wsb, be.stream()))
+        return roots, ts_ptr, ts, q_ptr, q_eid
+
+    # ------------------------------------------------------------- blocks
+    def block_build(self, root_start_ptr, counts, S_max, E_max, dst_offset, src_offset, with_edge_dst=False):
+        be = self.be
+        indptr, indices = be.empty(dst_offset + S_max + 1), be.empty(E_max)
+        edge_dst = be.empty(E_max) if with_edge_dst else None
+        self._ck(self.lib.block_build(be.ptr(root_start_ptr), be.ptr(counts), S_max, E_max, dst_offset,
+                                      src_offset, be.ptr(indptr), be.ptr(indices), be.ptr(edge_dst), be.stream()))
+        return indptr, indices, edge_dst
 
     # -------------------------------------------------------- time encode
     def time_encode(self, dt, w, b, dt_dtype=_abi.DT_I64, out=None, N_dev=None):

@@ -1,0 +1,253 @@
+"""Drop-in for the reference's pybind module `starrygl.lib.libstarrygl_comm`
+(csrc/srcs/starrygl/export.cu:20-253), sampler part: the same functions,
+classes, attribute names and argument order, running on libsgl_hot.so.
+
+Differences a caller can observe
+  * result attributes are views of the result's own tensors, not fresh copies
+    (export.cu:29-162 copies device-to-device on every attribute read);
+  * `root_start_ptr` / `root_end_ptr` both have S+1 entries: `root_start_ptr` is
+    the exclusive prefix (a CSC indptr), `root_end_ptr[s] = root_start_ptr[s+1]`
+    with a repeated last entry, so `ptr[:-1]` (graph.py:166-168) is per slot;
+  * `op='r'` starts a new local-id epoch and `op='f'` continues it, as
+    `AsyncGraphBlob` (graph.py:291) and the comment at sample.cu.hpp:1874 say;
+  * time windows of `get_seeds_in_chunks` are half open, [time_begin, time_end).
+"""
+import ctypes as C
+import queue
+import threading
+
+import torch
+
+from . import _abi, hot_path
+
+
+class TemporalRoot:
+    """export.cu:28-79 / sample.cu.hpp:849-871."""
+
+    def __init__(self, roots, ts_ptr, ts, q_ptr=None, q_eid=None):
+        e = roots.new_empty(0)
+        self.roots, self.ts_ptr, self.ts = roots, ts_ptr, ts
+        self.q_ptr = e if q_ptr is None else q_ptr
+        self.q_eid = e if q_eid is None else q_eid
+
+    @property
+    def root_num(self):
+        return int(self.roots.numel())
+
+    @property
+    def root_ts_num(self):
+        return int(self.ts.numel())
+
+    def __repr__(self):
+        return f"<TemporalRoot with {self.root_num} roots>"
+
+
+class NegativeRoot:
+    """export.cu:82-106 / sample.cu.hpp:872-881."""
+
+    def __init__(self, roots, ts):
+        self.roots, self.ts = roots, ts
+
+    @property
+    def root_num(self):
+        return int(self.roots.numel())
+
+    def __repr__(self):
+        return f"<NegativeRoot with {self.root_num} roots>"
+
+
+class TemporalNeighbor:
+    """export.cu:109-167 / sample.cu.hpp:882-915."""
+
+    def __init__(self, hop):
+        self.root_start_ptr, self.root_end_ptr = hop.root_start_ptr, hop.root_end_ptr
+        self.neighbors, self.neighbors_ts = hop.neighbors, hop.neighbors_ts
+        self.neighbors_eid, self.neighbors_dt = hop.neighbors_eid, hop.neighbors_dt
+
+    @property
+    def neighbor_num(self):
+        return int(self.neighbors.numel())
+
+    def __repr__(self):
+        return f"<TemporalNeighbor with {self.neighbor_num} neighbors>"
+
+
+class TemporalResult:
+    """export.cu:170-184 / sample.cu.hpp:916-934."""
+
+    def __init__(self, roots, neg_roots, neighbors_list, nodes_remapper_id=None):
+        self.roots, self.neg_roots, self.neighbors_list = roots, neg_roots, neighbors_list
+        self.nodes_remapper_id = roots.roots.new_empty(0) if nodes_remapper_id is None else nodes_remapper_id
+
+    @property
+    def neighbors(self):
+        return self.neighbors_list
+
+    def __repr__(self):
+        return f"<TemporalResult with {len(self.neighbors_list)} neighbor layers>"
+
+
+def _i64(t, device, name):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.dtype != torch.int64:
+        raise RuntimeError(f"{name} must be int64")          # sample.cu.hpp:1001-1013
+    return t.to(device).contiguous()
+
+
+class CUDAGraph:
+    """The sampler object of export.cu:186-227 on one HIP device."""
+
+    def __init__(self, hp, tcsr, chunk_size, mapper, stream=None, seed=1317):
+        self._hp, self._g = hp, tcsr
+        self._n, self._chunks = tcsr.n, int(chunk_size)
+        self._stream = stream
+        self._seed, self._queries = int(seed), 0
+        self._state = None
+        self._mapper = mapper
+        self._chunk_index = None
+        self._tasks, self._results = queue.Queue(), queue.Queue()
+        self._worker = None
+
+    # ---- direct (synchronous) entry points ---------------------------------
+    def get_negative_root(self, negative_root, negative_time):
+        dev = self._hp.be.device
+        return NegativeRoot(_i64(negative_root, dev, "negative_root"), _i64(negative_time, dev, "negative_time"))
+
+    def sample_src_in_chunks_khop(self, postive_root, negative_root, k, layers, allowed_offset, equal_root_time,
+                                  keep_root_time, sample_type, seed=None):
+        """k-hop sampling from explicit roots (sample.cu.hpp:1532-1716).  Ids in
+        the result are global; `submit_query` adds the remap."""
+        hp = self._hp
+        p = hp.params(sample_type, k, allowed_offset, equal_root_time, keep_root_time,
+                      seed=self._seed if seed is None else seed)
+        neg = negative_root if negative_root is not None else self._empty_neg()
+        res = hp.sample_khop(self._g, postive_root.roots, postive_root.ts_ptr, postive_root.ts, neg.roots, neg.ts,
+                             int(layers), p)
+        return TemporalResult(postive_root, neg, [TemporalNeighbor(h) for h in res.hops])
+
+    def get_seeds_in_chunks(self, chunks, time_begin, time_end, using_full_timestamp=False):
+        from .seeds import seeds_in_chunks
+        if using_full_timestamp:
+            raise NotImplementedError("using_full_timestamp (dense DTDG timestamps) is outside the CTDG hot path")
+        return seeds_in_chunks(self, chunks, int(time_begin), int(time_end))
+
+    def slice_by_chunk_ts(self, chunks, time_begin, time_end, using_full_timestamp=False, stream=0):
+        raise NotImplementedError("'cluster' slicing (sample.cu.hpp:1189-1299) is outside the k-hop hot path")
+
+    # ---- asynchronous FIFO pipeline (sample.cu.hpp:1856-2031) ---------------
+    def submit_query(self, time_start, time_end, chunk_list, test_generate_samples, test_generate_samples_ts,
+                     sample_type, layers, fanout, allowed_offset, equal_root_time, keep_root_time, op):
+        if sample_type == "cluster":
+            raise NotImplementedError("'cluster' sampling is outside the k-hop hot path")
+        if sample_type not in _abi.SAMPLE_TYPES:
+            raise RuntimeError("undefined sampling strategy")
+        if self._worker is None:
+            self._worker = threading.Thread(target=self._run, name="sgl-sampler", daemon=True)
+            self._worker.start()
+        fut = _Future()
+        self._results.put(fut)
+        self._tasks.put((fut, int(time_start), int(time_end), chunk_list, test_generate_samples,
+                         test_generate_samples_ts, sample_type, int(layers), int(fanout), int(allowed_offset),
+                         bool(equal_root_time), bool(keep_root_time), op, self._queries))
+        self._queries += 1
+
+    def get(self):
+        """Oldest unfinished query's result (blocks); a failed query re-raises here."""
+        return self._results.get().result()
+
+    def close(self):
+        if self._worker is not None:
+            self._tasks.put(None)
+            self._worker.join()
+            self._worker = None
+
+    def _run(self):
+        dev = self._hp.be.device
+        torch.cuda.set_device(dev)
+        stream = self._stream if isinstance(self._stream, torch.cuda.Stream) else torch.cuda.Stream(dev)
+        while True:
+            task = self._tasks.get()
+            if task is None:
+                return
+            fut = task[0]
+            try:
+                with torch.cuda.stream(stream):
+                    fut.set_result(self._execute(*task[1:]))
+            except BaseException as exc:  # forwarded to get(), like promise.set_exception
+                fut.set_exception(exc)
+
+    def _execute(self, t0, t1, chunk_list, neg_nodes, neg_ts, sample_type, layers, fanout, allowed_offset,
+                 equal_root_time, keep_root_time, op, query_index):
+        roots = self.get_seeds_in_chunks(chunk_list, t0, t1)
+        neg = self.get_negative_root(neg_nodes, neg_ts)
+        res = self.sample_src_in_chunks_khop(roots, neg, fanout, layers, allowed_offset, equal_root_time,
+                                             keep_root_time, sample_type, seed=self._seed + query_index)
+        return self.remap(res, reset=(op != "f"))
+
+    def remap(self, result, reset=True):
+        """Remapper::insert (sample.cu.hpp:1825-1852): roots, negatives and every
+        layer's neighbours become local ids, numbered per array in ascending id
+        order; nodes_remapper_id is the local -> global table of the epoch."""
+        hp = self._hp
+        if self._state is None:
+            self._state = hp.remap_state(self._n)
+            self._unique = None
+        arrays = [result.roots.roots, result.neg_roots.roots] + [l.neighbors for l in result.neighbors_list]
+        local, uniq, (total, before) = hp.unique_compact(arrays, _abi.UNIQUE_GROUPED, self._state, reset)
+        if reset or self._unique is None:
+            self._unique = uniq[:total]
+        else:
+            self._unique = torch.cat([self._unique[:before], uniq[before:total]])
+        result.roots = TemporalRoot(local[0], result.roots.ts_ptr, result.roots.ts, result.roots.q_ptr,
+                                    result.roots.q_eid)
+        result.neg_roots = NegativeRoot(local[1], result.neg_roots.ts)
+        for layer, loc in zip(result.neighbors_list, local[2:]):
+            layer.neighbors = loc
+        result.nodes_remapper_id = self._unique
+        torch.cuda.current_stream().synchronize()
+        return result
+
+    def _empty_neg(self):
+        e = torch.empty(0, dtype=torch.int64, device=self._hp.be.device)
+        return NegativeRoot(e, e)
+
+
+class _Future:
+    def __init__(self):
+        self._ev, self._val, self._exc = threading.Event(), None, None
+
+    def set_result(self, v):
+        self._val = v
+        self._ev.set()
+
+    def set_exception(self, e):
+        self._exc = e
+        self._ev.set()
+
+    def result(self):
+        self._ev.wait()
+        if self._exc is not None:
+            raise self._exc
+        return self._val
+
+
+def from_edge_index(n, chunk_size, src, dst, ts, eid, mapper=None, stream=0, rank=0):
+    """Build the T-CSR on device `rank` (export.cu:229-250).  Raises
+    RuntimeError-family exceptions for non-int64 input and out-of-range ids
+    (sample.cu.hpp:1001-1020, 1043-1062)."""
+    device = torch.device("cuda", int(rank))
+    hp = hot_path(device)
+    n, chunk_size = int(n), int(chunk_size)
+    src, dst, ts = (_i64(t, device, nm) for t, nm in ((src, "src"), (dst, "dst"), (ts, "ts")))
+    eid = None if eid is None else _i64(eid, device, "eid")
+    if not (src.numel() == dst.numel() == ts.numel()) or (eid is not None and eid.numel() != src.numel()):
+        raise RuntimeError("src, dst, ts and eid must have the same length")
+    if mapper is not None:
+        if mapper.numel() != n:
+            raise RuntimeError("row_chunk_mapper must have one entry per node")
+        if n > 0 and (int(mapper.min()) < 0 or int(mapper.max()) >= max(chunk_size, 1)):
+            raise IndexError("row_chunk_mapper names a chunk outside [0, chunk_size)")   # sample.cu.hpp:1059-1062
+    with torch.cuda.device(device):
+        g = hp.tcsr_build(n, src, dst, ts, eid)
+    return CUDAGraph(hp, g, chunk_size, mapper, stream if isinstance(stream, torch.cuda.Stream) else None)

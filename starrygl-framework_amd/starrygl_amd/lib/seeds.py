@@ -1,0 +1,40 @@
+"""Host side of seed extraction (Graph::get_seeds_in_chunks,
+csrc/include/starrygl/sample.cu.hpp:1303-1449): which chunks are selected and
+how many candidate nodes they hold is decided on the host from a host copy of
+chunk_ptr; the per-candidate work runs in libsgl_hot.so."""
+import numpy as np
+import torch
+
+
+def _chunk_index(graph):
+    """Lazily build (chunk_ptr, chunk_nodes) on the device + a host chunk_ptr."""
+    if graph._chunk_index is None:
+        hp, n, C = graph._hp, graph._n, max(graph._chunks, 1)
+        dev = hp.be.device
+        mapper = graph._mapper
+        if mapper is None:   # no mapper: every node in chunk 0
+            mapper = torch.zeros(n, dtype=torch.int64)
+        node_chunk = mapper.to(dev, torch.int64).contiguous()
+        chunk_ptr, chunk_nodes = hp.chunk_index(n, C, node_chunk)
+        graph._chunk_index = (chunk_ptr, chunk_nodes, chunk_ptr.cpu().numpy())
+    return graph._chunk_index
+
+
+def seeds_in_chunks(graph, chunks, t_begin, t_end):
+    from .libstarrygl_comm import TemporalRoot
+    hp = graph._hp
+    dev = hp.be.device
+    chunk_ptr, chunk_nodes, chunk_ptr_h = _chunk_index(graph)
+    if not isinstance(chunks, torch.Tensor):
+        raise TypeError("chunks must be a torch.Tensor")
+    chunks_h = chunks.detach().cpu().to(torch.int64).numpy().reshape(-1)
+    C = chunk_ptr_h.shape[0] - 1
+    if chunks_h.size and (chunks_h.min() < 0 or chunks_h.max() >= C):
+        raise IndexError("chunk id outside [0, chunk_size)")
+    sizes = chunk_ptr_h[chunks_h + 1] - chunk_ptr_h[chunks_h] if chunks_h.size else np.zeros(0, np.int64)
+    cand_off = np.zeros(chunks_h.size + 1, dtype=np.int64)
+    np.cumsum(sizes, out=cand_off[1:])
+    d_chunks = torch.from_numpy(chunks_h.copy()).to(dev)
+    d_off = torch.from_numpy(cand_off).to(dev)
+    out = hp.seeds(graph._g, chunk_ptr, chunk_nodes, d_chunks, d_off, int(cand_off[-1]), t_begin, t_end)
+    return TemporalRoot(*out)

@@ -1,0 +1,99 @@
+"""Host-side logic of the façade that needs no GPU: id codecs, id mappers, and
+the oracle's seed extraction / chunk index / block assembly against brute force."""
+import numpy as np
+import pytest
+import torch
+
+from starrygl_amd.utils.partition_book import DistRouteIndex, IDMapper, PartitionState
+from util import host_graph
+
+
+def test_dist_route_index_codec():
+    loc = torch.tensor([0, 5, 2**47 + 3, 2**48 - 1])
+    part = torch.tensor([0, 7, 16383, 1])
+    d = DistRouteIndex(loc, part)
+    assert torch.equal(d.loc, loc) and torch.equal(d.part, part) and not d.is_shared.any()
+    d.set_shared(torch.tensor([1, 3]))
+    assert d.is_shared.tolist() == [False, True, False, True]
+    assert torch.equal(d.loc, loc) and torch.equal(d.part, part)
+    assert torch.equal(DistRouteIndex(d.dist).dist, d.dist) and d.shape == loc.shape
+    # arithmetic spelled out
+    assert int(d.dist[1]) == 5 | (7 << 48) | (1 << 62)
+
+
+def test_idmapper_modes():
+    loc_ids = torch.tensor([10, 3, 7, 25])
+    m = IDMapper(loc_ids, num_master=2, mode="map", global_num=30)
+    assert m.to_local(torch.tensor([3, 25, 4, 10, 30])).tolist() == [1, 3, -1, 0, -1]
+    assert m.loc_nums == 4 and m.num_master == 2 and m.global_nums == 30
+    assert m.is_master_by_local(torch.tensor([0, 1, 2, -1])).tolist() == [True, True, False, False]
+    assert m.is_remote_ids(torch.tensor([10, 7, 4])).tolist() == [False, True, True]
+    assert m.is_store_local(torch.tensor([10, 7, 4])).tolist() == [True, True, False]
+    assert m.to_dist(torch.tensor([2, 0])).tolist() == [7, 10]
+    assert IDMapper(loc_ids, 4, "identity").to_local(torch.tensor([4, 9])).tolist() == [4, 9]
+    assert IDMapper(loc_ids, 4, "offset", offset=100).to_local(torch.tensor([104, 100])).tolist() == [4, 0]
+    enc = DistRouteIndex(torch.tensor([4, 9]), torch.tensor([3, 2]))
+    assert IDMapper(loc_ids, 4, "dist_route_index").to_local(enc.dist).tolist() == [4, 9]
+    assert IDMapper(loc_ids, 4, "identity").to_local(enc).tolist() == [4, 9]
+    with pytest.raises(ValueError):
+        IDMapper(loc_ids, 4, "hash")
+    dm = torch.arange(100, 104)
+    assert IDMapper(loc_ids, 4, "identity", dist_mapper=dm).to_dist(torch.tensor([1])).tolist() == [101]
+
+
+def test_partition_state():
+    st = PartitionState(torch.tensor([4, 2, 9]), 2, node_mode="map", num_nodes=10)
+    assert st.to_local_nid(torch.tensor([9, 4, 0])).tolist() == [2, 0, -1]
+    assert st.is_master_node_by_global(torch.tensor([9, 4])).tolist() == [False, True]
+    with pytest.raises(RuntimeError):
+        st.to_local_eid(torch.tensor([1]))
+    st2 = PartitionState(torch.tensor([4, 2, 9]), 2, loc_eids=torch.tensor([5, 6]), num_master_edges=1)
+    assert st2.to_local_eid(torch.tensor([6])).tolist() == [6]
+    assert st2.is_master_edge_by_local(torch.tensor([0, 1])).tolist() == [True, False]
+
+
+def _seed_brute(g, chunk_of, chunks, t0, t1):
+    roots, ts_ptr, ts, q_ptr, q_eid = [], [0], [], [0], []
+    for c in chunks:
+        for v in [v for v in range(g.n) if chunk_of[v] == c]:
+            ev = [e for e in range(g.row_ptr[v], g.row_ptr[v + 1]) if t0 <= g.ts[e] < t1]
+            if not ev:
+                continue
+            roots.append(v)
+            for t in sorted(set(g.ts[e] for e in ev)):
+                ts.append(t)
+                q_eid += [g.eid[e] for e in ev if g.ts[e] == t]
+                q_ptr.append(len(q_eid))
+            ts_ptr.append(len(ts))
+    return roots, ts_ptr, ts, q_ptr, q_eid
+
+
+def test_oracle_seeds_match_brute_force(oracle):
+    rng = np.random.default_rng(0)
+    n, m, C = 40, 600, 5
+    g = host_graph(oracle, n, rng.integers(0, n, m), rng.integers(0, n, m), rng.integers(0, 30, m))
+    chunk_of = rng.integers(0, C, n).astype(np.int64)
+    chunk_ptr, chunk_nodes = oracle.chunk_index(n, C, chunk_of)
+    assert np.array_equal(chunk_ptr, np.concatenate([[0], np.cumsum(np.bincount(chunk_of, minlength=C))]))
+    assert np.array_equal(chunk_nodes, np.argsort(chunk_of, kind="stable"))
+    for chunks, t0, t1 in [([0, 3], 5, 12), ([4, 4, 1], 0, 30), ([2], 29, 30), ([], 0, 30), ([1], 10, 10)]:
+        ch = np.array(chunks, dtype=np.int64)
+        sizes = chunk_ptr[ch + 1] - chunk_ptr[ch] if ch.size else np.zeros(0, np.int64)
+        off = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+        got = oracle.seeds(g, chunk_ptr, chunk_nodes, ch, off, int(off[-1]), t0, t1)
+        want = _seed_brute(g, chunk_of, chunks, t0, t1)
+        for a, b in zip(got, want):
+            assert a.tolist() == [int(x) for x in b]
+    with pytest.raises(IndexError):
+        oracle.chunk_index(3, 2, np.array([0, 2, 1], dtype=np.int64))
+
+
+def test_oracle_block_build(oracle):
+    rsp = np.array([0, 2, 2, 5], dtype=np.int64)
+    counts = np.array([3, 5, 0], dtype=np.int64)
+    indptr, indices, edst = oracle.block_build(rsp, counts, 3, 5, 4, 7, with_edge_dst=True)
+    assert indptr.tolist() == [0, 0, 0, 0, 0, 2, 2, 5]
+    assert indices.tolist() == [7, 8, 9, 10, 11]
+    assert edst.tolist() == [4, 4, 6, 6, 6]
+    # expanding indptr back gives edge_dst: the CSC and the COO view agree
+    assert np.repeat(np.arange(7), np.diff(indptr)).tolist() == edst.tolist()

@@ -1,0 +1,225 @@
+"""GPU: the Python façade (pyGraph / AsyncBlock / AsyncGraphBlob / DistNodeState /
+TimeEncoder / native-module mirror) against the CPU oracle and plain torch."""
+import numpy as np
+import pytest
+import torch
+
+from starrygl_amd.lib import _abi
+from starrygl_amd.utils import synth
+from util import host_graph, np_of, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def world(oracle, hot):
+    from starrygl_amd.graph.graph import pyGraph
+    n, m, C = 3000, 60_000, 8
+    src, dst, ts, eid = synth.graph_stream(n, m, 1.15, 100_000, 11)
+    rng = np.random.default_rng(1)
+    chunk_of = rng.integers(0, C, n).astype(np.int64)
+    # edges arrive shuffled: the façade builds the T-CSR itself
+    p = rng.permutation(m)
+    g = pyGraph(torch.from_numpy(src[p]), torch.from_numpy(dst[p]), torch.from_numpy(ts[p]), n, C,
+                eid=torch.from_numpy(eid[p]), chunk_mapper=torch.from_numpy(chunk_of))
+    hg = host_graph(oracle, n, src, dst, ts, eid)
+    cp, cn = oracle.chunk_index(n, C, chunk_of)
+    return dict(g=g, hg=hg, n=n, C=C, chunk_of=chunk_of, cp=cp, cn=cn, src=src, dst=dst, ts=ts)
+
+
+def _oracle_query(oracle, w, t0, t1, chunks, neg, neg_ts, policy, state, reset, seed):
+    ch = np.asarray(chunks, dtype=np.int64)
+    off = np.concatenate([[0], np.cumsum(w["cp"][ch + 1] - w["cp"][ch])]).astype(np.int64)
+    roots, ts_ptr, ts, q_ptr, q_eid = oracle.seeds(w["hg"], w["cp"], w["cn"], ch, off, int(off[-1]), t0, t1)
+    p = oracle.params(policy["sample_type"], policy["fanout"], policy.get("allowed_offset", -1),
+                      policy.get("equal_root_time", False), policy.get("keep_root_time", False), seed=seed)
+    res = oracle.sample_khop(w["hg"], roots, ts_ptr, ts, neg, neg_ts, policy["layers"], p)
+    arrays = [roots, neg] + [h.neighbors for h in res.hops]
+    local, uniq, (tot, before) = oracle.unique_compact(arrays, _abi.UNIQUE_GROUPED, state, reset)
+    return dict(roots=roots, ts_ptr=ts_ptr, ts=ts, q_ptr=q_ptr, q_eid=q_eid, res=res, local=local,
+                uniq=uniq, tot=tot, before=before)
+
+
+@pytest.mark.parametrize("sample_type", ["recent", "uniform"])
+def test_async_sample_matches_oracle_pipeline(oracle, world, sample_type):
+    g = world["g"]
+    policy = dict(sample_type=sample_type, layers=2, fanout=5, allowed_offset=-1, equal_root_time=False,
+                  keep_root_time=False)
+    rng = np.random.default_rng(5)
+    neg = rng.integers(0, world["n"], 200).astype(np.int64)
+    neg_ts = rng.integers(40_000, 60_000, 200).astype(np.int64)
+    kw = dict(test_generate_samples=torch.from_numpy(neg), test_generate_samples_ts=torch.from_numpy(neg_ts))
+    q0 = g.g._queries
+    g.async_sample(50_000, 52_000, torch.tensor([1, 5, 2]), policy, kw, op="r")
+    out = g.get_last_sample()
+    st = oracle.remap_state(world["n"])
+    want = _oracle_query(oracle, world, 50_000, 52_000, [1, 5, 2], neg, neg_ts, policy, st, True, seed=1317 + q0)
+    assert out.roots.root_num == want["roots"].shape[0] > 0
+    for f in ("ts_ptr", "ts", "q_ptr", "q_eid"):
+        assert np.array_equal(np_of(getattr(out.roots, f)), want[f]), f
+    assert np.array_equal(np_of(out.roots.roots), want["local"][0])
+    assert np.array_equal(np_of(out.neg_roots.roots), want["local"][1])
+    assert np.array_equal(np_of(out.nodes_remapper_id), want["uniq"][: want["tot"]])
+    assert len(out.neighbors) == 2 and out.neighbors is out.neighbors_list
+    for l, layer in enumerate(out.neighbors_list):
+        h = want["res"].hops[l]
+        assert np.array_equal(np_of(layer.neighbors), want["local"][2 + l])
+        for f in ("root_start_ptr", "root_end_ptr", "neighbors_ts", "neighbors_eid", "neighbors_dt"):
+            assert np.array_equal(np_of(getattr(layer, f)), getattr(h, f)), (l, f)
+        assert layer.neighbor_num == h.E
+    # local -> global round trip
+    assert np.array_equal(np_of(out.nodes_remapper_id)[np_of(out.neighbors[1].neighbors)], want["res"].hops[1].neighbors)
+
+
+def test_graph_blob_epochs_and_blocks(oracle, world):
+    from starrygl_amd.graph.graph import AsyncBlock, AsyncGraphBlob
+    g = world["g"]
+    policy = dict(sample_type="recent", layers=2, fanout=4, allowed_offset=-1, equal_root_time=False,
+                  keep_root_time=False)
+    t0s, t1s = [60_000, 61_000, 62_000], [61_000, 62_000, 63_000]
+    chunks = [torch.tensor([0, 1]), torch.tensor([2]), torch.tensor([7, 3])]
+    q0 = g.g._queries
+    blob = AsyncGraphBlob(g, t0s, t1s, chunks, policy)
+    st = oracle.remap_state(world["n"])
+    e = np.zeros(0, np.int64)
+    mapper_so_far = None
+    for i, ab in enumerate(blob.graph):
+        out = ab.value()
+        want = _oracle_query(oracle, world, t0s[i], t1s[i], chunks[i].tolist(), e, e, policy, st, i == 0, 1317 + q0 + i)
+        new = want["uniq"][want["before"]: want["tot"]]
+        mapper_so_far = new if i == 0 else np.concatenate([mapper_so_far, new])
+        assert np.array_equal(np_of(out.nodes_remapper_id), mapper_so_far)      # one id space across the blob
+        assert np.array_equal(np_of(out.roots.roots), want["local"][0])
+        root, neg, mfgs, nid = AsyncBlock.to_block(out.roots, out.neg_roots, out.neighbors, out.nodes_remapper_id)
+        assert len(mfgs) == 2
+        b1, b0 = mfgs            # reversed: outermost hop first
+        S0 = out.roots.root_ts_num
+        E0, E1 = out.neighbors[0].neighbor_num, out.neighbors[1].neighbor_num
+        assert (b0.num_dst_nodes(), b0.num_src_nodes(), b0.num_edges()) == (S0, S0 + E0, E0)
+        assert (b1.num_dst_nodes(), b1.num_src_nodes(), b1.num_edges()) == (S0 + E0, S0 + E0 + E1, E1)
+        ip0, ip1 = np_of(b0.indptr), np_of(b1.indptr)
+        assert np.array_equal(ip0, want["res"].hops[0].root_start_ptr)
+        assert np.array_equal(ip1, np.concatenate([np.zeros(S0, np.int64), want["res"].hops[1].root_start_ptr]))
+        assert np.array_equal(np_of(b1.indices), S0 + E0 + np.arange(E1))
+        # every edge of the outer block joins the sampled neighbour to the slot it was sampled for
+        nid1 = np_of(b1.srcdata["nid"])
+        dst_of_edge = np.repeat(np.arange(S0 + E0), np.diff(ip1))
+        assert np.array_equal(nid1[dst_of_edge], np.repeat(want["local"][2], np.diff(want["res"].hops[1].root_start_ptr)))
+        assert np.array_equal(np_of(b1.edata["dt"]), want["res"].hops[1].neighbors_dt)
+        assert np.array_equal(np_of(b0.srcdata["ts"])[:S0], want["ts"])
+
+
+def test_direct_khop_and_errors(oracle, world):
+    from starrygl_amd.lib.libstarrygl_comm import TemporalRoot, from_edge_index
+    g = world["g"].g
+    dev = torch.device("cuda:0")
+    roots = torch.tensor([5, 9, 100], device=dev)
+    root = TemporalRoot(roots, torch.arange(4, device=dev), torch.tensor([70_000, 80_000, 90_000], device=dev))
+    neg = g.get_negative_root(torch.tensor([1, 2]), torch.tensor([50_000, 50_001]))
+    res = g.sample_src_in_chunks_khop(root, neg, 3, 1, -1, False, False, "recent")
+    want = oracle.sample_khop(world["hg"], np.array([5, 9, 100]), np.arange(4), np.array([70_000, 80_000, 90_000]),
+                              np.array([1, 2]), np.array([50_000, 50_001]), 1, oracle.params("recent", 3))
+    assert np.array_equal(np_of(res.neighbors_list[0].neighbors), want.hops[0].neighbors)
+    with pytest.raises(RuntimeError, match="undefined sampling strategy"):
+        g.sample_src_in_chunks_khop(root, neg, 3, 1, -1, False, False, "nearest")
+    with pytest.raises(NotImplementedError):
+        g.slice_by_chunk_ts(torch.tensor([0]), 0, 1)
+    one = torch.tensor([0, 1])
+    with pytest.raises(IndexError):
+        from_edge_index(2, 1, one, torch.tensor([1, 2]), one, None)
+    with pytest.raises(RuntimeError):
+        from_edge_index(2, 1, one.int(), one, one, None)
+    with pytest.raises(IndexError):
+        from_edge_index(2, 2, one, one, one, None, torch.tensor([0, 2]))
+    # a failing query surfaces at get(), later queries still work
+    pg = world["g"]
+    pol = dict(sample_type="recent", layers=1, fanout=2)
+    pg.async_sample(0, 10, torch.tensor([99]), pol, {}, op="r")
+    pg.async_sample(0, 100_000, torch.tensor([0]), pol, {}, op="r")
+    with pytest.raises(IndexError):
+        pg.get_last_sample()
+    assert pg.get_last_sample().roots.root_num > 0
+    with pytest.raises(ValueError):
+        pg.async_sample(0, 1, torch.tensor([0]), dict(sample_type="recent", layers=1), {}, op="r")
+    with pytest.raises(TypeError):
+        pg.async_sample(0, 1, [0], pol)
+
+
+def test_neg_sampling_set():
+    from starrygl_amd.graph.graph import NegSamplingSet
+    pool = torch.arange(100, 200, device="cuda:0")
+    s = NegSamplingSet(pool).sample(50, 3)
+    assert s.shape == (50, 3) and int(s.min()) >= 100 and int(s.max()) < 200
+    with pytest.raises(TypeError):
+        NegSamplingSet([1, 2]).sample(1)
+
+
+@pytest.mark.parametrize("mode", ["identity", "map", "dist_route_index"])
+@pytest.mark.parametrize("tiered", [False, True])
+def test_dist_node_state(mode, tiered):
+    from starrygl_amd.cache.NodeState import DistNodeState
+    from starrygl_amd.utils.partition_book import DistRouteIndex, PartitionState
+    rng = np.random.default_rng(3)
+    rows, dim, G = 2000, 100, 5000
+    loc_ids = torch.from_numpy(rng.permutation(G)[:rows].astype(np.int64)) if mode == "map" else torch.arange(rows)
+    st = PartitionState(loc_ids, rows // 2, node_mode=mode, num_nodes=G)
+    hot = torch.from_numpy(rng.permutation(rows)[:300].astype(np.int64)) if tiered else None
+    ns = DistNodeState(st, dim, hot_ids=hot, ts_dtype=torch.int64 if tiered else torch.float32)
+    assert ns.data.is_pinned() and ns.data.shape == (rows, dim) and ns.ts.shape == (rows,)
+    ref_data, ref_ts = torch.zeros(rows, dim), torch.zeros(rows, dtype=ns.ts.dtype)
+    for it in range(3):
+        locs = torch.from_numpy(rng.permutation(rows)[:500].astype(np.int64))
+        gids = loc_ids[locs] if mode == "map" else locs
+        vals = torch.randn(500, dim)
+        t = torch.from_numpy(rng.integers(0, 10**6, 500)).to(ns.ts.dtype)
+        key = gids.cuda()
+        if mode == "dist_route_index":
+            key = DistRouteIndex(gids, torch.from_numpy(rng.integers(0, 8, 500))).dist.cuda()
+        ns.update(key, vals.cuda(), t.cuda())
+        ref_data[locs], ref_ts[locs] = vals, t
+        q_loc = torch.from_numpy(rng.integers(0, rows, 3000).astype(np.int64))
+        q = (loc_ids[q_loc] if mode == "map" else q_loc).cuda()
+        d, tt = ns[q]
+        assert d.is_cuda and torch.equal(d.cpu(), ref_data[q_loc]) and torch.equal(tt.cpu(), ref_ts[q_loc])
+        side = torch.cuda.Stream()
+        d2, _ = ns.prefetch(q, side)
+        side.synchronize()
+        assert torch.equal(d2.cpu(), ref_data[q_loc])
+    if mode == "map":        # ids that are not stored in this partition read as zero rows and are skipped by update
+        absent = torch.tensor(sorted(set(range(G)) - set(loc_ids.tolist()))[:7]).cuda()
+        d, tt = ns[absent]
+        assert not d.any() and not tt.any()
+        ns.update(absent, torch.ones(7, dim).cuda())
+    ns.to("cuda:0")
+    d, tt = ns[q]
+    assert torch.equal(d.cpu(), ref_data[q_loc]) and torch.equal(tt.cpu(), ref_ts[q_loc])
+    ns.reset()
+    assert not ns[q][0].any()
+
+
+def test_time_encoder_module():
+    from starrygl_amd.nn.model.time_encoder import TimeEncoder
+    enc = TimeEncoder(100).cuda()
+    assert set(enc.state_dict()) == {"w.weight", "w.bias"} and enc.w.weight.shape == (100, 1)
+    w_ref = torch.from_numpy((1.0 / 10 ** np.linspace(0, 9, 100, dtype=np.float32)).astype(np.float32))
+    assert torch.equal(enc.w.weight.detach().cpu().reshape(-1), w_ref) and not enc.w.bias.any()
+    dt = torch.randint(-2_600_000, 0, (4096,), device="cuda")
+    y = enc(dt)
+    ref = torch.cos(enc.w(dt.float().reshape(-1, 1)))
+    assert y.shape == (4096, 100) and (y - ref).abs().max().item() < 5e-4   # Linear may fuse multiply-add
+    assert enc(torch.zeros(5, device="cuda")).eq(1).all()
+    with torch.no_grad():
+        enc.w.bias.normal_()
+    y = enc(dt.reshape(64, 64))
+    ref = torch.cos(enc.w(dt.float().reshape(-1, 1)))
+    g = torch.randn_like(y)
+    gw, gb = torch.autograd.grad(y, [enc.w.weight, enc.w.bias], g)
+    rw, rb = torch.autograd.grad(ref, [enc.w.weight, enc.w.bias], g)
+    assert torch.allclose(gw, rw, rtol=1e-3, atol=1e-2 * rw.abs().max().item())
+    assert torch.allclose(gb, rb, rtol=1e-3, atol=1e-2 * rb.abs().max().item())
+    frozen = TimeEncoder(16, parameter_requires_grad=False).cuda()
+    assert not frozen.w.weight.requires_grad
+    want = 1.0 / 4.0 ** np.linspace(0, 4, 16, dtype=np.float32)
+    assert np.allclose(frozen.w.weight.detach().cpu().numpy().reshape(-1), want)
+    with pytest.raises(RuntimeError):
+        TimeEncoder(8)(torch.zeros(1))
