@@ -41,6 +41,9 @@ def main():
     ap.add_argument("--fanout", type=int, default=10)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--no-edge-feat", action="store_true", help="skip the 13.8 GB edge feature table (debug)")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run one 1 GiB device-to-device copy (known traffic) so that rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE readings can be scaled")
     ap.add_argument("--serial", action="store_true", help="capture the step as one serial chain of kernels")
     ap.add_argument("--eager", action="store_true", help="launch every kernel from the host instead of replaying a HIP graph")
     args = ap.parse_args()
@@ -148,6 +151,12 @@ def main():
     stage_inputs(0)
     body()
     torch.cuda.synchronize()
+    if args.pmc_calibration:
+        cal_src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+        cal_dst = torch.empty_like(cal_src)
+        cal_dst.copy_(cal_src)          # 1 GiB read + 1 GiB written
+        torch.cuda.synchronize()
+        del cal_src, cal_dst
     mode = "eager"
     graphs = None
     if not args.eager:
