@@ -320,7 +320,7 @@ int32_t sglo_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* roots,
                          int64_t* slot_node0, int64_t* slot_ts0,
                          const sgl_hop_out* outs, void* ws, size_t ws_bytes,
                          void* stream) {
-    if (!g || !p || !outs || R < 0 || S_pos < 0 || N_neg < 0 || layers < 0)
+    if (!g || !p || !outs || R < 0 || S_pos < 0 || N_neg < 0 || layers < 1)
         return fail(SGL_EINVAL, "sample_khop: null/negative");
     for (int64_t r = 0; r < R; ++r) {
         if (ts_ptr[r] > ts_ptr[r + 1] || ts_ptr[r] < 0 || ts_ptr[r + 1] > S_pos)

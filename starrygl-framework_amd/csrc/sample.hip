@@ -1,16 +1,25 @@
 // Temporal neighbour sampling over a T-CSR for gfx950.
 //
-// One hop = three launches on the caller's stream, no host synchronisation:
+// One hop = two (large hops: three) launches on the caller's stream, no host
+// synchronisation:
 //   count : a group of G lanes owns one (node, t) slot; the group finds the
 //           slot's candidate window with a (G+1)-ary cooperative search on the
 //           row's timestamp slice (ballot + popcount per step) and records the
-//           window start / length; the block writes the sum of its slot counts;
-//   scan  : one block turns the per-block sums into exclusive block offsets and
-//           publishes S, E and the number of out-of-range slots;
-//   fill  : the same grid copies (recent) or draws (uniform) the slot's edges
-//           into the ragged outputs with group-coalesced 8-byte accesses.
-// The slot count of hop l+1 is hop l's E, read from device memory, so a k-hop
-// call is a fixed launch sequence sized for the worst case.
+//           window start / length; a block walks a contiguous run of slots, G
+//           lanes per slot, BLOCK/G slots at a time, and writes the sum of its
+//           slot counts.  For hop 0 the slots are derived on the fly from the
+//           positive roots (expanded over their timestamp lists) and the
+//           negative roots, and written out for the caller;
+//   fill  : the same grid; a block first adds up the sums of the blocks before
+//           it (no inter-block waiting; beyond FUSED_PREFIX_MAX blocks a
+//           one-block scan kernel runs in between instead), then copies
+//           (recent) or draws (uniform) its slots' edges into the ragged
+//           outputs with group-coalesced 8-byte accesses.  The last block (or
+//           the scan kernel) publishes S, E and the number of bad slots.
+// The grid is capped at MAX_BLOCKS; the run length per block is derived on the
+// device from the live slot count, which for hop l+1 is hop l's E read from
+// device memory, so a k-hop call is a fixed launch sequence sized for the worst
+// case.
 //
 // Replaces static_recent_neighbor_num / recent_sample_single_hop_kernel /
 // static_neighbor_num / uniform_sample_single_hop_kernel and the thrust calls
@@ -20,7 +29,10 @@
 namespace sgl {
 namespace {
 
-constexpr int BLOCK = 256;
+constexpr int BLOCK = 256;          // 4 waves: 16 slots per block iteration at 16 lanes per slot
+constexpr int NWAVE = BLOCK / WAVE;
+constexpr int MAX_BLOCKS = 8192;   // grid cap of count/fill
+constexpr int FUSED_PREFIX_MAX = 1024;  // up to this many blocks a fill block adds up the sums before it itself
 constexpr int SCAN_BLOCK = 1024;
 
 struct HopArgs {
@@ -30,11 +42,23 @@ struct HopArgs {
     const int64_t* col;
     const int64_t* ts;
     const int64_t* eid;
-    // slots
+    // slots: explicit (slot_node/slot_ts), or - when roots != nullptr - derived from
+    // R positive roots over ts_ptr/root_ts followed by N_neg negatives, and then
+    // written to slot_node_out/slot_ts_out
     const int64_t* slot_node;
     const int64_t* slot_ts;
     int64_t S_max;
     const int64_t* S_dev;
+    const int64_t* roots;
+    const int64_t* ts_ptr;
+    const int64_t* root_ts;
+    const int64_t* neg_roots;
+    const int64_t* neg_ts;
+    int64_t R, S_pos;
+    int32_t derive;      // 1: slots come from roots/negatives
+    int32_t scanned;     // 1: scan_kernel wrote chunk_off and published the counts
+    int64_t* slot_node_out;
+    int64_t* slot_ts_out;
     // params
     int32_t type, k;
     int64_t allowed_offset;
@@ -43,8 +67,9 @@ struct HopArgs {
     // workspace
     int64_t* w_start;    // [S_max] first candidate position (recent: first copied edge)
     int64_t* w_len;      // [S_max] window length
-    int64_t* block_sum;  // [blocks] -> exclusive block offsets after the scan
-    int32_t* block_bad;  // [blocks]
+    int64_t* block_sum;  // [gridDim] edges counted by each block
+    int32_t* block_bad;  // [gridDim] out-of-range slots seen by each block
+    int64_t* chunk_off;  // [SCAN_BLOCK] written by scan_kernel: edges counted before each chunk of blocks
     // outputs
     int64_t* root_start_ptr;
     int64_t* root_end_ptr;
@@ -93,104 +118,173 @@ __device__ __forceinline__ int64_t group_lower_bound(const int64_t* __restrict__
     return lo;
 }
 
+// Slots [first, first + run) belong to block b; run is a multiple of the slots a
+// block handles per iteration so that iterations never straddle two blocks.
+__device__ __forceinline__ void block_run(int64_t S, int spb, int64_t* first, int64_t* run) {
+    int64_t r = ceil_div<int64_t>(S, (int64_t)gridDim.x);
+    r = ceil_div<int64_t>(r, spb) * spb;
+    if (r < spb) r = spb;
+    *run = r;
+    *first = (int64_t)blockIdx.x * r;
+}
+
+// (node, t) of slot s
+__device__ __forceinline__ void load_slot(const HopArgs& a, int64_t s, int64_t* v, int64_t* t) {
+    if (!a.derive) {
+        *v = a.slot_node[s];
+        *t = a.slot_ts[s];
+        return;
+    }
+    if (s >= a.S_pos) {
+        *v = a.neg_roots[s - a.S_pos];
+        *t = a.neg_ts[s - a.S_pos];
+        return;
+    }
+    *t = a.root_ts[s];
+    // root r with ts_ptr[r] <= s < ts_ptr[r+1].  One timestamp per root is the common
+    // case (ts_ptr[s] == s): the root is loaded speculatively beside the two pointers.
+    if (s < a.R) {
+        const int64_t p0 = a.ts_ptr[s], p1 = a.ts_ptr[s + 1], guess = a.roots[s];
+        if (p0 == s && p1 == s + 1) {
+            *v = guess;
+            return;
+        }
+    }
+    int64_t lo = 0, hi = a.R;
+    while (hi - lo > 1) {
+        const int64_t mid = lo + ((hi - lo) >> 1);
+        if (a.ts_ptr[mid] <= s) lo = mid; else hi = mid;
+    }
+    *v = a.roots[lo];
+}
+
 template <int G>
 __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
-    constexpr int SPB = BLOCK / G;  // slots per block
-    __shared__ int32_t s_cnt[SPB];
-    __shared__ int32_t s_bad[SPB];
-    const int64_t S = live_count(a.S_dev, a.S_max);
+    constexpr int SPB = BLOCK / G;  // slots per block iteration
+    __shared__ int32_t s_cnt[NWAVE];
+    __shared__ int32_t s_bad[NWAVE];
     const int gib = threadIdx.x / G;             // group in block
     const int lig = threadIdx.x % G;             // lane in group
-    const int gshift = (threadIdx.x % WAVE) / G * G;
-    const int64_t slot = (int64_t)blockIdx.x * SPB + gib;
-    if ((int64_t)blockIdx.x * SPB >= S) return;  // whole block past the live slots
-    bool active = slot < S;
-    int64_t v = 0, t = 0;
-    if (active) {
-        v = a.slot_node[slot];
-        t = a.slot_ts[slot];
-    }
-    const bool bad = active && (v < 0 || v >= a.n);
-    active = active && !bad;
-    int64_t rs = 0, re = 0;
-    if (active) {
-        rs = a.row_ptr[v];
-        re = a.row_ptr[v + 1];
-    }
-    const int64_t t_hi = t + (a.equal_root_time ? 1 : 0);
-    const int64_t hi = group_lower_bound<G>(a.ts, rs, re, t_hi, lig, gshift, active);
-    int64_t lo = rs;
-    if (a.allowed_offset >= 0)  // kernel argument: uniform across the wave
-        lo = group_lower_bound<G>(a.ts, rs, hi, t - a.allowed_offset, lig, gshift, active);
-    const int64_t len = hi - lo;
-    const int32_t c = (int32_t)(len < a.k ? len : a.k);
-    if (lig == 0) {
-        s_cnt[gib] = active ? c : 0;
-        s_bad[gib] = bad ? 1 : 0;
-        if (slot < S) {
+    const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    const int gshift = wlane / G * G;
+    // When the grid is not capped every block owns exactly SPB slots whatever the live
+    // count is: the slot can be loaded before the live count has arrived (one dependent
+    // memory round trip less).  Slots in [S, S_max) are allocated, their content is unused.
+    const bool fixed = (int64_t)gridDim.x * SPB >= a.S_max;
+    int64_t v0 = 0, t0 = 0;
+    const int64_t slot0 = (int64_t)blockIdx.x * SPB + gib;
+    if (fixed && slot0 < a.S_max) load_slot(a, slot0, &v0, &t0);
+    const int64_t S = live_count(a.S_dev, a.S_max);
+    int64_t first, run;
+    block_run(S, SPB, &first, &run);
+    int32_t sum = 0, nbad = 0;                   // per-wave partials, kept by lane 0 of each wave
+    for (int64_t it = first; it < first + run && it < S; it += SPB) {
+        const int64_t slot = it + gib;
+        bool active = slot < S;
+        int64_t v = v0, t = t0;
+        if (!fixed || it != first) {
+            v = t = 0;
+            if (active) load_slot(a, slot, &v, &t);
+        }
+        const bool bad = active && (v < 0 || v >= a.n);
+        active = active && !bad;
+        int64_t rs = 0, re = 0;
+        if (active) {
+            rs = a.row_ptr[v];
+            re = a.row_ptr[v + 1];
+        }
+        const int64_t t_hi = t + (a.equal_root_time ? 1 : 0);
+        const int64_t hi = group_lower_bound<G>(a.ts, rs, re, t_hi, lig, gshift, active);
+        int64_t lo = rs;
+        if (a.allowed_offset >= 0)  // kernel argument: uniform across the wave
+            lo = group_lower_bound<G>(a.ts, rs, hi, t - a.allowed_offset, lig, gshift, active);
+        const int64_t len = hi - lo;
+        const int32_t c = (int32_t)(len < a.k ? len : a.k);
+        if (lig == 0 && slot < S) {
             a.w_start[slot] = (a.type == SGL_SAMPLE_RECENT) ? hi - c : lo;
             a.w_len[slot] = active ? len : 0;
+            if (a.derive) {
+                a.slot_node_out[slot] = v;
+                a.slot_ts_out[slot] = t;
+            }
         }
+        // wave totals of c and of the bad flags (one contribution per group)
+        int32_t wc = (lig == 0 && active) ? c : 0;
+        int32_t wb = (lig == 0 && bad) ? 1 : 0;
+        for (int d = WAVE / 2; d > 0; d >>= 1) {
+            wc += __shfl(wc, wlane ^ d);
+            wb += __shfl(wb, wlane ^ d);
+        }
+        sum += wc;
+        nbad += wb;
+    }
+    if (wlane == 0) {
+        s_cnt[wid] = sum;
+        s_bad[wid] = nbad;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        int64_t sum = 0;
-        int32_t nbad = 0;
+        int64_t tot = 0;
+        int32_t totb = 0;
 #pragma unroll
-        for (int i = 0; i < SPB; ++i) {
-            sum += s_cnt[i];
-            nbad += s_bad[i];
+        for (int i = 0; i < NWAVE; ++i) {
+            tot += s_cnt[i];
+            totb += s_bad[i];
         }
-        a.block_sum[blockIdx.x] = sum;
-        a.block_bad[blockIdx.x] = nbad;
+        a.block_sum[blockIdx.x] = tot;
+        a.block_bad[blockIdx.x] = totb;
     }
 }
 
-// Exclusive scan of the live block sums by one block; publishes the counts and
-// the terminating entries of the two pointer arrays.
-__global__ __launch_bounds__(SCAN_BLOCK) void scan_kernel(HopArgs a, int spb) {
-    __shared__ int64_t s_part[SCAN_BLOCK];
-    __shared__ int32_t s_badp[SCAN_BLOCK];
-    const int64_t S = live_count(a.S_dev, a.S_max);
-    const int64_t nb = ceil_div<int64_t>(S, spb);
-    const int64_t per = ceil_div<int64_t>(nb, SCAN_BLOCK);
-    const int64_t b0 = (int64_t)threadIdx.x * per;
-    const int64_t b1 = b0 + per < nb ? b0 + per : nb;
-    int64_t sum = 0;
+// Prefix of the block sums at a granularity of CHUNK blocks, by one block (only
+// for grids beyond FUSED_PREFIX_MAX): chunk_off[c] = sum of block_sum[0 .. c*CHUNK).
+// Loads are coalesced and staged in LDS, thread t then owns the CHUNK consecutive
+// sums of chunk t, so a single shuffle scan over the thread totals suffices.  A
+// fill block adds the < CHUNK sums of its own chunk (one cache line) itself.
+// Publishes the counts and the terminating pointer entries.
+constexpr int CHUNK = MAX_BLOCKS / SCAN_BLOCK;
+__global__ __launch_bounds__(SCAN_BLOCK) void scan_kernel(HopArgs a, int nb) {
+    constexpr int NW = SCAN_BLOCK / WAVE;
+    __shared__ int32_t s_v[MAX_BLOCKS];
+    __shared__ int64_t s_w[NW];
+    __shared__ int32_t s_wb[NW];
+    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
     int32_t bad = 0;
-    for (int64_t b = b0; b < b1; ++b) {
-        sum += a.block_sum[b];
-        bad += a.block_bad[b];
+#pragma unroll
+    for (int r = 0; r < CHUNK; ++r) {
+        const int b = r * SCAN_BLOCK + threadIdx.x;
+        s_v[b] = b < nb ? (int32_t)a.block_sum[b] : 0;   // a block counts at most BLOCK/16 * fanout edges
+        if (b < nb) bad += a.block_bad[b];
     }
-    s_part[threadIdx.x] = sum;
-    s_badp[threadIdx.x] = bad;
+    const int64_t S = live_count(a.S_dev, a.S_max);
     __syncthreads();
-    // Hillis-Steele inclusive scan over the 1024 partials
-    for (int d = 1; d < SCAN_BLOCK; d <<= 1) {
-        int64_t x = 0;
-        int32_t y = 0;
-        if ((int)threadIdx.x >= d) {
-            x = s_part[threadIdx.x - d];
-            y = s_badp[threadIdx.x - d];
-        }
-        __syncthreads();
-        s_part[threadIdx.x] += x;
-        s_badp[threadIdx.x] += y;
-        __syncthreads();
+    int64_t sum = 0;
+#pragma unroll
+    for (int q = 0; q < CHUNK; ++q) sum += s_v[threadIdx.x * CHUNK + q];
+    int64_t inc = sum;
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const int64_t y = shfl_i64(inc, lane >= d ? lane - d : lane);
+        if (lane >= d) inc += y;
     }
-    int64_t run = s_part[threadIdx.x] - sum;  // exclusive prefix of this thread's chunk
-    for (int64_t b = b0; b < b1; ++b) {
-        const int64_t x = a.block_sum[b];
-        a.block_sum[b] = run;
-        run += x;
+    for (int d = WAVE / 2; d > 0; d >>= 1) bad += __shfl(bad, lane ^ d);
+    if (lane == WAVE - 1) s_w[wid] = inc;
+    if (lane == 0) s_wb[wid] = bad;
+    __syncthreads();
+    int64_t off = inc - sum, total = 0;
+    int32_t bad_total = 0;
+#pragma unroll
+    for (int q = 0; q < NW; ++q) {
+        if (q < wid) off += s_w[q];
+        total += s_w[q];
+        bad_total += s_wb[q];
     }
-    if (threadIdx.x == SCAN_BLOCK - 1) {
-        const int64_t E = s_part[SCAN_BLOCK - 1];
+    a.chunk_off[threadIdx.x] = off;
+    if (threadIdx.x == 0) {
         a.counts[0] = S;
-        a.counts[1] = E;
-        a.counts[2] = s_badp[SCAN_BLOCK - 1];
-        a.root_start_ptr[S] = E;
-        a.root_end_ptr[S] = E;
+        a.counts[1] = total;
+        a.counts[2] = bad_total;
+        a.root_start_ptr[S] = total;
+        a.root_end_ptr[S] = total;
     }
 }
 
@@ -218,117 +312,170 @@ __device__ __forceinline__ int64_t bounded(uint64_t bits, int64_t range) {
 template <int G>
 __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     constexpr int SPB = BLOCK / G;
-    __shared__ int64_t s_off[SPB];
-    const int64_t S = live_count(a.S_dev, a.S_max);
+    __shared__ int64_t s_red[NWAVE];
+    __shared__ int32_t s_redb[NWAVE];
+    __shared__ int32_t s_wtot[2][NWAVE];  // per-wave edge totals of an iteration, double buffered
     const int gib = threadIdx.x / G;
     const int lig = threadIdx.x % G;
-    const int gshift = (threadIdx.x % WAVE) / G * G;
-    const int wlane = threadIdx.x % WAVE;
-    const int64_t slot = (int64_t)blockIdx.x * SPB + gib;
-    if ((int64_t)blockIdx.x * SPB >= S) return;
-    const bool active = slot < S;
+    const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    const int gshift = wlane / G * G;
+    const int32_t k = a.k;
+    // first iteration's slot data: loaded before the live count arrives when the grid is
+    // not capped (see count_kernel), and before the prefix sum, so the loads overlap both
+    const bool fixed = (int64_t)gridDim.x * SPB >= a.S_max;
+    int64_t slot = (int64_t)blockIdx.x * SPB + gib;
     int64_t start = 0, len = 0, t = 0;
-    if (active) {
+    if (fixed && slot < a.S_max) {
         start = a.w_start[slot];
         len = a.w_len[slot];
-        t = a.slot_ts[slot];
+        t = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
     }
-    const int32_t k = a.k;
-    const int32_t c = (int32_t)(len < k ? len : k);
-    // exclusive prefix of c over the block's slots
-    if (lig == 0) s_off[gib] = c;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int64_t run = a.block_sum[blockIdx.x];
-#pragma unroll
-        for (int i = 0; i < SPB; ++i) {
-            const int64_t x = s_off[i];
-            s_off[i] = run;
-            run += x;
-        }
-    }
-    __syncthreads();
-    const int64_t off = s_off[gib];
-    if (active && lig == 0) {
-        a.root_start_ptr[slot] = off;
-        a.root_end_ptr[slot] = off + c;
-    }
-    if (a.type == SGL_SAMPLE_RECENT) {
+    const int64_t S = live_count(a.S_dev, a.S_max);
+    int64_t first, run;
+    block_run(S, SPB, &first, &run);
+    bool active = first < S && first + gib < S;
+    if (!fixed) {
+        slot = first + gib;
         if (active) {
-            for (int32_t j = lig; j < c; j += G) {
-                const int64_t e = start + j;
-                const int64_t ets = a.ts[e];
-                a.nbr[off + j] = a.col[e];
-                a.nbr_ts[off + j] = ets;
-                a.nbr_eid[off + j] = a.eid[e];
-                a.nbr_dt[off + j] = ets - t;
+            start = a.w_start[slot];
+            len = a.w_len[slot];
+            t = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
+        }
+    }
+    if (!active) start = len = t = 0;   // speculative loads of slots beyond the live count
+    // exclusive prefix of this block: read it (scan_kernel ran) or add up the sums of
+    // the blocks before it
+    int64_t run_off = 0;
+    if (a.scanned) {
+        constexpr int CH = MAX_BLOCKS / SCAN_BLOCK;
+        const int c0 = (int)blockIdx.x / CH * CH;
+        run_off = a.chunk_off[blockIdx.x / CH];
+#pragma unroll
+        for (int q = 0; q < CH - 1; ++q)
+            if (c0 + q < (int)blockIdx.x) run_off += a.block_sum[c0 + q];
+    } else {
+        int64_t part = 0;
+        int32_t partb = 0;
+        const bool last = blockIdx.x == gridDim.x - 1;
+        for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += BLOCK) {
+            part += a.block_sum[b];
+            if (last) partb += a.block_bad[b];
+        }
+        for (int d = WAVE / 2; d > 0; d >>= 1) {
+            part += shfl_i64(part, wlane ^ d);
+            partb += __shfl(partb, wlane ^ d);
+        }
+        if (wlane == 0) {
+            s_red[wid] = part;
+            s_redb[wid] = partb;
+        }
+        __syncthreads();
+        int32_t bad_total = 0;
+#pragma unroll
+        for (int q = 0; q < NWAVE; ++q) {
+            run_off += s_red[q];
+            bad_total += s_redb[q];
+        }
+        if (last && threadIdx.x == 0) {
+            const int64_t E = run_off + a.block_sum[blockIdx.x];
+            a.counts[0] = S;
+            a.counts[1] = E;
+            a.counts[2] = bad_total + a.block_bad[blockIdx.x];
+            a.root_start_ptr[S] = E;
+            a.root_end_ptr[S] = E;
+        }
+    }
+    int par = 0;
+    for (int64_t it = first; it < first + run && it < S; it += SPB, par ^= 1) {
+        if (it != first) {
+            slot = it + gib;
+            active = slot < S;
+            start = len = t = 0;
+            if (active) {
+                start = a.w_start[slot];
+                len = a.w_len[slot];
+                t = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
             }
         }
-        return;
-    }
-    // ---- uniform: needs k <= G (checked on the host) ------------------------
-    const bool draw = active && len > k;  // uniform inside the group
-    int64_t sel = lig;                    // offset inside the window; copy path: identity
-    int32_t rank = lig;
-    const bool any_draw = __any(draw);
-    if (any_draw) {                       // wave-uniform branch
-        int64_t tj = 0;
-        if (draw && lig < k) {
-            const uint64_t bits = draw_bits(a.seed, a.hop, slot, lig);
-            tj = a.replace ? bounded(bits, len) : bounded(bits, len - k + lig + 1);
+        const int32_t c = (int32_t)(len < k ? len : k);
+        // exclusive prefix of c over the iteration's slots: scan inside the wave (one
+        // contribution per group), then add the totals of the waves before this one
+        int32_t inc = (lig == 0) ? c : 0;
+        for (int d = 1; d < WAVE; d <<= 1) {
+            const int32_t x = __shfl_up(inc, d);
+            if (wlane >= d) inc += x;
         }
-        if (a.replace) {
-            if (draw) sel = tj;  // draw order is kept
+        if (wlane == WAVE - 1) s_wtot[par][wid] = inc;
+        // exclusive prefix at the group's first lane, broadcast to the group
+        const int32_t excl = __shfl(inc - ((lig == 0) ? c : 0), wlane - lig);
+        __syncthreads();
+        int32_t wave_off = 0, iter_total = 0;
+#pragma unroll
+        for (int q = 0; q < NWAVE; ++q) {
+            const int32_t x = s_wtot[par][q];
+            if (q < wid) wave_off += x;
+            iter_total += x;
+        }
+        const int64_t off = run_off + wave_off + excl;
+        run_off += iter_total;
+        if (active && lig == 0) {
+            a.root_start_ptr[slot] = off;
+            a.root_end_ptr[slot] = off + c;
+        }
+        if (a.type == SGL_SAMPLE_RECENT) {
+            if (active) {
+                for (int32_t j = lig; j < c; j += G) {
+                    const int64_t e = start + j;
+                    const int64_t ets = a.ts[e];
+                    a.nbr[off + j] = a.col[e];
+                    a.nbr_ts[off + j] = ets;
+                    a.nbr_eid[off + j] = a.eid[e];
+                    a.nbr_dt[off + j] = ets - t;
+                }
+            }
         } else {
-            // Floyd: step j picks t_j from [0, len-k+j]; a repeat is replaced by len-k+j
-            int64_t mine = -1;
-            for (int32_t j = 0; j < k; ++j) {
-                const int64_t cand = shfl_i64(tj, (wlane - lig) + j);
-                const bool dup = group_ballot<G>(draw && lig < j && mine == cand, gshift) != 0;
-                if (lig == j) mine = dup ? (len - k + j) : cand;
+            // ---- uniform: needs k <= G (checked on the host) ------------------------
+            const bool draw = active && len > k;  // uniform inside the group
+            int64_t sel = lig;                    // offset inside the window; copy path: identity
+            int32_t rank = lig;
+            const bool any_draw = __any(draw);
+            if (any_draw) {                       // wave-uniform branch
+                int64_t tj = 0;
+                if (draw && lig < k) {
+                    const uint64_t bits = draw_bits(a.seed, a.hop, slot, lig);
+                    tj = a.replace ? bounded(bits, len) : bounded(bits, len - k + lig + 1);
+                }
+                if (a.replace) {
+                    if (draw) sel = tj;  // draw order is kept
+                } else {
+                    // Floyd: step j picks t_j from [0, len-k+j]; a repeat is replaced by len-k+j
+                    int64_t mine = -1;
+                    for (int32_t j = 0; j < k; ++j) {
+                        const int64_t cand = shfl_i64(tj, (wlane - lig) + j);
+                        const bool dup = group_ballot<G>(draw && lig < j && mine == cand, gshift) != 0;
+                        if (lig == j) mine = dup ? (len - k + j) : cand;
+                    }
+                    // rank among the k picks (all distinct) = output position
+                    int32_t r = 0;
+                    for (int32_t j = 0; j < k; ++j) {
+                        const int64_t other = shfl_i64(mine, (wlane - lig) + j);
+                        r += (other < mine) ? 1 : 0;
+                    }
+                    if (draw) {
+                        sel = mine;
+                        rank = r;
+                    }
+                }
             }
-            // rank among the k picks (all distinct) = output position
-            int32_t r = 0;
-            for (int32_t j = 0; j < k; ++j) {
-                const int64_t other = shfl_i64(mine, (wlane - lig) + j);
-                r += (other < mine) ? 1 : 0;
-            }
-            if (draw) {
-                sel = mine;
-                rank = r;
+            if (active && lig < c) {
+                const int64_t e = start + sel;
+                const int64_t ets = a.ts[e];
+                a.nbr[off + rank] = a.col[e];
+                a.nbr_ts[off + rank] = a.keep_root_time ? t : ets;
+                a.nbr_eid[off + rank] = a.eid[e];
+                a.nbr_dt[off + rank] = ets - t;
             }
         }
-    }
-    if (active && lig < c) {
-        const int64_t e = start + sel;
-        const int64_t ets = a.ts[e];
-        a.nbr[off + rank] = a.col[e];
-        a.nbr_ts[off + rank] = a.keep_root_time ? t : ets;
-        a.nbr_eid[off + rank] = a.eid[e];
-        a.nbr_dt[off + rank] = ets - t;
-    }
-}
-
-// Hop-0 slots: positives expanded over their timestamp lists, then negatives.
-__global__ void expand_roots_kernel(int64_t R, const int64_t* __restrict__ roots,
-                                    const int64_t* __restrict__ ts_ptr, int64_t S_pos,
-                                    const int64_t* __restrict__ root_ts, int64_t N_neg,
-                                    const int64_t* __restrict__ neg_roots,
-                                    const int64_t* __restrict__ neg_ts, int64_t* slot_node,
-                                    int64_t* slot_ts) {
-    const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (s < S_pos) {
-        // last r with ts_ptr[r] <= s
-        int64_t lo = 0, hi = R;  // answer in [lo, hi)
-        while (hi - lo > 1) {
-            const int64_t mid = lo + ((hi - lo) >> 1);
-            if (ts_ptr[mid] <= s) lo = mid; else hi = mid;
-        }
-        slot_node[s] = roots[lo];
-        slot_ts[s] = root_ts[s];
-    } else if (s < S_pos + N_neg) {
-        slot_node[s] = neg_roots[s - S_pos];
-        slot_ts[s] = neg_ts[s - S_pos];
     }
 }
 
@@ -342,12 +489,11 @@ int pick_group(const sgl_sample_params* p) {
 }
 
 size_t hop_workspace_bytes(int64_t S_max) {
-    // sized for the largest block grid: 64-lane groups, 4 slots per block
-    const int64_t blocks = ceil_div<int64_t>(S_max > 0 ? S_max : 1, BLOCK / 64);
     size_t b = 0;
     b += align_up((size_t)(S_max + 1) * 8) * 2;
-    b += align_up((size_t)blocks * 8);
-    b += align_up((size_t)blocks * 4);
+    b += align_up((size_t)MAX_BLOCKS * 8);
+    b += align_up((size_t)MAX_BLOCKS * 4);
+    b += align_up((size_t)SCAN_BLOCK * 8);
     return b + 1024;
 }
 
@@ -385,42 +531,52 @@ int32_t check_out(const sgl_hop_out* o, int64_t S_max, int32_t k) {
 }
 
 template <int G>
-int32_t launch_hop(const HopArgs& a, hipStream_t st) {
+int32_t launch_hop(HopArgs a, hipStream_t st) {
     constexpr int SPB = BLOCK / G;
-    const int64_t blocks64 = ceil_div<int64_t>(a.S_max > 0 ? a.S_max : 1, SPB);
-    if (blocks64 > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "sample: too many slots for one launch");
-    const unsigned blocks = (unsigned)blocks64;
-    if (a.S_max > 0) {
-        hipLaunchKernelGGL(count_kernel<G>, dim3(blocks), dim3(BLOCK), 0, st, a);
-        SGL_LAUNCH_CHECK();
-    }
-    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, a, SPB);
+    int64_t blocks = ceil_div<int64_t>(a.S_max > 0 ? a.S_max : 1, SPB);
+    if (blocks > MAX_BLOCKS) blocks = MAX_BLOCKS;
+    a.scanned = blocks > FUSED_PREFIX_MAX ? 1 : 0;
+    hipLaunchKernelGGL(count_kernel<G>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
     SGL_LAUNCH_CHECK();
-    if (a.S_max > 0 && a.k > 0) {
-        hipLaunchKernelGGL(fill_kernel<G>, dim3(blocks), dim3(BLOCK), 0, st, a);
+    if (a.scanned) {
+        hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, a, (int)blocks);
         SGL_LAUNCH_CHECK();
     }
+    hipLaunchKernelGGL(fill_kernel<G>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
+    SGL_LAUNCH_CHECK();
     return SGL_OK;
 }
 
-int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot_ts, int64_t S_max,
-                const int64_t* S_dev, const sgl_sample_params* p, const sgl_hop_out* out, void* ws,
+struct RootSpec {  // hop-0 slot source of the k-hop driver
+    int64_t R, S_pos;
+    const int64_t *roots, *ts_ptr, *root_ts, *neg_roots, *neg_ts;
+    int64_t *slot_node_out, *slot_ts_out;
+};
+
+int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot_ts, const RootSpec* derive,
+                int64_t S_max, const int64_t* S_dev, const sgl_sample_params* p, const sgl_hop_out* out, void* ws,
                 size_t ws_bytes, hipStream_t st) {
-    if (S_max > 0 && (!slot_node || !slot_ts)) return fail(SGL_EINVAL, "sample: slot array is NULL");
+    if (!derive && S_max > 0 && (!slot_node || !slot_ts)) return fail(SGL_EINVAL, "sample: slot array is NULL");
     if (ws_bytes < hop_workspace_bytes(S_max) || !ws)
         return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, hop_workspace_bytes(S_max));
     Arena ar(ws, ws_bytes);
-    HopArgs a;
+    HopArgs a{};
     a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid;
     a.slot_node = slot_node; a.slot_ts = slot_ts; a.S_max = S_max; a.S_dev = S_dev;
+    a.derive = derive ? 1 : 0;
+    if (derive) {
+        a.R = derive->R; a.S_pos = derive->S_pos; a.roots = derive->roots; a.ts_ptr = derive->ts_ptr;
+        a.root_ts = derive->root_ts; a.neg_roots = derive->neg_roots; a.neg_ts = derive->neg_ts;
+        a.slot_node_out = derive->slot_node_out; a.slot_ts_out = derive->slot_ts_out;
+    }
     a.type = p->type; a.k = p->fanout; a.allowed_offset = p->allowed_offset;
     a.equal_root_time = p->equal_root_time; a.keep_root_time = p->keep_root_time;
     a.replace = p->replace; a.hop = p->hop; a.seed = p->seed;
-    const int64_t max_blocks = ceil_div<int64_t>(S_max > 0 ? S_max : 1, BLOCK / 64);
     a.w_start = ar.take<int64_t>(S_max + 1);
     a.w_len = ar.take<int64_t>(S_max + 1);
-    a.block_sum = ar.take<int64_t>(max_blocks);
-    a.block_bad = ar.take<int32_t>(max_blocks);
+    a.block_sum = ar.take<int64_t>(MAX_BLOCKS);
+    a.block_bad = ar.take<int32_t>(MAX_BLOCKS);
+    a.chunk_off = ar.take<int64_t>(SCAN_BLOCK);
     if (!ar.ok()) return fail(SGL_ENOMEM, "sample: workspace too small");
     a.root_start_ptr = out->root_start_ptr; a.root_end_ptr = out->root_end_ptr;
     a.nbr = out->neighbors; a.nbr_ts = out->neighbors_ts; a.nbr_eid = out->neighbors_eid;
@@ -449,7 +605,7 @@ extern "C" int32_t sgl_sample_hop(const sgl_tcsr* g, const int64_t* slot_node, c
     if ((rc = check_params(p)) != SGL_OK) return rc;
     if (S_max < 0) return fail(SGL_EINVAL, "sample_hop: S_max < 0");
     if ((rc = check_out(out, S_max, p->fanout)) != SGL_OK) return rc;
-    return run_hop(g, slot_node, slot_ts, S_max, S_dev, p, out, ws, ws_bytes, as_stream(stream));
+    return run_hop(g, slot_node, slot_ts, nullptr, S_max, S_dev, p, out, ws, ws_bytes, as_stream(stream));
 }
 
 static int64_t worst_slots(int64_t S0, int32_t layer, int32_t k) {
@@ -480,7 +636,7 @@ extern "C" int32_t sgl_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* 
     int32_t rc;
     if ((rc = check_graph(g)) != SGL_OK) return rc;
     if ((rc = check_params(p)) != SGL_OK) return rc;
-    if (R < 0 || S_pos < 0 || N_neg < 0 || layers < 0) return fail(SGL_EINVAL, "sample_khop: negative size");
+    if (R < 0 || S_pos < 0 || N_neg < 0 || layers < 1) return fail(SGL_EINVAL, "sample_khop: negative size or layers < 1");
     if (S_pos > 0 && (R == 0 || !roots || !ts_ptr || !root_ts))
         return fail(SGL_EINVAL, "sample_khop: positive root array is NULL");
     if (N_neg > 0 && (!neg_roots || !neg_ts)) return fail(SGL_EINVAL, "sample_khop: negative root array is NULL");
@@ -493,20 +649,15 @@ extern "C" int32_t sgl_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* 
         if ((rc = check_out(&outs[l], s, p->fanout)) != SGL_OK) return rc;
     }
     hipStream_t st = as_stream(stream);
-    if (S0 > 0) {
-        const unsigned blocks = (unsigned)ceil_div<int64_t>(S0, 256);
-        hipLaunchKernelGGL(expand_roots_kernel, dim3(blocks), dim3(256), 0, st, R, roots, ts_ptr, S_pos,
-                           root_ts, N_neg, neg_roots, neg_ts, slot_node0, slot_ts0);
-        SGL_LAUNCH_CHECK();
-    }
-    const int64_t* sn = slot_node0;
-    const int64_t* stt = slot_ts0;
+    RootSpec spec{R, S_pos, roots, ts_ptr, root_ts, neg_roots, neg_ts, slot_node0, slot_ts0};
+    const int64_t* sn = nullptr;
+    const int64_t* stt = nullptr;
     const int64_t* S_dev = nullptr;
     for (int32_t l = 0; l < layers; ++l) {
         sgl_sample_params pl = *p;
         pl.hop = l;
         const int64_t s_max = worst_slots(S0, l, p->fanout);
-        rc = run_hop(g, sn, stt, s_max, S_dev, &pl, &outs[l], ws, ws_bytes, st);
+        rc = run_hop(g, sn, stt, l == 0 ? &spec : nullptr, s_max, S_dev, &pl, &outs[l], ws, ws_bytes, st);
         if (rc != SGL_OK) return rc;
         sn = outs[l].neighbors;
         stt = outs[l].neighbors_ts;
