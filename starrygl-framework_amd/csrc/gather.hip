@@ -58,7 +58,10 @@ __device__ __forceinline__ const char* resolve(const sgl_cache& c, int64_t id, i
     return static_cast<const char*>(c.cold) + key * c.row_bytes;
 }
 
-template <typename V>
+// NT: non-temporal loads and stores, for outputs much larger than the last-level
+// cache (measured: +5..13 % beyond ~0.5 GB, -15 % at 70 MB, so small calls keep
+// the cached path where repeated rows hit in L2).
+template <typename V, bool NT>
 __global__ __launch_bounds__(BLOCK) void gather_kernel(GatherArgs a) {
     extern __shared__ const char* s_src[];  // [rpb]
     __shared__ int32_t s_tier[3];
@@ -89,14 +92,17 @@ __global__ __launch_bounds__(BLOCK) void gather_kernel(GatherArgs a) {
                 const int32_t r = lc / cpr;
                 const int32_t part = lc - r * cpr;
                 const V* src = reinterpret_cast<const V*>(s_src[r]);
-                if (src != nullptr) v = src[part];
+                if (src != nullptr) v = NT ? __builtin_nontemporal_load(src + part) : src[part];
             }
             val[u] = v;
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int32_t lc = base + u * BLOCK + threadIdx.x;
-            if (lc < total) dst[lc] = val[u];
+            if (lc < total) {
+                if (NT) __builtin_nontemporal_store(val[u], dst + lc);
+                else dst[lc] = val[u];
+            }
         }
     }
     if (a.stats != nullptr && threadIdx.x < 3 && s_tier[threadIdx.x] != 0)
@@ -205,11 +211,12 @@ extern "C" int32_t sgl_gather(const sgl_cache* c, const int64_t* ids, int64_t N_
     if (blocks > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "gather: too many rows for one launch");
     const size_t shmem = (size_t)rpb * sizeof(char*);
     hipStream_t st = as_stream(stream);
-    switch (vec) {
-        case 16: hipLaunchKernelGGL(gather_kernel<u32x4>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
-        case 8: hipLaunchKernelGGL(gather_kernel<u32x2>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
-        default: hipLaunchKernelGGL(gather_kernel<uint32_t>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
-    }
+    const bool nt = (double)N_max * (double)c->row_bytes >= 256.0 * 1024 * 1024;
+    const dim3 grid((unsigned)blocks), blk(BLOCK);
+    if (vec == 16 && nt) hipLaunchKernelGGL((gather_kernel<u32x4, true>), grid, blk, shmem, st, a);
+    else if (vec == 16) hipLaunchKernelGGL((gather_kernel<u32x4, false>), grid, blk, shmem, st, a);
+    else if (vec == 8) hipLaunchKernelGGL((gather_kernel<u32x2, false>), grid, blk, shmem, st, a);
+    else hipLaunchKernelGGL((gather_kernel<uint32_t, false>), grid, blk, shmem, st, a);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }

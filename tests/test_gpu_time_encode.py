@@ -43,3 +43,19 @@ def test_time_encode_f32_input_and_device_count(oracle, hot):
                     out=out, N_dev=n_dev)
     got = np_of(out)
     assert np.abs(got[:777] - want[:777]).max() <= TOL and not got[777:].any()
+
+
+def test_time_encode_is_within_one_ulp_everywhere(oracle, hot):
+    """denser check of the in-kernel cosine: <= 1 ulp (1.2e-7 absolute, |y| <= 1) against the
+    correctly rounded oracle over small, mid-range and huge arguments, including the
+    library fallback beyond 2^45."""
+    rng = np.random.default_rng(0)
+    dt = np.concatenate([rng.integers(-50, 50, 2000), rng.integers(-10**7, 10**7, 20_000),
+                         rng.integers(-2**44, 2**44, 20_000), rng.integers(-2**62, 2**62, 2000),
+                         np.array([2**45, 2**46, -(2**63) + 1, 2**63 - 1])]).astype(np.int64)
+    w, b = _w(100), rng.standard_normal(100).astype(np.float32)
+    want = oracle.time_encode(dt, w, b)
+    got = np_of(hot.time_encode(to_dev(hot, dt), to_dev(hot, w, "f32"), to_dev(hot, b, "f32")))
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    assert err.max() <= 1.2e-7, err.max()
+    assert (got == want).mean() > 0.99
