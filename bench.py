@@ -30,6 +30,196 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def _time_launches(torch, fn, reps=10, warm=2):
+    """Average duration (ms) of `fn` launched `reps` times back to back between one
+    pair of HIP events on the current stream."""
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def workload_cache_stress(hot, torch, np, synth, rows=50_000_000, dim=128, n_req=2_000_000, hot_frac=0.10):
+    """configs[2]: 50M x 128 bf16 table, hottest 10 % of rows (Zipf(1.1) access rank) in HBM,
+    the rest in pinned host memory, 2M Zipf(1.1) requests per batch."""
+    dev = hot.be.device
+    row_bytes = dim * 2
+    hot_rows = int(rows * hot_frac)
+    t0 = time.time()
+    # access rank r -> row id through an affine permutation (odd multiplier mod 2^k would need a
+    # power-of-two table; a random offset rotation keeps hot rows non-contiguous in id space)
+    g = torch.Generator(device=dev).manual_seed(3)
+    rank_to_id = torch.randperm(rows, device=dev, generator=g)
+    hot_slot = torch.full((rows,), -1, dtype=torch.int32, device=dev)
+    hot_slot[rank_to_id[:hot_rows]] = torch.arange(hot_rows, dtype=torch.int32, device=dev)
+    # row content: bf16 bit pattern derived from the row id (any bit pattern is a valid payload)
+    def content(ids):
+        base = (ids * 2654435761 % 65521).to(torch.int32).unsqueeze(1)
+        return ((base + torch.arange(dim, device=dev, dtype=torch.int32)) & 0x7FFF).to(torch.int16)
+    hot_tab = torch.empty((hot_rows, dim), dtype=torch.int16, device=dev)
+    for lo in range(0, hot_rows, 1 << 20):
+        hot_tab[lo: lo + (1 << 20)] = content(rank_to_id[lo: min(lo + (1 << 20), hot_rows)])
+    cold = torch.empty((rows, dim), dtype=torch.int16, pin_memory=True)
+    for lo in range(0, rows, 1 << 22):
+        hi = min(lo + (1 << 22), rows)
+        cold[lo:hi].copy_(content(torch.arange(lo, hi, device=dev)))
+    torch.cuda.synchronize()
+    log(f"[c3] tables ready in {time.time() - t0:.1f}s (hot {hot_rows * row_bytes / 1e9:.2f} GB HBM, cold {rows * row_bytes / 1e9:.1f} GB pinned)")
+    cache = hot.cache(row_bytes, hot_tab, rows=rows, cold=cold, hot_slot=hot_slot)
+    ranks = torch.from_numpy(synth.zipf_requests(rows, n_req, 1.1, 5)).to(dev)
+    ids_mixed = rank_to_id[ranks]
+    ids_hit = rank_to_id[ranks[ranks < hot_rows]][: n_req]
+    if ids_hit.numel() < n_req:
+        ids_hit = ids_hit.repeat((n_req + ids_hit.numel() - 1) // ids_hit.numel())[:n_req]
+    miss_ranks = ranks[ranks >= hot_rows]
+    ids_miss = rank_to_id[miss_ranks]
+    out = torch.empty((n_req, dim), dtype=torch.int16, device=dev)
+    stats = hot.be.zeros(3)
+    hot.gather(cache, ids_mixed, out, stats=stats)
+    n_hot, n_cold, n_abs = stats.cpu().tolist()
+    # byte-exact check of a sample against the generating formula
+    chk = torch.arange(0, n_req, 97, device=dev)
+    assert torch.equal(out[chk], content(ids_mixed[chk])), "cache stress gather: output differs from the table content"
+    dup = 1.0 - torch.unique(ids_mixed).numel() / n_req
+    per_row = 8 + 4 + 2 * row_bytes          # id + index entry + row read + row written
+    res = {"rows": rows, "row_bytes": row_bytes, "requests": n_req, "hit_fraction": n_hot / n_req,
+           "duplicate_fraction": round(dup, 4)}
+    ms = _time_launches(torch, lambda: hot.gather(cache, ids_hit, out))
+    res["all_hit"] = {"ms": round(ms, 4), "GBps": round(n_req * per_row / ms / 1e6, 1),
+                      "frac_of_hbm_peak": round(n_req * per_row / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    ms = _time_launches(torch, lambda: hot.gather(cache, ids_mixed, out), reps=5)
+    res["mixed"] = {"ms": round(ms, 4), "GBps": round(n_req * per_row / ms / 1e6, 1)}
+    if ids_miss.numel() > 0:
+        om = out[: ids_miss.numel()]
+        ms = _time_launches(torch, lambda: hot.gather(cache, ids_miss, om), reps=5)
+        res["miss_only"] = {"rows": int(ids_miss.numel()), "ms": round(ms, 4),
+                            "host_read_GBps": round(ids_miss.numel() * row_bytes / ms / 1e6, 2)}
+        # the practical PCIe roof: one pinned -> device copy of the same number of bytes
+        nb = ids_miss.numel()
+        ms = _time_launches(torch, lambda: om.copy_(cold[:nb], non_blocking=True), reps=5)
+        res["miss_only"]["memcpy_h2d_same_bytes_GBps"] = round(nb * row_bytes / ms / 1e6, 2)
+    return res
+
+
+def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=2000, k=10, remote=0.30, steps=30):
+    """configs[4]: one GPU's share of a partitioned TGN step: 1-hop recent-10 sampling, gather of
+    memory (+ int64 last update), node and edge features, cos time encoding to 100 dims.  30 % of
+    the node rows (memory, node features) are served from pinned host memory; edge features are
+    all HBM resident here (a 41 GB pinned mirror is not allocated)."""
+    dev = hot.be.device
+    t0 = time.time()
+    src, dst, ts, eid, row_ptr = synth.graph_by_degree(n, m, 1.1, 1 << 40, 20245)
+    D = lambda a, dt="i64": hot.be.asarray(a, dt)
+    dg = hot.tcsr_from_sorted(n, D(row_ptr), D(dst), D(ts), D(eid), validate=False)
+    gen = torch.Generator(device=dev).manual_seed(5)
+    rng = np.random.default_rng(9)
+    is_remote = torch.from_numpy(rng.random(n) < remote)
+    local_ids = torch.nonzero(~is_remote).reshape(-1)
+    slot = torch.full((n,), -1, dtype=torch.int32)
+    slot[local_ids] = torch.arange(local_ids.numel(), dtype=torch.int32)
+    slot = slot.to(dev)
+
+    def tiered(full_dev):      # -> (cache, keep-alive)
+        cold = torch.empty(full_dev.shape, dtype=full_dev.dtype, pin_memory=True)
+        cold.copy_(full_dev)
+        hot_t = full_dev[local_ids.to(dev)].contiguous()
+        return hot_t, cold
+
+    mem = torch.randn((n, 100), device=dev, generator=gen)
+    mem_ts = torch.randint(0, 1 << 40, (n,), device=dev, generator=gen)
+    nfeat = torch.randn((n, 100), device=dev, generator=gen)
+    mem_hot, mem_cold = tiered(mem)
+    ts_hot, ts_cold = tiered(mem_ts)
+    nf_hot, nf_cold = tiered(nfeat)
+    c_mem = hot.cache(400, mem_hot, rows=n, cold=mem_cold, hot_slot=slot, ts_hot=ts_hot, ts_cold=ts_cold)
+    c_nf = hot.cache(400, nf_hot, rows=n, cold=nf_cold, hot_slot=slot)
+    del mem, nfeat
+    efeat = torch.empty((m, 172), device=dev)
+    for lo in range(0, m, 1 << 22):
+        efeat[lo: lo + (1 << 22)].normal_(generator=gen)
+    c_ef = hot.cache(688, efeat)
+    torch.cuda.synchronize()
+    log(f"[c5] graph + tables ready in {time.time() - t0:.1f}s")
+    order = np.argsort(ts, kind="stable")
+    NB = 16
+    starts = np.sort(rng.integers(m // 2, m - B, NB))
+    bt = [synth.link_batch(src[order[s: s + B]], dst[order[s: s + B]], ts[order[s: s + B]], 0, B, n, B, rng) for s in starts]
+    roots, root_ts = D(np.stack([b[0] for b in bt])), D(np.stack([b[2] for b in bt]))
+    neg, neg_ts = D(np.stack([b[3] for b in bt])), D(np.stack([b[4] for b in bt]))
+    ts_ptr = D(bt[0][1])
+    S0 = 3 * B
+    p = hot.params("recent", k)
+    kr = hot.khop_buffers(S0, 1, k)
+    state = hot.remap_state(n)
+    local = [hot.be.empty(S0), hot.be.empty(S0 * k)]
+    ubuf, U = hot.be.empty(S0 + S0 * k), hot.be.zeros(2)
+    S0_dev = D(np.array([S0], dtype=np.int64))
+    o_mem = torch.empty((S0 + S0 * k, 100), device=dev)
+    o_ts = hot.be.empty(S0 + S0 * k)
+    o_nf = torch.empty((S0 + S0 * k, 100), device=dev)
+    o_ef = torch.empty((S0 * k, 172), device=dev)
+    w = torch.from_numpy((1.0 / 10 ** np.linspace(0, 9, 100, dtype=np.float32)).astype(np.float32)).to(dev)
+    bias = torch.zeros(100, device=dev)
+    o_te = torch.empty((S0 * k, 100), device=dev)
+    s_in = [torch.empty_like(x[0]) for x in (roots, root_ts, neg, neg_ts)]
+    hot._workspace(hot.lib.unique_workspace_bytes(n, 2, (_abi.i64 * 2)(S0, S0 * k)))
+    E = kr.hops[0].counts[1:2]
+    acc = torch.zeros(2, dtype=torch.int64, device=dev)
+
+    def body():
+        hot.sample_khop(dg, s_in[0], ts_ptr, s_in[1], s_in[2], s_in[3], 1, p, finalize=False, out=kr)
+        hot.unique_compact([kr.slot_node0, kr.hops[0].neighbors], _abi.UNIQUE_SORTED, state, True,
+                           lens_dev=[S0_dev, E], out_arrays=local, finalize=False, unique_out=ubuf, U_out=U)
+        hot.gather(c_mem, ubuf, o_mem, out_ts=o_ts, N_dev=U[0:1])
+        hot.gather(c_nf, ubuf, o_nf, N_dev=U[0:1])
+        hot.gather(c_ef, kr.hops[0].neighbors_eid, o_ef, N_dev=E)
+        hot.time_encode(kr.hops[0].neighbors_dt, w, bias, out=o_te, N_dev=E)
+        acc[0:1].add_(E); acc[1:2].add_(U[0:1])
+
+    def stage(b):
+        for dst_, src_ in zip(s_in, (roots, root_ts, neg, neg_ts)):
+            dst_.copy_(src_[b])
+
+    stage(0); body(); torch.cuda.synchronize()
+    side = torch.cuda.Stream(); side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        body()
+    torch.cuda.current_stream().wait_stream(side); torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        body()
+    for i in range(3):
+        stage(i % NB); graph.replay()
+    torch.cuda.synchronize(); acc.zero_(); torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for i in range(steps):
+        stage(i % NB); graph.replay()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t1
+    e_tot, u_tot = acc.cpu().tolist()
+    # stage timings (eager, back to back)
+    stage(0); body(); torch.cuda.synchronize()
+    e1, u1 = int(E.item()), int(U[0].item())
+    res = {"nodes": n, "edges": m, "roots_per_batch": S0, "remote_row_fraction": remote, "steps": steps,
+           "ms_per_step": round(wall / steps * 1e3, 4), "sampled_edges_per_s": round(e_tot / wall, 1),
+           "edges_per_step": e_tot / steps, "unique_nodes_per_step": u_tot / steps}
+    ms = _time_launches(torch, lambda: hot.time_encode(kr.hops[0].neighbors_dt, w, bias, out=o_te, N_dev=E))
+    res["time_encode"] = {"ms": round(ms, 4), "rows": e1, "GBps": round(e1 * 408 / ms / 1e6, 1)}
+    ms = _time_launches(torch, lambda: hot.gather(c_ef, kr.hops[0].neighbors_eid, o_ef, N_dev=E))
+    res["gather_edge_feat"] = {"ms": round(ms, 4), "rows": e1, "GBps": round(e1 * 1384 / ms / 1e6, 1)}
+    ms = _time_launches(torch, lambda: hot.gather(c_mem, ubuf, o_mem, out_ts=o_ts, N_dev=U[0:1]))
+    res["gather_memory_30pct_host"] = {"ms": round(ms, 4), "rows": u1, "GBps": round(u1 * (8 + 4 + 800 + 16) / ms / 1e6, 1)}
+    ms = _time_launches(torch, lambda: hot.sample_khop(dg, s_in[0], ts_ptr, s_in[1], s_in[2], s_in[3], 1, p, finalize=False, out=kr))
+    res["sample_recent_1hop"] = {"ms": round(ms, 4), "edges_per_s": round(e1 / ms * 1e3, 1)}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -41,6 +231,9 @@ def main():
     ap.add_argument("--fanout", type=int, default=10)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--no-edge-feat", action="store_true", help="skip the 13.8 GB edge feature table (debug)")
+    ap.add_argument("--workload", default="all", choices=["c2", "c3", "c5", "all"],
+                    help="c2 = the headline workload (always run); 'all' adds the cache stress test (c3) and the "
+                         "TGN step (c5) as extra_workloads")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (known traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings can be scaled")
@@ -260,11 +453,19 @@ def main():
         for kk in v:
             v[kk] = float(round(v[kk], 4))
     dom = "gather_edge_feat_hop2" if edge_cache is not None else "gather_node_feat"
-    ach = stages[dom]["GBps"]
+    # the dominant kernel alone: 20 launches back to back between one pair of HIP events on the stream
+    # it is launched on (the per-stage figures above carry one graph launch + one event pair each)
+    stage_inputs(W % NB)
+    st_recent(); st_unique()
+    torch.cuda.synchronize()
+    dom_ms = _time_launches(torch, st_edge1 if edge_cache is not None else st_node, reps=20)
+    c_now = kr.counts.cpu().numpy()
+    dom_bytes = float(c_now[4]) * (8 + 1376) if edge_cache is not None else float(U[0].item()) * (8 + 800)
+    ach = round(dom_bytes / dom_ms / 1e6, 1)
     roofline = {"kernel": "gather_kernel<u32x4> (" + dom + ")", "bound": "hbm", "achieved": ach,
                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
-                "avg_launch_ms": stages[dom]["ms"],
-                "algorithmic_bytes_per_launch": int(b_e1 if edge_cache is not None else b_node)}
+                "avg_launch_ms": round(dom_ms, 5), "launches_timed": 20,
+                "algorithmic_bytes_per_launch": int(dom_bytes)}
 
     # ---- CPU baseline: the oracle's 2-hop recent sampler on the host cores, same batches
     cpu = None
@@ -294,6 +495,48 @@ def main():
                "kind": "port", "sample": f"{nb_cpu} batches of {S0} roots, {edges_cpu} edges in {t_cpu:.2f}s",
                "gpu_over_cpu_sampler": round(stages["sample_recent_2hop"]["edges_per_s"] / (edges_cpu / t_cpu), 1)}
 
+    extra = {}
+    has_edge_feat = edge_cache is not None
+    # sampler throughput when several mini-batches are sampled by one call (what a loader with a
+    # prefetch queue, or an AsyncGraphBlob of several windows, can do): same graph, same batches
+    scaling = []
+    for mult in (1, 4, 16, 64):
+        idx = [(W + i) % NB for i in range(mult)]
+        r_ = torch.cat([roots[i] for i in idx]); rt_ = torch.cat([root_ts[i] for i in idx])
+        n_ = torch.cat([neg[i] for i in idx]); nt_ = torch.cat([neg_ts[i] for i in idx])
+        tp_ = torch.arange(r_.numel() + 1, dtype=torch.int64, device=dev)
+        kb = hot.khop_buffers(S0 * mult, 2, k)
+        fn = lambda: hot.sample_khop(dg, r_, tp_, rt_, n_, nt_, 2, p_rec, finalize=False, out=kb)
+        ms = _time_launches(torch, fn, reps=10)
+        cnt = kb.counts.cpu().numpy()
+        e_ = int(cnt[1] + cnt[4])
+        scaling.append({"batches_per_call": mult, "roots": S0 * mult, "edges": e_, "ms": round(ms, 4),
+                        "edges_per_s": round(e_ / ms * 1e3, 1),
+                        "GBps": round((samp_bytes(S0 * mult, cnt[1]) + samp_bytes(cnt[1], cnt[4])) / ms / 1e6, 1)})
+        del kb
+    extra["sampler scaling (2-hop recent 10x10, several batches per call)"] = scaling
+    if args.workload != "c2":
+        # free the headline workload's tables first
+        del node_feat, edge_feat, node_cache, edge_cache, e_out, node_out, dg
+        graphs = g_step = None
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+    for name, fn in (("configs[2] cache stress", lambda: workload_cache_stress(hot, torch, np, synth)),
+                     ("configs[4] tgn step", lambda: workload_tgn_step(hot, torch, np, synth, _abi))):
+        key = "c3" if "cache" in name else "c5"
+        if args.workload not in (key, "all"):
+            continue
+        try:
+            t_w = time.time()
+            extra[name] = fn()
+            extra[name]["wall_s"] = round(time.time() - t_w, 1)
+        except Exception as exc:      # the headline line is still printed
+            extra[name] = {"error": f"{type(exc).__name__}: {exc}"}
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+
     out = {
         "metric": "sampled edges/sec (2-hop recent & uniform) + feature-gather GB/s vs HBM peak",
         "value": round(value, 1), "unit": "sampled edges/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -302,9 +545,9 @@ def main():
         "config": {"workload": "configs[1]: 1M nodes / 20M edges Zipf(1.1) out-degree, batches of 4000 events + 4000 "
                                "negatives (12000 roots): 2-hop recent 10x10 + unique + node/edge gather + 2-hop uniform 10x10",
                    "nodes": n, "edges": m, "roots_per_batch": S0, "fanout": [k, k],
-                   "node_feat": "100xfp32", "edge_feat": "172xfp32" if edge_cache is not None else None},
+                   "node_feat": "100xfp32", "edge_feat": "172xfp32" if has_edge_feat else None},
         "edges_per_step": {"recent": float(np.mean(e_rec)), "uniform": float(np.mean(e_uni))},
-        "stages": stages, "roofline": roofline, "cpu_baseline": cpu,
+        "stages": stages, "roofline": roofline, "cpu_baseline": cpu, "extra_workloads": extra,
     }
     print(json.dumps(out), flush=True)
 

@@ -18,6 +18,10 @@ namespace {
 
 constexpr int BLOCK = 256;
 constexpr int UNROLL = 4;
+// Grids are capped and blocks walk tiles with a grid stride: the live row count is a
+// device value, and launching the worst-case number of blocks costs ~0.2 ns per dead
+// block (10 us for 50 000 of them), more than the whole copy of a small batch.
+constexpr int MAX_GRID = 4096;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -66,45 +70,48 @@ __global__ __launch_bounds__(BLOCK) void gather_kernel(GatherArgs a) {
     extern __shared__ const char* s_src[];  // [rpb]
     __shared__ int32_t s_tier[3];
     const int64_t N = live_count(a.N_dev, a.N_max);
-    const int64_t row0 = (int64_t)blockIdx.x * a.rpb;
-    if (row0 >= N) return;
-    const int32_t rows = (int32_t)((N - row0) < a.rpb ? (N - row0) : a.rpb);
     if (threadIdx.x < 3) s_tier[threadIdx.x] = 0;
-    __syncthreads();
-    for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
-        int64_t ts;
-        int tier;
-        s_src[r] = resolve(a.c, a.ids[row0 + r], &ts, &tier);
-        if (a.out_ts != nullptr) a.out_ts[row0 + r] = ts;
-        if (a.stats != nullptr) atomicAdd(&s_tier[tier], 1);
-    }
-    __syncthreads();
     const int32_t cpr = a.cpr;
-    const int32_t total = rows * cpr;
-    V* __restrict__ dst = reinterpret_cast<V*>(a.out + row0 * a.c.row_bytes);
-    for (int32_t base = 0; base < total; base += BLOCK * UNROLL) {
-        V val[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int32_t lc = base + u * BLOCK + threadIdx.x;
-            V v = {};
-            if (lc < total) {
-                const int32_t r = lc / cpr;
-                const int32_t part = lc - r * cpr;
-                const V* src = reinterpret_cast<const V*>(s_src[r]);
-                if (src != nullptr) v = NT ? __builtin_nontemporal_load(src + part) : src[part];
-            }
-            val[u] = v;
+    const int64_t first_row = (int64_t)blockIdx.x * a.rpb;
+    if (a.stats != nullptr) __syncthreads();  // s_tier is zero before the first atomicAdd
+    for (int64_t row0 = first_row; row0 < N; row0 += (int64_t)gridDim.x * a.rpb) {
+        const int32_t rows = (int32_t)((N - row0) < a.rpb ? (N - row0) : a.rpb);
+        if (row0 != first_row) __syncthreads();  // s_src of the previous tile has been consumed
+        for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
+            int64_t ts;
+            int tier;
+            s_src[r] = resolve(a.c, a.ids[row0 + r], &ts, &tier);
+            if (a.out_ts != nullptr) a.out_ts[row0 + r] = ts;
+            if (a.stats != nullptr) atomicAdd(&s_tier[tier], 1);
         }
+        __syncthreads();
+        const int32_t total = rows * cpr;
+        V* __restrict__ dst = reinterpret_cast<V*>(a.out + row0 * a.c.row_bytes);
+        for (int32_t base = 0; base < total; base += BLOCK * UNROLL) {
+            V val[UNROLL];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int32_t lc = base + u * BLOCK + threadIdx.x;
-            if (lc < total) {
-                if (NT) __builtin_nontemporal_store(val[u], dst + lc);
-                else dst[lc] = val[u];
+            for (int u = 0; u < UNROLL; ++u) {
+                const int32_t lc = base + u * BLOCK + threadIdx.x;
+                V v = {};
+                if (lc < total) {
+                    const int32_t r = lc / cpr;
+                    const int32_t part = lc - r * cpr;
+                    const V* src = reinterpret_cast<const V*>(s_src[r]);
+                    if (src != nullptr) v = NT ? __builtin_nontemporal_load(src + part) : src[part];
+                }
+                val[u] = v;
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int32_t lc = base + u * BLOCK + threadIdx.x;
+                if (lc < total) {
+                    if (NT) __builtin_nontemporal_store(val[u], dst + lc);
+                    else dst[lc] = val[u];
+                }
             }
         }
     }
+    if (a.stats != nullptr) __syncthreads();
     if (a.stats != nullptr && threadIdx.x < 3 && s_tier[threadIdx.x] != 0)
         atomicAdd(reinterpret_cast<unsigned long long*>(a.stats + threadIdx.x),
                   (unsigned long long)s_tier[threadIdx.x]);
@@ -126,34 +133,35 @@ struct ScatterArgs {
 template <typename V>
 __global__ __launch_bounds__(BLOCK) void scatter_kernel(ScatterArgs a) {
     extern __shared__ char* s_dst[];
-    const int64_t row0 = (int64_t)blockIdx.x * a.rpb;
-    if (row0 >= a.N) return;
-    const int32_t rows = (int32_t)((a.N - row0) < a.rpb ? (a.N - row0) : a.rpb);
-    for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
-        int64_t ts_unused;
-        int tier;
-        const char* p = resolve(a.c, a.ids[row0 + r], &ts_unused, &tier);
-        char* d = nullptr;
-        if (tier == 0) {
-            const int64_t slot = (p - static_cast<const char*>(a.c.hot)) / a.c.row_bytes;
-            d = a.hot_rw + slot * a.c.row_bytes;
-            if (a.ts != nullptr && a.ts_hot_rw != nullptr) a.ts_hot_rw[slot] = a.ts[row0 + r];
-        } else if (tier == 1) {
-            const int64_t loc = (p - static_cast<const char*>(a.c.cold)) / a.c.row_bytes;
-            d = a.cold_rw + loc * a.c.row_bytes;
-            if (a.ts != nullptr && a.ts_cold_rw != nullptr) a.ts_cold_rw[loc] = a.ts[row0 + r];
+    for (int64_t row0 = (int64_t)blockIdx.x * a.rpb; row0 < a.N; row0 += (int64_t)gridDim.x * a.rpb) {
+        const int32_t rows = (int32_t)((a.N - row0) < a.rpb ? (a.N - row0) : a.rpb);
+        __syncthreads();
+        for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
+            int64_t ts_unused;
+            int tier;
+            const char* p = resolve(a.c, a.ids[row0 + r], &ts_unused, &tier);
+            char* d = nullptr;
+            if (tier == 0) {
+                const int64_t slot = (p - static_cast<const char*>(a.c.hot)) / a.c.row_bytes;
+                d = a.hot_rw + slot * a.c.row_bytes;
+                if (a.ts != nullptr && a.ts_hot_rw != nullptr) a.ts_hot_rw[slot] = a.ts[row0 + r];
+            } else if (tier == 1) {
+                const int64_t loc = (p - static_cast<const char*>(a.c.cold)) / a.c.row_bytes;
+                d = a.cold_rw + loc * a.c.row_bytes;
+                if (a.ts != nullptr && a.ts_cold_rw != nullptr) a.ts_cold_rw[loc] = a.ts[row0 + r];
+            }
+            s_dst[r] = d;
         }
-        s_dst[r] = d;
-    }
-    __syncthreads();
-    const int32_t cpr = a.cpr;
-    const int32_t total = rows * cpr;
-    const V* __restrict__ src = reinterpret_cast<const V*>(a.values + row0 * a.c.row_bytes);
-    for (int32_t lc = threadIdx.x; lc < total; lc += BLOCK) {
-        const int32_t r = lc / cpr;
-        const int32_t part = lc - r * cpr;
-        V* d = reinterpret_cast<V*>(s_dst[r]);
-        if (d != nullptr) d[part] = src[lc];
+        __syncthreads();
+        const int32_t cpr = a.cpr;
+        const int32_t total = rows * cpr;
+        const V* __restrict__ src = reinterpret_cast<const V*>(a.values + row0 * a.c.row_bytes);
+        for (int32_t lc = threadIdx.x; lc < total; lc += BLOCK) {
+            const int32_t r = lc / cpr;
+            const int32_t part = lc - r * cpr;
+            V* d = reinterpret_cast<V*>(s_dst[r]);
+            if (d != nullptr) d[part] = src[lc];
+        }
     }
 }
 
@@ -207,7 +215,10 @@ extern "C" int32_t sgl_gather(const sgl_cache* c, const int64_t* ids, int64_t N_
     int64_t rpb = (int64_t)BLOCK * UNROLL / a.cpr;
     rpb = rpb < 1 ? 1 : (rpb > 1024 ? 1024 : rpb);
     a.rpb = (int32_t)rpb;
-    const int64_t blocks = ceil_div<int64_t>(N_max, rpb);
+    // a device-side live count usually is far below the capacity: cap the grid; a host-known
+    // count gets one block per tile (measured 15 % faster on 2M-row gathers than striding)
+    int64_t blocks = ceil_div<int64_t>(N_max, rpb);
+    if (N_dev != nullptr && blocks > MAX_GRID) blocks = MAX_GRID;
     if (blocks > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "gather: too many rows for one launch");
     const size_t shmem = (size_t)rpb * sizeof(char*);
     hipStream_t st = as_stream(stream);
@@ -240,8 +251,8 @@ extern "C" int32_t sgl_scatter_update(const sgl_cache* c, void* hot_rw, void* co
     int64_t rpb = (int64_t)BLOCK * UNROLL / a.cpr;
     rpb = rpb < 1 ? 1 : (rpb > 1024 ? 1024 : rpb);
     a.rpb = (int32_t)rpb;
-    const int64_t blocks = ceil_div<int64_t>(N, rpb);
-    if (blocks > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "scatter_update: too many rows for one launch");
+    int64_t blocks = ceil_div<int64_t>(N, rpb);
+    if (blocks > 0x3FFFFFll) blocks = 0x3FFFFFll;
     const size_t shmem = (size_t)rpb * sizeof(char*);
     hipStream_t st = as_stream(stream);
     switch (vec) {

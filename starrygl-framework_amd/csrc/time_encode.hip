@@ -69,32 +69,34 @@ template <int VEC>
 __global__ __launch_bounds__(BLOCK) void time_encode_kernel(TEArgs a) {
     __shared__ float s_x[MAX_RPB];
     const int64_t N = live_count(a.N_dev, a.N_max);
-    const int64_t row0 = (int64_t)blockIdx.x * a.rpb;
-    if (row0 >= N) return;
-    const int32_t rows = (int32_t)((N - row0) < a.rpb ? (N - row0) : a.rpb);
-    for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
-        s_x[r] = a.dt_dtype == SGL_DT_I64 ? (float)static_cast<const int64_t*>(a.dt)[row0 + r]
-                                           : static_cast<const float*>(a.dt)[row0 + r];
-    }
-    __syncthreads();
     const int32_t cpr = a.dim / VEC;
-    const int32_t total = rows * cpr;
-    float* __restrict__ dst = a.out + row0 * a.dim;
-    for (int32_t lc = threadIdx.x; lc < total; lc += BLOCK) {
-        const int32_t r = lc / cpr;
-        const int32_t j = (lc - r * cpr) * VEC;
-        const float x = s_x[r];
-        if constexpr (VEC == 4) {
-            const f32x4 w = *reinterpret_cast<const f32x4*>(a.w + j);
-            const f32x4 b = *reinterpret_cast<const f32x4*>(a.b + j);
-            f32x4 y;
-            y.x = enc(w.x, x, b.x);
-            y.y = enc(w.y, x, b.y);
-            y.z = enc(w.z, x, b.z);
-            y.w = enc(w.w, x, b.w);
-            reinterpret_cast<f32x4*>(dst)[lc] = y;
-        } else {
-            dst[lc] = enc(a.w[j], x, a.b[j]);
+    // capped grid, tiles walked with a grid stride (dead blocks of a worst-case grid are not free)
+    for (int64_t row0 = (int64_t)blockIdx.x * a.rpb; row0 < N; row0 += (int64_t)gridDim.x * a.rpb) {
+        const int32_t rows = (int32_t)((N - row0) < a.rpb ? (N - row0) : a.rpb);
+        __syncthreads();
+        for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
+            s_x[r] = a.dt_dtype == SGL_DT_I64 ? (float)static_cast<const int64_t*>(a.dt)[row0 + r]
+                                               : static_cast<const float*>(a.dt)[row0 + r];
+        }
+        __syncthreads();
+        const int32_t total = rows * cpr;
+        float* __restrict__ dst = a.out + row0 * a.dim;
+        for (int32_t lc = threadIdx.x; lc < total; lc += BLOCK) {
+            const int32_t r = lc / cpr;
+            const int32_t j = (lc - r * cpr) * VEC;
+            const float x = s_x[r];
+            if constexpr (VEC == 4) {
+                const f32x4 w = *reinterpret_cast<const f32x4*>(a.w + j);
+                const f32x4 b = *reinterpret_cast<const f32x4*>(a.b + j);
+                f32x4 y;
+                y.x = enc(w.x, x, b.x);
+                y.y = enc(w.y, x, b.y);
+                y.z = enc(w.z, x, b.z);
+                y.w = enc(w.w, x, b.w);
+                reinterpret_cast<f32x4*>(dst)[lc] = y;
+            } else {
+                dst[lc] = enc(a.w[j], x, a.b[j]);
+            }
         }
     }
 }
@@ -119,8 +121,9 @@ extern "C" int32_t sgl_time_encode(const void* dt, int32_t dt_dtype, int64_t N_m
     int64_t rpb = (int64_t)BLOCK * 4 / cpr;
     rpb = rpb < 1 ? 1 : (rpb > MAX_RPB ? MAX_RPB : rpb);
     a.rpb = (int32_t)rpb;
-    const int64_t blocks = ceil_div<int64_t>(N_max, rpb);
-    if (blocks > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "time_encode: too many rows for one launch");
+    int64_t blocks = ceil_div<int64_t>(N_max, rpb);
+    if (N_dev != nullptr && blocks > 8192) blocks = 8192;   // live count usually far below capacity
+    if (blocks > 0x3FFFFFll) blocks = 0x3FFFFFll;
     hipStream_t st = as_stream(stream);
     if (vec4)
         hipLaunchKernelGGL(time_encode_kernel<4>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);

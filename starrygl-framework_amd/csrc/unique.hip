@@ -33,6 +33,7 @@ constexpr int BLOCK = 256;
 constexpr int MAXG = 8;
 constexpr int TILE = BLOCK;            // bitmap words per block in reduce/assign (one per thread)
 constexpr int SCAN_BLOCK = 1024;
+constexpr int MAX_GRID = 2048;         // grid cap of the per-id kernels (grid-stride loops)
 constexpr int FUSED_SCAN_MAX = 4096;   // up to this many tiles assign sums the preceding tiles itself
 constexpr size_t HEADER_BYTES = 256;
 
@@ -83,19 +84,6 @@ struct Arrays {
     int64_t start[MAXG + 1];  // flat index space over len_max
 };
 
-__device__ __forceinline__ bool locate(const Arrays& a, int64_t t, int* g_out, int64_t* i_out) {
-    if (t >= a.start[a.G]) return false;
-    int g = 0;
-#pragma unroll
-    for (int q = 1; q < MAXG; ++q)
-        if (q < a.G && t >= a.start[q]) g = q;
-    const int64_t i = t - a.start[g];
-    if (i >= live_count(a.len_dev[g], a.len_max[g])) return false;
-    *g_out = g;
-    *i_out = i;
-    return true;
-}
-
 __global__ void init_state_kernel(State s) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -112,14 +100,22 @@ __global__ void init_state_kernel(State s) {
 // MI355X: testing the bit first, or folding the block's ids through an LDS
 // hash set first, both lengthen the dependent chain and run 2-3x slower.)
 __global__ __launch_bounds__(BLOCK) void mark_kernel(State s, Arrays a, int reset) {
-    const int64_t t = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
-    int g;
-    int64_t i;
-    if (!locate(a, t, &g, &i)) return;
-    const int64_t id = a.ids[g][i];
-    if (id < 0 || id >= s.universe) return;
-    if ((uint32_t)(s.table[id] >> 32) == eff_stamp(s, reset)) return;  // numbered earlier in this epoch
-    atomicOr(reinterpret_cast<unsigned long long*>(&s.bitmap[id >> 6]), 1ull << (id & 63));
+    const uint32_t stamp = eff_stamp(s, reset);
+    // Flat index space over the arrays' capacities, walked array by array with a grid
+    // stride bounded by each array's LIVE length: capacities are worst cases (slots x
+    // fanout), so most of the index space is dead.
+#pragma unroll
+    for (int g = 0; g < MAXG; ++g) {
+        if (g >= a.G) continue;
+        const int64_t len = live_count(a.len_dev[g], a.len_max[g]);
+        const int64_t* __restrict__ ids = a.ids[g];
+        for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < len; i += (int64_t)gridDim.x * BLOCK) {
+            const int64_t id = ids[i];
+            if (id < 0 || id >= s.universe) continue;
+            if ((uint32_t)(s.table[id] >> 32) == stamp) continue;  // numbered earlier in this epoch
+            atomicOr(reinterpret_cast<unsigned long long*>(&s.bitmap[id >> 6]), 1ull << (id & 63));
+        }
+    }
 }
 
 __global__ __launch_bounds__(BLOCK) void reduce_kernel(State s, int64_t* tile_sum) {
@@ -228,17 +224,23 @@ __global__ void commit_kernel(State s, int reset, int first, int has_new, int64_
 }
 
 __global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a) {
-    const int64_t t = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
-    int g;
-    int64_t i;
-    if (!locate(a, t, &g, &i)) return;
-    const int64_t id = a.ids[g][i];
-    int64_t local = -1;
-    if (id >= 0 && id < s.universe) {
-        const uint64_t e = s.table[id];
-        if ((uint32_t)(e >> 32) == (uint32_t)(s.hdr->epoch & 0xFFFFFFFFull)) local = (int64_t)(e & 0xFFFFFFFFull);
+    const uint32_t stamp = (uint32_t)(s.hdr->epoch & 0xFFFFFFFFull);
+#pragma unroll
+    for (int g = 0; g < MAXG; ++g) {
+        if (g >= a.G) continue;
+        const int64_t len = live_count(a.len_dev[g], a.len_max[g]);
+        const int64_t* ids = a.ids[g];   // may alias out[g]
+        int64_t* out = a.out[g];
+        for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < len; i += (int64_t)gridDim.x * BLOCK) {
+            const int64_t id = ids[i];
+            int64_t local = -1;
+            if (id >= 0 && id < s.universe) {
+                const uint64_t e = s.table[id];
+                if ((uint32_t)(e >> 32) == stamp) local = (int64_t)(e & 0xFFFFFFFFull);
+            }
+            out[i] = local;
+        }
     }
-    a.out[g][i] = local;
 }
 
 size_t dense_workspace_bytes(int64_t universe) {
@@ -332,8 +334,9 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
         }
         const int64_t sub_total = sub.start[sub.G];
         if (sub_total == 0 || universe == 0) continue;
-        hipLaunchKernelGGL(mark_kernel, dim3((unsigned)ceil_div<int64_t>(sub_total, BLOCK)), dim3(BLOCK), 0, st,
-                           s, sub, rst);
+        int64_t mb = ceil_div<int64_t>(sub_total, BLOCK);
+        if (mb > MAX_GRID) mb = MAX_GRID;
+        hipLaunchKernelGGL(mark_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, sub, rst);
         SGL_LAUNCH_CHECK();
         hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
         SGL_LAUNCH_CHECK();
@@ -355,7 +358,9 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
         SGL_LAUNCH_CHECK();
     }
     if (total > 0) {
-        hipLaunchKernelGGL(lookup_kernel, dim3((unsigned)ceil_div<int64_t>(total, BLOCK)), dim3(BLOCK), 0, st, s, all);
+        int64_t lb = ceil_div<int64_t>(total, BLOCK);
+        if (lb > MAX_GRID) lb = MAX_GRID;
+        hipLaunchKernelGGL(lookup_kernel, dim3((unsigned)lb), dim3(BLOCK), 0, st, s, all);
         SGL_LAUNCH_CHECK();
     }
     return SGL_OK;
