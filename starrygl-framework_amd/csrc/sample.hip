@@ -479,13 +479,17 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     }
 }
 
-int pick_group(const sgl_sample_params* p) {
+// Lanes per slot.  Uniform needs fanout <= G (one lane per draw).  Recent copies any
+// fanout with any G; with many slots 8 lanes per slot keep twice as many slots in
+// flight per compute unit, which is what bounds a launch once the slots exceed one
+// wave-residency round (8192 waves): 53k slots run ~25 % faster than with 16 lanes.
+int pick_group(const sgl_sample_params* p, int64_t S_max) {
     if (p->type == SGL_SAMPLE_UNIFORM) {
         if (p->fanout <= 16) return 16;
         if (p->fanout <= 32) return 32;
         return 64;
     }
-    return 16;
+    return S_max >= 32768 ? 8 : 16;
 }
 
 size_t hop_workspace_bytes(int64_t S_max) {
@@ -581,7 +585,8 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
     a.root_start_ptr = out->root_start_ptr; a.root_end_ptr = out->root_end_ptr;
     a.nbr = out->neighbors; a.nbr_ts = out->neighbors_ts; a.nbr_eid = out->neighbors_eid;
     a.nbr_dt = out->neighbors_dt; a.counts = out->counts;
-    switch (pick_group(p)) {
+    switch (pick_group(p, S_max)) {
+        case 8: return launch_hop<8>(a, st);
         case 16: return launch_hop<16>(a, st);
         case 32: return launch_hop<32>(a, st);
         default: return launch_hop<64>(a, st);

@@ -119,3 +119,15 @@ def test_error_codes(hot):
     p.type = 9
     assert hot.lib.sample_khop(None, 0, None, None, 0, None, 0, None, None, 1, C.byref(p), None, None, None,
                                None, 0, None) == _abi.SGL_EINVAL
+
+
+@pytest.mark.parametrize("sample_type", ["recent", "uniform"])
+def test_large_hops(oracle, hot, sample_type):
+    """> 32k slots per hop: the recent strategy switches to 8 lanes per slot, grids
+    beyond 1024 blocks use the one-block scan, beyond 8192 blocks every block walks
+    several slot groups; a 200k-edge hub row keeps the multi-step search in play."""
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 2_000, 600_000, 1.05, 10**9, 17, hub=200_000)
+    rng = np.random.default_rng(4)
+    b = synth.link_batch(src, dst, ts, 500_000, 502_000, g.n, 2000, rng)          # 6k roots -> ~60k -> ~600k slots
+    got, want = _run_both(oracle, hot, g, dg, *b, 3, sample_type=sample_type, fanout=10, seed=5)
+    assert want.hops[1].S > 32768 and want.hops[2].S > 8192 * 32
