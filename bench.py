@@ -24,6 +24,9 @@ for _p in (ROOT, os.path.join(ROOT, "starrygl-framework_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per gathered 688-byte row of the hop-2 edge-feature gather, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of this script (summary and commands: profiles/gather_kernel_configs1_hbm_traffic.md)
+MEASURED_HBM_BYTES_PER_ROW = {"read": 657.8, "write": 702.5}
 
 
 def log(*a):
@@ -463,7 +466,8 @@ def main():
     dom_bytes = float(c_now[4]) * (8 + 1376) if edge_cache is not None else float(U[0].item()) * (8 + 800)
     ach = round(dom_bytes / dom_ms / 1e6, 1)
     roofline = {"kernel": "gather_kernel<u32x4> (" + dom + ")", "bound": "hbm", "achieved": ach,
-                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
+                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4),
+                "traffic": (int(dom_bytes / (8 + 1376) * sum(MEASURED_HBM_BYTES_PER_ROW.values())) if edge_cache is not None else None),
                 "avg_launch_ms": round(dom_ms, 5), "launches_timed": 20,
                 "algorithmic_bytes_per_launch": int(dom_bytes)}
 
@@ -547,6 +551,8 @@ def main():
                    "nodes": n, "edges": m, "roots_per_batch": S0, "fanout": [k, k],
                    "node_feat": "100xfp32", "edge_feat": "172xfp32" if has_edge_feat else None},
         "edges_per_step": {"recent": float(np.mean(e_rec)), "uniform": float(np.mean(e_uni))},
+        "mean_rows_per_step": {"gather_node_feat": float(np.mean(cl[:, 4])), "gather_edge_feat_hop1": float(np.mean(cl[:, 0])),
+                               "gather_edge_feat_hop2": float(np.mean(cl[:, 1]))},
         "stages": stages, "roofline": roofline, "cpu_baseline": cpu, "extra_workloads": extra,
     }
     print(json.dumps(out), flush=True)

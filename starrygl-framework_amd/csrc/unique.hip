@@ -101,20 +101,31 @@ __global__ void init_state_kernel(State s) {
 // hash set first, both lengthen the dependent chain and run 2-3x slower.)
 __global__ __launch_bounds__(BLOCK) void mark_kernel(State s, Arrays a, int reset) {
     const uint32_t stamp = eff_stamp(s, reset);
-    // Flat index space over the arrays' capacities, walked array by array with a grid
-    // stride bounded by each array's LIVE length: capacities are worst cases (slots x
-    // fanout), so most of the index space is dead.
+    // Index i is processed for every array at once (loads of the different arrays are
+    // independent and issue together: one dependent chain id -> table -> atomic per
+    // thread instead of one per array), with a grid stride bounded by the longest LIVE
+    // length: capacities are worst cases (slots x fanout), most of them is dead.
+    int64_t len[MAXG];
+    int64_t max_len = 0;
 #pragma unroll
     for (int g = 0; g < MAXG; ++g) {
-        if (g >= a.G) continue;
-        const int64_t len = live_count(a.len_dev[g], a.len_max[g]);
-        const int64_t* __restrict__ ids = a.ids[g];
-        for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < len; i += (int64_t)gridDim.x * BLOCK) {
-            const int64_t id = ids[i];
-            if (id < 0 || id >= s.universe) continue;
-            if ((uint32_t)(s.table[id] >> 32) == stamp) continue;  // numbered earlier in this epoch
-            atomicOr(reinterpret_cast<unsigned long long*>(&s.bitmap[id >> 6]), 1ull << (id & 63));
+        len[g] = g < a.G ? live_count(a.len_dev[g], a.len_max[g]) : 0;
+        max_len = len[g] > max_len ? len[g] : max_len;
+    }
+    for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < max_len; i += (int64_t)gridDim.x * BLOCK) {
+        int64_t id[MAXG];
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) id[g] = (g < a.G && i < len[g]) ? a.ids[g][i] : -1;
+        uint64_t e[MAXG];
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) {
+            const bool ok = id[g] >= 0 && id[g] < s.universe;
+            e[g] = ok ? s.table[id[g]] : ((uint64_t)stamp << 32);   // out of range: treated as already numbered
         }
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g)
+            if ((uint32_t)(e[g] >> 32) != stamp)
+                atomicOr(reinterpret_cast<unsigned long long*>(&s.bitmap[id[g] >> 6]), 1ull << (id[g] & 63));
     }
 }
 
@@ -225,21 +236,24 @@ __global__ void commit_kernel(State s, int reset, int first, int has_new, int64_
 
 __global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a) {
     const uint32_t stamp = (uint32_t)(s.hdr->epoch & 0xFFFFFFFFull);
+    int64_t len[MAXG];
+    int64_t max_len = 0;
 #pragma unroll
     for (int g = 0; g < MAXG; ++g) {
-        if (g >= a.G) continue;
-        const int64_t len = live_count(a.len_dev[g], a.len_max[g]);
-        const int64_t* ids = a.ids[g];   // may alias out[g]
-        int64_t* out = a.out[g];
-        for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < len; i += (int64_t)gridDim.x * BLOCK) {
-            const int64_t id = ids[i];
-            int64_t local = -1;
-            if (id >= 0 && id < s.universe) {
-                const uint64_t e = s.table[id];
-                if ((uint32_t)(e >> 32) == stamp) local = (int64_t)(e & 0xFFFFFFFFull);
-            }
-            out[i] = local;
-        }
+        len[g] = g < a.G ? live_count(a.len_dev[g], a.len_max[g]) : 0;
+        max_len = len[g] > max_len ? len[g] : max_len;
+    }
+    for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < max_len; i += (int64_t)gridDim.x * BLOCK) {
+        int64_t id[MAXG];
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) id[g] = (g < a.G && i < len[g]) ? a.ids[g][i] : -1;   // ids may alias out
+        uint64_t e[MAXG];
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) e[g] = (id[g] >= 0 && id[g] < s.universe) ? s.table[id[g]] : 0ull;
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g)
+            if (g < a.G && i < len[g])
+                a.out[g][i] = ((uint32_t)(e[g] >> 32) == stamp) ? (int64_t)(e[g] & 0xFFFFFFFFull) : -1;
     }
 }
 
@@ -334,7 +348,9 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
         }
         const int64_t sub_total = sub.start[sub.G];
         if (sub_total == 0 || universe == 0) continue;
-        int64_t mb = ceil_div<int64_t>(sub_total, BLOCK);
+        int64_t longest = 0;
+        for (int g = 0; g < sub.G; ++g) longest = sub.len_max[g] > longest ? sub.len_max[g] : longest;
+        int64_t mb = ceil_div<int64_t>(longest, BLOCK);
         if (mb > MAX_GRID) mb = MAX_GRID;
         hipLaunchKernelGGL(mark_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, sub, rst);
         SGL_LAUNCH_CHECK();
@@ -358,7 +374,9 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
         SGL_LAUNCH_CHECK();
     }
     if (total > 0) {
-        int64_t lb = ceil_div<int64_t>(total, BLOCK);
+        int64_t longest = 0;
+        for (int g = 0; g < all.G; ++g) longest = all.len_max[g] > longest ? all.len_max[g] : longest;
+        int64_t lb = ceil_div<int64_t>(longest, BLOCK);
         if (lb > MAX_GRID) lb = MAX_GRID;
         hipLaunchKernelGGL(lookup_kernel, dim3((unsigned)lb), dim3(BLOCK), 0, st, s, all);
         SGL_LAUNCH_CHECK();
