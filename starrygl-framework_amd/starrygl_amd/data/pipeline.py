@@ -1,0 +1,201 @@
+"""One mini-batch of the temporal hot path as a single pre-planned unit.
+
+The reference assembles a training batch in its (unpublished) `starrygl.data`
+package: `AsyncPipelineLoader` asks the graph engine for samples and a
+`GraphCollator` turns them into blocks plus feature / memory futures
+(call sites: test/test.py:201-221, test/test_dataloader.py:119-149; consumers
+starrygl/nn/model/tgn.py:119-196).  `MiniBatchPipeline` is that unit for one GPU:
+
+    roots (+ negatives) -> k-hop sampling -> unique / local ids -> node, memory
+    and edge row gathers -> cos time encoding of every hop's dt
+
+All buffers are allocated once for the worst case, no stage synchronises with
+the host, live sizes stay on the device; with `use_graph=True` the whole chain
+is captured into one HIP graph on the first batch and replayed afterwards (a
+batch then costs a few small copies plus one graph launch).
+"""
+import torch
+
+from ..graph.graph import Block
+from ..lib import _abi, hot_path
+
+
+class MiniBatch:
+    """Result of one pipeline run.  Device tensors are worst-case sized until
+    `finalize()` reads the live counts once and narrows them."""
+
+    def __init__(self, pipe):
+        self._p = pipe
+        self.final = False
+
+    def finalize(self):
+        if self.final:
+            return self
+        p = self._p
+        c = p.kr.counts.cpu().tolist()
+        u_total = int(p.U[0].item())
+        bad = sum(c[3 * l + 2] for l in range(p.layers))
+        if bad:
+            raise IndexError(f"sgl status {_abi.SGL_ERANGE}: {bad} sampling slots name a node outside [0,n)")
+        self.S = [c[3 * l] for l in range(p.layers)]
+        self.E = [c[3 * l + 1] for l in range(p.layers)]
+        self.num_unique = u_total
+        self.slot_node, self.slot_ts = p.kr.slot_node0[: self.S[0]], p.kr.slot_ts0[: self.S[0]]
+        self.slot_local = p.local[0][: self.S[0]]
+        self.nid_mapper = p.ubuf[:u_total]
+        self.hops = []
+        for l, h in enumerate(p.kr.hops):
+            S, E = self.S[l], self.E[l]
+            self.hops.append(dict(root_start_ptr=h.root_start_ptr[: S + 1], root_end_ptr=h.root_end_ptr[: S + 1],
+                                  neighbors=h.neighbors[:E], neighbors_local=p.local[1 + l][:E],
+                                  neighbors_ts=h.neighbors_ts[:E], neighbors_eid=h.neighbors_eid[:E],
+                                  neighbors_dt=h.neighbors_dt[:E]))
+        self.node_data = {k: v[:u_total] for k, v in p.node_out.items()}
+        self.node_ts = {k: v[:u_total] for k, v in p.node_ts_out.items()}
+        self.edge_data = [{k: v[l][: self.E[l]] for k, v in p.edge_out.items()} for l in range(p.layers)]
+        self.time_feat = [t[: self.E[l]] for l, t in enumerate(p.te_out)] if p.te_out else None
+        self.final = True
+        return self
+
+    def blocks(self, self_loop=True):
+        """Message-flow blocks, outermost hop first (AsyncBlock.to_block order);
+        node ids inside the blocks are LOCAL ids (rows of node_data)."""
+        self.finalize()
+        hp = self._p.hp
+        last_nodes, last_ts = self.slot_local, self.slot_ts
+        out = []
+        for l, h in enumerate(self.hops):
+            S, E, n_prev = self.S[l], self.E[l], int(last_nodes.numel())
+            dst_off = n_prev - S if self_loop else 0
+            num_dst = n_prev if self_loop else S
+            src_off = num_dst if self_loop else 0
+            counts = self._p.kr.hops[l].counts
+            indptr, indices, _ = hp.block_build(h["root_start_ptr"], counts, S, E, dst_off, src_off)
+            b = Block(indptr, indices, src_off + E, num_dst)
+            if self_loop:
+                b.srcdata["nid"] = torch.cat([last_nodes, h["neighbors_local"]])
+                b.srcdata["ts"] = torch.cat([last_ts, h["neighbors_ts"]])
+            else:
+                b.srcdata["nid"], b.srcdata["ts"] = h["neighbors_local"], h["neighbors_ts"]
+            b.edata["eid"], b.edata["dt"] = h["neighbors_eid"], h["neighbors_dt"]
+            for k, v in self.edge_data[l].items():
+                b.edata[k] = v
+            if self.time_feat is not None:
+                b.edata["time_feat"] = self.time_feat[l]
+            last_nodes, last_ts = b.srcdata["nid"], b.srcdata["ts"]
+            out.append(b)
+        out.reverse()
+        return out
+
+
+class MiniBatchPipeline:
+    def __init__(self, graph, num_pos_slots, num_neg, layers, fanout, sample_type="recent", node_tables=None,
+                 edge_tables=None, time_encoder=None, allowed_offset=-1, equal_root_time=False,
+                 keep_root_time=False, seed=0, use_graph=True):
+        """graph: the native graph object (`pyGraph.g`, i.e. `CUDAGraph`).
+        num_pos_slots / num_neg: positive root timestamps and negatives per batch
+        (fixed, they size every buffer).  node_tables / edge_tables: name ->
+        `sgl_cache` (from `HotPath.cache`) gathered for the unique nodes / the
+        sampled edge ids; a node table with timestamps also yields node_ts[name].
+        time_encoder: (w, b) fp32 device tensors, or a TimeEncoder module."""
+        self.g = graph
+        self.hp = hp = graph._hp
+        self.dev = hp.be.device
+        self.layers, self.fanout = int(layers), int(fanout)
+        self.S_pos, self.N_neg = int(num_pos_slots), int(num_neg)
+        self.S0 = self.S_pos + self.N_neg
+        self.p = hp.params(sample_type, fanout, allowed_offset, equal_root_time, keep_root_time, seed=seed)
+        self.node_tables, self.edge_tables = dict(node_tables or {}), dict(edge_tables or {})
+        if time_encoder is not None and not isinstance(time_encoder, tuple):
+            time_encoder = (time_encoder.w.weight.detach().reshape(-1).contiguous(),
+                            time_encoder.w.bias.detach().contiguous())
+        self.te = time_encoder
+        be = hp.be
+        # static inputs
+        self.in_roots, self.in_ts = be.empty(self.S_pos), be.empty(self.S_pos)
+        self.in_neg, self.in_neg_ts = be.empty(self.N_neg), be.empty(self.N_neg)
+        self.ts_ptr = torch.arange(self.S_pos + 1, dtype=torch.int64, device=self.dev)
+        # outputs
+        self.kr = hp.khop_buffers(self.S0, self.layers, self.fanout)
+        caps = [self.S0] + [self.S0 * self.fanout ** (l + 1) for l in range(self.layers)]
+        self.local = [be.empty(c) for c in caps]
+        self.ucap = min(sum(caps), graph._n)
+        self.ubuf, self.U = be.empty(max(self.ucap, 1)), be.zeros(2)
+        self.state = hp.remap_state(graph._n)
+        self.S0_dev = torch.tensor([self.S0], dtype=torch.int64, device=self.dev)
+        f32 = torch.float32
+        self.node_out, self.node_ts_out, self.edge_out = {}, {}, {}
+        for name, c in self.node_tables.items():
+            self.node_out[name] = torch.empty((self.ucap, c.row_bytes), dtype=torch.uint8, device=self.dev)
+            if c.ts_hot or c.ts_cold:
+                self.node_ts_out[name] = be.empty(self.ucap)
+        for name, c in self.edge_tables.items():
+            self.edge_out[name] = [torch.empty((caps[l + 1], c.row_bytes), dtype=torch.uint8, device=self.dev)
+                                   for l in range(self.layers)]
+        self.te_out = None
+        if self.te is not None:
+            dim = int(self.te[0].numel())
+            self.te_out = [torch.empty((caps[l + 1], dim), dtype=f32, device=self.dev) for l in range(self.layers)]
+        self._views = {}
+        hp._workspace(hp.lib.unique_workspace_bytes(graph._n, 1 + self.layers,
+                                                    (_abi.i64 * (1 + self.layers))(*caps)))
+        self.use_graph, self._graph = use_graph, None
+
+    def view(self, name, dtype):
+        """Reinterpret the byte output buffers of table `name` as rows of `dtype`."""
+        key = (name, dtype)
+        if key not in self._views:
+            if name in self.node_out:
+                self.node_out[name] = self.node_out[name].view(dtype)
+            if name in self.edge_out:
+                self.edge_out[name] = [t.view(dtype) for t in self.edge_out[name]]
+            self._views[key] = True
+        return self
+
+    def _chain(self):
+        hp, kr = self.hp, self.kr
+        hp.sample_khop(self.g._g, self.in_roots, self.ts_ptr, self.in_ts, self.in_neg, self.in_neg_ts, self.layers,
+                       self.p, finalize=False, out=kr)
+        arrays = [kr.slot_node0] + [h.neighbors for h in kr.hops]
+        lens = [self.S0_dev] + [h.counts[1:2] for h in kr.hops]
+        hp.unique_compact(arrays, _abi.UNIQUE_SORTED, self.state, True, lens_dev=lens, out_arrays=self.local,
+                          finalize=False, unique_out=self.ubuf, U_out=self.U)
+        for name, c in self.node_tables.items():
+            hp.gather(c, self.ubuf, self.node_out[name], out_ts=self.node_ts_out.get(name), N_dev=self.U[0:1])
+        for l, h in enumerate(kr.hops):
+            for name, c in self.edge_tables.items():
+                hp.gather(c, h.neighbors_eid, self.edge_out[name][l], N_dev=h.counts[1:2])
+            if self.te is not None:
+                hp.time_encode(h.neighbors_dt, self.te[0], self.te[1], out=self.te_out[l], N_dev=h.counts[1:2])
+
+    def run(self, roots, root_ts, neg_roots=None, neg_ts=None):
+        """Enqueue one batch (asynchronous).  `roots`/`root_ts`: S_pos ids and
+        timestamps (one timestamp per root); `neg_roots`/`neg_ts`: N_neg each."""
+        if roots.numel() != self.S_pos or root_ts.numel() != self.S_pos:
+            raise ValueError(f"this pipeline was planned for {self.S_pos} positive slots")
+        if self.N_neg and (neg_roots is None or neg_roots.numel() != self.N_neg or neg_ts.numel() != self.N_neg):
+            raise ValueError(f"this pipeline was planned for {self.N_neg} negatives")
+        self.in_roots.copy_(roots, non_blocking=True)
+        self.in_ts.copy_(root_ts, non_blocking=True)
+        if self.N_neg:
+            self.in_neg.copy_(neg_roots, non_blocking=True)
+            self.in_neg_ts.copy_(neg_ts, non_blocking=True)
+        if not self.use_graph:
+            self._chain()
+        elif self._graph is None:
+            self._chain()                      # warm-up outside capture (also the result of this call)
+            torch.cuda.current_stream(self.dev).synchronize()
+            side = torch.cuda.Stream(self.dev)
+            side.wait_stream(torch.cuda.current_stream(self.dev))
+            with torch.cuda.stream(side):
+                self._chain()
+            torch.cuda.current_stream(self.dev).wait_stream(side)
+            torch.cuda.current_stream(self.dev).synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self._chain()
+            self._graph = g
+            g.replay()
+        else:
+            self._graph.replay()
+        return MiniBatch(self)

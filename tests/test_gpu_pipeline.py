@@ -1,0 +1,60 @@
+"""GPU: the pre-planned mini-batch unit (sample -> unique -> gathers -> time encoding),
+eager and as a replayed HIP graph, against the CPU oracle stage by stage."""
+import numpy as np
+import pytest
+import torch
+
+from starrygl_amd.lib import _abi
+from starrygl_amd.utils import synth
+from util import host_graph, np_of, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+@pytest.mark.parametrize("sample_type", ["recent", "uniform"])
+def test_pipeline_matches_oracle(oracle, hot, use_graph, sample_type):
+    from starrygl_amd.data import MiniBatchPipeline
+    from starrygl_amd.lib.libstarrygl_comm import from_edge_index
+    n, m, B = 4000, 80_000, 300
+    src, dst, ts, eid = synth.graph_stream(n, m, 1.15, 500_000, 21)
+    hg = host_graph(oracle, n, src, dst, ts, eid)
+    g = from_edge_index(n, 1, *(torch.from_numpy(x) for x in (src, dst, ts, eid)))
+    rng = np.random.default_rng(2)
+    mem = rng.standard_normal((n, 100)).astype(np.float32)
+    mem_ts = rng.integers(0, 10**6, n).astype(np.int64)
+    efeat = rng.standard_normal((m, 172)).astype(np.float32)
+    hot_ids = rng.permutation(n)[: n // 4]
+    slot = np.full(n, -1, np.int32); slot[hot_ids] = np.arange(hot_ids.size, dtype=np.int32)
+    c_mem = hot.cache(400, to_dev(hot, mem[hot_ids], "f32"), rows=n, cold=torch.from_numpy(mem).pin_memory(),
+                      hot_slot=to_dev(hot, slot, "i32"), ts_hot=to_dev(hot, mem_ts[hot_ids]),
+                      ts_cold=torch.from_numpy(mem_ts).pin_memory())
+    c_ef = hot.cache(688, to_dev(hot, efeat, "f32"))
+    w = (1.0 / 10 ** np.linspace(0, 9, 100, dtype=np.float32)).astype(np.float32)
+    b = rng.standard_normal(100).astype(np.float32)
+    pipe = MiniBatchPipeline(g, 2 * B, B, 2, 5, sample_type, node_tables={"mem": c_mem}, edge_tables={"f": c_ef},
+                             time_encoder=(to_dev(hot, w, "f32"), to_dev(hot, b, "f32")), seed=9, use_graph=use_graph)
+    pipe.view("mem", torch.float32).view("f", torch.float32)
+    for lo in (20_000, 50_000, 79_000, 30_000):
+        roots, ts_ptr, root_ts, neg, neg_ts = synth.link_batch(src, dst, ts, lo, lo + B, n, B, rng)
+        mb = pipe.run(to_dev(hot, roots), to_dev(hot, root_ts), to_dev(hot, neg), to_dev(hot, neg_ts)).finalize()
+        want = oracle.sample_khop(hg, roots, ts_ptr, root_ts, neg, neg_ts, 2, oracle.params(sample_type, 5, seed=9))
+        arrays = [want.slot_node0] + [h.neighbors for h in want.hops]
+        loc, uniq, _ = oracle.unique_compact(arrays, _abi.UNIQUE_SORTED, None, True)
+        assert mb.E == [h.E for h in want.hops] and mb.num_unique == uniq.shape[0]
+        assert np.array_equal(np_of(mb.nid_mapper), uniq) and np.array_equal(np_of(mb.slot_local), loc[0])
+        assert np.array_equal(np_of(mb.node_data["mem"]), mem[uniq])
+        assert np.array_equal(np_of(mb.node_ts["mem"]), mem_ts[uniq])
+        for l, h in enumerate(want.hops):
+            assert np.array_equal(np_of(mb.hops[l]["neighbors_local"]), loc[1 + l])
+            assert np.array_equal(np_of(mb.hops[l]["neighbors_eid"]), h.neighbors_eid)
+            assert np.array_equal(np_of(mb.edge_data[l]["f"]), efeat[h.neighbors_eid])
+            y = oracle.time_encode(h.neighbors_dt, w, b)
+            assert np.abs(np_of(mb.time_feat[l]) - y).max() <= 1e-6
+        blocks = mb.blocks()
+        assert [bk.num_edges() for bk in blocks] == mb.E[::-1]
+        outer = blocks[0]
+        assert outer.num_dst_nodes() == mb.S[0] + mb.E[0] and outer.num_src_nodes() == mb.S[0] + mb.E[0] + mb.E[1]
+        assert np.array_equal(uniq[np_of(outer.srcdata["nid"])[-mb.E[1]:]], want.hops[1].neighbors)
+    with pytest.raises(ValueError):
+        pipe.run(to_dev(hot, roots[:5]), to_dev(hot, root_ts[:5]), to_dev(hot, neg), to_dev(hot, neg_ts))
