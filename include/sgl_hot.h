@@ -298,6 +298,21 @@ int32_t sgl_block_build(const int64_t* root_start_ptr, const int64_t* counts,
                         int64_t src_offset, int64_t* indptr, int64_t* indices,
                         int64_t* edge_dst, void* stream);
 
+/* -------------------------------------------------- latest event per node */
+/* For N events with dense keys local[i] in [0, U) (local ids from
+ * sgl_unique_compact) and timestamps ts[i]: max_ts[u] = max of ts over the
+ * events of key u, arg[u] = the smallest event index attaining it (first
+ * occurrence wins ties, as torch_scatter.scatter_max does on the CPU); keys
+ * without events get max_ts = INT64_MIN, arg = -1.  Events with local[i]
+ * outside [0, U) are ignored.  Replaces index.unique + scatter_max of
+ * mailbox.get_update_mail / set_mailbox_local
+ * (starrygl/nn/memory/mailbox.py:41-47, 78-83).  N = *N_dev, U = *U_dev when
+ * given (<= N_max, U_max). */
+int32_t sgl_segment_max_ts(const int64_t* local, const int64_t* ts,
+                           int64_t N_max, const int64_t* N_dev,
+                           int64_t U_max, const int64_t* U_dev,
+                           int64_t* max_ts, int64_t* arg, void* stream);
+
 /* ----------------------------------------------------------- time encoding */
 #define SGL_DT_I64 0
 #define SGL_DT_F32 1

@@ -680,3 +680,26 @@ int32_t sglo_block_build(const int64_t* root_start_ptr, const int64_t* counts, i
         }
     return SGL_OK;
 }
+
+/* -------------------------------------------------- latest event per node */
+
+/* Reference: unq, inv = index.unique(return_inverse=True);
+ * max_ts, idx = torch_scatter.scatter_max(mail_ts, inv, 0)
+ * (starrygl/nn/memory/mailbox.py:78-83).  Ties: the first event wins. */
+int32_t sglo_segment_max_ts(const int64_t* local, const int64_t* ts, int64_t N_max,
+                            const int64_t* N_dev, int64_t U_max, const int64_t* U_dev,
+                            int64_t* max_ts, int64_t* arg, void* stream) {
+    (void)stream;
+    if (N_max < 0 || U_max < 0 || (N_max > 0 && (!local || !ts)) || (U_max > 0 && (!max_ts || !arg)))
+        return fail(SGL_EINVAL, "segment_max_ts: null");
+    int64_t N = N_dev ? *N_dev : N_max, U = U_dev ? *U_dev : U_max;
+    if (N > N_max) N = N_max;
+    if (U > U_max) U = U_max;
+    for (int64_t u = 0; u < U; ++u) { max_ts[u] = INT64_MIN; arg[u] = -1; }
+    for (int64_t i = 0; i < N; ++i) {
+        int64_t u = local[i];
+        if (u < 0 || u >= U) continue;
+        if (arg[u] < 0 || ts[i] > max_ts[u]) { max_ts[u] = ts[i]; arg[u] = i; }
+    }
+    return SGL_OK;
+}

@@ -199,3 +199,66 @@ extern "C" int32_t sgl_block_build(const int64_t* root_start_ptr, const int64_t*
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }
+
+// ---- latest event per node (mailbox update reduce) ---------------------------
+namespace sgl {
+namespace {
+
+__global__ void segmax_init_kernel(int64_t U_max, const int64_t* U_dev, int64_t* max_ts, int64_t* arg) {
+    const int64_t U = live_count(U_dev, U_max);
+    for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < U; u += (int64_t)gridDim.x * blockDim.x) {
+        max_ts[u] = INT64_MIN;
+        arg[u] = INT64_MAX;
+    }
+}
+
+// pass 1: max_ts[u] = max ts (atomics spread over the keys)
+__global__ void segmax_max_kernel(const int64_t* __restrict__ local, const int64_t* __restrict__ ts, int64_t N_max,
+                                  const int64_t* N_dev, int64_t U_max, const int64_t* U_dev, int64_t* max_ts) {
+    const int64_t N = live_count(N_dev, N_max), U = live_count(U_dev, U_max);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < N; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t u = local[i];
+        if (u >= 0 && u < U) atomicMax(reinterpret_cast<long long*>(&max_ts[u]), (long long)ts[i]);
+    }
+}
+
+// pass 2: arg[u] = smallest i with ts[i] == max_ts[u]
+__global__ void segmax_arg_kernel(const int64_t* __restrict__ local, const int64_t* __restrict__ ts, int64_t N_max,
+                                  const int64_t* N_dev, int64_t U_max, const int64_t* U_dev,
+                                  const int64_t* __restrict__ max_ts, int64_t* arg) {
+    const int64_t N = live_count(N_dev, N_max), U = live_count(U_dev, U_max);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < N; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t u = local[i];
+        if (u >= 0 && u < U && ts[i] == max_ts[u]) atomicMin(reinterpret_cast<long long*>(&arg[u]), (long long)i);
+    }
+}
+
+__global__ void segmax_fix_kernel(int64_t U_max, const int64_t* U_dev, int64_t* arg) {
+    const int64_t U = live_count(U_dev, U_max);
+    for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < U; u += (int64_t)gridDim.x * blockDim.x)
+        if (arg[u] == INT64_MAX) arg[u] = -1;
+}
+
+}  // namespace
+}  // namespace sgl
+
+extern "C" int32_t sgl_segment_max_ts(const int64_t* local, const int64_t* ts, int64_t N_max, const int64_t* N_dev,
+                                      int64_t U_max, const int64_t* U_dev, int64_t* max_ts, int64_t* arg,
+                                      void* stream) {
+    if (N_max < 0 || U_max < 0) return fail(SGL_EINVAL, "segment_max_ts: negative size");
+    if ((N_max > 0 && (!local || !ts)) || (U_max > 0 && (!max_ts || !arg))) return fail(SGL_EINVAL, "segment_max_ts: NULL array");
+    if (U_max == 0) return SGL_OK;
+    hipStream_t st = as_stream(stream);
+    auto grid = [](int64_t n) { int64_t b = ceil_div<int64_t>(n > 0 ? n : 1, BLOCK); return dim3((unsigned)(b > 2048 ? 2048 : b)); };
+    hipLaunchKernelGGL(segmax_init_kernel, grid(U_max), dim3(BLOCK), 0, st, U_max, U_dev, max_ts, arg);
+    SGL_LAUNCH_CHECK();
+    if (N_max > 0) {
+        hipLaunchKernelGGL(segmax_max_kernel, grid(N_max), dim3(BLOCK), 0, st, local, ts, N_max, N_dev, U_max, U_dev, max_ts);
+        SGL_LAUNCH_CHECK();
+        hipLaunchKernelGGL(segmax_arg_kernel, grid(N_max), dim3(BLOCK), 0, st, local, ts, N_max, N_dev, U_max, U_dev, max_ts, arg);
+        SGL_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(segmax_fix_kernel, grid(U_max), dim3(BLOCK), 0, st, U_max, U_dev, arg);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}

@@ -287,6 +287,16 @@ class HotPath:
                                       src_offset, be.ptr(indptr), be.ptr(indices), be.ptr(edge_dst), be.stream()))
         return indptr, indices, edge_dst
 
+    # ------------------------------------------------------ latest by key
+    def segment_max_ts(self, local, ts, U, N_dev=None, U_dev=None):
+        """-> (max_ts[U], arg[U]): per dense key the largest timestamp and the first
+        event index attaining it."""
+        be = self.be
+        max_ts, arg = be.empty(max(U, 1)), be.empty(max(U, 1))
+        self._ck(self.lib.segment_max_ts(be.ptr(local), be.ptr(ts), int(local.shape[0]), be.ptr(N_dev), int(U),
+                                         be.ptr(U_dev), be.ptr(max_ts), be.ptr(arg), be.stream()))
+        return max_ts[:U], arg[:U]
+
     # -------------------------------------------------------- time encode
     def time_encode(self, dt, w, b, dt_dtype=_abi.DT_I64, out=None, N_dev=None):
         be, N, dim = self.be, int(dt.shape[0]), int(w.shape[0])

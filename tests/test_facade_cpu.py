@@ -97,3 +97,15 @@ def test_oracle_block_build(oracle):
     assert edst.tolist() == [4, 4, 6, 6, 6]
     # expanding indptr back gives edge_dst: the CSC and the COO view agree
     assert np.repeat(np.arange(7), np.diff(indptr)).tolist() == edst.tolist()
+
+
+def test_oracle_segment_max_ts(oracle):
+    rng = np.random.default_rng(3)
+    local = rng.integers(-1, 12, 500).astype(np.int64)      # -1 and 10, 11 are outside [0, 10)
+    ts = rng.integers(0, 20, 500).astype(np.int64)          # many ties
+    mx, arg = oracle.segment_max_ts(local, ts, 10)
+    for u in range(10):
+        pos = np.flatnonzero(local == u)
+        assert mx[u] == ts[pos].max() and arg[u] == pos[np.argmax(ts[pos])]     # argmax = first occurrence
+    mx, arg = oracle.segment_max_ts(np.array([0, 0], np.int64), np.array([5, 7], np.int64), 3)
+    assert arg.tolist() == [1, -1, -1] and mx[0] == 7 and mx[1] == np.iinfo(np.int64).min

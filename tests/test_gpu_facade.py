@@ -223,3 +223,45 @@ def test_time_encoder_module():
     assert np.allclose(frozen.w.weight.detach().cpu().numpy().reshape(-1), want)
     with pytest.raises(RuntimeError):
         TimeEncoder(8)(torch.zeros(1))
+
+
+def test_segment_max_and_mailbox(oracle, hot):
+    rng = np.random.default_rng(6)
+    local = rng.integers(-2, 3005, 200_000).astype(np.int64)
+    ts = rng.integers(-50, 50, 200_000).astype(np.int64)
+    mx, arg = hot.segment_max_ts(to_dev(hot, local), to_dev(hot, ts), 3000)
+    omx, oarg = oracle.segment_max_ts(local, ts, 3000)
+    assert np.array_equal(np_of(mx), omx) and np.array_equal(np_of(arg), oarg)
+
+    from starrygl_amd.nn.memory.mailbox import mailbox
+    n, size, d_out, d_e, B = 500, 2, 8, 4, 300
+    mb = mailbox(n, size, d_out, d_e, device="cuda:0")
+    assert mb.shape == (n, size, 2 * d_out + d_e)
+    ref_box, ref_ts, ref_pos = np.zeros((n, size, 20), np.float32), np.zeros((n, size), np.float32), np.zeros(n, np.int64)
+    for it in range(4):
+        src, dst = rng.integers(0, n, B), rng.integers(0, n, B)
+        t = np.sort(rng.integers(0, 50, B)).astype(np.float32) + it * 50
+        ef, ms, md = (rng.standard_normal((B, k)).astype(np.float32) for k in (d_e, d_out, d_out))
+        T = lambda a: torch.from_numpy(a).cuda()
+        index, mail, mail_ts = mb.get_update_mail(T(src), T(dst), T(t), T(ef), T(ms), T(md))
+        # numpy restatement: mails of both endpoints, per node the mail with the largest ts (first on ties)
+        idx_all = np.concatenate([src, dst])
+        mails = np.concatenate([np.concatenate([ms, md, ef], 1), np.concatenate([md, ms, ef], 1)], 0)
+        ts_all = np.concatenate([t, t])
+        uniq = np.unique(idx_all)
+        pick = np.array([np.flatnonzero(idx_all == u)[np.argmax(ts_all[idx_all == u])] for u in uniq])
+        assert np.array_equal(np_of(index), uniq)
+        assert np.array_equal(np_of(mail), mails[pick]) and np.array_equal(np_of(mail_ts), ts_all[pick])
+        mb.set_mailbox_local(index, mail, mail_ts)
+        ref_box[uniq, ref_pos[uniq]] = mails[pick]
+        ref_ts[uniq, ref_pos[uniq]] = ts_all[pick]
+        ref_pos[uniq] = (ref_pos[uniq] + 1) % size
+        assert np.array_equal(np_of(mb.mailbox), ref_box) and np.array_equal(np_of(mb.mailbox_ts), ref_ts)
+        assert np.array_equal(np_of(mb.next_mail_pos), ref_pos)
+    m, mt = mb.get_message(torch.tensor([3, 4]).cuda())
+    assert np.array_equal(np_of(m), ref_box[[3, 4]])
+    # 'max' reduction inside set_mailbox_local de-duplicates first
+    mb.reset()
+    idx = torch.tensor([7, 7, 9]).cuda()
+    mb.set_mailbox_local(idx, torch.arange(60, dtype=torch.float32).reshape(3, 20).cuda(), torch.tensor([1.0, 5.0, 2.0]).cuda(), "max")
+    assert np_of(mb.mailbox)[7, 0, 0] == 20 and np_of(mb.mailbox_ts)[7, 0] == 5 and np_of(mb.mailbox)[9, 0, 0] == 40
