@@ -231,6 +231,24 @@ int32_t sgl_gather(const sgl_cache* c, const int64_t* ids, int64_t N_max,
                    const int64_t* N_dev, void* out, int64_t* out_ts,
                    int64_t* stats, void* stream);
 
+/* Several gathers in ONE launch (up to SGL_GATHER_MAX_SEGMENTS): each segment is
+ * what one sgl_gather call takes.  A training step gathers node features, memory
+ * rows and the edge features of every hop; on small batches each launch costs
+ * more than its copy, and host-tier segments overlap their PCIe latency with the
+ * HBM segments.  Every row size must be a multiple of 16 bytes and every table
+ * and output 16-byte aligned (SGL_ENOTSUP otherwise: use sgl_gather). */
+#define SGL_GATHER_MAX_SEGMENTS 8
+typedef struct sgl_gather_seg {
+    const sgl_cache* cache;
+    const int64_t*   ids;
+    int64_t          N_max;
+    const int64_t*   N_dev;   /* optional device live count */
+    void*            out;
+    int64_t*         out_ts;  /* optional */
+} sgl_gather_seg;
+int32_t sgl_gather_multi(int32_t num_segments, const sgl_gather_seg* segs,
+                         void* stream);
+
 /* Scatter rows back (replaces DistNodeState.update, NodeState.py:46-61):
  * ids that are not resident are skipped.  Duplicate ids: the highest i wins
  * is NOT guaranteed; callers pass unique ids (as the reference's callers do). */

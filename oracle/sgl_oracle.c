@@ -703,3 +703,15 @@ int32_t sglo_segment_max_ts(const int64_t* local, const int64_t* ts, int64_t N_m
     }
     return SGL_OK;
 }
+
+/* Several gathers at once: by definition the same as one sglo_gather per segment. */
+int32_t sglo_gather_multi(int32_t T, const sgl_gather_seg* segs, void* stream) {
+    if (T < 0 || (T > 0 && !segs)) return fail(SGL_EINVAL, "gather_multi: bad segment list");
+    if (T > SGL_GATHER_MAX_SEGMENTS) return fail(SGL_ENOTSUP, "gather_multi: too many segments");
+    for (int32_t t = 0; t < T; ++t) {
+        int32_t rc = sglo_gather(segs[t].cache, segs[t].ids, segs[t].N_max, segs[t].N_dev, segs[t].out,
+                                 segs[t].out_ts, NULL, stream);
+        if (rc != SGL_OK) return rc;
+    }
+    return SGL_OK;
+}

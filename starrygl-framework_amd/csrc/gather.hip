@@ -117,6 +117,66 @@ __global__ __launch_bounds__(BLOCK) void gather_kernel(GatherArgs a) {
                   (unsigned long long)s_tier[threadIdx.x]);
 }
 
+
+struct MultiSeg {
+    sgl_cache c;
+    const int64_t* ids;
+    int64_t N_max;
+    const int64_t* N_dev;
+    char* out;
+    int64_t* out_ts;
+    int32_t rpb, cpr;
+};
+struct MultiArgs {
+    int32_t T;
+    MultiSeg seg[SGL_GATHER_MAX_SEGMENTS];
+};
+
+// Several gathers in one launch: every block walks its grid-stride share of the
+// tiles of segment 0, then of segment 1, ...  16-byte chunks only.
+__global__ __launch_bounds__(BLOCK) void gather_multi_kernel(MultiArgs m) {
+    extern __shared__ const char* s_src[];
+#pragma unroll 1
+    for (int t = 0; t < m.T; ++t) {
+        const MultiSeg& a = m.seg[t];
+        const int64_t N = live_count(a.N_dev, a.N_max);
+        const int32_t cpr = a.cpr;
+        for (int64_t row0 = (int64_t)blockIdx.x * a.rpb; row0 < N; row0 += (int64_t)gridDim.x * a.rpb) {
+            const int32_t rows = (int32_t)((N - row0) < a.rpb ? (N - row0) : a.rpb);
+            __syncthreads();  // s_src of the previous tile has been consumed
+            for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
+                int64_t ts;
+                int tier;
+                s_src[r] = resolve(a.c, a.ids[row0 + r], &ts, &tier);
+                if (a.out_ts != nullptr) a.out_ts[row0 + r] = ts;
+            }
+            __syncthreads();
+            const int32_t total = rows * cpr;
+            u32x4* __restrict__ dst = reinterpret_cast<u32x4*>(a.out + row0 * a.c.row_bytes);
+            for (int32_t base = 0; base < total; base += BLOCK * UNROLL) {
+                u32x4 val[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    const int32_t lc = base + u * BLOCK + threadIdx.x;
+                    u32x4 v = {};
+                    if (lc < total) {
+                        const int32_t r = lc / cpr;
+                        const int32_t part = lc - r * cpr;
+                        const u32x4* src = reinterpret_cast<const u32x4*>(s_src[r]);
+                        if (src != nullptr) v = src[part];
+                    }
+                    val[u] = v;
+                }
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    const int32_t lc = base + u * BLOCK + threadIdx.x;
+                    if (lc < total) dst[lc] = val[u];
+                }
+            }
+        }
+    }
+}
+
 struct ScatterArgs {
     sgl_cache c;
     char* hot_rw;
@@ -228,6 +288,41 @@ extern "C" int32_t sgl_gather(const sgl_cache* c, const int64_t* ids, int64_t N_
     else if (vec == 16) hipLaunchKernelGGL((gather_kernel<u32x4, false>), grid, blk, shmem, st, a);
     else if (vec == 8) hipLaunchKernelGGL((gather_kernel<u32x2, false>), grid, blk, shmem, st, a);
     else hipLaunchKernelGGL((gather_kernel<uint32_t, false>), grid, blk, shmem, st, a);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}
+
+
+extern "C" int32_t sgl_gather_multi(int32_t T, const sgl_gather_seg* segs, void* stream) {
+    if (T < 0 || (T > 0 && !segs)) return fail(SGL_EINVAL, "gather_multi: bad segment list");
+    if (T > SGL_GATHER_MAX_SEGMENTS) return fail(SGL_ENOTSUP, "gather_multi: more than %d segments", SGL_GATHER_MAX_SEGMENTS);
+    MultiArgs m;
+    m.T = 0;
+    int64_t max_rpb = 1, want_blocks = 1;
+    for (int32_t t = 0; t < T; ++t) {
+        const sgl_gather_seg& g = segs[t];
+        int32_t rc;
+        if ((rc = check_cache(g.cache)) != SGL_OK) return rc;
+        if (g.N_max < 0) return fail(SGL_EINVAL, "gather_multi: N_max < 0");
+        if (g.N_max == 0) continue;
+        if (!g.ids || !g.out) return fail(SGL_EINVAL, "gather_multi: ids/out is NULL");
+        if (pick_vec(g.cache->row_bytes, {g.cache->hot, g.cache->cold, g.out}) != 16)
+            return fail(SGL_ENOTSUP, "gather_multi: segment %d is not 16-byte aligned / sized", t);
+        MultiSeg& a = m.seg[m.T++];
+        a.c = *g.cache; a.ids = g.ids; a.N_max = g.N_max; a.N_dev = g.N_dev;
+        a.out = static_cast<char*>(g.out); a.out_ts = g.out_ts;
+        a.cpr = (int32_t)(g.cache->row_bytes / 16);
+        int64_t rpb = (int64_t)BLOCK * UNROLL / a.cpr;
+        rpb = rpb < 1 ? 1 : (rpb > 1024 ? 1024 : rpb);
+        a.rpb = (int32_t)rpb;
+        max_rpb = rpb > max_rpb ? rpb : max_rpb;
+        const int64_t b = ceil_div<int64_t>(g.N_max, rpb);
+        want_blocks = b > want_blocks ? b : want_blocks;
+    }
+    if (m.T == 0) return SGL_OK;
+    if (want_blocks > MAX_GRID) want_blocks = MAX_GRID;
+    hipLaunchKernelGGL(gather_multi_kernel, dim3((unsigned)want_blocks), dim3(BLOCK), (size_t)max_rpb * sizeof(char*),
+                       as_stream(stream), m);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }

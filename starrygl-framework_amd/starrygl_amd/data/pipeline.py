@@ -140,6 +140,7 @@ class MiniBatchPipeline:
         hp._workspace(hp.lib.unique_workspace_bytes(graph._n, 1 + self.layers,
                                                     (_abi.i64 * (1 + self.layers))(*caps)))
         self.use_graph, self._graph = use_graph, None
+        self._plans, self._slow = None, []
 
     def view(self, name, dtype):
         """Reinterpret the byte output buffers of table `name` as rows of `dtype`."""
@@ -160,11 +161,19 @@ class MiniBatchPipeline:
         lens = [self.S0_dev] + [h.counts[1:2] for h in kr.hops]
         hp.unique_compact(arrays, _abi.UNIQUE_SORTED, self.state, True, lens_dev=lens, out_arrays=self.local,
                           finalize=False, unique_out=self.ubuf, U_out=self.U)
-        for name, c in self.node_tables.items():
-            hp.gather(c, self.ubuf, self.node_out[name], out_ts=self.node_ts_out.get(name), N_dev=self.U[0:1])
+        if self._plans is None:      # every gather of the batch in as few launches as possible
+            segs = [(c, self.ubuf, self.node_out[name], self.node_ts_out.get(name), self.U[0:1])
+                    for name, c in self.node_tables.items()]
+            segs += [(c, h.neighbors_eid, self.edge_out[name][l], None, h.counts[1:2])
+                     for l, h in enumerate(kr.hops) for name, c in self.edge_tables.items()]
+            fast = [s for s in segs if s[0].row_bytes % 16 == 0]
+            self._slow = [s for s in segs if s[0].row_bytes % 16 != 0]
+            self._plans = [hp.gather_plan(fast[i: i + 8]) for i in range(0, len(fast), 8)]
+        for plan in self._plans:
+            hp.gather_multi(plan)
+        for c, ids, out, out_ts, n_dev in self._slow:
+            hp.gather(c, ids, out, out_ts=out_ts, N_dev=n_dev)
         for l, h in enumerate(kr.hops):
-            for name, c in self.edge_tables.items():
-                hp.gather(c, h.neighbors_eid, self.edge_out[name][l], N_dev=h.counts[1:2])
             if self.te is not None:
                 hp.time_encode(h.neighbors_dt, self.te[0], self.te[1], out=self.te_out[l], N_dev=h.counts[1:2])
 

@@ -42,6 +42,10 @@ class Cache(C.Structure):
                 ("ts_hot", vp), ("ts_cold", vp)]
 
 
+class GatherSeg(C.Structure):
+    _fields_ = [("cache", C.POINTER(Cache)), ("ids", vp), ("N_max", i64), ("N_dev", vp), ("out", vp), ("out_ts", vp)]
+
+
 class SeedQuery(C.Structure):
     _fields_ = [("chunk_ptr", vp), ("chunk_nodes", vp), ("num_chunks", i64), ("chunks", vp),
                 ("cand_off", vp), ("n_cand", i64), ("t_begin", i64), ("t_end", i64)]
@@ -67,6 +71,7 @@ PROTOTYPES = {
     "unique_compact": (i32, [vp, i64, i32, i32, i32, P(vp), P(i64), P(vp), P(vp),
                              vp, i64, vp, vp, sz, vp]),
     "gather": (i32, [P(Cache), vp, i64, vp, vp, vp, vp, vp]),
+    "gather_multi": (i32, [i32, P(GatherSeg), vp]),
     "scatter_update": (i32, [P(Cache), vp, vp, vp, vp, vp, i64, vp, vp, vp]),
     "chunk_index_workspace_bytes": (sz, [i64]),
     "chunk_index_build": (i32, [i64, i64, vp, vp, vp, vp, sz, vp]),

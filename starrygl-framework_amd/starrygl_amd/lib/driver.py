@@ -9,7 +9,7 @@ library with the same ABI on host memory.
 import ctypes as C
 
 from . import _abi
-from ._abi import (TCSR, Cache, HopOut, SampleParams, SeedQuery, check, i64, vp)
+from ._abi import (TCSR, Cache, GatherSeg, HopOut, SampleParams, SeedQuery, check, i64, vp)
 
 
 class TorchBackend:
@@ -245,6 +245,20 @@ class HotPath:
         self._ck(self.lib.gather(C.byref(cache), be.ptr(ids), int(ids.shape[0]), be.ptr(N_dev),
                                  be.ptr(out), be.ptr(out_ts), be.ptr(stats), be.stream()))
         return out
+
+    def gather_plan(self, segments):
+        """Pre-marshalled argument block for `gather_multi`: segments is a list of
+        (cache, ids, out, out_ts or None, N_dev or None)."""
+        be = self.be
+        arr = (GatherSeg * len(segments))()
+        for i, (c, ids, out, out_ts, n_dev) in enumerate(segments):
+            arr[i] = GatherSeg(C.pointer(c), be.ptr(ids), int(ids.shape[0]), be.ptr(n_dev), be.ptr(out), be.ptr(out_ts))
+        arr._keep = segments
+        return arr
+
+    def gather_multi(self, plan):
+        """All segments of `plan` (from gather_plan) in one launch."""
+        self._ck(self.lib.gather_multi(len(plan), plan, self.be.stream()))
 
     def scatter_update(self, cache, hot_rw, cold_rw, ts_hot_rw, ts_cold_rw, ids, values, ts=None):
         be = self.be

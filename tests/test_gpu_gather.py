@@ -133,3 +133,40 @@ def test_scatter_update_roundtrip(oracle, hot):
     hot.gather(cache, to_dev(hot, ids), out)
     keep = ids_bad >= 0
     assert np.array_equal(np_of(out)[keep], vals[keep])
+
+
+def test_gather_multi_equals_single_gathers(oracle, hot):
+    """three segments (tiered 400 B rows with timestamps and a device-side count, all-HBM 688 B
+    rows, all-HBM 256 B rows) in one launch == three sgl_gather calls, byte for byte."""
+    rng = np.random.default_rng(11)
+    rows = 6000
+    full, h, c, slot = _tables(rows, 100, np.float32, 0.3, 1)
+    ts_full = rng.integers(0, 10**9, rows).astype(np.int64)
+    ts_hot = np.zeros(h.shape[0], np.int64); ts_hot[slot[slot >= 0]] = ts_full[slot >= 0]
+    c0, keep0 = _dev_cache(hot, full, h, c, slot, ts_hot=to_dev(hot, ts_hot), ts_cold=torch.from_numpy(ts_full).pin_memory())
+    t1 = rng.standard_normal((9000, 172)).astype(np.float32)
+    t2 = rng.integers(0, 2**16, (3000, 128), dtype=np.uint16)
+    d1, d2 = torch.from_numpy(t1).cuda(), torch.from_numpy(t2).cuda()
+    c1, c2 = hot.cache(688, d1), hot.cache(256, d2)
+    ids = [rng.integers(-1, rows + 1, 20_000).astype(np.int64), rng.integers(0, 9000, 50_000).astype(np.int64),
+           rng.integers(0, 3000, 7).astype(np.int64)]
+    d_ids = [to_dev(hot, x) for x in ids]
+    live0 = to_dev(hot, np.array([12_345], dtype=np.int64))
+    outs = [torch.zeros((20_000, 100), device="cuda"), torch.empty((50_000, 172), device="cuda"),
+            torch.empty((7, 128), dtype=torch.uint16, device="cuda")]
+    out_ts = hot.be.zeros(20_000)
+    plan = hot.gather_plan([(c0, d_ids[0], outs[0], out_ts, live0), (c1, d_ids[1], outs[1], None, None),
+                            (c2, d_ids[2], outs[2], None, None)])
+    hot.gather_multi(plan)
+    ref0, ref_ts = torch.zeros((20_000, 100), device="cuda"), hot.be.zeros(20_000)
+    hot.gather(c0, d_ids[0], ref0, out_ts=ref_ts, N_dev=live0)
+    assert torch.equal(outs[0], ref0) and torch.equal(out_ts, ref_ts) and not np_of(outs[0])[12_345:].any()
+    ok = (ids[0][:12_345] >= 0) & (ids[0][:12_345] < rows)
+    assert np.array_equal(np_of(outs[0])[:12_345][ok], full[ids[0][:12_345][ok]])
+    assert np.array_equal(np_of(out_ts)[:12_345][ok], ts_full[ids[0][:12_345][ok]])
+    assert np.array_equal(np_of(outs[1]), t1[ids[1]]) and np.array_equal(np_of(outs[2]), t2[ids[2]])
+    # rows that are not a multiple of 16 bytes are refused (the single-gather entry point takes them)
+    c3 = hot.cache(12, torch.zeros((10, 3), device="cuda"))
+    bad = hot.gather_plan([(c3, d_ids[2], torch.zeros((7, 3), device="cuda"), None, None)])
+    with pytest.raises(RuntimeError):
+        hot.gather_multi(bad)
