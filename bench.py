@@ -24,9 +24,10 @@ for _p in (ROOT, os.path.join(ROOT, "starrygl-framework_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per gathered 688-byte row of the hop-2 edge-feature gather, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs of this script (summary and commands: profiles/gather_kernel_configs1_hbm_traffic.md)
-MEASURED_HBM_BYTES_PER_ROW = {"read": 657.8, "write": 702.5}
+# HBM bytes moved per algorithmic byte by the step's gather launch (node rows + hop-1 + hop-2 edge rows),
+# from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (summary and commands:
+# profiles/gather_multi_kernel_configs1_hbm_traffic.md)
+MEASURED_HBM_PER_ALGORITHMIC_BYTE = {"read": 0.994, "write": 1.002}
 
 
 def log(*a):
@@ -225,6 +226,87 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     return res
 
 
+def workload_large_partition(hot, torch, np, synth, _abi, n=100_000_000, m=1_000_000_000, R=50_000, k=20):
+    """configs[3]: one 100M-node / 1B-edge T-CSR (24.8 GB), batches of 50 000 roots with uniform
+    timestamps, 2-hop most-recent 20x20, unique + compaction of every sampled id (dense-table and
+    hash-set path), block construction.  The graph is generated on the device; roots are sources
+    of uniformly drawn edges and destinations follow the out-degree law, so that second-hop slots
+    have neighbours to return and a batch samples about 17M edges."""
+    dev, T_BITS = hot.be.device, 36
+    t0 = time.time()
+    row_ptr, col, ts, eid, key = synth.graph_by_degree_device(torch, dev, n, m, 1.05, 1_000_000, T_BITS, 20243)
+    g = hot.tcsr_from_sorted(n, row_ptr, col, ts, eid, validate=True)
+    gen = torch.Generator(device=dev).manual_seed(1)
+    NB = 4
+    roots = [key[torch.randint(0, m, (R,), device=dev, generator=gen)] >> T_BITS for _ in range(NB)]
+    root_ts = [torch.randint(0, 1 << T_BITS, (R,), device=dev, generator=gen) for _ in range(NB)]
+    max_deg = int((row_ptr[1:] - row_ptr[:-1]).max())
+    del key
+    torch.cuda.synchronize()
+    log(f"[c4] graph ready in {time.time() - t0:.1f}s (max degree {max_deg})")
+    empty, ts_ptr = hot.be.empty(0), torch.arange(R + 1, device=dev)
+    p = hot.params("recent", k)
+    kr = hot.khop_buffers(R, 2, k)
+    caps = [R, R * k, R * k * k]
+    local = [hot.be.empty(c) for c in caps]
+    ubuf, U = hot.be.empty(sum(caps)), hot.be.zeros(2)
+    state = hot.remap_state(n)
+    R_dev = torch.tensor([R], device=dev)
+    hot._workspace(hot.lib.unique_workspace_bytes(n, 3, (_abi.i64 * 3)(*caps)))
+    res = {"nodes": n, "edges": m, "roots_per_batch": R, "fanout": [k, k], "max_degree": max_deg}
+
+    def sample(b):
+        hot.sample_khop(g, roots[b], ts_ptr, root_ts[b], empty, empty, 2, p, finalize=False, out=kr)
+
+    def arrays():
+        return [kr.slot_node0, kr.hops[0].neighbors, kr.hops[1].neighbors]
+
+    def lens():
+        return [R_dev, kr.hops[0].counts[1:2], kr.hops[1].counts[1:2]]
+
+    def unique_dense():
+        hot.unique_compact(arrays(), _abi.UNIQUE_GROUPED, state, True, lens_dev=lens(), out_arrays=local,
+                           finalize=False, unique_out=ubuf, U_out=U)
+
+    def blocks():
+        off = 0
+        for h in kr.hops:
+            hot.block_build(h.root_start_ptr, h.counts, h.cap_slots, h.cap_edges, off, off + h.cap_slots)
+
+    ms_s, e_tot = [], 0
+    for b in range(NB):
+        ms_s.append(_time_launches(torch, lambda: sample(b), reps=5, warm=1))
+        c = kr.counts.cpu().numpy()
+        e_tot += int(c[1] + c[4])
+    sample(0)
+    c = kr.counts.cpu().numpy()
+    E0, E1 = int(c[1]), int(c[4])
+    ms = float(np.mean(ms_s))
+    samp_bytes = lambda S, E: S * 48 + E * 56
+    res["sample_recent_2hop"] = {"ms": round(ms, 4), "edges_per_batch": e_tot / NB,
+                                 "edges_per_s": round(e_tot / NB / ms * 1e3, 1),
+                                 "GBps": round((samp_bytes(R, E0) + samp_bytes(E0, E1)) / ms / 1e6, 1)}
+    ids_in = R + E0 + E1
+    ms = _time_launches(torch, unique_dense, reps=5, warm=1)
+    u = int(U[0].item())
+    res["unique_compact_dense_table"] = {"ms": round(ms, 4), "ids": ids_in, "unique": u,
+                                         "ids_per_s": round(ids_in / ms * 1e3, 1),
+                                         "GBps": round((16 * ids_in + 8 * u) / ms / 1e6, 1)}
+    live = [a[:l] for a, l in zip(arrays(), (R, E0, E1))]
+
+    def unique_hash():
+        hot.unique_compact(live, _abi.UNIQUE_SORTED, None, True, out_arrays=[x[:a.numel()] for x, a in zip(local, live)],
+                           finalize=False, unique_out=ubuf, U_out=U)
+
+    ms = _time_launches(torch, unique_hash, reps=3, warm=1)
+    res["unique_compact_hash_set"] = {"ms": round(ms, 4), "ids": ids_in, "ids_per_s": round(ids_in / ms * 1e3, 1),
+                                      "GBps": round((16 * ids_in + 8 * u) / ms / 1e6, 1)}
+    ms = _time_launches(torch, blocks, reps=5, warm=1)
+    res["block_build_2_layers"] = {"ms": round(ms, 4), "edges": E0 + E1,
+                                   "GBps": round((8 * (E0 + E1) + 16 * (R + E0)) / ms / 1e6, 1)}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -236,9 +318,9 @@ def main():
     ap.add_argument("--fanout", type=int, default=10)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--no-edge-feat", action="store_true", help="skip the 13.8 GB edge feature table (debug)")
-    ap.add_argument("--workload", default="all", choices=["c2", "c3", "c5", "all"],
-                    help="c2 = the headline workload (always run); 'all' adds the cache stress test (c3) and the "
-                         "TGN step (c5) as extra_workloads")
+    ap.add_argument("--workload", default="all", choices=["c2", "c3", "c4", "c5", "all"],
+                    help="c2 = the headline workload (always run); 'all' adds the cache stress test (c3), the "
+                         "1B-edge partition (c4) and the TGN step (c5) as extra_workloads")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (known traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings can be scaled")
@@ -293,11 +375,13 @@ def main():
 
     p_rec = hot.params("recent", k)
     p_uni = hot.params("uniform", k, seed=20242)
-    kr, ku = hot.khop_buffers(S0, 2, k), hot.khop_buffers(S0, 2, k)
+    # every device-side count of a step lives in one array, so that one add accumulates them all
+    live = torch.zeros(14, dtype=torch.int64, device=dev)     # recent S,E,bad x2 | uniform S,E,bad x2 | U_total, U_before
+    kr, ku = hot.khop_buffers(S0, 2, k, counts=live[0:6]), hot.khop_buffers(S0, 2, k, counts=live[6:12])
     state = hot.remap_state(n)
     total_ids = S0 + S0 * k + S0 * k * k
     local = [hot.be.empty(S0), hot.be.empty(S0 * k), hot.be.empty(S0 * k * k)]
-    ubuf, U = hot.be.empty(min(total_ids, n)), hot.be.zeros(2)
+    ubuf, U = hot.be.empty(min(total_ids, n)), live[12:14]
     S0_dev = D(np.array([S0], dtype=np.int64))
     node_out = torch.empty((min(total_ids, n), 100), device=dev)
     e_out = [torch.empty((S0 * k, 172), device=dev), torch.empty((S0 * k * k, 172), device=dev)] if edge_cache else None
@@ -305,13 +389,16 @@ def main():
     hot._workspace(max(hot.lib.sample_khop_workspace_bytes(S0, 2, k),
                        hot.lib.unique_workspace_bytes(n, 3, (_abi.i64 * 3)(S0, S0 * k, S0 * k * k))))
 
-    # static input buffers: a step copies its batch here (4 small D2D copies), the stages read them
-    s_roots, s_root_ts, s_neg, s_neg_ts = (torch.empty_like(roots[0]), torch.empty_like(root_ts[0]),
-                                           torch.empty_like(neg[0]), torch.empty_like(neg_ts[0]))
-    acc = torch.zeros(5, dtype=torch.int64, device=dev)   # running sums of E0, E1 (recent), E0, E1 (uniform), U
+    # static input buffer: a step copies its batch here (one D2D copy of the packed roots, root
+    # times, negatives and their times), the stages read views of it
+    packed = torch.cat([roots, root_ts, neg, neg_ts], dim=1).contiguous()
+    s_all = torch.empty_like(packed[0])
+    s_roots, s_root_ts, s_neg, s_neg_ts = torch.split(s_all, [roots.shape[1], root_ts.shape[1], neg.shape[1], neg_ts.shape[1]])
+    acc = torch.zeros(14, dtype=torch.int64, device=dev)  # running sums of `live`
+    ACC = [1, 4, 7, 10, 12]                               # E0, E1 (recent), E0, E1 (uniform), U
 
     def stage_inputs(b):
-        s_roots.copy_(roots[b]); s_root_ts.copy_(root_ts[b]); s_neg.copy_(neg[b]); s_neg_ts.copy_(neg_ts[b])
+        s_all.copy_(packed[b])
 
     def st_recent():
         hot.sample_khop(dg, s_roots, ts_ptr, s_root_ts, s_neg, s_neg_ts, 2, p_rec, finalize=False, out=kr)
@@ -336,7 +423,7 @@ def main():
         hot.sample_khop(dg, s_roots, ts_ptr, s_root_ts, s_neg, s_neg_ts, 2, p_uni, finalize=False, out=ku)
 
     def st_account():
-        acc[0:2].add_(kr.counts[1::3]); acc[2:4].add_(ku.counts[1::3]); acc[4:5].add_(U[0:1])
+        acc.add_(live)
 
     stages_fn = [st_recent, st_unique, st_node, st_edge0, st_edge1, st_uniform]
     # in the step itself the three gathers are one launch
@@ -417,7 +504,7 @@ def main():
         run_step()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t_start
-    tot = acc.cpu().numpy().astype(np.float64)
+    tot = acc.cpu().numpy()[ACC].astype(np.float64)
     # ---- per-stage GPU time: the same K steps, HIP events between the stages
     NEV = len(stages_fn) + 1
     evs = [[torch.cuda.Event(enable_timing=True) for _ in range(NEV)] for _ in range(K)]
@@ -429,7 +516,7 @@ def main():
         for j in range(len(stages_fn)):
             graphs[j].replay() if graphs is not None else stages_fn[j]()
             evs[i][j + 1].record()
-        cnt_log[i, 0:2].copy_(kr.counts[1::3]); cnt_log[i, 2:4].copy_(ku.counts[1::3]); cnt_log[i, 4:5].copy_(U[0:1])
+        cnt_log[i].copy_(live[ACC])
     torch.cuda.synchronize()
     cl = cnt_log.cpu().numpy()
     assert np.array_equal(cl.sum(axis=0).astype(np.float64), tot), "the two passes over the batches disagree"
@@ -461,21 +548,49 @@ def main():
     for v in stages.values():
         for kk in v:
             v[kk] = float(round(v[kk], 4))
-    dom = "gather_edge_feat_hop2" if edge_cache is not None else "gather_node_feat"
-    # the dominant kernel alone: 20 launches back to back between one pair of HIP events on the stream
-    # it is launched on (the per-stage figures above carry one graph launch + one event pair each)
-    stage_inputs(W % NB)
-    st_recent(); st_unique()
-    torch.cuda.synchronize()
-    dom_ms = _time_launches(torch, st_edge1 if edge_cache is not None else st_node, reps=20)
-    c_now = kr.counts.cpu().numpy()
-    dom_bytes = float(c_now[4]) * (8 + 1376) if edge_cache is not None else float(U[0].item()) * (8 + 800)
+    # the dominant kernel alone: the step's gather launch (all three row lists in one launch), 20
+    # launches back to back between one pair of HIP events on the stream it is launched on (the
+    # per-stage figures above carry one graph launch + one event pair each).  Every launch gathers
+    # a different batch's rows, as consecutive steps do: repeating one batch would re-read rows
+    # that the previous launch left in the 256 MB last-level cache.
+    NR = 20
+    rl_plans, rl_rows = [], np.zeros(3)
+    for i in range(NR):
+        stage_inputs((W + i) % NB)
+        st_recent(); st_unique()
+        c_now = live.cpu().numpy()
+        u_, e0_, e1_ = int(c_now[12]), int(c_now[1]), int(c_now[4])
+        rl_rows += (u_, e0_, e1_)
+        if edge_cache is not None:
+            rl_plans.append(hot.gather_plan([(node_cache, ubuf[:u_].clone(), node_out, None, None),
+                                             (edge_cache, kr.hops[0].neighbors_eid[:e0_].clone(), e_out[0], None, None),
+                                             (edge_cache, kr.hops[1].neighbors_eid[:e1_].clone(), e_out[1], None, None)]))
+        else:
+            rl_plans.append(ubuf[:u_].clone())
+    rl_rows /= NR
+
+    def rl_launches():
+        for pl in rl_plans:
+            hot.gather_multi(pl) if edge_cache is not None else hot.gather(node_cache, pl, node_out)
+
+    rl_launches()
+    dom_ms = _time_launches(torch, rl_launches, reps=1, warm=1) / NR
+    if edge_cache is not None:
+        rd = rl_rows[0] * (8 + 400) + (rl_rows[1] + rl_rows[2]) * (8 + 688)
+        wr = rl_rows[0] * 400 + (rl_rows[1] + rl_rows[2]) * 688
+        dom = "gather_multi_kernel (node rows + hop-1 + hop-2 edge rows of one step)"
+        traffic = int(rd * MEASURED_HBM_PER_ALGORITHMIC_BYTE["read"] + wr * MEASURED_HBM_PER_ALGORITHMIC_BYTE["write"])
+    else:
+        rd, wr, traffic = rl_rows[0] * (8 + 400), rl_rows[0] * 400, None
+        dom = "gather_kernel<u32x4> (node rows)"
+    dom_bytes = rd + wr
     ach = round(dom_bytes / dom_ms / 1e6, 1)
-    roofline = {"kernel": "gather_kernel<u32x4> (" + dom + ")", "bound": "hbm", "achieved": ach,
+    roofline = {"kernel": dom, "bound": "hbm", "achieved": ach,
                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4),
-                "traffic": (int(dom_bytes / (8 + 1376) * sum(MEASURED_HBM_BYTES_PER_ROW.values())) if edge_cache is not None else None),
-                "avg_launch_ms": round(dom_ms, 5), "launches_timed": 20,
-                "algorithmic_bytes_per_launch": int(dom_bytes)}
+                "traffic": traffic, "avg_launch_ms": round(dom_ms, 5), "launches_timed": NR,
+                "algorithmic_bytes_per_launch": int(dom_bytes),
+                "mean_rows_per_launch": {"node": rl_rows[0], "edge_hop1": rl_rows[1], "edge_hop2": rl_rows[2]}}
+    del rl_plans
 
     # ---- CPU baseline: the oracle's 2-hop recent sampler on the host cores, same batches
     cpu = None
@@ -533,8 +648,9 @@ def main():
         gc.collect()
         torch.cuda.empty_cache()
     for name, fn in (("configs[2] cache stress", lambda: workload_cache_stress(hot, torch, np, synth)),
+                     ("configs[3] large partition", lambda: workload_large_partition(hot, torch, np, synth, _abi)),
                      ("configs[4] tgn step", lambda: workload_tgn_step(hot, torch, np, synth, _abi))):
-        key = "c3" if "cache" in name else "c5"
+        key = {"configs[2]": "c3", "configs[3]": "c4", "configs[4]": "c5"}[name[:10]]
         if args.workload not in (key, "all"):
             continue
         try:

@@ -154,12 +154,14 @@ class HotPath:
             out.finalize(*be.tolist(out.counts))
         return out
 
-    def khop_buffers(self, S0, layers, fanout):
-        """Worst-case output buffers of a k-hop call; reusable across calls."""
+    def khop_buffers(self, S0, layers, fanout, counts=None):
+        """Worst-case output buffers of a k-hop call; reusable across calls.  `counts`
+        (int64[3 * layers], zeroed) may be a slice of a larger array of the caller's."""
         be = self.be
         slot_node0, slot_ts0 = be.empty(S0), be.empty(S0)
         outs, cap = [], S0
-        counts = be.zeros(3 * max(layers, 1))
+        if counts is None:
+            counts = be.zeros(3 * max(layers, 1))
         for l in range(layers):
             outs.append(HopResult(be, cap, cap * fanout, counts[3 * l: 3 * l + 3]))
             cap *= fanout

@@ -1,7 +1,9 @@
 """Synthetic power-law temporal graphs and request streams (numpy, seeded).
 
 These generate the workloads the benchmark and the tests run on; every array
-is int64 unless stated.  Nothing here touches the GPU.
+is int64 unless stated.  Everything is numpy on the host except
+`graph_by_degree_device`, which builds graphs too large for that with torch on
+the device it is given.
 """
 import numpy as np
 
@@ -86,3 +88,53 @@ def zipf_requests(rows, count, a, seed):
         b = 1.0 - a
         r = (1.0 + u * ((rows + 1.0) ** b - 1.0)) ** (1.0 / b)
     return np.clip(np.floor(r).astype(np.int64) - 1, 0, rows - 1)
+
+
+def graph_by_degree_device(torch, device, n, m, a, max_deg, t_bits, seed, dst_by_degree=True):
+    """A T-CSR of n nodes and m edges generated on `device` with torch: out-degree
+    Zipf(a) by rank, capped at max_deg and scaled to sum m, node ids a random
+    permutation of the ranks; timestamps uniform in [0, 2^t_bits), ascending
+    inside every row; destinations drawn in proportion to out-degree (or
+    uniformly); eid = storage position.  Needs bit_length(n - 1) + t_bits <= 63.
+    Returns (row_ptr, col, ts, eid, key) with key[e] = src[e] << t_bits | ts[e],
+    ascending over the whole edge list: a searchsorted over it finds any row's
+    time window without walking the CSR."""
+    assert max(int(n - 1).bit_length(), 1) + t_bits <= 63
+    gen = torch.Generator(device=device).manual_seed(seed)
+    w = torch.arange(1, n + 1, device=device, dtype=torch.float64).pow_(-a)
+
+    def degrees(c):
+        return torch.clamp((w * c).floor_(), max=float(max_deg)).to(torch.int64)
+
+    lo, hi = 0.0, max_deg / float(w[-1])
+    for _ in range(60):           # largest scale whose floor-and-cap degrees stay within m
+        mid = 0.5 * (lo + hi)
+        if int(degrees(mid).sum()) <= m:
+            lo = mid
+        else:
+            hi = mid
+    deg_rank = degrees(lo)
+    rest = m - int(deg_rank.sum())
+    deg_rank += rest // n
+    if rest % n:
+        deg_rank[n - rest % n:] += 1          # the remainder goes to the tail ranks, one edge each
+    del w
+    ids = torch.randperm(n, device=device, generator=gen)
+    deg = torch.empty_like(deg_rank)
+    deg[ids] = deg_rank
+    del ids, deg_rank
+    row_ptr = torch.zeros(n + 1, dtype=torch.int64, device=device)
+    torch.cumsum(deg, 0, out=row_ptr[1:])
+    key = torch.repeat_interleave(torch.arange(n, device=device), deg, output_size=m)
+    del deg
+    key.mul_(1 << t_bits)
+    key.add_(torch.randint(0, 1 << t_bits, (m,), device=device, generator=gen))
+    key = torch.sort(key).values
+    ts = key & ((1 << t_bits) - 1)
+    if dst_by_degree:
+        col = key[torch.randint(0, m, (m,), device=device, generator=gen)]
+        col >>= t_bits
+    else:
+        col = torch.randint(0, n, (m,), device=device, generator=gen)
+    eid = torch.arange(m, device=device)
+    return row_ptr, col, ts, eid, key
