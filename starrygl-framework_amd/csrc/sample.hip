@@ -4,7 +4,8 @@
 // synchronisation:
 //   count : a group of G lanes owns one (node, t) slot; the group finds the
 //           slot's candidate window with a (G+1)-ary cooperative search on the
-//           row's timestamp slice (ballot + popcount per step) and records the
+//           row's timestamp slice (ballot + popcount per step; G = 1, a plain
+//           binary search per lane, for very large hops) and records the
 //           window start / length; a block walks a contiguous run of slots, G
 //           lanes per slot, BLOCK/G slots at a time, and writes the sum of its
 //           slot counts.  For hop 0 the slots are derived on the fly from the
@@ -57,6 +58,7 @@ struct HopArgs {
     int64_t R, S_pos;
     int32_t derive;      // 1: slots come from roots/negatives
     int32_t scanned;     // 1: scan_kernel wrote chunk_off and published the counts
+    int32_t align;       // a block's run of slots is a multiple of this (both kernels of a hop agree on it)
     int64_t* slot_node_out;
     int64_t* slot_ts_out;
     // params
@@ -99,7 +101,12 @@ __device__ __forceinline__ int64_t group_lower_bound(const int64_t* __restrict__
                 pred = ts[lo + ((int64_t)(lig + 1) * len) / (G + 1)] < key;
             }
         }
-        const int c = __popcll(group_ballot<G>(pred, gshift));
+        int c;
+        if constexpr (G == 1) {
+            c = pred ? 1 : 0;     // one lane per slot: plain binary search, no exchange between lanes
+        } else {
+            c = __popcll(group_ballot<G>(pred, gshift));
+        }
         if (!done) {
             if (last) {
                 lo += c;
@@ -118,8 +125,9 @@ __device__ __forceinline__ int64_t group_lower_bound(const int64_t* __restrict__
     return lo;
 }
 
-// Slots [first, first + run) belong to block b; run is a multiple of the slots a
-// block handles per iteration so that iterations never straddle two blocks.
+// Slots [first, first + run) belong to block b; run is a multiple of `spb`, itself a
+// multiple of the slots either kernel of the hop handles per block iteration, so that
+// iterations never straddle two blocks and both kernels see the same partition.
 __device__ __forceinline__ void block_run(int64_t S, int spb, int64_t* first, int64_t* run) {
     int64_t r = ceil_div<int64_t>(S, (int64_t)gridDim.x);
     r = ceil_div<int64_t>(r, spb) * spb;
@@ -170,13 +178,13 @@ __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
     // When the grid is not capped every block owns exactly SPB slots whatever the live
     // count is: the slot can be loaded before the live count has arrived (one dependent
     // memory round trip less).  Slots in [S, S_max) are allocated, their content is unused.
-    const bool fixed = (int64_t)gridDim.x * SPB >= a.S_max;
+    const bool fixed = a.align == SPB && (int64_t)gridDim.x * SPB >= a.S_max;
     int64_t v0 = 0, t0 = 0;
     const int64_t slot0 = (int64_t)blockIdx.x * SPB + gib;
     if (fixed && slot0 < a.S_max) load_slot(a, slot0, &v0, &t0);
     const int64_t S = live_count(a.S_dev, a.S_max);
     int64_t first, run;
-    block_run(S, SPB, &first, &run);
+    block_run(S, a.align, &first, &run);
     int32_t sum = 0, nbad = 0;                   // per-wave partials, kept by lane 0 of each wave
     for (int64_t it = first; it < first + run && it < S; it += SPB) {
         const int64_t slot = it + gib;
@@ -322,7 +330,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     const int32_t k = a.k;
     // first iteration's slot data: loaded before the live count arrives when the grid is
     // not capped (see count_kernel), and before the prefix sum, so the loads overlap both
-    const bool fixed = (int64_t)gridDim.x * SPB >= a.S_max;
+    const bool fixed = a.align == SPB && (int64_t)gridDim.x * SPB >= a.S_max;
     int64_t slot = (int64_t)blockIdx.x * SPB + gib;
     int64_t start = 0, len = 0, t = 0;
     if (fixed && slot < a.S_max) {
@@ -332,7 +340,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     }
     const int64_t S = live_count(a.S_dev, a.S_max);
     int64_t first, run;
-    block_run(S, SPB, &first, &run);
+    block_run(S, a.align, &first, &run);
     bool active = first < S && first + gib < S;
     if (!fixed) {
         slot = first + gib;
@@ -424,13 +432,30 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
         }
         if (a.type == SGL_SAMPLE_RECENT) {
             if (active) {
-                for (int32_t j = lig; j < c; j += G) {
-                    const int64_t e = start + j;
-                    const int64_t ets = a.ts[e];
-                    a.nbr[off + j] = a.col[e];
-                    a.nbr_ts[off + j] = ets;
-                    a.nbr_eid[off + j] = a.eid[e];
-                    a.nbr_dt[off + j] = ets - t;
+                // up to ROUNDS * G edges per pass, every load issued before the first store
+                constexpr int ROUNDS = 4;
+                for (int32_t j0 = lig; j0 < c; j0 += ROUNDS * G) {
+                    int64_t ets[ROUNDS], dst[ROUNDS], id[ROUNDS];
+#pragma unroll
+                    for (int r = 0; r < ROUNDS; ++r) {
+                        const int32_t j = j0 + r * G;
+                        if (j < c) {
+                            const int64_t e = start + j;
+                            ets[r] = a.ts[e];
+                            dst[r] = a.col[e];
+                            id[r] = a.eid[e];
+                        }
+                    }
+#pragma unroll
+                    for (int r = 0; r < ROUNDS; ++r) {
+                        const int32_t j = j0 + r * G;
+                        if (j < c) {
+                            a.nbr[off + j] = dst[r];
+                            a.nbr_ts[off + j] = ets[r];
+                            a.nbr_eid[off + j] = id[r];
+                            a.nbr_dt[off + j] = ets[r] - t;
+                        }
+                    }
                 }
             }
         } else {
@@ -492,6 +517,14 @@ int pick_group(const sgl_sample_params* p, int64_t S_max) {
     return S_max >= 32768 ? 8 : 16;
 }
 
+// Lanes per slot of the window search.  A hop that fits a few wave-residency rounds is
+// bound by the length of one slot's chain of dependent loads: the G lanes of the copy
+// group search together, (G+1)-ary.  A hop of several hundred thousand slots is bound by
+// the number of loads in flight and by their count: one lane per slot (plain binary
+// search) keeps 8x the slots in flight and issues ~2.5x fewer loads than 8 lanes do
+// (857k slots over rows of up to 1M edges: 187 us against 330 us).
+int pick_search_group(int Gf, int64_t S_max) { return S_max >= 262144 ? 1 : Gf; }
+
 size_t hop_workspace_bytes(int64_t S_max) {
     size_t b = 0;
     b += align_up((size_t)(S_max + 1) * 8) * 2;
@@ -534,19 +567,42 @@ int32_t check_out(const sgl_hop_out* o, int64_t S_max, int32_t k) {
     return SGL_OK;
 }
 
-template <int G>
-int32_t launch_hop(HopArgs a, hipStream_t st) {
-    constexpr int SPB = BLOCK / G;
-    int64_t blocks = ceil_div<int64_t>(a.S_max > 0 ? a.S_max : 1, SPB);
+using HopKernel = void (*)(HopArgs);
+
+HopKernel count_fn(int G) {
+    switch (G) {
+        case 1: return count_kernel<1>;
+        case 2: return count_kernel<2>;
+        case 4: return count_kernel<4>;
+        case 8: return count_kernel<8>;
+        case 16: return count_kernel<16>;
+        case 32: return count_kernel<32>;
+        default: return count_kernel<64>;
+    }
+}
+
+HopKernel fill_fn(int G) {
+    switch (G) {
+        case 8: return fill_kernel<8>;
+        case 16: return fill_kernel<16>;
+        case 32: return fill_kernel<32>;
+        default: return fill_kernel<64>;
+    }
+}
+
+// Gc lanes per slot search, Gf lanes per slot copy or draw
+int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf) {
+    a.align = BLOCK / (Gc < Gf ? Gc : Gf);
+    int64_t blocks = ceil_div<int64_t>(a.S_max > 0 ? a.S_max : 1, a.align);
     if (blocks > MAX_BLOCKS) blocks = MAX_BLOCKS;
     a.scanned = blocks > FUSED_PREFIX_MAX ? 1 : 0;
-    hipLaunchKernelGGL(count_kernel<G>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
+    hipLaunchKernelGGL(count_fn(Gc), dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
     SGL_LAUNCH_CHECK();
     if (a.scanned) {
         hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, a, (int)blocks);
         SGL_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(fill_kernel<G>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
+    hipLaunchKernelGGL(fill_fn(Gf), dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }
@@ -585,12 +641,8 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
     a.root_start_ptr = out->root_start_ptr; a.root_end_ptr = out->root_end_ptr;
     a.nbr = out->neighbors; a.nbr_ts = out->neighbors_ts; a.nbr_eid = out->neighbors_eid;
     a.nbr_dt = out->neighbors_dt; a.counts = out->counts;
-    switch (pick_group(p, S_max)) {
-        case 8: return launch_hop<8>(a, st);
-        case 16: return launch_hop<16>(a, st);
-        case 32: return launch_hop<32>(a, st);
-        default: return launch_hop<64>(a, st);
-    }
+    const int Gf = pick_group(p, S_max);
+    return launch_hop(a, st, pick_search_group(Gf, S_max), Gf);
 }
 
 }  // namespace
