@@ -301,6 +301,40 @@ int32_t sgl_seeds_fill(const sgl_tcsr* g, const sgl_seed_query* q,
                        int64_t* q_ptr, int64_t* q_eid, void* workspace,
                        size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------- sub-graph slice ("cluster" mode) */
+/* The sub-graph of a chunk set over a time window (replaces
+ * count_edges_kernel / write_edges_kernel / mark_chunks_exists_kernel and
+ * Graph::slice_by_chunk_ts, sample.cu.hpp:115-120, 299-515, 1189-1299; the
+ * 'cluster' branch of the query worker, :1953-1961).  Candidates and window
+ * as for the seeds: the nodes of the selected chunks in chunk-list order, edges
+ * with t_begin <= ts < t_end.  A candidate with a non-empty window becomes a
+ * node of the slice; of its window edges those whose destination lies in a
+ * selected chunk (node_chunk[col[e]] selected) are kept, in storage order.
+ *   nodes[R], ts_ptr[R+1] : slice nodes and their ranges in ts[]
+ *   ts[T], edge_ptr[T+1]  : per node a list of timestamps; entry s owns the
+ *                           kept edges [edge_ptr[s], edge_ptr[s+1]), exactly
+ *                           those kept edges of the node with timestamp ts[s]
+ *   col/col_ts/col_eid[E] : the kept edges
+ * full_timestamps == 0: ts[] lists the distinct timestamps of the node's window
+ * edges (kept or not).  full_timestamps == 1 (discrete-time snapshots, what the
+ * query worker asks for): every node lists all integers t_begin .. t_end-1, so
+ * T = R * (t_end - t_begin).
+ *   sgl_slice_count -> totals[0..2] = {R, T, E};   (caller allocates)
+ *   sgl_slice_fill.
+ * node_chunk: device [g->n] chunk id of every node, in [0, total_chunks). */
+size_t  sgl_slice_workspace_bytes(int64_t n_cand, int64_t total_chunks);
+int32_t sgl_slice_count(const sgl_tcsr* g, const sgl_seed_query* q,
+                        const int64_t* node_chunk, int64_t total_chunks,
+                        int32_t full_timestamps, int64_t* totals,
+                        void* workspace, size_t workspace_bytes, void* stream);
+int32_t sgl_slice_fill(const sgl_tcsr* g, const sgl_seed_query* q,
+                       const int64_t* node_chunk, int64_t total_chunks,
+                       int32_t full_timestamps, const int64_t* totals,
+                       int64_t* nodes, int64_t* ts_ptr, int64_t* ts,
+                       int64_t* edge_ptr, int64_t* col, int64_t* col_ts,
+                       int64_t* col_eid, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
 /* --------------------------------------------------------- block building */
 /* Message-flow block of one layer in CSC form (replaces the tensor algebra of
  * AsyncBlock.to_block, starrygl/graph/graph.py:153-271, and

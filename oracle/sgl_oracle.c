@@ -659,6 +659,94 @@ int32_t sglo_seeds_fill(const sgl_tcsr* g, const sgl_seed_query* q, const int64_
     return seeds_walk(g, q, NULL, roots, ts_ptr, ts, q_ptr, q_eid);
 }
 
+/* ------------------------------------------- sub-graph slice ("cluster" mode) */
+
+size_t sglo_slice_workspace_bytes(int64_t n_cand, int64_t total_chunks) { (void)n_cand; (void)total_chunks; return 0; }
+
+/* Walks the candidates in output order and counts (nodes == NULL) or writes.
+ * Reference: count_edges_kernel / write_edges_kernel (sample.cu.hpp:299-515):
+ * per chunk, per node of the chunk, the edge range of the time window
+ * (lower_bound / upper_bound, :347-348); the node is listed when the range is
+ * not empty (:349-351); timestamps are counted where col_ts changes (:358-366)
+ * or, with use_full_timestamps, as t_end - t_begin per node (:352-355); an edge
+ * is written when the chunk of its destination is selected (:370-377, 497-503);
+ * out_ts_ptr holds, per listed timestamp, the offset of its first written edge
+ * (:487-491; every integer of a gap maps to the next edge's offset, :462-470).
+ * The window is t_begin <= ts < t_end as for the seeds. */
+static int32_t slice_walk(const sgl_tcsr* g, const sgl_seed_query* q, const int64_t* node_chunk,
+                          int64_t total_chunks, int32_t full, int64_t* totals, int64_t* nodes,
+                          int64_t* ts_ptr, int64_t* ts, int64_t* edge_ptr, int64_t* col, int64_t* col_ts,
+                          int64_t* col_eid) {
+    uint8_t* member = (uint8_t*)calloc((size_t)total_chunks + 1, 1);
+    if (!member) return fail(SGL_ENOMEM, "malloc");
+    for (int64_t p = 0; p < q->num_chunks; ++p)
+        if (q->chunks[p] >= 0 && q->chunks[p] < total_chunks) member[q->chunks[p]] = 1;
+    int64_t R = 0, T = 0, E = 0;
+    const int write = ts_ptr != NULL;
+    for (int64_t p = 0; p < q->num_chunks; ++p) {
+        const int64_t c = q->chunks[p];
+        const int64_t a = q->chunk_ptr[c], b = q->chunk_ptr[c + 1];
+        if (q->cand_off[p + 1] - q->cand_off[p] != b - a) {
+            free(member);
+            return fail(SGL_EINVAL, "slice: cand_off is not the prefix of the selected chunk sizes");
+        }
+        for (int64_t x = a; x < b; ++x) {
+            const int64_t v = q->chunk_nodes[x];
+            const int64_t rs = g->row_ptr[v], re = g->row_ptr[v + 1];
+            const int64_t lo = lower_bound_ts(g->ts, rs, re, q->t_begin);
+            const int64_t hi = lower_bound_ts(g->ts, lo, re, q->t_end);
+            if (hi <= lo) continue;
+            if (write) { nodes[R] = v; ts_ptr[R] = T; }
+            int64_t next_t = q->t_begin;      /* full mode: first integer not yet listed */
+            for (int64_t e = lo; e < hi; ++e) {
+                const int64_t t = g->ts[e];
+                if (full) {
+                    for (; next_t <= t; ++next_t) {
+                        if (write) { ts[T] = next_t; edge_ptr[T] = E; }
+                        ++T;
+                    }
+                } else if (e == lo || t != g->ts[e - 1]) {
+                    if (write) { ts[T] = t; edge_ptr[T] = E; }
+                    ++T;
+                }
+                const int64_t dc = node_chunk[g->col[e]];
+                if (dc >= 0 && dc < total_chunks && member[dc]) {
+                    if (write) { col[E] = g->col[e]; col_ts[E] = t; col_eid[E] = g->eid[e]; }
+                    ++E;
+                }
+            }
+            if (full)
+                for (; next_t < q->t_end; ++next_t) {
+                    if (write) { ts[T] = next_t; edge_ptr[T] = E; }
+                    ++T;
+                }
+            ++R;
+        }
+    }
+    free(member);
+    if (write) { ts_ptr[R] = T; edge_ptr[T] = E; }
+    if (totals) { totals[0] = R; totals[1] = T; totals[2] = E; }
+    return SGL_OK;
+}
+
+int32_t sglo_slice_count(const sgl_tcsr* g, const sgl_seed_query* q, const int64_t* node_chunk,
+                         int64_t total_chunks, int32_t full_timestamps, int64_t* totals, void* ws,
+                         size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (!g || !q || !totals || total_chunks < 0) return fail(SGL_EINVAL, "slice_count: null");
+    if (full_timestamps && q->t_end < q->t_begin) return fail(SGL_EINVAL, "slice: t_end < t_begin");
+    return slice_walk(g, q, node_chunk, total_chunks, full_timestamps, totals, NULL, NULL, NULL, NULL, NULL, NULL, NULL);
+}
+
+int32_t sglo_slice_fill(const sgl_tcsr* g, const sgl_seed_query* q, const int64_t* node_chunk,
+                        int64_t total_chunks, int32_t full_timestamps, const int64_t* totals, int64_t* nodes,
+                        int64_t* ts_ptr, int64_t* ts, int64_t* edge_ptr, int64_t* col, int64_t* col_ts,
+                        int64_t* col_eid, void* ws, size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream; (void)totals;
+    if (!g || !q || !ts_ptr || !edge_ptr || total_chunks < 0) return fail(SGL_EINVAL, "slice_fill: null");
+    return slice_walk(g, q, node_chunk, total_chunks, full_timestamps, NULL, nodes, ts_ptr, ts, edge_ptr, col, col_ts, col_eid);
+}
+
 /* --------------------------------------------------------- block building */
 
 /* Reference: AsyncBlock.to_block builds ('csc', (indptr, indices, [])) with

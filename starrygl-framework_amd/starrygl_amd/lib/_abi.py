@@ -78,6 +78,9 @@ PROTOTYPES = {
     "seeds_workspace_bytes": (sz, [i64]),
     "seeds_count": (i32, [P(TCSR), P(SeedQuery), vp, vp, sz, vp]),
     "seeds_fill": (i32, [P(TCSR), P(SeedQuery), vp, vp, vp, vp, vp, vp, vp, sz, vp]),
+    "slice_workspace_bytes": (sz, [i64, i64]),
+    "slice_count": (i32, [P(TCSR), P(SeedQuery), vp, i64, i32, vp, vp, sz, vp]),
+    "slice_fill": (i32, [P(TCSR), P(SeedQuery), vp, i64, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]),
     "block_build": (i32, [vp, vp, i64, i64, i64, i64, vp, vp, vp, vp]),
     "segment_max_ts": (i32, [vp, vp, i64, vp, i64, vp, vp, vp, vp]),
     "time_encode": (i32, [vp, i32, i64, vp, vp, vp, i32, vp, vp]),

@@ -294,6 +294,26 @@ class HotPath:
                                      be.ptr(ts), be.ptr(q_ptr), be.ptr(q_eid), be.ptr(ws), wsb, be.stream()))
         return roots, ts_ptr, ts, q_ptr, q_eid
 
+    def slice(self, g, chunk_ptr, chunk_nodes, node_chunk, chunks, cand_off, n_cand, t_begin, t_end,
+              full_timestamps=False):
+        """Sub-graph of the selected chunks over [t_begin, t_end)
+        -> (nodes, ts_ptr, ts, edge_ptr, col, col_ts, col_eid)."""
+        be = self.be
+        q = SeedQuery(be.ptr(chunk_ptr), be.ptr(chunk_nodes), int(chunks.shape[0]), be.ptr(chunks),
+                      be.ptr(cand_off), int(n_cand), int(t_begin), int(t_end))
+        total_chunks, full = int(chunk_ptr.shape[0]) - 1, int(bool(full_timestamps))
+        totals = be.zeros(3)
+        ws, wsb = self._workspace(self.lib.slice_workspace_bytes(n_cand, total_chunks))
+        self._ck(self.lib.slice_count(C.byref(g.view), C.byref(q), be.ptr(node_chunk), total_chunks, full,
+                                      be.ptr(totals), be.ptr(ws), wsb, be.stream()))
+        R, T, E = be.tolist(totals)
+        nodes, ts_ptr, ts, edge_ptr = be.empty(R), be.empty(R + 1), be.empty(T), be.empty(T + 1)
+        col, col_ts, col_eid = be.empty(E), be.empty(E), be.empty(E)
+        self._ck(self.lib.slice_fill(C.byref(g.view), C.byref(q), be.ptr(node_chunk), total_chunks, full,
+                                     be.ptr(totals), be.ptr(nodes), be.ptr(ts_ptr), be.ptr(ts), be.ptr(edge_ptr),
+                                     be.ptr(col), be.ptr(col_ts), be.ptr(col_eid), be.ptr(ws), wsb, be.stream()))
+        return nodes, ts_ptr, ts, edge_ptr, col, col_ts, col_eid
+
     # ------------------------------------------------------------- blocks
     def block_build(self, root_start_ptr, counts, S_max, E_max, dst_offset, src_offset, with_edge_dst=False):
         be = self.be

@@ -10,7 +10,8 @@ Differences a caller can observe
     with a repeated last entry, so `ptr[:-1]` (graph.py:166-168) is per slot;
   * `op='r'` starts a new local-id epoch and `op='f'` continues it, as
     `AsyncGraphBlob` (graph.py:291) and the comment at sample.cu.hpp:1874 say;
-  * time windows of `get_seeds_in_chunks` are half open, [time_begin, time_end).
+  * time windows of `get_seeds_in_chunks` and `slice_by_chunk_ts` are half open,
+    [time_begin, time_end).
 """
 import ctypes as C
 import queue
@@ -63,6 +64,14 @@ class TemporalNeighbor:
         self.root_start_ptr, self.root_end_ptr = hop.root_start_ptr, hop.root_end_ptr
         self.neighbors, self.neighbors_ts = hop.neighbors, hop.neighbors_ts
         self.neighbors_eid, self.neighbors_dt = hop.neighbors_eid, hop.neighbors_dt
+
+    @classmethod
+    def from_arrays(cls, root_start_ptr, root_end_ptr, neighbors, neighbors_ts, neighbors_eid, neighbors_dt):
+        self = cls.__new__(cls)
+        self.root_start_ptr, self.root_end_ptr = root_start_ptr, root_end_ptr
+        self.neighbors, self.neighbors_ts = neighbors, neighbors_ts
+        self.neighbors_eid, self.neighbors_dt = neighbors_eid, neighbors_dt
+        return self
 
     @property
     def neighbor_num(self):
@@ -133,14 +142,13 @@ class CUDAGraph:
         return seeds_in_chunks(self, chunks, int(time_begin), int(time_end))
 
     def slice_by_chunk_ts(self, chunks, time_begin, time_end, using_full_timestamp=False, stream=0):
-        raise NotImplementedError("'cluster' slicing (sample.cu.hpp:1189-1299) is outside the k-hop hot path")
+        from .seeds import slice_in_chunks
+        return slice_in_chunks(self, chunks, int(time_begin), int(time_end), bool(using_full_timestamp))
 
     # ---- asynchronous FIFO pipeline (sample.cu.hpp:1856-2031) ---------------
     def submit_query(self, time_start, time_end, chunk_list, test_generate_samples, test_generate_samples_ts,
                      sample_type, layers, fanout, allowed_offset, equal_root_time, keep_root_time, op):
-        if sample_type == "cluster":
-            raise NotImplementedError("'cluster' sampling is outside the k-hop hot path")
-        if sample_type not in _abi.SAMPLE_TYPES:
+        if sample_type != "cluster" and sample_type not in _abi.SAMPLE_TYPES:
             raise RuntimeError("undefined sampling strategy")
         if self._worker is None:
             self._worker = threading.Thread(target=self._run, name="sgl-sampler", daemon=True)
@@ -179,6 +187,8 @@ class CUDAGraph:
 
     def _execute(self, t0, t1, chunk_list, neg_nodes, neg_ts, sample_type, layers, fanout, allowed_offset,
                  equal_root_time, keep_root_time, op, query_index):
+        if sample_type == "cluster":     # sample.cu.hpp:1953-1961: dense timestamps, no negatives
+            return self.remap(self.slice_by_chunk_ts(chunk_list, t0, t1, True), reset=(op != "f"))
         roots = self.get_seeds_in_chunks(chunk_list, t0, t1)
         neg = self.get_negative_root(neg_nodes, neg_ts)
         res = self.sample_src_in_chunks_khop(roots, neg, fanout, layers, allowed_offset, equal_root_time,

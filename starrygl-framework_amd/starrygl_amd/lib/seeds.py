@@ -16,15 +16,14 @@ def _chunk_index(graph):
             mapper = torch.zeros(n, dtype=torch.int64)
         node_chunk = mapper.to(dev, torch.int64).contiguous()
         chunk_ptr, chunk_nodes = hp.chunk_index(n, C, node_chunk)
-        graph._chunk_index = (chunk_ptr, chunk_nodes, chunk_ptr.cpu().numpy())
+        graph._chunk_index = (chunk_ptr, chunk_nodes, chunk_ptr.cpu().numpy(), node_chunk)
     return graph._chunk_index
 
 
-def seeds_in_chunks(graph, chunks, t_begin, t_end):
-    from .libstarrygl_comm import TemporalRoot
-    hp = graph._hp
-    dev = hp.be.device
-    chunk_ptr, chunk_nodes, chunk_ptr_h = _chunk_index(graph)
+def _candidates(graph, chunks):
+    """-> (device chunk ids, device exclusive prefix of their sizes, candidate count)."""
+    dev = graph._hp.be.device
+    chunk_ptr_h = _chunk_index(graph)[2]
     if not isinstance(chunks, torch.Tensor):
         raise TypeError("chunks must be a torch.Tensor")
     chunks_h = chunks.detach().cpu().to(torch.int64).numpy().reshape(-1)
@@ -34,7 +33,27 @@ def seeds_in_chunks(graph, chunks, t_begin, t_end):
     sizes = chunk_ptr_h[chunks_h + 1] - chunk_ptr_h[chunks_h] if chunks_h.size else np.zeros(0, np.int64)
     cand_off = np.zeros(chunks_h.size + 1, dtype=np.int64)
     np.cumsum(sizes, out=cand_off[1:])
-    d_chunks = torch.from_numpy(chunks_h.copy()).to(dev)
-    d_off = torch.from_numpy(cand_off).to(dev)
-    out = hp.seeds(graph._g, chunk_ptr, chunk_nodes, d_chunks, d_off, int(cand_off[-1]), t_begin, t_end)
+    return torch.from_numpy(chunks_h.copy()).to(dev), torch.from_numpy(cand_off).to(dev), int(cand_off[-1])
+
+
+def seeds_in_chunks(graph, chunks, t_begin, t_end):
+    from .libstarrygl_comm import TemporalRoot
+    chunk_ptr, chunk_nodes = _chunk_index(graph)[:2]
+    d_chunks, d_off, n_cand = _candidates(graph, chunks)
+    out = graph._hp.seeds(graph._g, chunk_ptr, chunk_nodes, d_chunks, d_off, n_cand, t_begin, t_end)
     return TemporalRoot(*out)
+
+
+def slice_in_chunks(graph, chunks, t_begin, t_end, full_timestamps):
+    """Graph::slice_by_chunk_ts (sample.cu.hpp:1189-1299): the selected chunks'
+    nodes with edges in [t_begin, t_end) as roots (one timestamp list per node)
+    and, as the single neighbour layer, the window edges whose destination lies
+    in a selected chunk; `root_start_ptr` indexes them per (node, timestamp)."""
+    from .libstarrygl_comm import NegativeRoot, TemporalNeighbor, TemporalResult, TemporalRoot
+    chunk_ptr, chunk_nodes, _, node_chunk = _chunk_index(graph)
+    d_chunks, d_off, n_cand = _candidates(graph, chunks)
+    nodes, ts_ptr, ts, edge_ptr, col, col_ts, col_eid = graph._hp.slice(
+        graph._g, chunk_ptr, chunk_nodes, node_chunk, d_chunks, d_off, n_cand, t_begin, t_end, full_timestamps)
+    e = nodes.new_empty(0)
+    layer = TemporalNeighbor.from_arrays(edge_ptr, torch.cat([edge_ptr[1:], edge_ptr[-1:]]), col, col_ts, col_eid, e)
+    return TemporalResult(TemporalRoot(nodes, ts_ptr, ts), NegativeRoot(e, e), [layer])

@@ -88,6 +88,47 @@ def test_oracle_seeds_match_brute_force(oracle):
         oracle.chunk_index(3, 2, np.array([0, 2, 1], dtype=np.int64))
 
 
+def _slice_brute(g, chunk_of, chunks, t0, t1, full):
+    sel = set(chunks)
+    nodes, ts_ptr, ts, edge_ptr, col, col_ts, col_eid = [], [0], [], [], [], [], []
+    for c in chunks:
+        for v in [v for v in range(g.n) if chunk_of[v] == c]:
+            ev = [e for e in range(g.row_ptr[v], g.row_ptr[v + 1]) if t0 <= g.ts[e] < t1]
+            if not ev:
+                continue
+            nodes.append(v)
+            for t in (range(t0, t1) if full else sorted(set(g.ts[e] for e in ev))):
+                ts.append(t)
+                edge_ptr.append(len(col))
+                for e in ev:
+                    if g.ts[e] == t and chunk_of[g.col[e]] in sel:
+                        col.append(g.col[e]); col_ts.append(g.ts[e]); col_eid.append(g.eid[e])
+            ts_ptr.append(len(ts))
+    edge_ptr.append(len(col))
+    return nodes, ts_ptr, ts, edge_ptr, col, col_ts, col_eid
+
+
+def test_oracle_slice_matches_brute_force(oracle):
+    rng = np.random.default_rng(4)
+    n, m, C = 40, 900, 5
+    g = host_graph(oracle, n, rng.integers(0, n, m), rng.integers(0, n, m), rng.integers(0, 30, m))
+    chunk_of = rng.integers(0, C, n).astype(np.int64)
+    chunk_ptr, chunk_nodes = oracle.chunk_index(n, C, chunk_of)
+    for chunks, t0, t1 in [([0, 3], 5, 12), ([4, 1, 2], 0, 30), ([2], 29, 30), ([], 0, 30), ([1], 10, 10),
+                           ([0, 1, 2, 3, 4], 3, 9)]:
+        ch = np.array(chunks, dtype=np.int64)
+        sizes = chunk_ptr[ch + 1] - chunk_ptr[ch] if ch.size else np.zeros(0, np.int64)
+        off = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+        for full in (False, True):
+            got = oracle.slice(g, chunk_ptr, chunk_nodes, chunk_of, ch, off, int(off[-1]), t0, t1, full)
+            want = _slice_brute(g, chunk_of, chunks, t0, t1, full)
+            for a, b in zip(got, want):
+                assert a.tolist() == [int(x) for x in b], (chunks, t0, t1, full)
+            # with every chunk selected no edge of the window is dropped
+            if len(chunks) == C:
+                assert got[4].shape[0] == int(((g.ts >= t0) & (g.ts < t1)).sum())
+
+
 def test_oracle_block_build(oracle):
     rsp = np.array([0, 2, 2, 5], dtype=np.int64)
     counts = np.array([3, 5, 0], dtype=np.int64)

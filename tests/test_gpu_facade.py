@@ -122,8 +122,8 @@ def test_direct_khop_and_errors(oracle, world):
     assert np.array_equal(np_of(res.neighbors_list[0].neighbors), want.hops[0].neighbors)
     with pytest.raises(RuntimeError, match="undefined sampling strategy"):
         g.sample_src_in_chunks_khop(root, neg, 3, 1, -1, False, False, "nearest")
-    with pytest.raises(NotImplementedError):
-        g.slice_by_chunk_ts(torch.tensor([0]), 0, 1)
+    with pytest.raises(IndexError):
+        g.slice_by_chunk_ts(torch.tensor([world["C"]]), 0, 1)
     one = torch.tensor([0, 1])
     with pytest.raises(IndexError):
         from_edge_index(2, 1, one, torch.tensor([1, 2]), one, None)
@@ -143,6 +143,35 @@ def test_direct_khop_and_errors(oracle, world):
         pg.async_sample(0, 1, torch.tensor([0]), dict(sample_type="recent", layers=1), {}, op="r")
     with pytest.raises(TypeError):
         pg.async_sample(0, 1, [0], pol)
+
+
+@pytest.mark.parametrize("full", [False, True])
+def test_slice_by_chunk_ts_matches_oracle(oracle, world, full):
+    g = world["g"]
+    for chunks, t0, t1 in [([1, 5, 2], 50_000, 50_400), ([0, 1, 2, 3, 4, 5, 6, 7], 10_000, 10_250), ([3], 99_000, 100_000),
+                           ([6, 0], 70_000, 70_001), ([], 0, 10), ([4], 500, 500)]:
+        ch = np.asarray(chunks, dtype=np.int64)
+        off = np.concatenate([[0], np.cumsum(world["cp"][ch + 1] - world["cp"][ch])]).astype(np.int64)
+        want = oracle.slice(world["hg"], world["cp"], world["cn"], world["chunk_of"], ch, off, int(off[-1]), t0, t1, full)
+        out = g.g.slice_by_chunk_ts(torch.tensor(chunks, dtype=torch.int64), t0, t1, full)
+        layer = out.neighbors_list[0]
+        got = (out.roots.roots, out.roots.ts_ptr, out.roots.ts, layer.root_start_ptr, layer.neighbors,
+               layer.neighbors_ts, layer.neighbors_eid)
+        for a, b in zip(got, want):
+            assert np.array_equal(np_of(a), b), (chunks, t0, t1)
+        assert np.array_equal(np_of(layer.root_end_ptr)[:-1], want[3][1:])
+    assert want[0].shape[0] == 0                                      # the empty window
+    # through the query queue: dense timestamps, ids remapped per array (roots, then neighbours)
+    g.async_sample(50_000, 50_020, torch.tensor([1, 5, 2]), {"sample_type": "cluster"}, {}, op="r")
+    out = g.get_last_sample()
+    ch = np.array([1, 5, 2], dtype=np.int64)
+    off = np.concatenate([[0], np.cumsum(world["cp"][ch + 1] - world["cp"][ch])]).astype(np.int64)
+    want = oracle.slice(world["hg"], world["cp"], world["cn"], world["chunk_of"], ch, off, int(off[-1]), 50_000, 50_020, True)
+    assert out.roots.root_ts_num == want[0].shape[0] * 20 > 0
+    ids = np_of(out.nodes_remapper_id)
+    assert np.array_equal(ids[np_of(out.roots.roots)], want[0])
+    assert np.array_equal(ids[np_of(out.neighbors_list[0].neighbors)], want[4])
+    assert np.array_equal(np_of(out.neighbors_list[0].root_start_ptr), want[3])
 
 
 def test_neg_sampling_set():
