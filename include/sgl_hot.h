@@ -350,6 +350,31 @@ int32_t sgl_block_build(const int64_t* root_start_ptr, const int64_t* counts,
                         int64_t src_offset, int64_t* indptr, int64_t* indices,
                         int64_t* edge_dst, void* stream);
 
+/* ------------------------------------------------ batch materialisation */
+/* np.unique over (id, timestamp) records with return_inverse (replaces
+ * _get_unique_pairs and, over the concatenation of two lists,
+ * _merge_and_map_nodes, prepare_sample.py:205-213, 231-246): uniq_ids/uniq_ts
+ * [U] ascend in (id, ts), signed order; inverse[i] is the place of pair i in
+ * them; U_dev[0] = U.  Capacity of the three outputs: N_max.  N = *N_dev when
+ * given. */
+size_t  sgl_unique_pairs_workspace_bytes(int64_t N_max);
+int32_t sgl_unique_pairs(const int64_t* ids, const int64_t* ts, int64_t N_max,
+                         const int64_t* N_dev, int64_t* uniq_ids,
+                         int64_t* uniq_ts, int64_t* inverse, int64_t* U_dev,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/* Edge order and pointer array of a CSC block from (destination, timestamp)
+ * pairs (replaces _build_csc_from_pairs, prepare_sample.py:215-229): perm is
+ * the stable order np.lexsort((ts, dst_local)), indptr[d] the number of edges
+ * with destination below d (d = 0 .. num_dst).  dst_local must lie in
+ * [0, num_dst).  E = *E_dev when given. */
+size_t  sgl_csc_from_pairs_workspace_bytes(int64_t E_max);
+int32_t sgl_csc_from_pairs(const int64_t* dst_local, const int64_t* ts,
+                           int64_t E_max, const int64_t* E_dev,
+                           int64_t num_dst, int64_t* indptr, int64_t* perm,
+                           void* workspace, size_t workspace_bytes,
+                           void* stream);
+
 /* -------------------------------------------------- latest event per node */
 /* For N events with dense keys local[i] in [0, U) (local ids from
  * sgl_unique_compact) and timestamps ts[i]: max_ts[u] = max of ts over the

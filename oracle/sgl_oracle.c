@@ -747,6 +747,69 @@ int32_t sglo_slice_fill(const sgl_tcsr* g, const sgl_seed_query* q, const int64_
     return slice_walk(g, q, node_chunk, total_chunks, full_timestamps, NULL, nodes, ts_ptr, ts, edge_ptr, col, col_ts, col_eid);
 }
 
+/* ------------------------------------------------ batch materialisation */
+
+typedef struct { int64_t a, b, pos; } rec3;
+
+static int rec3_cmp(const void* x, const void* y) {
+    const rec3* p = (const rec3*)x; const rec3* q = (const rec3*)y;
+    if (p->a != q->a) return p->a < q->a ? -1 : 1;
+    if (p->b != q->b) return p->b < q->b ? -1 : 1;
+    return p->pos < q->pos ? -1 : (p->pos > q->pos ? 1 : 0);
+}
+
+size_t sglo_unique_pairs_workspace_bytes(int64_t N_max) { (void)N_max; return 0; }
+
+/* Reference: _get_unique_pairs (prepare_sample.py:205-213): np.unique of
+ * records (id, ts) with return_inverse - records ascend by id, then ts. */
+int32_t sglo_unique_pairs(const int64_t* ids, const int64_t* ts, int64_t N_max, const int64_t* N_dev,
+                          int64_t* uniq_ids, int64_t* uniq_ts, int64_t* inverse, int64_t* U_dev, void* ws,
+                          size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (N_max < 0 || !U_dev) return fail(SGL_EINVAL, "unique_pairs: bad argument");
+    const int64_t N = N_dev ? (*N_dev < N_max ? *N_dev : N_max) : N_max;
+    rec3* r = (rec3*)malloc((size_t)(N > 0 ? N : 1) * sizeof(rec3));
+    if (!r) return fail(SGL_ENOMEM, "malloc");
+    for (int64_t i = 0; i < N; ++i) { r[i].a = ids[i]; r[i].b = ts[i]; r[i].pos = i; }
+    qsort(r, (size_t)N, sizeof(rec3), rec3_cmp);
+    int64_t U = 0;
+    for (int64_t i = 0; i < N; ++i) {
+        if (i == 0 || r[i].a != r[i - 1].a || r[i].b != r[i - 1].b) {
+            uniq_ids[U] = r[i].a; uniq_ts[U] = r[i].b; ++U;
+        }
+        inverse[r[i].pos] = U - 1;
+    }
+    free(r);
+    U_dev[0] = U;
+    return SGL_OK;
+}
+
+size_t sglo_csc_from_pairs_workspace_bytes(int64_t E_max) { (void)E_max; return 0; }
+
+/* Reference: _build_csc_from_pairs (prepare_sample.py:215-229): perm =
+ * np.lexsort((ts, dst_local)) (stable), indptr = cumsum of the per-destination
+ * counts. */
+int32_t sglo_csc_from_pairs(const int64_t* dst_local, const int64_t* ts, int64_t E_max, const int64_t* E_dev,
+                            int64_t num_dst, int64_t* indptr, int64_t* perm, void* ws, size_t ws_bytes,
+                            void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (E_max < 0 || num_dst < 0 || !indptr) return fail(SGL_EINVAL, "csc_from_pairs: bad argument");
+    const int64_t E = E_dev ? (*E_dev < E_max ? *E_dev : E_max) : E_max;
+    rec3* r = (rec3*)malloc((size_t)(E > 0 ? E : 1) * sizeof(rec3));
+    if (!r) return fail(SGL_ENOMEM, "malloc");
+    for (int64_t d = 0; d <= num_dst; ++d) indptr[d] = 0;
+    for (int64_t i = 0; i < E; ++i) {
+        r[i].a = dst_local[i]; r[i].b = ts[i]; r[i].pos = i;
+        if (dst_local[i] < 0 || dst_local[i] >= num_dst) { free(r); return fail(SGL_ERANGE, "csc_from_pairs: destination outside [0, num_dst)"); }
+        indptr[dst_local[i] + 1] += 1;
+    }
+    qsort(r, (size_t)E, sizeof(rec3), rec3_cmp);
+    for (int64_t i = 0; i < E; ++i) perm[i] = r[i].pos;
+    for (int64_t d = 0; d < num_dst; ++d) indptr[d + 1] += indptr[d];
+    free(r);
+    return SGL_OK;
+}
+
 /* --------------------------------------------------------- block building */
 
 /* Reference: AsyncBlock.to_block builds ('csc', (indptr, indices, [])) with

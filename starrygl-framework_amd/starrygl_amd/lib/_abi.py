@@ -78,6 +78,10 @@ PROTOTYPES = {
     "seeds_workspace_bytes": (sz, [i64]),
     "seeds_count": (i32, [P(TCSR), P(SeedQuery), vp, vp, sz, vp]),
     "seeds_fill": (i32, [P(TCSR), P(SeedQuery), vp, vp, vp, vp, vp, vp, vp, sz, vp]),
+    "unique_pairs_workspace_bytes": (sz, [i64]),
+    "unique_pairs": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, vp, sz, vp]),
+    "csc_from_pairs_workspace_bytes": (sz, [i64]),
+    "csc_from_pairs": (i32, [vp, vp, i64, vp, i64, vp, vp, vp, sz, vp]),
     "slice_workspace_bytes": (sz, [i64, i64]),
     "slice_count": (i32, [P(TCSR), P(SeedQuery), vp, i64, i32, vp, vp, sz, vp]),
     "slice_fill": (i32, [P(TCSR), P(SeedQuery), vp, i64, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]),

@@ -323,6 +323,28 @@ class HotPath:
                                       src_offset, be.ptr(indptr), be.ptr(indices), be.ptr(edge_dst), be.stream()))
         return indptr, indices, edge_dst
 
+    # ------------------------------------------------- (id, ts) pair algebra
+    def unique_pairs(self, ids, ts, N_dev=None):
+        """-> (uniq_ids[U], uniq_ts[U], inverse[N]): np.unique over (id, ts) records with
+        return_inverse (one synchronising read of U)."""
+        be, N = self.be, int(ids.shape[0])
+        uid, uts, inv, U = be.empty(max(N, 1)), be.empty(max(N, 1)), be.empty(max(N, 1)), be.zeros(1)
+        ws, wsb = self._workspace(self.lib.unique_pairs_workspace_bytes(N))
+        self._ck(self.lib.unique_pairs(be.ptr(ids), be.ptr(ts), N, be.ptr(N_dev), be.ptr(uid), be.ptr(uts),
+                                       be.ptr(inv), be.ptr(U), be.ptr(ws), wsb, be.stream()))
+        u = be.tolist(U)[0]
+        n = N if N_dev is None else min(N, be.tolist(N_dev)[0])
+        return uid[:u], uts[:u], inv[:n]
+
+    def csc_from_pairs(self, dst_local, ts, num_dst, E_dev=None):
+        """-> (indptr[num_dst + 1], perm[E]): the stable (dst_local, ts) edge order."""
+        be, E = self.be, int(dst_local.shape[0])
+        indptr, perm = be.empty(num_dst + 1), be.empty(max(E, 1))
+        ws, wsb = self._workspace(self.lib.csc_from_pairs_workspace_bytes(E))
+        self._ck(self.lib.csc_from_pairs(be.ptr(dst_local), be.ptr(ts), E, be.ptr(E_dev), int(num_dst),
+                                         be.ptr(indptr), be.ptr(perm), be.ptr(ws), wsb, be.stream()))
+        return indptr, perm[:E]
+
     # ------------------------------------------------------ latest by key
     def segment_max_ts(self, local, ts, U, N_dev=None, U_dev=None):
         """-> (max_ts[U], arg[U]): per dense key the largest timestamp and the first

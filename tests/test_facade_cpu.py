@@ -150,3 +150,44 @@ def test_oracle_segment_max_ts(oracle):
         assert mx[u] == ts[pos].max() and arg[u] == pos[np.argmax(ts[pos])]     # argmax = first occurrence
     mx, arg = oracle.segment_max_ts(np.array([0, 0], np.int64), np.array([5, 7], np.int64), 3)
     assert arg.tolist() == [1, -1, -1] and mx[0] == 7 and mx[1] == np.iinfo(np.int64).min
+
+
+def test_oracle_pair_unique_and_csc_order(oracle):
+    """np.unique over (id, ts) records and np.lexsort((ts, dst)) are the routines the reference calls
+    (prepare_sample.py:205-229); the oracle's restatement must equal them."""
+    rng = np.random.default_rng(6)
+    dt = np.dtype([("id", np.int64), ("ts", np.int64)])
+    for n in (0, 1, 2, 900):
+        ids, ts = rng.integers(-9, 40, n).astype(np.int64), rng.integers(-4, 12, n).astype(np.int64)
+        c = np.empty(n, dtype=dt)
+        c["id"], c["ts"] = ids, ts
+        u, inv = np.unique(c, return_inverse=True)
+        g_id, g_ts, g_inv = oracle.unique_pairs(ids, ts)
+        assert np.array_equal(g_id, u["id"]) and np.array_equal(g_ts, u["ts"]) and np.array_equal(g_inv, inv.reshape(-1))
+        d = rng.integers(0, 25, n).astype(np.int64)
+        indptr, perm = oracle.csc_from_pairs(d, ts, 25)
+        assert np.array_equal(perm, np.lexsort((ts, d)))
+        assert np.array_equal(indptr, np.concatenate([[0], np.cumsum(np.bincount(d, minlength=25))]))
+    with pytest.raises(IndexError):
+        oracle.csc_from_pairs(np.array([3], np.int64), np.array([0], np.int64), 3)
+
+
+def test_slot_and_batch_files_round_trip(tmp_path):
+    from starrygl_amd.data import offline
+    src, dst, ts = torch.arange(5), torch.arange(5) + 1, torch.arange(5) * 10
+    offline.write_slot(tmp_path / "slot_0001_sub_0000.pt", src, dst, ts, torch.arange(5), torch.tensor([2, 7]), 1, 12)
+    d = offline.read_slot(tmp_path / "slot_0001_sub_0000.pt")
+    assert sorted(d) == sorted(offline.SLOT_KEYS) and d["slot_id"] == 1 and d["chunk_id"] == 12
+    assert torch.equal(d["dst"], dst) and torch.equal(d["cid"], torch.tensor([2, 7]))
+    torch.save({"src": src}, tmp_path / "bad.pt")
+    with pytest.raises(KeyError):
+        offline.read_slot(tmp_path / "bad.pt")
+    batch = [{"gids": src, "ts": ts, "inv_map": src, "num_neg": 2, "task_label": "neg_set", "comm_plan": [None, None]},
+             {"indptr": torch.tensor([0, 1, 1, 2, 2, 2]), "indices": torch.tensor([0, 3]), "eid": torch.tensor([9, 8]),
+              "edge_ts": torch.tensor([1, 2]), "edge_dt": torch.tensor([1.0, 2.0]), "gids": src, "ts": ts}]
+    offline.write_batch(tmp_path / "b.pt", batch)
+    back = offline.read_batch(tmp_path / "b.pt")
+    assert back[0]["task_label"] == "neg_set" and back[0]["comm_plan"] == [None, None]
+    assert torch.equal(back[1]["indptr"], batch[1]["indptr"]) and back[1]["edge_dt"].dtype == torch.float32
+    blk = offline.batch_to_blocks(back)[0]
+    assert blk.num_dst_nodes() == 5 and blk.num_edges() == 2 and torch.equal(blk.edata["eid"], torch.tensor([9, 8]))
