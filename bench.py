@@ -640,6 +640,9 @@ def main():
                         "GBps": round((samp_bytes(S0 * mult, cnt[1]) + samp_bytes(cnt[1], cnt[4])) / ms / 1e6, 1)})
         del kb
     extra["sampler scaling (2-hop recent 10x10, several batches per call)"] = scaling
+    if cpu is not None:     # the same ratio when one call samples several mini-batches (same graph, same batches)
+        cpu["gpu_over_cpu_sampler_by_batches_per_call"] = {str(r["batches_per_call"]): round(r["edges_per_s"] / cpu["value"], 1)
+                                                           for r in scaling}
     if args.workload != "c2":
         # free the headline workload's tables first
         del node_feat, edge_feat, node_cache, edge_cache, e_out, node_out, dg, multi

@@ -317,7 +317,7 @@ __device__ __forceinline__ int64_t bounded(uint64_t bits, int64_t range) {
     return (int64_t)__umul64hi(bits, (uint64_t)range);
 }
 
-template <int G>
+template <int G, bool UNIFORM>
 __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     constexpr int SPB = BLOCK / G;
     __shared__ int64_t s_red[NWAVE];
@@ -430,7 +430,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
             a.root_start_ptr[slot] = off;
             a.root_end_ptr[slot] = off + c;
         }
-        if (a.type == SGL_SAMPLE_RECENT) {
+        if constexpr (!UNIFORM) {
             if (active) {
                 // up to ROUNDS * G edges per pass, every load issued before the first store
                 constexpr int ROUNDS = 4;
@@ -581,13 +581,15 @@ HopKernel count_fn(int G) {
     }
 }
 
-HopKernel fill_fn(int G) {
-    switch (G) {
-        case 8: return fill_kernel<8>;
-        case 16: return fill_kernel<16>;
-        case 32: return fill_kernel<32>;
-        default: return fill_kernel<64>;
+HopKernel fill_fn(int G, bool uniform) {
+    if (uniform) {
+        switch (G) {
+            case 16: return fill_kernel<16, true>;
+            case 32: return fill_kernel<32, true>;
+            default: return fill_kernel<64, true>;
+        }
     }
+    return G == 8 ? fill_kernel<8, false> : fill_kernel<16, false>;
 }
 
 // Gc lanes per slot search, Gf lanes per slot copy or draw
@@ -602,7 +604,7 @@ int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf) {
         hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, a, (int)blocks);
         SGL_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(fill_fn(Gf), dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
+    hipLaunchKernelGGL(fill_fn(Gf, a.type == SGL_SAMPLE_UNIFORM), dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }
