@@ -324,6 +324,8 @@ def main():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (known traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings can be scaled")
+    ap.add_argument("--no-fused-mark", action="store_true",
+                    help="unique runs its own marking pass instead of the sampler recording the ids it emits")
     ap.add_argument("--serial", action="store_true", help="capture the step as one serial chain of kernels")
     ap.add_argument("--eager", action="store_true", help="launch every kernel from the host instead of replaying a HIP graph")
     args = ap.parse_args()
@@ -400,13 +402,18 @@ def main():
     def stage_inputs(b):
         s_all.copy_(packed[b])
 
+    # in the step the recent sampler also records the ids it emits as pending in the remap state, so
+    # that the unique stage starts at its second pass (one launch less per step)
+    p_rec_mark = hot.marking(p_rec, state) if not args.no_fused_mark else p_rec
+
     def st_recent():
-        hot.sample_khop(dg, s_roots, ts_ptr, s_root_ts, s_neg, s_neg_ts, 2, p_rec, finalize=False, out=kr)
+        hot.sample_khop(dg, s_roots, ts_ptr, s_root_ts, s_neg, s_neg_ts, 2, p_rec_mark, finalize=False, out=kr)
 
     def st_unique():
         hot.unique_compact([kr.slot_node0, kr.hops[0].neighbors, kr.hops[1].neighbors], _abi.UNIQUE_SORTED, state,
                            True, lens_dev=[S0_dev, kr.hops[0].counts[1:2], kr.hops[1].counts[1:2]],
-                           out_arrays=local, finalize=False, unique_out=ubuf, U_out=U)
+                           out_arrays=local, finalize=False, unique_out=ubuf, U_out=U,
+                           premarked=not args.no_fused_mark)
 
     def st_node():
         hot.gather(node_cache, ubuf, node_out, N_dev=U[0:1])
@@ -470,16 +477,23 @@ def main():
         else:
             # independent stages become parallel branches of the graph: the uniform sampler
             # runs beside the recent one -> unique -> gathers chain
-            br = [torch.cuda.Stream()]
+            # The uniform sampler is independent of the recent -> unique -> gather chain: it is a
+            # second branch of the graph, captured after the chain.  (Kernels of two branches hardly
+            # overlap on this part, and the runtime issues branches in creation order: capturing the
+            # independent branch first delays the chain and costs ~10 % of the step; two graphs on
+            # two streams, or the edge gather on a branch beside unique, were slower as well.)
+            br = torch.cuda.Stream()
             with torch.cuda.graph(g_step):
                 cur = torch.cuda.current_stream()
-                br[0].wait_stream(cur)
-                with torch.cuda.stream(br[0]):
-                    st_uniform()
+                ev0 = torch.cuda.Event()
+                ev0.record(cur)
                 st_recent()
                 st_unique()
                 st_gathers()
-                cur.wait_stream(br[0])
+                br.wait_event(ev0)
+                with torch.cuda.stream(br):
+                    st_uniform()
+                cur.wait_stream(br)
                 st_account()
         graphs = []
         for f in stages_fn:
@@ -487,7 +501,7 @@ def main():
             with torch.cuda.graph(gs):
                 f()
             graphs.append(gs)
-        mode = "hipgraph" if args.serial else "hipgraph, uniform sampler on a parallel branch"
+        mode = "hipgraph" if args.serial else "hipgraph, uniform sampler on a second branch"
         run_step = g_step.replay
     else:
         run_step = body
@@ -604,7 +618,7 @@ def main():
         # parity of batch 0 against the GPU result (the oracle as the checker)
         want = ora.sample_khop(hg, *bt[W % NB], 2, po)
         stage_inputs(W % NB)
-        st_recent()
+        st_recent(); st_unique()      # (the pair: the sampler's pending ids are consumed by unique)
         c = kr.counts.cpu().numpy()
         assert int(c[1]) == want.hops[0].E and int(c[4]) == want.hops[1].E, "GPU and oracle disagree on edge counts"
         assert np.array_equal(kr.hops[1].neighbors_eid[: int(c[4])].cpu().numpy(), want.hops[1].neighbors_eid)

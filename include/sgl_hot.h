@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define SGL_ABI_VERSION 1
+#define SGL_ABI_VERSION 2
 
 /* ------------------------------------------------------------------ status */
 #define SGL_OK        0
@@ -103,6 +103,16 @@ typedef struct sgl_sample_params {
     int32_t  replace;         /* uniform only: 1 = k iid draws (may repeat)    */
     int32_t  hop;             /* RNG stream selector for sgl_sample_hop        */
     uint64_t seed;            /* Philox4x32-10 key                             */
+    /* Optional fusion with the unique stage (no counterpart in the reference,
+     * whose Remapper marks ids in a pass of its own, sample.cu.hpp:1719-1760):
+     * when mark_state is a state of sgl_remap_init over mark_universe ids, the
+     * sampler also records every id it emits - the hop-0 slot nodes of
+     * sgl_sample_khop and the neighbours of every hop - as pending in that
+     * state, which is the first pass of sgl_unique_compact.  The next
+     * sgl_unique_compact on the state must then be the one over exactly those
+     * arrays, with reset = 1 and mode SGL_UNIQUE_SORTED | SGL_UNIQUE_PREMARKED. */
+    void*    mark_state;      /* NULL: off                                     */
+    int64_t  mark_universe;
 } sgl_sample_params;
 
 /* One hop's result, caller-allocated (replaces TemporalNeighbor,
@@ -163,6 +173,9 @@ int32_t sgl_sample_khop(const sgl_tcsr* g,
 /* ------------------------------------------------------ unique / compaction */
 #define SGL_UNIQUE_SORTED  0 /* all arrays form one group: == np.unique(return_inverse) */
 #define SGL_UNIQUE_GROUPED 1 /* per array: ids new to the epoch, ascending, appended    */
+#define SGL_UNIQUE_PREMARKED 0x100 /* flag, with SGL_UNIQUE_SORTED, reset = 1 and a dense state:
+                                    * the sampler has already recorded the arrays' ids as
+                                    * pending (sgl_sample_params.mark_state)              */
 
 /* Persistent remap state over a dense id universe [0, universe): the
  * replacement of Remapper's id_mapper/global_mask tables and epoch counter

@@ -400,6 +400,11 @@ int32_t sglo_unique_compact(void* state, int64_t universe_arg, int32_t reset, in
     (void)ws; (void)ws_bytes; (void)stream;
     if (G < 0 || (G > 0 && (!ids || !len_max || !local_out)) || !U_dev)
         return fail(SGL_EINVAL, "unique_compact: null");
+    /* PREMARKED only tells the HIP library that the sampler already did its first pass; the
+     * result is defined by the arrays alone, so the restatement just numbers them. */
+    if ((mode & SGL_UNIQUE_PREMARKED) && ((mode & ~SGL_UNIQUE_PREMARKED) != SGL_UNIQUE_SORTED || !reset || !state))
+        return fail(SGL_EINVAL, "unique_compact: PREMARKED needs the dense state, SORTED mode and reset = 1");
+    mode &= ~SGL_UNIQUE_PREMARKED;
     if (mode != SGL_UNIQUE_SORTED && mode != SGL_UNIQUE_GROUPED)
         return fail(SGL_EINVAL, "unique_compact: bad mode");
     if (!state && !reset) return fail(SGL_ENOTSUP, "unique_compact: hash path needs reset=1");

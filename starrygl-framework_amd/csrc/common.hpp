@@ -52,6 +52,24 @@ struct Arena {
 // ---- device helpers ---------------------------------------------------------
 #if defined(__HIPCC__)
 
+// Layout of a remap state (sgl_remap_init): header, table[universe] of 8-byte entries, then the
+// "pending" set: one flag byte per id for universes up to REMAP_BYTE_FLAGS_MAX ids (set by plain
+// stores), one bit per id beyond (set by atomicOr; sweeping a byte per id would cost more there
+// than the atomics do).  unique.hip owns the state; the sampler only sets flags.
+constexpr size_t REMAP_HEADER_BYTES = 256;
+constexpr int64_t REMAP_BYTE_FLAGS_MAX = 1ll << 24;
+inline bool remap_byte_flags(int64_t universe) { return universe <= REMAP_BYTE_FLAGS_MAX; }
+inline void* remap_flags(void* state, int64_t universe) {
+    return static_cast<char*>(state) + REMAP_HEADER_BYTES + (size_t)universe * 8;
+}
+__device__ __forceinline__ void remap_set_pending(void* flags, int bytes, int64_t id) {
+    if (bytes) {
+        static_cast<uint8_t*>(flags)[id] = 1;
+    } else {
+        atomicOr(static_cast<unsigned long long*>(flags) + (id >> 6), 1ull << (id & 63));
+    }
+}
+
 // Ballot restricted to the G-lane group that starts at bit `gshift` of the wave.
 template <int G>
 __device__ __forceinline__ uint64_t group_ballot(bool pred, int gshift) {

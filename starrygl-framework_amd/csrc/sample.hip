@@ -66,6 +66,9 @@ struct HopArgs {
     int64_t allowed_offset;
     int32_t equal_root_time, keep_root_time, replace, hop;
     uint64_t seed;
+    void* mark;          // pending-id flags of a remap state, or nullptr
+    int64_t mark_universe;
+    int32_t mark_bytes;  // 1: a flag byte per id, 0: a bit per id
     // workspace
     int64_t* w_start;    // [S_max] first candidate position (recent: first copied edge)
     int64_t* w_len;      // [S_max] window length
@@ -123,6 +126,11 @@ __device__ __forceinline__ int64_t group_lower_bound(const int64_t* __restrict__
         }
     }
     return lo;
+}
+
+// Records `id` as pending in the remap state (as unique.hip's mark pass does)
+__device__ __forceinline__ void mark_id(const HopArgs& a, int64_t id) {
+    if (id >= 0 && id < a.mark_universe) remap_set_pending(a.mark, a.mark_bytes, id);
 }
 
 // Slots [first, first + run) belong to block b; run is a multiple of `spb`, itself a
@@ -214,6 +222,7 @@ __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
             if (a.derive) {
                 a.slot_node_out[slot] = v;
                 a.slot_ts_out[slot] = t;
+                if (a.mark != nullptr) mark_id(a, v);
             }
         }
         // wave totals of c and of the bad flags (one contribution per group)
@@ -451,6 +460,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
                         const int32_t j = j0 + r * G;
                         if (j < c) {
                             a.nbr[off + j] = dst[r];
+                            if (a.mark != nullptr) mark_id(a, dst[r]);
                             a.nbr_ts[off + j] = ets[r];
                             a.nbr_eid[off + j] = id[r];
                             a.nbr_dt[off + j] = ets[r] - t;
@@ -494,8 +504,9 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
             }
             if (active && lig < c) {
                 const int64_t e = start + sel;
-                const int64_t ets = a.ts[e];
-                a.nbr[off + rank] = a.col[e];
+                const int64_t ets = a.ts[e], dst = a.col[e];
+                a.nbr[off + rank] = dst;
+                if (a.mark != nullptr) mark_id(a, dst);
                 a.nbr_ts[off + rank] = a.keep_root_time ? t : ets;
                 a.nbr_eid[off + rank] = a.eid[e];
                 a.nbr_dt[off + rank] = ets - t;
@@ -539,6 +550,8 @@ int32_t check_params(const sgl_sample_params* p) {
     if (p->type != SGL_SAMPLE_RECENT && p->type != SGL_SAMPLE_UNIFORM)
         return fail(SGL_ENOTSUP, "undefined sampling strategy");
     if (p->fanout < 0) return fail(SGL_EINVAL, "sample: fanout < 0");
+    if (p->mark_state && (p->mark_universe < 0 || p->mark_universe > 0xFFFFFFFFll))
+        return fail(SGL_EINVAL, "sample: bad mark_universe");
     if (p->type == SGL_SAMPLE_UNIFORM && p->fanout > SGL_UNIFORM_MAX_FANOUT)
         return fail(SGL_ENOTSUP, "uniform fanout %d > %d", p->fanout, SGL_UNIFORM_MAX_FANOUT);
     return SGL_OK;
@@ -634,6 +647,9 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
     a.type = p->type; a.k = p->fanout; a.allowed_offset = p->allowed_offset;
     a.equal_root_time = p->equal_root_time; a.keep_root_time = p->keep_root_time;
     a.replace = p->replace; a.hop = p->hop; a.seed = p->seed;
+    a.mark = p->mark_state ? remap_flags(p->mark_state, p->mark_universe) : nullptr;
+    a.mark_universe = p->mark_universe;
+    a.mark_bytes = remap_byte_flags(p->mark_universe) ? 1 : 0;
     a.w_start = ar.take<int64_t>(S_max + 1);
     a.w_len = ar.take<int64_t>(S_max + 1);
     a.block_sum = ar.take<int64_t>(MAX_BLOCKS);

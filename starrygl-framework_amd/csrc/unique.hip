@@ -2,15 +2,18 @@
 //
 // Dense-universe path (ids in [0, universe), `state` given):
 //   the persistent state holds a 64-bit table entry per id
-//   (epoch << 32 | local id) and a bitmap of universe bits.  Per group
-//     mark   : ids whose table entry is not of the current epoch set their bit
-//              (atomicOr), duplicates collapse for free;
-//     reduce : per-tile popcount sums;
-//     assign : every set bit gets local id = base + rank of the bit, which is
+//   (epoch << 32 | local id) and a "pending" flag per id: a byte for universes
+//   of up to 16M ids, a bit beyond.  Per group
+//     mark   : ids whose table entry is not of the current epoch set their flag
+//              (plain byte store, or atomicOr on the bitmap), duplicates
+//              collapse for free;
+//     reduce : per-tile popcount sums over the flag words;
+//     assign : every set flag gets local id = base + rank of the flag, which is
 //              the ascending-id order the reference obtains by sort + unique;
 //              the entry, the local->global list and the cleared word are
 //              written in the same pass;
-//     commit : the call's epoch and id count become the committed ones;
+//     commit : the call's epoch and id count become the committed ones (the
+//              last group's commit is done by one thread of the lookup launch);
 //   then one lookup launch rewrites every input array through the table.
 //   No sort, no hash probing; the result is deterministic.
 //
@@ -31,11 +34,11 @@ namespace {
 
 constexpr int BLOCK = 256;
 constexpr int MAXG = 8;
-constexpr int TILE = BLOCK;            // bitmap words per block in reduce/assign (one per thread)
+constexpr int TILE = BLOCK;            // flag words (8 ids each) per block in reduce/assign (one per thread)
 constexpr int SCAN_BLOCK = 1024;
 constexpr int MAX_GRID = 2048;         // grid cap of the per-id kernels (grid-stride loops)
 constexpr int FUSED_SCAN_MAX = 4096;   // up to this many tiles assign sums the preceding tiles itself
-constexpr size_t HEADER_BYTES = 256;
+constexpr size_t HEADER_BYTES = REMAP_HEADER_BYTES;
 
 struct Header {
     uint64_t epoch;     // committed epoch (low 32 bits are stamped into the table)
@@ -45,15 +48,17 @@ struct Header {
 struct State {
     Header* hdr;
     uint64_t* table;
-    uint64_t* bitmap;
+    uint64_t* bitmap;   // the pending flags, one byte per id, addressed as 8-byte words by reduce/assign
     int64_t universe, words;
+    int32_t bytes;      // 1: a flag byte per id (8 ids per word), 0: a bit per id (64 ids per word)
 };
 
 State carve(void* state, int64_t universe) {
     State s;
     char* p = static_cast<char*>(state);
     s.universe = universe;
-    s.words = ceil_div<int64_t>(universe, 64);
+    s.bytes = remap_byte_flags(universe) ? 1 : 0;
+    s.words = ceil_div<int64_t>(universe, s.bytes ? 8 : 64);
     s.hdr = reinterpret_cast<Header*>(p);
     s.table = reinterpret_cast<uint64_t*>(p + HEADER_BYTES);
     s.bitmap = s.table + universe;
@@ -95,10 +100,13 @@ __global__ void init_state_kernel(State s) {
     }
 }
 
-// Sets the bitmap bit of every id that has no local id in this epoch yet: one
-// id per thread and an unconditional fire-and-forget atomicOr.  (Measured on
-// MI355X: testing the bit first, or folding the block's ids through an LDS
-// hash set first, both lengthen the dependent chain and run 2-3x slower.)
+// Sets the flag of every id that has no local id in this epoch yet: one id per
+// thread and an unconditional fire-and-forget store / atomicOr.  (Measured on
+// MI355X: on a small universe the atomics of a batch serialise on the few cache
+// lines of the bitmap and cost twice what byte stores do; on a 100M-id universe
+// sweeping a byte per id in reduce/assign costs more than the atomics.  Testing
+// the flag first, or folding the block's ids through an LDS hash set first,
+// lengthens the dependent chain and runs 2-3x slower in both layouts.)
 __global__ __launch_bounds__(BLOCK) void mark_kernel(State s, Arrays a, int reset) {
     const uint32_t stamp = eff_stamp(s, reset);
     // Index i is processed for every array at once (loads of the different arrays are
@@ -125,7 +133,7 @@ __global__ __launch_bounds__(BLOCK) void mark_kernel(State s, Arrays a, int rese
 #pragma unroll
         for (int g = 0; g < MAXG; ++g)
             if ((uint32_t)(e[g] >> 32) != stamp)
-                atomicOr(reinterpret_cast<unsigned long long*>(&s.bitmap[id[g] >> 6]), 1ull << (id[g] & 63));
+                remap_set_pending(s.bitmap, s.bytes, id[g]);
     }
 }
 
@@ -174,7 +182,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void scan_tiles_kernel(int64_t* tile_su
 // adds up the tiles before it.
 __global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* tile_sum, int64_t nt,
                                                        int scanned, int reset, int64_t* unique_out,
-                                                       int64_t unique_capacity, int64_t* U_dev) {
+                                                       int64_t unique_capacity, int64_t* U_dev, uint32_t* stamp_ws) {
     __shared__ int64_t s_red[BLOCK / WAVE];
     __shared__ int32_t s_wave[BLOCK / WAVE];
     const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
@@ -205,17 +213,19 @@ __global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* t
         if (q < wid) wave_off += s_wave[q];
         block_total += s_wave[q];
     }
-    if (blockIdx.x == nt - 1 && threadIdx.x == 0) {  // publish the counts of this call
+    if (blockIdx.x == nt - 1 && threadIdx.x == 0) {  // publish the counts and the stamp of this call
         U_dev[0] = base + tile_off + block_total;
+        stamp_ws[0] = eff_stamp(s, reset);
     }
     if (c == 0) return;
     int64_t local = base + tile_off + wave_off + (inc - c);
     const uint64_t stamp = (uint64_t)eff_stamp(s, reset) << 32;
-    const int64_t id0 = w * 64;
+    const int64_t id0 = w * (s.bytes ? 8 : 64);
+    const int shift = s.bytes ? 3 : 0;
     while (word) {
         const int bit = __ffsll((unsigned long long)word) - 1;
         word &= word - 1;
-        const int64_t id = id0 + bit;
+        const int64_t id = id0 + (bit >> shift);
         s.table[id] = stamp | (uint64_t)(uint32_t)local;
         if (local < unique_capacity) unique_out[local] = id;
         ++local;
@@ -225,7 +235,7 @@ __global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* t
 
 // Makes the call's epoch and id count the committed ones.  `first`: U_dev[1]
 // (ids numbered before this call) is recorded.  `has_new` == 0: no assign ran.
-__global__ void commit_kernel(State s, int reset, int first, int has_new, int64_t* U_dev) {
+__device__ __forceinline__ void commit(const State& s, int reset, int first, int has_new, int64_t* U_dev) {
     const int64_t base = eff_base(s, reset);
     const uint64_t epoch = eff_epoch(s, reset);
     if (first) U_dev[1] = base;
@@ -234,8 +244,18 @@ __global__ void commit_kernel(State s, int reset, int first, int has_new, int64_
     s.hdr->id_count = U_dev[0];
 }
 
-__global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a) {
-    const uint32_t stamp = (uint32_t)(s.hdr->epoch & 0xFFFFFFFFull);
+__global__ void commit_kernel(State s, int reset, int first, int has_new, int64_t* U_dev) {
+    commit(s, reset, first, has_new, U_dev);
+}
+
+// Rewrites every input array through the table.  `fold` != 0: the call's last commit
+// has not run yet; the kernel takes the stamp from `stamp_ws` (written by the single
+// thread of stamp_kernel / assign's publisher before this launch, never from the header)
+// and thread 0 of block 0 commits, so no thread of this launch reads what it writes.
+__global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a, int fold, int reset, int first, int has_new,
+                                                       const uint32_t* stamp_ws, int64_t* U_dev) {
+    const uint32_t stamp = fold ? stamp_ws[0] : (uint32_t)(s.hdr->epoch & 0xFFFFFFFFull);
+    if (fold && blockIdx.x == 0 && threadIdx.x == 0) commit(s, reset, first, has_new, U_dev);
     int64_t len[MAXG];
     int64_t max_len = 0;
 #pragma unroll
@@ -258,8 +278,8 @@ __global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a) {
 }
 
 size_t dense_workspace_bytes(int64_t universe) {
-    const int64_t words = ceil_div<int64_t>(universe, 64);
-    return align_up((size_t)(ceil_div<int64_t>(words, TILE) + 2) * 8) + 256;
+    const int64_t words = ceil_div<int64_t>(universe, remap_byte_flags(universe) ? 8 : 64);
+    return align_up((size_t)(ceil_div<int64_t>(words, TILE) + 2) * 8) + 512;
 }
 
 }  // namespace
@@ -269,7 +289,7 @@ using namespace sgl;
 
 extern "C" size_t sgl_remap_state_bytes(int64_t universe) {
     if (universe < 0) return 0;
-    return HEADER_BYTES + (size_t)universe * 8 + (size_t)ceil_div<int64_t>(universe, 64) * 8 + 8;
+    return HEADER_BYTES + (size_t)universe * 8 + (size_t)ceil_div<int64_t>(universe, remap_byte_flags(universe) ? 8 : 64) * 8 + 8;
 }
 
 extern "C" int32_t sgl_remap_init(void* state, size_t state_bytes, int64_t universe, void* stream) {
@@ -298,7 +318,11 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
                                       void* ws, size_t ws_bytes, void* stream) {
     if (G < 0 || (G > 0 && (!ids || !len_max || !local_out)) || !U_dev)
         return fail(SGL_EINVAL, "unique_compact: NULL argument");
+    const bool premarked = (mode & SGL_UNIQUE_PREMARKED) != 0;
+    mode &= ~SGL_UNIQUE_PREMARKED;
     if (mode != SGL_UNIQUE_SORTED && mode != SGL_UNIQUE_GROUPED) return fail(SGL_EINVAL, "unique_compact: bad mode");
+    if (premarked && (mode != SGL_UNIQUE_SORTED || !reset || !state))
+        return fail(SGL_EINVAL, "unique_compact: PREMARKED needs the dense state, SORTED mode and reset = 1");
     if (G > MAXG) return fail(SGL_ENOTSUP, "unique_compact: more than %d arrays", MAXG);
     if (unique_capacity < 0 || (unique_capacity > 0 && !unique_out))
         return fail(SGL_EINVAL, "unique_compact: unique_out is NULL");
@@ -334,10 +358,20 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
     if (ceil_div<int64_t>(total, BLOCK) > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "unique_compact: too many ids");
 
     int64_t* tile_sum = ar.take<int64_t>(nt + 2);
+    uint32_t* stamp_ws = ar.take<uint32_t>(4);
     if (!ar.ok()) return fail(SGL_ENOMEM, "unique_compact: workspace too small");
     const int n_groups = (mode == SGL_UNIQUE_SORTED) ? (G > 0 ? 1 : 0) : G;
-    int first = 1, rst = reset ? 1 : 0;
+    // groups that have anything to number; the commit of the last one is folded into the
+    // lookup launch (one launch less per call), the others commit with a kernel of their own
+    int runnable[MAXG], n_run = 0;
     for (int grp = 0; grp < n_groups; ++grp) {
+        const int64_t sub_total = (mode == SGL_UNIQUE_GROUPED) ? all.len_max[grp] : total;
+        if (sub_total > 0 && universe > 0) runnable[n_run++] = grp;
+    }
+    const bool fold = n_run > 0 && total > 0;
+    int first = 1, rst = reset ? 1 : 0;
+    for (int r = 0; r < n_run; ++r) {
+        const int grp = runnable[r];
         Arrays sub = all;
         if (mode == SGL_UNIQUE_GROUPED) {  // only array `grp`
             sub.G = 1;
@@ -346,14 +380,14 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
             sub.start[0] = 0;
             for (int g = 1; g <= MAXG; ++g) sub.start[g] = sub.len_max[0];
         }
-        const int64_t sub_total = sub.start[sub.G];
-        if (sub_total == 0 || universe == 0) continue;
         int64_t longest = 0;
         for (int g = 0; g < sub.G; ++g) longest = sub.len_max[g] > longest ? sub.len_max[g] : longest;
         int64_t mb = ceil_div<int64_t>(longest, BLOCK);
         if (mb > MAX_GRID) mb = MAX_GRID;
-        hipLaunchKernelGGL(mark_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, sub, rst);
-        SGL_LAUNCH_CHECK();
+        if (!premarked) {
+            hipLaunchKernelGGL(mark_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, sub, rst);
+            SGL_LAUNCH_CHECK();
+        }
         hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
         SGL_LAUNCH_CHECK();
         const int scanned = nt > FUSED_SCAN_MAX ? 1 : 0;
@@ -362,14 +396,15 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
             SGL_LAUNCH_CHECK();
         }
         hipLaunchKernelGGL(assign_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, scanned, rst,
-                           unique_out, unique_capacity, U_dev);
+                           unique_out, unique_capacity, U_dev, stamp_ws);
         SGL_LAUNCH_CHECK();
+        if (fold && r == n_run - 1) break;   // committed by the lookup launch below
         hipLaunchKernelGGL(commit_kernel, dim3(1), dim3(1), 0, st, s, rst, first, 1, U_dev);
         SGL_LAUNCH_CHECK();
         first = 0;
         rst = 0;  // the epoch has been opened; later groups continue it
     }
-    if (first) {  // nothing was numbered: still open the epoch / report the counts
+    if (n_run == 0) {  // nothing was numbered: still open the epoch / report the counts
         hipLaunchKernelGGL(commit_kernel, dim3(1), dim3(1), 0, st, s, rst, 1, 0, U_dev);
         SGL_LAUNCH_CHECK();
     }
@@ -378,7 +413,8 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
         for (int g = 0; g < all.G; ++g) longest = all.len_max[g] > longest ? all.len_max[g] : longest;
         int64_t lb = ceil_div<int64_t>(longest, BLOCK);
         if (lb > MAX_GRID) lb = MAX_GRID;
-        hipLaunchKernelGGL(lookup_kernel, dim3((unsigned)lb), dim3(BLOCK), 0, st, s, all);
+        hipLaunchKernelGGL(lookup_kernel, dim3((unsigned)lb), dim3(BLOCK), 0, st, s, all, fold ? 1 : 0, rst, first, 1,
+                           stamp_ws, U_dev);
         SGL_LAUNCH_CHECK();
     }
     return SGL_OK;

@@ -122,6 +122,8 @@ class MiniBatchPipeline:
         self.ucap = min(sum(caps), graph._n)
         self.ubuf, self.U = be.empty(max(self.ucap, 1)), be.zeros(2)
         self.state = hp.remap_state(graph._n)
+        # the sampler records the ids it emits as pending in the remap state: unique skips its first pass
+        self.p = hp.marking(self.p, self.state)
         self.S0_dev = torch.tensor([self.S0], dtype=torch.int64, device=self.dev)
         f32 = torch.float32
         self.node_out, self.node_ts_out, self.edge_out = {}, {}, {}
@@ -160,7 +162,7 @@ class MiniBatchPipeline:
         arrays = [kr.slot_node0] + [h.neighbors for h in kr.hops]
         lens = [self.S0_dev] + [h.counts[1:2] for h in kr.hops]
         hp.unique_compact(arrays, _abi.UNIQUE_SORTED, self.state, True, lens_dev=lens, out_arrays=self.local,
-                          finalize=False, unique_out=self.ubuf, U_out=self.U)
+                          finalize=False, unique_out=self.ubuf, U_out=self.U, premarked=True)
         if self._plans is None:      # every gather of the batch in as few launches as possible
             segs = [(c, self.ubuf, self.node_out[name], self.node_ts_out.get(name), self.U[0:1])
                     for name, c in self.node_tables.items()]

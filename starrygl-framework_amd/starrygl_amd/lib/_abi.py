@@ -5,12 +5,12 @@ header declares.  The product library exports them as ``sgl_*``.
 """
 import ctypes as C
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
 UNIFORM_MAX_FANOUT = 64
-UNIQUE_SORTED, UNIQUE_GROUPED = 0, 1
+UNIQUE_SORTED, UNIQUE_GROUPED, UNIQUE_PREMARKED = 0, 1, 0x100
 DT_I64, DT_F32 = 0, 1
 
 SAMPLE_TYPES = {"recent": SAMPLE_RECENT, "uniform": SAMPLE_UNIFORM}
@@ -25,7 +25,8 @@ class TCSR(C.Structure):
 class SampleParams(C.Structure):
     _fields_ = [("type", i32), ("fanout", i32), ("allowed_offset", i64),
                 ("equal_root_time", i32), ("keep_root_time", i32),
-                ("replace", i32), ("hop", i32), ("seed", u64)]
+                ("replace", i32), ("hop", i32), ("seed", u64),
+                ("mark_state", vp), ("mark_universe", i64)]
 
 
 class HopOut(C.Structure):

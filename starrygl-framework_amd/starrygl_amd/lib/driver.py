@@ -141,7 +141,16 @@ class HotPath:
             sample_type = _abi.SAMPLE_TYPES[sample_type]
         return SampleParams(int(sample_type), int(fanout), int(allowed_offset),
                             int(bool(equal_root_time)), int(bool(keep_root_time)),
-                            int(bool(replace)), int(hop), int(seed) & (2**64 - 1))
+                            int(bool(replace)), int(hop), int(seed) & (2**64 - 1), None, 0)
+
+    def marking(self, p, state):
+        """Copy of the sampling parameters `p` that makes the sampler record every id it
+        emits as pending in the remap `state`: the following `unique_compact(..., state,
+        reset=True, premarked=True)` over the sampled arrays then skips its first pass."""
+        q = SampleParams.from_buffer_copy(p)
+        q.mark_state, q.mark_universe = self.be.ptr(state.buf), state.universe
+        q._keep = state
+        return q
 
     def sample_hop(self, g, slot_node, slot_ts, p, S_dev=None, finalize=True):
         be, S = self.be, int(slot_node.shape[0])
@@ -197,7 +206,8 @@ class HotPath:
         return RemapState(st, universe)
 
     def unique_compact(self, arrays, mode=_abi.UNIQUE_SORTED, state=None, reset=True,
-                       lens_dev=None, out_arrays=None, finalize=True, unique_out=None, U_out=None):
+                       lens_dev=None, out_arrays=None, finalize=True, unique_out=None, U_out=None,
+                       premarked=False):
         be, G = self.be, len(arrays)
         len_max = (i64 * max(G, 1))(*[int(a.shape[0]) for a in arrays])
         total = sum(len_max[:G])
@@ -219,7 +229,8 @@ class HotPath:
         universe = 0 if state is None else state.universe
         ws, wsb = self._workspace(self.lib.unique_workspace_bytes(universe, G, len_max))
         self._ck(self.lib.unique_compact(None if state is None else be.ptr(state.buf), universe,
-                                         int(bool(reset)), int(mode), G, ids, len_max, ldev, outs,
+                                         int(bool(reset)), int(mode) | (_abi.UNIQUE_PREMARKED if premarked else 0),
+                                         G, ids, len_max, ldev, outs,
                                          be.ptr(unique), cap, be.ptr(U), be.ptr(ws), wsb,
                                          be.stream()))
         if state is not None:

@@ -131,3 +131,38 @@ def test_large_hops(oracle, hot, sample_type):
     b = synth.link_batch(src, dst, ts, 500_000, 502_000, g.n, 2000, rng)          # 6k roots -> ~60k -> ~600k slots
     got, want = _run_both(oracle, hot, g, dg, *b, 3, sample_type=sample_type, fanout=10, seed=5)
     assert want.hops[1].S > 32768 and want.hops[2].S > 8192 * 32
+
+
+@pytest.mark.parametrize("sample_type,fanout,layers", [("recent", 10, 2), ("uniform", 10, 2), ("recent", 20, 1), ("uniform", 33, 1)])
+def test_sampler_marks_ids_for_unique(oracle, hot, sample_type, fanout, layers):
+    """The sampler records what it emits as pending in a remap state; the unique call that follows
+    skips its first pass.  Same local ids and unique list as the oracle's ordinary unique over the
+    sampled arrays; the state is clean afterwards (an ordinary call on it still agrees)."""
+    from starrygl_amd.lib import _abi
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 10_000, 160_000, 1.2, 2_600_000, 20240)
+    rng = np.random.default_rng(5)
+    state, ostate = hot.remap_state(g.n), oracle.remap_state(g.n)
+    for lo in (80_000, 159_400):
+        roots, ts_ptr, root_ts, neg, neg_ts = synth.link_batch(src, dst, ts, lo, lo + 600, g.n, 600, rng)
+        roots[:3] = [g.n + 5, -2, 7]                        # out-of-range roots: no neighbours, local id -1
+        kw = dict(sample_type=sample_type, fanout=fanout, seed=3 + lo)
+        want = oracle.sample_khop(g, roots, ts_ptr, root_ts, neg, neg_ts, layers, oracle.params(**kw), finalize=False)
+        cnt = want.counts
+        wa = [want.slot_node0] + [h.neighbors[: int(cnt[3 * l + 1])] for l, h in enumerate(want.hops)]
+        wl, wu, (wt, _) = oracle.unique_compact([x.copy() for x in wa], _abi.UNIQUE_SORTED, ostate, True)
+        p = hot.marking(hot.params(**kw), state)
+        got = hot.sample_khop(dg, to_dev(hot, roots), to_dev(hot, ts_ptr), to_dev(hot, root_ts), to_dev(hot, neg),
+                              to_dev(hot, neg_ts), layers, p, finalize=False)
+        arrays = [got.slot_node0] + [h.neighbors for h in got.hops]
+        lens = [to_dev(hot, np.array([roots.size + neg.size]))] + [h.counts[1:2] for h in got.hops]
+        gl, gu, (gt, gb) = hot.unique_compact(arrays, _abi.UNIQUE_SORTED, state, True, lens_dev=lens, premarked=True)
+        assert (gt, gb) == (wt, 0) and np.array_equal(np_of(gu), wu[:wt])
+        for a, b in zip(gl, wl):
+            assert np.array_equal(np_of(a)[: b.size], b)
+        assert np_of(gl[0])[:3].tolist()[:2] == [-1, -1]
+        # an ordinary call afterwards: nothing left pending from the sampler
+        extra = rng.integers(0, g.n, 1000).astype(np.int64)
+        l2, u2, (t2, _) = hot.unique_compact([to_dev(hot, extra)], _abi.UNIQUE_SORTED, state, True)
+        assert np.array_equal(np_of(u2), np.unique(extra)) and t2 == np.unique(extra).size
+    with pytest.raises(ValueError):
+        hot.unique_compact([to_dev(hot, extra)], _abi.UNIQUE_GROUPED, state, True, premarked=True)
