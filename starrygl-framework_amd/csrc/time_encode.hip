@@ -33,32 +33,32 @@ struct TEArgs {
 
 // cos of an fp32 argument, accurate to < 1 ulp of the fp32 result for every
 // magnitude the path produces (|a| up to 2^40 and beyond): the argument is reduced
-// in double precision by multiples of pi/2 (two-constant Cody-Waite, exact through
-// FMA), then one degree-5 polynomial in r^2 is evaluated whose coefficients are
-// chosen by the quadrant (sine or cosine series).  About 12 fp64 operations, which
-// is ~1.8x faster on gfx950 than the library cosf whose large-argument path does a
-// Payne-Hanek reduction, and it never leaves the HBM-write-bound regime for small
-// dims.  Arguments beyond 2^45 (not reachable from int64 timestamps times w <= 1
-// in practice) take the library routine.
+// in double precision by multiples of pi (two-constant Cody-Waite, exact through
+// FMA) to r in [-pi/2, pi/2]; then cos(r) = 1 - 2 sin^2(r/2) with one odd
+// polynomial for sin on [-pi/4, pi/4] - no quadrant-dependent coefficients, so no
+// selects - and the sign (-1)^n is applied by a multiply.  About 20 fp64
+// operations, all straight-line.  The library cosf takes ~2.5x as long (its
+// large-argument path is a Payne-Hanek reduction).  Arguments beyond 2^45 (not
+// reachable from int64 timestamps times w <= 1 in practice) take the library routine.
 __device__ __forceinline__ float cos_f32(float af) {
     if (!(__builtin_fabsf(af) < 3.5e13f)) return cosf(af);   // also NaN / inf
     const double x = (double)af;
-    const double n = __builtin_rint(x * 0.63661977236758134308);        // 2/pi
-    double r = __builtin_fma(-n, 1.57079632679489655800e+00, x);        // pi/2, high part
-    r = __builtin_fma(-n, 6.12323399573676603587e-17, r);               // pi/2, low part
-    const int q = (int)(long long)n;
-    const bool odd = q & 1;                                             // quadrants 1, 3: +-sin(r)
-    const double r2 = r * r;
-    // sin(r) = r + r*r2*S(r2), cos(r) = 1 + r2*C(r2) on [-pi/4, pi/4]
-    double h = odd ? -2.505210838544171878e-08 : -2.755731922398589065e-07;   // -1/11! : -1/10!
-    h = __builtin_fma(h, r2, odd ? 2.755731922398589065e-06 : 2.480158730158730159e-05);   //  1/9!  :  1/8!
-    h = __builtin_fma(h, r2, odd ? -1.984126984126984127e-04 : -1.388888888888888889e-03); // -1/7!  : -1/6!
-    h = __builtin_fma(h, r2, odd ? 8.333333333333333333e-03 : 4.166666666666666667e-02);   //  1/5!  :  1/4!
-    h = __builtin_fma(h, r2, odd ? -1.666666666666666667e-01 : -0.5);                      // -1/3!  : -1/2!
-    double y = __builtin_fma(h, odd ? r * r2 : r2, odd ? r : 1.0);
-    // cos(r + q*pi/2): q=0 cos, q=1 -sin, q=2 -cos, q=3 sin
-    y = (((q + 1) & 2) != 0) ? -y : y;
-    return (float)y;
+    const double n = __builtin_rint(x * 0.31830988618379067154);        // 1/pi
+    double r = __builtin_fma(-n, 3.14159265358979311600e+00, x);        // pi, high part
+    r = __builtin_fma(-n, 1.22464679914735317723e-16, r);               // pi, low part
+    const double h = 0.5 * r, h2 = h * h;
+    // sin(h) = h + h*h2*S(h2) on [-pi/4, pi/4]
+    double p = -2.505210838544171878e-08;                               // -1/11!
+    p = __builtin_fma(p, h2, 2.755731922398589065e-06);                 //  1/9!
+    p = __builtin_fma(p, h2, -1.984126984126984127e-04);                // -1/7!
+    p = __builtin_fma(p, h2, 8.333333333333333333e-03);                 //  1/5!
+    p = __builtin_fma(p, h2, -1.666666666666666667e-01);                // -1/3!
+    const double sn = __builtin_fma(p, h * h2, h);
+    const double c = __builtin_fma(-2.0 * sn, sn, 1.0);                 // cos(r)
+    // (-1)^n: n/2 has fraction 0 (even) or 1/2 (odd)
+    const double half = 0.5 * n;
+    const double frac = half - __builtin_floor(half);
+    return (float)(c * __builtin_fma(-4.0, frac, 1.0));
 }
 
 __device__ __forceinline__ float enc(float w, float x, float b) {
@@ -81,8 +81,12 @@ __global__ __launch_bounds__(BLOCK) void time_encode_kernel(TEArgs a) {
         __syncthreads();
         const int32_t total = rows * cpr;
         float* __restrict__ dst = a.out + row0 * a.dim;
+        const float inv_cpr = 1.0f / (float)cpr;
         for (int32_t lc = threadIdx.x; lc < total; lc += BLOCK) {
-            const int32_t r = lc / cpr;
+            // lc / cpr for lc < 2^16 (a tile has at most MAX_RPB * BLOCK chunks): one multiply and a fix-up
+            int32_t r = (int32_t)(((float)lc + 0.5f) * inv_cpr);
+            r -= (r * cpr > lc) ? 1 : 0;
+            r += ((r + 1) * cpr <= lc) ? 1 : 0;
             const int32_t j = (lc - r * cpr) * VEC;
             const float x = s_x[r];
             if constexpr (VEC == 4) {
