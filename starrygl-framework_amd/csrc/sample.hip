@@ -534,7 +534,11 @@ int pick_group(const sgl_sample_params* p, int64_t S_max) {
 // the number of loads in flight and by their count: one lane per slot (plain binary
 // search) keeps 8x the slots in flight and issues ~2.5x fewer loads than 8 lanes do
 // (857k slots over rows of up to 1M edges: 187 us against 330 us).
-int pick_search_group(int Gf, int64_t S_max) { return S_max >= 262144 ? 1 : Gf; }
+int pick_search_group(int Gf, int64_t S_max) {
+    if (S_max >= 262144) return 1;
+    if (S_max >= 32768 && Gf > 8) return 8;   // as the recent strategy: one wave-residency round for the search
+    return Gf;
+}
 
 size_t hop_workspace_bytes(int64_t S_max) {
     size_t b = 0;
