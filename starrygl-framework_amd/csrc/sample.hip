@@ -626,6 +626,238 @@ int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf) {
     return SGL_OK;
 }
 
+
+// ---------------------------------------------------------------------------------------
+// Two hops of the recent strategy in one launch, for the latency regime (a few thousand to
+// 32768 root slots, fanout <= 16): the multi-launch path spends most of such a call on launch
+// floors and on re-reading what the previous kernel just wrote.
+//
+// A group of 16 lanes owns one root slot.  The group finds the root's window together and
+// takes its c <= k edges, one per lane; lane j then finds the window of "its" hop-2 slot
+// (neighbour j at its timestamp) with a plain binary search, so a root and all its hop-2
+// slots are counted without leaving registers.  Output offsets need the number of edges of
+// all earlier slots: the block publishes its totals in a 64-bit descriptor right after its
+// searches and adds up the descriptors of all blocks before it as they appear (a block waits
+// only for blocks with a smaller index, which the dispatcher started no later than itself,
+// and for nothing those blocks wait for).  The wait is bounded: after FUSED_SPIN_LIMIT polls
+// a lane gives up and counts[2] of hop 0 is poisoned, so every wave exits whatever happens.  Then the group writes
+// hop 1 (one edge per lane) and copies each hop-2 slot's edges with all its lanes.
+//
+// Descriptor: published flag (2 bits) | bad root slots (16) | hop-1 edges (22) | hop-2 edges (24);
+// the fields cannot overflow for <= 32768 slots and fanout <= 16, so packed values add.
+constexpr int FG = 16;
+constexpr int FSPB = BLOCK / FG;
+constexpr int64_t FUSED_MAX_SLOTS = 32768;
+constexpr int FUSED_SPIN_LIMIT = 1 << 20;
+constexpr uint64_t ST_AGG = 1ull << 62, ST_MASK = 3ull << 62;
+constexpr int SH_E0 = 24, SH_BAD = 46;
+constexpr uint64_t M_E1 = (1ull << 24) - 1, M_E0 = (1ull << 22) - 1, M_BAD = (1ull << 16) - 1;
+
+struct Fused2Args {
+    HopArgs h;            // graph, roots, parameters, hop-0 outputs
+    int64_t* rsp1;        // hop-1 outputs
+    int64_t* rep1;
+    int64_t* nbr1;
+    int64_t* nbr_ts1;
+    int64_t* nbr_eid1;
+    int64_t* nbr_dt1;
+    int64_t* counts1;
+    unsigned long long* desc;   // [gridDim] zeroed by fused_clear_kernel
+};
+
+__global__ void fused_clear_kernel(unsigned long long* desc, int n, int64_t* counts1) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) desc[i] = 0ull;
+    if (i == 0) counts1[2] = 0;
+}
+
+// First index in [lo, hi) with ts[idx] >= key, by one lane.  (Wider searches - 8-ary per lane,
+// several probes per lane in the group search - were measured slower here: the searches are
+// bound by the number of scattered loads, not by the number of rounds.)
+__device__ __forceinline__ int64_t lane_lower_bound(const int64_t* __restrict__ ts, int64_t lo, int64_t hi, int64_t key) {
+    while (lo < hi) {
+        const int64_t mid = lo + ((hi - lo) >> 1);
+        if (ts[mid] < key) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+__global__ __launch_bounds__(BLOCK) void fused2_recent_kernel(Fused2Args f) {
+    const HopArgs& a = f.h;
+    __shared__ uint64_t s_grp[FSPB];
+    __shared__ uint64_t s_red[NWAVE];
+    __shared__ int s_gave[NWAVE];
+    const int gib = threadIdx.x / FG, lig = threadIdx.x % FG;
+    const int wlane = threadIdx.x % WAVE;
+    const int gshift = wlane / FG * FG, gbase = wlane - lig;
+    const int32_t k = a.k;
+    const int64_t S = a.S_max;
+    const int64_t slot = (int64_t)blockIdx.x * FSPB + gib;
+    const bool in_range = slot < S;
+    int64_t v = 0, t = 0;
+    if (in_range) load_slot(a, slot, &v, &t);
+    const bool bad = in_range && (v < 0 || v >= a.n);
+    const bool active = in_range && !bad;
+    if (in_range && lig == 0) {
+        a.slot_node_out[slot] = v;
+        a.slot_ts_out[slot] = t;
+        if (a.mark != nullptr) mark_id(a, v);
+    }
+    // ---- hop 1: the root's window, one edge per lane
+    int64_t rs = 0, re = 0;
+    if (active) {
+        rs = a.row_ptr[v];
+        re = a.row_ptr[v + 1];
+    }
+    const int64_t eq = a.equal_root_time ? 1 : 0;
+    const int64_t hi = group_lower_bound<FG>(a.ts, rs, re, t + eq, lig, gshift, active);
+    int64_t lo = rs;
+    if (a.allowed_offset >= 0) lo = group_lower_bound<FG>(a.ts, rs, hi, t - a.allowed_offset, lig, gshift, active);
+    const int64_t len = hi - lo;
+    const int32_t c = active ? (int32_t)(len < k ? len : k) : 0;
+    const bool e_on = lig < c;
+    int64_t nbr = 0, ets = 0, id = 0;
+    if (e_on) {
+        const int64_t e = hi - c + lig;
+        nbr = a.col[e];
+        ets = a.ts[e];
+        id = a.eid[e];
+    }
+    // ---- hop 2: lane j counts the slot (neighbour j, its timestamp)
+    int64_t start2 = 0;
+    int32_t c2 = 0;
+    if (e_on) {
+        if (nbr >= 0 && nbr < a.n) {
+            const int64_t rs2 = a.row_ptr[nbr], re2 = a.row_ptr[nbr + 1];
+            const int64_t hi2 = lane_lower_bound(a.ts, rs2, re2, ets + eq);
+            int64_t lo2 = rs2;
+            if (a.allowed_offset >= 0) lo2 = lane_lower_bound(a.ts, rs2, hi2, ets - a.allowed_offset);
+            const int64_t len2 = hi2 - lo2;
+            c2 = (int32_t)(len2 < k ? len2 : k);
+            start2 = hi2 - c2;
+        } else {
+            atomicAdd(reinterpret_cast<unsigned long long*>(&f.counts1[2]), 1ull);
+        }
+    }
+    // exclusive prefix of c2 inside the group, group total
+    int32_t inc2 = c2;
+    for (int d = 1; d < FG; d <<= 1) {
+        const int32_t x = __shfl_up(inc2, d, FG);
+        if (lig >= d) inc2 += x;
+    }
+    const int32_t C2 = __shfl(inc2, FG - 1, FG);
+    if (lig == 0) s_grp[gib] = ((uint64_t)(bad ? 1 : 0) << SH_BAD) | ((uint64_t)c << SH_E0) | (uint64_t)C2;
+    __syncthreads();
+    uint64_t gpre = 0, btotal = 0;
+#pragma unroll
+    for (int q = 0; q < FSPB; ++q) {
+        const uint64_t x = s_grp[q];
+        if (q < gib) gpre += x;
+        btotal += x;
+    }
+    // ---- totals of all earlier blocks: publish this block's, then add up theirs as they appear
+    // (every block publishes right after its searches, so nobody waits for a chain of blocks)
+    const int64_t b = blockIdx.x;
+    if (threadIdx.x == 0)
+        __hip_atomic_store(&f.desc[b], ST_AGG | btotal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint64_t part = 0;
+    int gave_up = 0;
+    for (int64_t idx = threadIdx.x; idx < b; idx += BLOCK) {
+        uint64_t d;
+        int spins = 0;
+        while (((d = __hip_atomic_load(&f.desc[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) & ST_MASK) == 0) {
+            if (++spins > FUSED_SPIN_LIMIT) {
+                gave_up = 1;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        part += d & ~ST_MASK;
+    }
+    for (int dd = WAVE / 2; dd > 0; dd >>= 1) {
+        part += (uint64_t)shfl_i64((int64_t)part, wlane ^ dd);
+        gave_up |= __shfl(gave_up, wlane ^ dd);
+    }
+    if (wlane == 0) {
+        s_red[threadIdx.x / WAVE] = part;
+        s_gave[threadIdx.x / WAVE] = gave_up;
+    }
+    __syncthreads();
+    uint64_t prefix = 0;
+    gave_up = 0;
+#pragma unroll
+    for (int q = 0; q < NWAVE; ++q) {
+        prefix += s_red[q];
+        gave_up |= s_gave[q];
+    }
+    if (threadIdx.x == 0) {
+        if (gave_up) a.counts[2] = INT64_MAX;         // poisoned: reading the result reports an error
+        if (b == (int64_t)gridDim.x - 1) {            // totals of the call
+            const uint64_t tot = prefix + btotal;
+            const int64_t E0 = (int64_t)((tot >> SH_E0) & M_E0), E1 = (int64_t)(tot & M_E1);
+            a.counts[0] = S;
+            a.counts[1] = E0;
+            if (!gave_up) a.counts[2] = (int64_t)((tot >> SH_BAD) & M_BAD);
+            a.root_start_ptr[S] = E0;
+            a.root_end_ptr[S] = E0;
+            f.counts1[0] = E0;
+            f.counts1[1] = E1;
+            f.rsp1[E0] = E1;
+            f.rep1[E0] = E1;
+        }
+    }
+    const uint64_t P = prefix + gpre;
+    const int64_t off1 = (int64_t)((P >> SH_E0) & M_E0);
+    const int64_t off2 = (int64_t)(P & M_E1) + (inc2 - c2);
+    // ---- hop-1 outputs
+    if (in_range && lig == 0) {
+        a.root_start_ptr[slot] = off1;
+        a.root_end_ptr[slot] = off1 + c;
+    }
+    if (e_on) {
+        const int64_t o = off1 + lig;
+        a.nbr[o] = nbr;
+        if (a.mark != nullptr) mark_id(a, nbr);
+        a.nbr_ts[o] = ets;
+        a.nbr_eid[o] = id;
+        a.nbr_dt[o] = ets - t;
+        f.rsp1[o] = off2;
+        f.rep1[o] = off2 + c2;
+    }
+    // ---- hop-2 outputs: slot j of the group is copied by all its lanes (c2 <= k <= 16 edges),
+    // four slots per pass with every load issued before the first store
+    constexpr int PASS = 4;
+    for (int32_t j0 = 0; j0 < k; j0 += PASS) {
+        int64_t o2[PASS], t2[PASS], ets2[PASS], dst2[PASS], id2[PASS];
+        bool on[PASS];
+#pragma unroll
+        for (int r = 0; r < PASS; ++r) {
+            const int src = gbase + ((j0 + r) & (FG - 1));
+            const int64_t st2 = shfl_i64(start2, src);
+            o2[r] = shfl_i64(off2, src) + lig;
+            t2[r] = shfl_i64(ets, src);
+            const int32_t cc = __shfl(c2, src);
+            on[r] = j0 + r < c && lig < cc;
+            if (on[r]) {
+                const int64_t e = st2 + lig;
+                ets2[r] = a.ts[e];
+                dst2[r] = a.col[e];
+                id2[r] = a.eid[e];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < PASS; ++r) {
+            if (on[r]) {
+                f.nbr1[o2[r]] = dst2[r];
+                if (a.mark != nullptr) mark_id(a, dst2[r]);
+                f.nbr_ts1[o2[r]] = ets2[r];
+                f.nbr_eid1[o2[r]] = id2[r];
+                f.nbr_dt1[o2[r]] = ets2[r] - t2[r];
+            }
+        }
+    }
+}
+
 struct RootSpec {  // hop-0 slot source of the k-hop driver
     int64_t R, S_pos;
     const int64_t *roots, *ts_ptr, *root_ts, *neg_roots, *neg_ts;
@@ -665,6 +897,42 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
     a.nbr_dt = out->neighbors_dt; a.counts = out->counts;
     const int Gf = pick_group(p, S_max);
     return launch_hop(a, st, pick_search_group(Gf, S_max), Gf);
+}
+
+
+int32_t run_fused2(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, const sgl_sample_params* p,
+                   const sgl_hop_out* outs, void* ws, size_t ws_bytes, hipStream_t st) {
+    if (ws_bytes < hop_workspace_bytes(S0) || !ws)
+        return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, hop_workspace_bytes(S0));
+    Arena ar(ws, ws_bytes);
+    Fused2Args f{};
+    HopArgs& a = f.h;
+    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid;
+    a.S_max = S0; a.derive = 1;
+    a.R = spec->R; a.S_pos = spec->S_pos; a.roots = spec->roots; a.ts_ptr = spec->ts_ptr;
+    a.root_ts = spec->root_ts; a.neg_roots = spec->neg_roots; a.neg_ts = spec->neg_ts;
+    a.slot_node_out = spec->slot_node_out; a.slot_ts_out = spec->slot_ts_out;
+    a.type = p->type; a.k = p->fanout; a.allowed_offset = p->allowed_offset;
+    a.equal_root_time = p->equal_root_time; a.keep_root_time = p->keep_root_time;
+    a.replace = p->replace; a.hop = 0; a.seed = p->seed;
+    a.mark = p->mark_state ? remap_flags(p->mark_state, p->mark_universe) : nullptr;
+    a.mark_universe = p->mark_universe;
+    a.mark_bytes = remap_byte_flags(p->mark_universe) ? 1 : 0;
+    a.root_start_ptr = outs[0].root_start_ptr; a.root_end_ptr = outs[0].root_end_ptr;
+    a.nbr = outs[0].neighbors; a.nbr_ts = outs[0].neighbors_ts; a.nbr_eid = outs[0].neighbors_eid;
+    a.nbr_dt = outs[0].neighbors_dt; a.counts = outs[0].counts;
+    f.rsp1 = outs[1].root_start_ptr; f.rep1 = outs[1].root_end_ptr;
+    f.nbr1 = outs[1].neighbors; f.nbr_ts1 = outs[1].neighbors_ts; f.nbr_eid1 = outs[1].neighbors_eid;
+    f.nbr_dt1 = outs[1].neighbors_dt; f.counts1 = outs[1].counts;
+    const int blocks = (int)ceil_div<int64_t>(S0, FSPB);
+    f.desc = reinterpret_cast<unsigned long long*>(ar.take<int64_t>(blocks));
+    if (!ar.ok()) return fail(SGL_ENOMEM, "sample: workspace too small");
+    hipLaunchKernelGGL(fused_clear_kernel, dim3((unsigned)ceil_div<int>(blocks, BLOCK)), dim3(BLOCK), 0, st, f.desc, blocks,
+                       f.counts1);
+    SGL_LAUNCH_CHECK();
+    hipLaunchKernelGGL(fused2_recent_kernel, dim3((unsigned)blocks), dim3(BLOCK), 0, st, f);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
 }
 
 }  // namespace
@@ -729,6 +997,9 @@ extern "C" int32_t sgl_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* 
     }
     hipStream_t st = as_stream(stream);
     RootSpec spec{R, S_pos, roots, ts_ptr, root_ts, neg_roots, neg_ts, slot_node0, slot_ts0};
+    if (layers == 2 && p->type == SGL_SAMPLE_RECENT && p->fanout >= 1 && p->fanout <= FG && S0 >= 1 &&
+        S0 <= FUSED_MAX_SLOTS)
+        return run_fused2(g, &spec, S0, p, outs, ws, ws_bytes, st);
     const int64_t* sn = nullptr;
     const int64_t* stt = nullptr;
     const int64_t* S_dev = nullptr;
