@@ -166,3 +166,24 @@ def test_sampler_marks_ids_for_unique(oracle, hot, sample_type, fanout, layers):
         assert np.array_equal(np_of(u2), np.unique(extra)) and t2 == np.unique(extra).size
     with pytest.raises(ValueError):
         hot.unique_compact([to_dev(hot, extra)], _abi.UNIQUE_GROUPED, state, True, premarked=True)
+
+
+@pytest.mark.parametrize("fanout", [1, 9, 16, 17])
+def test_two_hop_recent_single_launch_boundaries(oracle, hot, fanout):
+    """2-hop recent calls of up to 32768 root slots and fanout <= 16 run as one kernel; slot counts
+    around the group / block / limit boundaries and fanouts on both sides of the limit must agree
+    with the oracle like every other path."""
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 3_000, 90_000, 1.15, 10**6, 23, hub=20_000)
+    rng = np.random.default_rng(9)
+    for S0 in (1, 15, 16, 17, 255, 256, 257, 32768, 32769):
+        n_neg = S0 // 3
+        roots = rng.integers(0, g.n, S0 - n_neg).astype(np.int64)
+        root_ts = rng.integers(0, 10**6, S0 - n_neg).astype(np.int64)
+        ts_ptr = np.arange(S0 - n_neg + 1, dtype=np.int64)
+        neg = rng.integers(0, g.n, n_neg).astype(np.int64)
+        neg_ts = rng.integers(0, 10**6, n_neg).astype(np.int64)
+        if S0 > 32768 and fanout > 9:
+            continue                      # 32769 * 17^2 edges: more than this test needs to allocate
+        got, want = _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, neg, neg_ts, 2, sample_type="recent",
+                              fanout=fanout, equal_root_time=bool(S0 % 2))
+        assert got.hops[1].E == want.hops[1].E
