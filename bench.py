@@ -478,16 +478,18 @@ def main():
             # independent stages become parallel branches of the graph: the uniform sampler
             # runs beside the recent one -> unique -> gathers chain
             # The uniform sampler is independent of the recent -> unique -> gather chain: it is a
-            # second branch of the graph, captured after the chain.  (Kernels of two branches hardly
-            # overlap on this part, and the runtime issues branches in creation order: capturing the
+            # second branch of the graph, forked after the recent sampler (both samplers are single
+            # kernels whose blocks wait for each other's totals: running them side by side only makes
+            # them wait longer) and captured after the chain.  (Kernels of two branches hardly overlap
+            # on this part, and the runtime issues branches in creation order: capturing the
             # independent branch first delays the chain and costs ~10 % of the step; two graphs on
             # two streams, or the edge gather on a branch beside unique, were slower as well.)
             br = torch.cuda.Stream()
             with torch.cuda.graph(g_step):
                 cur = torch.cuda.current_stream()
+                st_recent()
                 ev0 = torch.cuda.Event()
                 ev0.record(cur)
-                st_recent()
                 st_unique()
                 st_gathers()
                 br.wait_event(ev0)

@@ -628,7 +628,7 @@ int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf) {
 
 
 // ---------------------------------------------------------------------------------------
-// Two hops of the recent strategy in one launch, for the latency regime (a few thousand to
+// Two hops in one launch, for the latency regime (a few thousand to
 // 32768 root slots, fanout <= 16): the multi-launch path spends most of such a call on launch
 // floors and on re-reading what the previous kernel just wrote.
 //
@@ -682,8 +682,11 @@ __device__ __forceinline__ int64_t lane_lower_bound(const int64_t* __restrict__ 
     return lo;
 }
 
-__global__ __launch_bounds__(BLOCK) void fused2_recent_kernel(Fused2Args f) {
+template <bool UNIFORM>
+__global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
     const HopArgs& a = f.h;
+    // uniform: the draws of a hop-2 slot are made by the slot's lane; its k picks live here, pick-major
+    __shared__ int64_t s_pick[UNIFORM ? FG * BLOCK : 1];
     __shared__ uint64_t s_grp[FSPB];
     __shared__ uint64_t s_red[NWAVE];
     __shared__ int s_gave[NWAVE];
@@ -716,25 +719,67 @@ __global__ __launch_bounds__(BLOCK) void fused2_recent_kernel(Fused2Args f) {
     const int64_t len = hi - lo;
     const int32_t c = active ? (int32_t)(len < k ? len : k) : 0;
     const bool e_on = lig < c;
+    int64_t pos = hi - c + lig;      // recent: the last c window edges, lane j takes the j-th of them
+    if constexpr (UNIFORM) {
+        // as fill_kernel: lane j draws, Floyd's subset, rank = output place; then the picks are
+        // handed round so that lane j holds the pick of output place j
+        const bool draw = active && len > k;
+        int64_t sel = lig;
+        int32_t rank = lig;
+        if (__any(draw)) {
+            int64_t tj = 0;
+            if (draw && lig < k) {
+                const uint64_t bits = draw_bits(a.seed, 0, slot, lig);
+                tj = a.replace ? bounded(bits, len) : bounded(bits, len - k + lig + 1);
+            }
+            if (a.replace) {
+                if (draw) sel = tj;
+            } else {
+                int64_t mine = -1;
+                for (int32_t j = 0; j < k; ++j) {
+                    const int64_t cand = shfl_i64(tj, gbase + j);
+                    const bool dup = group_ballot<FG>(draw && lig < j && mine == cand, gshift) != 0;
+                    if (lig == j) mine = dup ? (len - k + j) : cand;
+                }
+                int32_t r = 0;
+                for (int32_t j = 0; j < k; ++j) {
+                    const int64_t other = shfl_i64(mine, gbase + j);
+                    r += (other < mine) ? 1 : 0;
+                }
+                if (draw) {
+                    sel = mine;
+                    rank = r;
+                }
+            }
+            int64_t placed = sel;
+            for (int32_t j = 0; j < k; ++j) {
+                const int64_t sj = shfl_i64(sel, gbase + j);
+                const int32_t rj = __shfl(rank, gbase + j);
+                if (rj == lig) placed = sj;
+            }
+            sel = placed;
+        }
+        pos = lo + sel;
+    }
     int64_t nbr = 0, ets = 0, id = 0;
     if (e_on) {
-        const int64_t e = hi - c + lig;
-        nbr = a.col[e];
-        ets = a.ts[e];
-        id = a.eid[e];
+        nbr = a.col[pos];
+        ets = a.ts[pos];
+        id = a.eid[pos];
     }
-    // ---- hop 2: lane j counts the slot (neighbour j, its timestamp)
-    int64_t start2 = 0;
+    // ---- hop 2: lane j counts the slot (neighbour j, its timestamp - or the root's, keep_root_time)
+    const int64_t t2 = (UNIFORM && a.keep_root_time) ? t : ets;
+    int64_t start2 = 0, len2 = 0;
     int32_t c2 = 0;
     if (e_on) {
         if (nbr >= 0 && nbr < a.n) {
             const int64_t rs2 = a.row_ptr[nbr], re2 = a.row_ptr[nbr + 1];
-            const int64_t hi2 = lane_lower_bound(a.ts, rs2, re2, ets + eq);
+            const int64_t hi2 = lane_lower_bound(a.ts, rs2, re2, t2 + eq);
             int64_t lo2 = rs2;
-            if (a.allowed_offset >= 0) lo2 = lane_lower_bound(a.ts, rs2, hi2, ets - a.allowed_offset);
-            const int64_t len2 = hi2 - lo2;
+            if (a.allowed_offset >= 0) lo2 = lane_lower_bound(a.ts, rs2, hi2, t2 - a.allowed_offset);
+            len2 = hi2 - lo2;
             c2 = (int32_t)(len2 < k ? len2 : k);
-            start2 = hi2 - c2;
+            start2 = UNIFORM ? lo2 : hi2 - c2;
         } else {
             atomicAdd(reinterpret_cast<unsigned long long*>(&f.counts1[2]), 1ull);
         }
@@ -818,28 +863,73 @@ __global__ __launch_bounds__(BLOCK) void fused2_recent_kernel(Fused2Args f) {
         const int64_t o = off1 + lig;
         a.nbr[o] = nbr;
         if (a.mark != nullptr) mark_id(a, nbr);
-        a.nbr_ts[o] = ets;
+        a.nbr_ts[o] = t2;
         a.nbr_eid[o] = id;
         a.nbr_dt[o] = ets - t;
         f.rsp1[o] = off2;
         f.rep1[o] = off2 + c2;
     }
+    if constexpr (UNIFORM) {
+        // the draws of hop-2 slot (off1 + lig), by its lane: the slot index is the counter of the
+        // generator, so they can only be made now.  Picks ascend (Floyd + insertion sort), or keep
+        // the draw order when drawing with replacement.
+        const bool draw2 = e_on && len2 > k;
+        const int64_t s2 = off1 + lig;
+        if (__any(draw2)) {
+            // picks in registers (all indices are compile-time constants), placed by rank at the end
+            int64_t pk[FG];
+#pragma unroll
+            for (int j = 0; j < FG; ++j) {
+                pk[j] = INT64_MAX;
+                if (j < k) {
+                    const uint64_t bits = draw_bits(a.seed, 1, s2, j);
+                    if (a.replace) {
+                        pk[j] = bounded(bits, len2 > 0 ? len2 : 1);
+                    } else {
+                        int64_t pj = bounded(bits, len2 - k + j + 1 > 0 ? len2 - k + j + 1 : 1);
+                        bool dup = false;
+#pragma unroll
+                        for (int i = 0; i < j; ++i) dup |= pk[i] == pj;
+                        pk[j] = dup ? len2 - k + j : pj;
+                    }
+                }
+            }
+            if (draw2) {
+#pragma unroll
+                for (int j = 0; j < FG; ++j) {
+                    if (j < k) {
+                        int32_t place = j;            // with replacement: the draw order
+                        if (!a.replace) {             // distinct picks: ascending
+                            place = 0;
+#pragma unroll
+                            for (int i = 0; i < FG; ++i) place += (i != j && pk[i] < pk[j]) ? 1 : 0;
+                        }
+                        s_pick[place * BLOCK + threadIdx.x] = pk[j];
+                    }
+                }
+            }
+        }
+        if (e_on && !draw2)
+            for (int32_t j = 0; j < c2; ++j) s_pick[j * BLOCK + threadIdx.x] = j;   // the whole window, in storage order
+        __syncthreads();
+    }
     // ---- hop-2 outputs: slot j of the group is copied by all its lanes (c2 <= k <= 16 edges),
     // four slots per pass with every load issued before the first store
     constexpr int PASS = 4;
     for (int32_t j0 = 0; j0 < k; j0 += PASS) {
-        int64_t o2[PASS], t2[PASS], ets2[PASS], dst2[PASS], id2[PASS];
+        int64_t o2[PASS], tt[PASS], ets2[PASS], dst2[PASS], id2[PASS];
         bool on[PASS];
 #pragma unroll
         for (int r = 0; r < PASS; ++r) {
             const int src = gbase + ((j0 + r) & (FG - 1));
             const int64_t st2 = shfl_i64(start2, src);
             o2[r] = shfl_i64(off2, src) + lig;
-            t2[r] = shfl_i64(ets, src);
+            tt[r] = shfl_i64(t2, src);
             const int32_t cc = __shfl(c2, src);
             on[r] = j0 + r < c && lig < cc;
             if (on[r]) {
-                const int64_t e = st2 + lig;
+                int64_t e = st2 + lig;
+                if constexpr (UNIFORM) e = st2 + s_pick[lig * BLOCK + (threadIdx.x - lig) + ((j0 + r) & (FG - 1))];
                 ets2[r] = a.ts[e];
                 dst2[r] = a.col[e];
                 id2[r] = a.eid[e];
@@ -850,9 +940,9 @@ __global__ __launch_bounds__(BLOCK) void fused2_recent_kernel(Fused2Args f) {
             if (on[r]) {
                 f.nbr1[o2[r]] = dst2[r];
                 if (a.mark != nullptr) mark_id(a, dst2[r]);
-                f.nbr_ts1[o2[r]] = ets2[r];
+                f.nbr_ts1[o2[r]] = (UNIFORM && a.keep_root_time) ? tt[r] : ets2[r];
                 f.nbr_eid1[o2[r]] = id2[r];
-                f.nbr_dt1[o2[r]] = ets2[r] - t2[r];
+                f.nbr_dt1[o2[r]] = ets2[r] - tt[r];
             }
         }
     }
@@ -930,7 +1020,10 @@ int32_t run_fused2(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, const sg
     hipLaunchKernelGGL(fused_clear_kernel, dim3((unsigned)ceil_div<int>(blocks, BLOCK)), dim3(BLOCK), 0, st, f.desc, blocks,
                        f.counts1);
     SGL_LAUNCH_CHECK();
-    hipLaunchKernelGGL(fused2_recent_kernel, dim3((unsigned)blocks), dim3(BLOCK), 0, st, f);
+    if (p->type == SGL_SAMPLE_UNIFORM)
+        hipLaunchKernelGGL(fused2_kernel<true>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, f);
+    else
+        hipLaunchKernelGGL(fused2_kernel<false>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, f);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }
@@ -997,7 +1090,7 @@ extern "C" int32_t sgl_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* 
     }
     hipStream_t st = as_stream(stream);
     RootSpec spec{R, S_pos, roots, ts_ptr, root_ts, neg_roots, neg_ts, slot_node0, slot_ts0};
-    if (layers == 2 && p->type == SGL_SAMPLE_RECENT && p->fanout >= 1 && p->fanout <= FG && S0 >= 1 &&
+    if (layers == 2 && p->fanout >= 1 && p->fanout <= FG && S0 >= 1 &&
         S0 <= FUSED_MAX_SLOTS)
         return run_fused2(g, &spec, S0, p, outs, ws, ws_bytes, st);
     const int64_t* sn = nullptr;
