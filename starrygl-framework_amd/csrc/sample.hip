@@ -22,6 +22,9 @@
 // device memory, so a k-hop call is a fixed launch sequence sized for the worst
 // case.
 //
+// 2-hop calls of at most 32768 root slots and fanout <= 16 - a training mini-batch -
+// take a different route: one kernel does both hops (see fused2_kernel below).
+//
 // Replaces static_recent_neighbor_num / recent_sample_single_hop_kernel /
 // static_neighbor_num / uniform_sample_single_hop_kernel and the thrust calls
 // between them (csrc/include/starrygl/sample.cu.hpp:706-827, 1532-1716).
