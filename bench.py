@@ -638,6 +638,17 @@ def main():
 
     extra = {}
     has_edge_feat = edge_cache is not None
+    # what a plain device-to-device copy reaches on this box (read + written bytes per second): the
+    # practical ceiling for the gather kernels, which move the same bytes through an indirection
+    roof = {}
+    for mb in (128, 1024):
+        a_ = torch.empty(mb << 20, dtype=torch.uint8, device=dev)
+        b_ = [torch.empty_like(a_) for _ in range(2)]
+        it = iter(range(10 ** 9))
+        ms = _time_launches(torch, lambda: b_[next(it) & 1].copy_(a_), reps=10)
+        roof[f"{mb} MB"] = round(2 * (mb << 20) / ms / 1e6, 1)
+        del a_, b_
+    extra["device copy GB/s (read + write)"] = roof
     # sampler throughput when several mini-batches are sampled by one call (what a loader with a
     # prefetch queue, or an AsyncGraphBlob of several windows, can do): same graph, same batches
     scaling = []
