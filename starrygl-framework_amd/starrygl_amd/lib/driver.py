@@ -101,14 +101,18 @@ class HotPath:
         self.lib, self.be = lib, backend
         if lib.abi_version() != _abi.ABI_VERSION:
             raise RuntimeError("sgl ABI version mismatch")
-        self._ws = None
+        self._ws = {}
 
     # ------------------------------------------------------------ helpers
     def _workspace(self, nbytes):
+        """Scratch memory for one call, kept per stream: calls ordered on one stream may share
+        it, calls on different streams (the query worker's and the caller's, say) must not."""
         nbytes = max(int(nbytes), 256)
-        if self._ws is None or self.be.nbytes(self._ws) < nbytes:
-            self._ws = self.be.empty(nbytes, "u8")
-        return self._ws, self.be.nbytes(self._ws)
+        key = self.be.stream()
+        ws = self._ws.get(key)
+        if ws is None or self.be.nbytes(ws) < nbytes:
+            ws = self._ws[key] = self.be.empty(nbytes, "u8")
+        return ws, self.be.nbytes(ws)
 
     def _ck(self, rc):
         check(self.lib, rc)
