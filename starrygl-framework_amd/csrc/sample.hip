@@ -877,19 +877,37 @@ __global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
         // generator, so they can only be made now.  Picks ascend (Floyd + insertion sort), or keep
         // the draw order when drawing with replacement.
         const bool draw2 = e_on && len2 > k;
-        const int64_t s2 = off1 + lig;
+        const uint32_t dmask = (uint32_t)group_ballot<FG>(draw2, gshift);    // the group's drawing slots
         if (__any(draw2)) {
-            // picks in registers (all indices are compile-time constants), placed by rank at the end
+            // 1. the raw draws of all drawing slots of the group, spread over its 16 lanes (the
+            //    generator is most of the cost: a lane that drew all k of its own slot would leave
+            //    the lanes of non-drawing slots idle for k rounds)
+            const int nd = __popc(dmask);
+            for (int d = lig; __any(d < nd * k); d += FG) {
+                if (d < nd * k) {
+                    const int q = d / k, j = d - q * k;
+                    uint32_t mm = dmask;                 // lane of the q-th drawing slot
+                    for (int i = 0; i < q; ++i) mm &= mm - 1;
+                    const int owner = __ffs(mm) - 1;
+                    const uint64_t bits = draw_bits(a.seed, 1, off1 + owner, j);
+                    s_pick[j * BLOCK + (threadIdx.x - lig) + owner] = (int64_t)bits;
+                }
+            }
+        }
+        __syncthreads();
+        if (__any(draw2)) {
+            // 2. the slot's lane turns its k raw draws into picks (registers, compile-time indices)
+            //    and places them by rank
             int64_t pk[FG];
 #pragma unroll
             for (int j = 0; j < FG; ++j) {
                 pk[j] = INT64_MAX;
-                if (j < k) {
-                    const uint64_t bits = draw_bits(a.seed, 1, s2, j);
+                if (j < k && draw2) {
+                    const uint64_t bits = (uint64_t)s_pick[j * BLOCK + threadIdx.x];
                     if (a.replace) {
-                        pk[j] = bounded(bits, len2 > 0 ? len2 : 1);
+                        pk[j] = bounded(bits, len2);
                     } else {
-                        int64_t pj = bounded(bits, len2 - k + j + 1 > 0 ? len2 - k + j + 1 : 1);
+                        int64_t pj = bounded(bits, len2 - k + j + 1);
                         bool dup = false;
 #pragma unroll
                         for (int i = 0; i < j; ++i) dup |= pk[i] == pj;
