@@ -334,7 +334,11 @@ int32_t sgl_seeds_fill(const sgl_tcsr* g, const sgl_seed_query* q,
  * T = R * (t_end - t_begin).
  *   sgl_slice_count -> totals[0..2] = {R, T, E};   (caller allocates)
  *   sgl_slice_fill.
- * node_chunk: device [g->n] chunk id of every node, in [0, total_chunks). */
+ * node_chunk: device [g->n] chunk id of every node, in [0, total_chunks); NULL
+ * keeps every window edge (no destination filter), which with
+ * full_timestamps = 1 is get_seeds_in_chunks' using_full_timestamp mode
+ * (filter_seeds_kernel, sample.cu.hpp:575-578): nodes/ts_ptr/ts are the roots,
+ * edge_ptr/col_eid their q_ptr/q_eid. */
 size_t  sgl_slice_workspace_bytes(int64_t n_cand, int64_t total_chunks);
 int32_t sgl_slice_count(const sgl_tcsr* g, const sgl_seed_query* q,
                         const int64_t* node_chunk, int64_t total_chunks,

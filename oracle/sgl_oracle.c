@@ -714,8 +714,8 @@ static int32_t slice_walk(const sgl_tcsr* g, const sgl_seed_query* q, const int6
                     if (write) { ts[T] = t; edge_ptr[T] = E; }
                     ++T;
                 }
-                const int64_t dc = node_chunk[g->col[e]];
-                if (dc >= 0 && dc < total_chunks && member[dc]) {
+                const int64_t dc = node_chunk ? node_chunk[g->col[e]] : -1;
+                if (!node_chunk || (dc >= 0 && dc < total_chunks && member[dc])) {
                     if (write) { col[E] = g->col[e]; col_ts[E] = t; col_eid[E] = g->eid[e]; }
                     ++E;
                 }

@@ -88,6 +88,7 @@ __device__ __forceinline__ int64_t candidate_node(const sgl_seed_query& q, int64
 // 1 when the chunk of node `dst` is selected; chunk ids outside the table count as not selected
 __device__ __forceinline__ bool dst_selected(const SliceWs& w, const int64_t* __restrict__ node_chunk, int64_t total_chunks,
                                              int64_t dst) {
+    if (node_chunk == nullptr) return true;          // no destination filter
     const int64_t c = node_chunk[dst];
     return c >= 0 && c < total_chunks && w.member[c] != 0;
 }
@@ -194,7 +195,7 @@ __global__ void empty_slice_kernel(int64_t* totals) { totals[0] = totals[1] = to
 int32_t check(const sgl_tcsr* g, const sgl_seed_query* q, const int64_t* node_chunk, int64_t total_chunks, int32_t full) {
     if (!g || !q) return fail(SGL_EINVAL, "slice: NULL graph or query");
     if (q->num_chunks < 0 || q->n_cand < 0 || total_chunks < 0) return fail(SGL_EINVAL, "slice: negative size");
-    if (q->n_cand > 0 && (!q->chunk_ptr || !q->chunk_nodes || !q->chunks || !q->cand_off || !g->row_ptr || !node_chunk))
+    if (q->n_cand > 0 && (!q->chunk_ptr || !q->chunk_nodes || !q->chunks || !q->cand_off || !g->row_ptr))
         return fail(SGL_EINVAL, "slice: NULL array");
     if (full && q->t_end < q->t_begin) return fail(SGL_EINVAL, "slice: t_end < t_begin");
     if (ceil_div<int64_t>(q->n_cand + 1, CPB) > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "slice: too many candidates");

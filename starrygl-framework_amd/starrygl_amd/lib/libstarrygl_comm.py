@@ -137,9 +137,7 @@ class CUDAGraph:
 
     def get_seeds_in_chunks(self, chunks, time_begin, time_end, using_full_timestamp=False):
         from .seeds import seeds_in_chunks
-        if using_full_timestamp:
-            raise NotImplementedError("using_full_timestamp (dense DTDG timestamps) is outside the CTDG hot path")
-        return seeds_in_chunks(self, chunks, int(time_begin), int(time_end))
+        return seeds_in_chunks(self, chunks, int(time_begin), int(time_end), bool(using_full_timestamp))
 
     def slice_by_chunk_ts(self, chunks, time_begin, time_end, using_full_timestamp=False, stream=0):
         from .seeds import slice_in_chunks

@@ -36,10 +36,17 @@ def _candidates(graph, chunks):
     return torch.from_numpy(chunks_h.copy()).to(dev), torch.from_numpy(cand_off).to(dev), int(cand_off[-1])
 
 
-def seeds_in_chunks(graph, chunks, t_begin, t_end):
+def seeds_in_chunks(graph, chunks, t_begin, t_end, full_timestamps=False):
+    """`full_timestamps`: every root lists all integers of [t_begin, t_end) as its timestamps
+    (discrete-time snapshots; filter_seeds_kernel, sample.cu.hpp:575-578) instead of the distinct
+    timestamps of its events."""
     from .libstarrygl_comm import TemporalRoot
     chunk_ptr, chunk_nodes = _chunk_index(graph)[:2]
     d_chunks, d_off, n_cand = _candidates(graph, chunks)
+    if full_timestamps:
+        nodes, ts_ptr, ts, q_ptr, _, _, q_eid = graph._hp.slice(graph._g, chunk_ptr, chunk_nodes, None, d_chunks, d_off,
+                                                                n_cand, t_begin, t_end, True)
+        return TemporalRoot(nodes, ts_ptr, ts, q_ptr, q_eid)
     out = graph._hp.seeds(graph._g, chunk_ptr, chunk_nodes, d_chunks, d_off, n_cand, t_begin, t_end)
     return TemporalRoot(*out)
 

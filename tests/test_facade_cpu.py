@@ -127,6 +127,19 @@ def test_oracle_slice_matches_brute_force(oracle):
             # with every chunk selected no edge of the window is dropped
             if len(chunks) == C:
                 assert got[4].shape[0] == int(((g.ts >= t0) & (g.ts < t1)).sum())
+            # without a destination filter: the seeds of the same query (full: one entry per integer time)
+            free = oracle.slice(g, chunk_ptr, chunk_nodes, None, ch, off, int(off[-1]), t0, t1, full)
+            roots, ts_ptr, ts_, q_ptr, q_eid = _seed_brute(g, chunk_of, chunks, t0, t1)
+            assert free[0].tolist() == [int(x) for x in roots]
+            if not full:
+                for a, b in zip((free[1], free[2], free[3], free[6]), (ts_ptr, ts_, q_ptr, q_eid)):
+                    assert a.tolist() == [int(x) for x in b]
+            else:
+                assert free[2].tolist() == list(range(t0, t1)) * len(roots) and free[6].tolist() == [int(x) for x in q_eid]
+                cnt = np.diff(free[3]).reshape(len(roots), -1) if roots else np.zeros((0, 0))
+                for r, v in enumerate(roots):                 # events per (root, integer time)
+                    row = g.ts[g.row_ptr[v]: g.row_ptr[v + 1]]
+                    assert cnt[r].tolist() == [int((row == t).sum()) for t in range(t0, t1)]
 
 
 def test_oracle_block_build(oracle):

@@ -161,6 +161,14 @@ def test_slice_by_chunk_ts_matches_oracle(oracle, world, full):
             assert np.array_equal(np_of(a), b), (chunks, t0, t1)
         assert np.array_equal(np_of(layer.root_end_ptr)[:-1], want[3][1:])
     assert want[0].shape[0] == 0                                      # the empty window
+    # seeds with dense timestamps = the slice without a destination filter
+    ch = np.array([1, 5, 2], dtype=np.int64)
+    off = np.concatenate([[0], np.cumsum(world["cp"][ch + 1] - world["cp"][ch])]).astype(np.int64)
+    want = oracle.slice(world["hg"], world["cp"], world["cn"], None, ch, off, int(off[-1]), 50_000, 50_030, True)
+    r = g.g.get_seeds_in_chunks(torch.tensor([1, 5, 2]), 50_000, 50_030, True)
+    for a, b in zip((r.roots, r.ts_ptr, r.ts, r.q_ptr, r.q_eid), (want[0], want[1], want[2], want[3], want[6])):
+        assert np.array_equal(np_of(a), b)
+    assert r.root_ts_num == 30 * r.root_num > 0
     # through the query queue: dense timestamps, ids remapped per array (roots, then neighbours)
     g.async_sample(50_000, 50_020, torch.tensor([1, 5, 2]), {"sample_type": "cluster"}, {}, op="r")
     out = g.get_last_sample()
