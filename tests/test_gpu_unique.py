@@ -26,7 +26,9 @@ def _both(oracle, hot, arrays, mode, universe, calls=1, resets=None):
 
 
 @pytest.mark.parametrize("universe,sizes", [(1000, (50, 500, 5000)), (1_000_000, (12_000, 120_000, 1_200_000)),
-                                            (77, (0, 10, 0)), (64, (64,)), (65, (1,)), (5_000_000, (100,))])
+                                            (77, (0, 10, 0)), (64, (64,)), (65, (1,)), (5_000_000, (100,)),
+                                            # both sides of the flag-byte / flag-bit layout switch (2^24 ids)
+                                            (1 << 24, (3000, 70_000)), ((1 << 24) + 1, (3000, 70_000))])
 def test_sorted_matches_numpy_unique(oracle, hot, universe, sizes):
     rng = np.random.default_rng(universe)
     arrs = [rng.integers(0, universe, s).astype(np.int64) for s in sizes]
