@@ -106,3 +106,28 @@ def test_two_hop_recent_unique_block_at_full_size(hot, big):
         assert int(indptr[-1]) == h.E and bool((deg[:dst_offset] == 0).all())
         assert torch.equal(torch.repeat_interleave(torch.arange(deg.numel(), device=dev), deg, output_size=h.E), edge_dst)
         assert torch.equal(indices, torch.arange(h.E, device=dev) + h.S + dst_offset)
+
+
+def test_tcsr_build_at_full_size(hot):
+    """T-CSR build from 1B shuffled edges (100M nodes): row_ptr is the cumulated degree sequence, the
+    permutation returned as eid maps every output edge to its input edge, rows ascend in (ts, eid)."""
+    dev = hot.be.device
+    free, _ = torch.cuda.mem_get_info(dev)
+    if free < 160 << 30:
+        pytest.skip("needs 160 GB of free HBM")
+    gen = torch.Generator(device=dev).manual_seed(3)
+    src = torch.randint(0, N, (M,), device=dev, generator=gen)
+    dst = torch.randint(0, N, (M,), device=dev, generator=gen)
+    ts = torch.randint(0, 1 << 20, (M,), device=dev, generator=gen)      # ~1000 edges per timestamp: plenty of ties
+    g = hot.tcsr_build(N, src, dst, ts, None)
+    deg = torch.bincount(src, minlength=N)
+    assert int(g.row_ptr[0]) == 0 and torch.equal(g.row_ptr[1:] - g.row_ptr[:-1], deg)
+    assert torch.equal(g.col, dst[g.eid]) and torch.equal(g.ts, ts[g.eid])
+    rows = torch.repeat_interleave(torch.arange(N, device=dev), deg, output_size=M)
+    assert torch.equal(rows, src[g.eid])
+    del deg
+    same = rows[1:] == rows[:-1]
+    del rows
+    assert bool((g.ts[1:][same] >= g.ts[:-1][same]).all())
+    tie = same & (g.ts[1:] == g.ts[:-1])
+    assert int(tie.sum()) > 0 and bool((g.eid[1:][tie] > g.eid[:-1][tie]).all())
