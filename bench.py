@@ -564,6 +564,20 @@ def main():
     for v in stages.values():
         for kk in v:
             v[kk] = float(round(v[kk], 4))
+    # the other two routes of the unique stage on one batch's ids, launched on their own (eager, back to
+    # back): the dense-table route with its own marking pass, and the hash-set route (arbitrary ids, no table)
+    stage_inputs(W % NB)
+    st_recent(); st_unique()
+    c_now = live.cpu().numpy()
+    arrs = [kr.slot_node0, kr.hops[0].neighbors[: int(c_now[1])], kr.hops[1].neighbors[: int(c_now[4])]]
+    outs_ = [x[: a.numel()] for x, a in zip(local, arrs)]
+    n_ids = sum(a.numel() for a in arrs)
+    u_alt = hot.be.zeros(2)
+    for tag, st_ in (("unique_compact_dense_own_marking", state), ("unique_compact_hash_set", None)):
+        ms = _time_launches(torch, lambda: hot.unique_compact(arrs, _abi.UNIQUE_SORTED, st_, True, out_arrays=outs_,
+                                                              finalize=False, unique_out=ubuf, U_out=u_alt), reps=10)
+        stages[tag] = {"ms": round(ms, 4), "ids_per_s": round(n_ids / ms * 1e3, 1)}
+    st_recent(); st_unique()      # leave the state as a step does
     # the dominant kernel alone: the step's gather launch (all three row lists in one launch), 20
     # launches back to back between one pair of HIP events on the stream it is launched on (the
     # per-stage figures above carry one graph launch + one event pair each).  Every launch gathers
