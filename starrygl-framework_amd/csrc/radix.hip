@@ -24,6 +24,7 @@ constexpr int WAVES = BLOCK / WAVE;
 constexpr int RADIX = 256;
 constexpr int SCAN_BLOCK = 1024;
 constexpr int SCAN_TILE = 2048;
+constexpr int64_t SCAN_SINGLE_MAX = 16384;   // up to here one block scans the whole input
 
 __global__ __launch_bounds__(BLOCK) void hist_kernel(const uint64_t* __restrict__ keys, int64_t n_max,
                                                      const int64_t* n_dev, int shift, int64_t nb,
@@ -126,13 +127,15 @@ __global__ __launch_bounds__(BLOCK) void scan_reduce_kernel(const int64_t* __res
     }
 }
 
-__global__ __launch_bounds__(SCAN_BLOCK) void scan_single_kernel(int64_t* data, int64_t n, int64_t* total_out) {
+// One block scans n values: thread t owns a contiguous run.  `in` may equal `out`.
+__global__ __launch_bounds__(SCAN_BLOCK) void scan_single_kernel(const int64_t* in, int64_t* out, int64_t n,
+                                                                 int64_t* total_out) {
     __shared__ int64_t s_part[SCAN_BLOCK];
     const int64_t per = ceil_div<int64_t>(n, SCAN_BLOCK);
     const int64_t b0 = (int64_t)threadIdx.x * per;
     const int64_t b1 = b0 + per < n ? b0 + per : n;
     int64_t sum = 0;
-    for (int64_t b = b0; b < b1; ++b) sum += data[b];
+    for (int64_t b = b0; b < b1; ++b) sum += in[b];
     s_part[threadIdx.x] = sum;
     __syncthreads();
     for (int d = 1; d < SCAN_BLOCK; d <<= 1) {
@@ -144,8 +147,8 @@ __global__ __launch_bounds__(SCAN_BLOCK) void scan_single_kernel(int64_t* data, 
     }
     int64_t run = s_part[threadIdx.x] - sum;
     for (int64_t b = b0; b < b1; ++b) {
-        const int64_t x = data[b];
-        data[b] = run;
+        const int64_t x = in[b];
+        out[b] = run;
         run += x;
     }
     if (threadIdx.x == SCAN_BLOCK - 1 && total_out != nullptr) *total_out = s_part[SCAN_BLOCK - 1];
@@ -195,9 +198,14 @@ int32_t exclusive_scan_i64(const int64_t* in, int64_t* out, int64_t n, int64_t* 
     int64_t* tile_sum = static_cast<int64_t*>(ws);
     const int64_t nt = ceil_div<int64_t>(n > 0 ? n : 1, SCAN_TILE);
     if (nt > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "scan: too many elements");
+    if (n <= SCAN_SINGLE_MAX) {   // short inputs: one launch instead of three
+        hipLaunchKernelGGL(scan_single_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, in, out, n, total_out);
+        SGL_LAUNCH_CHECK();
+        return SGL_OK;
+    }
     hipLaunchKernelGGL(scan_reduce_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, in, n, tile_sum);
     SGL_LAUNCH_CHECK();
-    hipLaunchKernelGGL(scan_single_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, tile_sum, nt, total_out);
+    hipLaunchKernelGGL(scan_single_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, tile_sum, tile_sum, nt, total_out);
     SGL_LAUNCH_CHECK();
     hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, in, n, tile_sum, out);
     SGL_LAUNCH_CHECK();
