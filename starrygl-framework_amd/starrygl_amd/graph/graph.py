@@ -62,12 +62,12 @@ class pyGraph:
         neg = test_generate_kwargs.get("test_generate_samples", empty).to(dev)
         neg_ts = test_generate_kwargs.get("test_generate_samples_ts", empty).to(dev)
         if policy["sample_type"] == "cluster":
-            return self.g.submit_query(time_start, time_end, chunk_list.to(dev), neg, neg_ts, "cluster",
+            return self.g.submit_query(time_start, time_end, chunk_list, neg, neg_ts, "cluster",
                                        1, 0, 0, 0, 0, op)
         for key in ("fanout", "layers"):
             if key not in policy:
                 raise ValueError(f"policy must contain '{key}' for non-c sampling")
-        return self.g.submit_query(time_start, time_end, chunk_list.to(dev), neg, neg_ts, policy["sample_type"],
+        return self.g.submit_query(time_start, time_end, chunk_list, neg, neg_ts, policy["sample_type"],
                                    policy["layers"], policy["fanout"], policy.get("allowed_offset", -1),
                                    policy.get("equal_root_time", False), policy.get("keep_root_time", False), op)
 
@@ -136,7 +136,8 @@ class AsyncBlock:
         hp = hot_path(dev)
         # hop-0 slots: every (root, timestamp) pair, then the negatives
         reps = root.ts_ptr[1:] - root.ts_ptr[:-1]
-        last_nodes = torch.cat([torch.repeat_interleave(root.roots, reps), neg_roots.roots])
+        last_nodes = torch.cat([torch.repeat_interleave(root.roots, reps, output_size=int(root.ts.numel())),
+                                neg_roots.roots])
         last_ts = torch.cat([root.ts, neg_roots.ts])
         mfgs = []
         for layer in neighbors:

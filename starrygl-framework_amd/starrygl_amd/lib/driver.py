@@ -390,10 +390,11 @@ class KHopResult:
         self.hp, self.slot_node0, self.slot_ts0, self.hops = hp, slot_node0, slot_ts0, hops
         self.counts, self.final = counts, False
 
-    def finalize(self):
-        """Read the per-hop device counts (one synchronising copy) and narrow."""
+    def finalize(self, counts_host=None):
+        """Read the per-hop device counts (one synchronising copy, unless the caller
+        already has them on the host) and narrow."""
         if not self.final:
-            c = self.hp.be.tolist(self.counts)
+            c = self.hp.be.tolist(self.counts) if counts_host is None else list(counts_host)
             for l, h in enumerate(self.hops):
                 h.finalize(*c[3 * l: 3 * l + 3])
             S0 = getattr(self, "S0_live", None)

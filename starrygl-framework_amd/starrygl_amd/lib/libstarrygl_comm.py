@@ -124,16 +124,23 @@ class CUDAGraph:
         return NegativeRoot(_i64(negative_root, dev, "negative_root"), _i64(negative_time, dev, "negative_time"))
 
     def sample_src_in_chunks_khop(self, postive_root, negative_root, k, layers, allowed_offset, equal_root_time,
-                                  keep_root_time, sample_type, seed=None):
+                                  keep_root_time, sample_type, seed=None, _defer=None):
         """k-hop sampling from explicit roots (sample.cu.hpp:1532-1716).  Ids in
-        the result are global; `submit_query` adds the remap."""
+        the result are global; `submit_query` adds the remap.  (`_defer`: the query
+        worker passes a device array for the counts and reads them later, together with
+        the unique count, in one copy.)"""
         hp = self._hp
         p = hp.params(sample_type, k, allowed_offset, equal_root_time, keep_root_time,
                       seed=self._seed if seed is None else seed)
         neg = negative_root if negative_root is not None else self._empty_neg()
-        res = hp.sample_khop(self._g, postive_root.roots, postive_root.ts_ptr, postive_root.ts, neg.roots, neg.ts,
-                             int(layers), p)
-        return TemporalResult(postive_root, neg, [TemporalNeighbor(h) for h in res.hops])
+        if _defer is None:
+            res = hp.sample_khop(self._g, postive_root.roots, postive_root.ts_ptr, postive_root.ts, neg.roots, neg.ts,
+                                 int(layers), p)
+            return TemporalResult(postive_root, neg, [TemporalNeighbor(h) for h in res.hops])
+        S0 = int(postive_root.ts.numel() + neg.roots.numel())
+        out = hp.khop_buffers(S0, int(layers), int(k), counts=_defer)
+        return hp.sample_khop(self._g, postive_root.roots, postive_root.ts_ptr, postive_root.ts, neg.roots, neg.ts,
+                              int(layers), p, finalize=False, out=out)
 
     def get_seeds_in_chunks(self, chunks, time_begin, time_end, using_full_timestamp=False):
         from .seeds import seeds_in_chunks
@@ -189,9 +196,37 @@ class CUDAGraph:
             return self.remap(self.slice_by_chunk_ts(chunk_list, t0, t1, True), reset=(op != "f"))
         roots = self.get_seeds_in_chunks(chunk_list, t0, t1)
         neg = self.get_negative_root(neg_nodes, neg_ts)
-        res = self.sample_src_in_chunks_khop(roots, neg, fanout, layers, allowed_offset, equal_root_time,
-                                             keep_root_time, sample_type, seed=self._seed + query_index)
-        return self.remap(res, reset=(op != "f"))
+        if layers < 1:
+            raise ValueError("layers must be at least 1")
+        # sampling and unique are chained on the device; their counts come back in one copy
+        hp = self._hp
+        live = hp.be.zeros(3 * layers + 2)
+        kr = self.sample_src_in_chunks_khop(roots, neg, fanout, layers, allowed_offset, equal_root_time,
+                                            keep_root_time, sample_type, seed=self._seed + query_index,
+                                            _defer=live[: 3 * layers])
+        arrays = [roots.roots, neg.roots] + [h.neighbors for h in kr.hops]
+        lens = [None, None] + [h.counts[1:2] for h in kr.hops]
+        return self._remap_arrays(roots, neg, kr, arrays, lens, live, reset=(op != "f"))
+
+    def _remap_arrays(self, roots, neg, kr, arrays, lens, live, reset):
+        hp, L = self._hp, len(kr.hops)
+        if self._state is None:
+            self._state = hp.remap_state(self._n)
+            self._unique = None
+        local, uniq, _ = hp.unique_compact(arrays, _abi.UNIQUE_GROUPED, self._state, reset, lens_dev=lens,
+                                           finalize=False, U_out=live[3 * L:])
+        vals = hp.be.tolist(live)
+        kr.finalize(vals[: 3 * L])
+        total, before = vals[3 * L], vals[3 * L + 1]
+        self._unique = uniq[:total] if (reset or self._unique is None) else torch.cat([self._unique[:before],
+                                                                                        uniq[before:total]])
+        res = TemporalResult(TemporalRoot(local[0], roots.ts_ptr, roots.ts, roots.q_ptr, roots.q_eid),
+                             NegativeRoot(local[1], neg.ts), [TemporalNeighbor(h) for h in kr.hops])
+        for layer, loc in zip(res.neighbors_list, local[2:]):
+            layer.neighbors = loc[: layer.neighbors.numel()]
+        res.nodes_remapper_id = self._unique
+        torch.cuda.current_stream().synchronize()
+        return res
 
     def remap(self, result, reset=True):
         """Remapper::insert (sample.cu.hpp:1825-1852): roots, negatives and every
