@@ -808,6 +808,26 @@ __global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
     const int64_t b = blockIdx.x;
     if (threadIdx.x == 0)
         __hip_atomic_store(&f.desc[b], ST_AGG | btotal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // recent: what a hop-2 slot copies is known before its output place is, so the loads are issued
+    // now (after the block has published) and are in flight while it waits for the totals of the blocks before it
+    constexpr int PRE = 8;     // slots preloaded (registers: 6 per slot); the rest is loaded afterwards
+    int64_t pre_ts[UNIFORM ? 1 : PRE], pre_col[UNIFORM ? 1 : PRE], pre_eid[UNIFORM ? 1 : PRE];
+    if constexpr (!UNIFORM) {
+#pragma unroll
+        for (int j = 0; j < PRE; ++j) {
+            pre_ts[j] = pre_col[j] = pre_eid[j] = 0;
+            if (j < k) {
+                const int64_t st2 = shfl_i64(start2, gbase + j);
+                const int32_t cc = __shfl(c2, gbase + j);
+                if (j < c && lig < cc) {
+                    const int64_t e = st2 + lig;
+                    pre_ts[j] = a.ts[e];
+                    pre_col[j] = a.col[e];
+                    pre_eid[j] = a.eid[e];
+                }
+            }
+        }
+    }
     uint64_t part = 0;
     int gave_up = 0;
     for (int64_t idx = threadIdx.x; idx < b; idx += BLOCK) {
@@ -934,10 +954,28 @@ __global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
             for (int32_t j = 0; j < c2; ++j) s_pick[j * BLOCK + threadIdx.x] = j;   // the whole window, in storage order
         __syncthreads();
     }
-    // ---- hop-2 outputs: slot j of the group is copied by all its lanes (c2 <= k <= 16 edges),
-    // four slots per pass with every load issued before the first store
+    // ---- hop-2 outputs: slot j of the group is copied by all its lanes (c2 <= k <= 16 edges)
+    if constexpr (!UNIFORM) {
+#pragma unroll
+        for (int j = 0; j < PRE; ++j) {
+            if (j < k) {
+                const int64_t o2 = shfl_i64(off2, gbase + j) + lig;
+                const int64_t tt = shfl_i64(t2, gbase + j);
+                const int32_t cc = __shfl(c2, gbase + j);
+                if (j < c && lig < cc) {
+                    f.nbr1[o2] = pre_col[j];
+                    if (a.mark != nullptr) mark_id(a, pre_col[j]);
+                    f.nbr_ts1[o2] = pre_ts[j];
+                    f.nbr_eid1[o2] = pre_eid[j];
+                    f.nbr_dt1[o2] = pre_ts[j] - tt;
+                }
+            }
+        }
+    }
+    // uniform, and the slots beyond the preloaded ones: four slots per pass with every load issued
+    // before the first store
     constexpr int PASS = 4;
-    for (int32_t j0 = 0; j0 < k; j0 += PASS) {
+    for (int32_t j0 = UNIFORM ? 0 : PRE; j0 < k; j0 += PASS) {
         int64_t o2[PASS], tt[PASS], ets2[PASS], dst2[PASS], id2[PASS];
         bool on[PASS];
 #pragma unroll
