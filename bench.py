@@ -521,6 +521,19 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t_start
     tot = acc.cpu().numpy()[ACC].astype(np.float64)
+    # ---- spread of the step time: the same K steps once more, one HIP event pair per step
+    sev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
+    for i in range(K):
+        stage_inputs((W + i) % NB)
+        sev[i][0].record()
+        run_step()
+        sev[i][1].record()
+    torch.cuda.synchronize()
+    acc.zero_()
+    step_ms = np.array([a_.elapsed_time(b_) for a_, b_ in sev])
+    step_spread = {"p10": round(float(np.percentile(step_ms, 10)), 4), "median": round(float(np.median(step_ms)), 4),
+                   "p90": round(float(np.percentile(step_ms, 90)), 4),
+                   "note": "GPU time of one step between two HIP events (batch upload excluded)"}
     # ---- per-stage GPU time: the same K steps, HIP events between the stages
     NEV = len(stages_fn) + 1
     evs = [[torch.cuda.Event(enable_timing=True) for _ in range(NEV)] for _ in range(K)]
@@ -646,8 +659,25 @@ def main():
             t_cpu += time.perf_counter() - t1
             edges_cpu += r.hops[0].E + r.hops[1].E
             nb_cpu += 1
+        # the same sampler on one thread (a tenth of the time budget)
+        cdll.sglo_set_num_threads(1)
+        t_one, edges_one, nb_one = 0.0, 0, 0
+        while t_one < args.cpu_seconds / 10:
+            t1 = time.perf_counter()
+            r = ora.sample_khop(hg, *bt[nb_one % NB], 2, po)
+            t_one += time.perf_counter() - t1
+            edges_one += r.hops[0].E + r.hops[1].E
+            nb_one += 1
+        cdll.sglo_set_num_threads(threads)
+        cpu_model = "unknown"
+        try:
+            with open("/proc/cpuinfo") as fh:
+                cpu_model = next((ln.split(":", 1)[1].strip() for ln in fh if ln.startswith("model name")), "unknown")
+        except OSError:
+            pass
         cpu = {"value": round(edges_cpu / t_cpu, 1), "unit": "sampled edges/s (2-hop recent 10x10)", "cores": threads,
                "kind": "port", "sample": f"{nb_cpu} batches of {S0} roots, {edges_cpu} edges in {t_cpu:.2f}s",
+               "cpu_model": cpu_model, "one_thread_value": round(edges_one / t_one, 1),
                "gpu_over_cpu_sampler": round(stages["sample_recent_2hop"]["edges_per_s"] / (edges_cpu / t_cpu), 1)}
 
     extra = {}
@@ -710,7 +740,7 @@ def main():
     out = {
         "metric": "sampled edges/sec (2-hop recent & uniform) + feature-gather GB/s vs HBM peak",
         "value": round(value, 1), "unit": "sampled edges/s", "n_gpus": 1, "steps": K, "warmup": W,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 4), "step_ms_spread": step_spread, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int64", "data": "synthetic", "launch_mode": mode,
         "config": {"workload": "configs[1]: 1M nodes / 20M edges Zipf(1.1) out-degree, batches of 4000 events + 4000 "
                                "negatives (12000 roots): 2-hop recent 10x10 + unique + node/edge gather + 2-hop uniform 10x10",
