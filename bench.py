@@ -326,6 +326,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE readings can be scaled")
     ap.add_argument("--no-fused-mark", action="store_true",
                     help="unique runs its own marking pass instead of the sampler recording the ids it emits")
+    ap.add_argument("--separate-samplers", action="store_true",
+                    help="one library call per sampler (the uniform one on a second graph branch) instead of one call for both")
     ap.add_argument("--serial", action="store_true", help="capture the step as one serial chain of kernels")
     ap.add_argument("--eager", action="store_true", help="launch every kernel from the host instead of replaying a HIP graph")
     args = ap.parse_args()
@@ -429,6 +431,9 @@ def main():
     def st_uniform():
         hot.sample_khop(dg, s_roots, ts_ptr, s_root_ts, s_neg, s_neg_ts, 2, p_uni, finalize=False, out=ku)
 
+    def st_samplers():      # both 2-hop samplers of the step in one library call (one launch)
+        hot.sample_khop_multi(dg, s_roots, ts_ptr, s_root_ts, s_neg, s_neg_ts, 2, [p_rec_mark, p_uni], [kr, ku])
+
     def st_account():
         acc.add_(live)
 
@@ -447,7 +452,10 @@ def main():
             st_node()
 
     def body():
-        st_recent(); st_unique(); st_gathers(); st_uniform()
+        if args.separate_samplers:
+            st_recent(); st_unique(); st_gathers(); st_uniform()
+        else:
+            st_samplers(); st_unique(); st_gathers()
         st_account()
 
     K, W = args.steps, args.warmup
@@ -471,7 +479,7 @@ def main():
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         g_step = torch.cuda.CUDAGraph()
-        if args.serial:
+        if args.serial or not args.separate_samplers:
             with torch.cuda.graph(g_step):
                 body()
         else:
@@ -503,7 +511,8 @@ def main():
             with torch.cuda.graph(gs):
                 f()
             graphs.append(gs)
-        mode = "hipgraph" if args.serial else "hipgraph, uniform sampler on a second branch"
+        mode = ("hipgraph, both samplers in one launch" if not args.separate_samplers else
+                "hipgraph" if args.serial else "hipgraph, uniform sampler on a second branch")
         run_step = g_step.replay
     else:
         run_step = body

@@ -170,6 +170,27 @@ int32_t sgl_sample_khop(const sgl_tcsr* g,
                         const sgl_hop_out* outs,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* Q k-hop calls over the same roots in one library call: query q samples with
+ * p[q] into outs[q * layers + l], l < layers; slot_node0/slot_ts0 are written
+ * once (all queries expand the same roots).  This is what a loader issues when
+ * one mini-batch is sampled under several policies - the reference submits them
+ * one after the other (AsyncGraphBlob, graph.py:274-293; Graph::submit_query,
+ * sample.cu.hpp:1903-1928).  Results equal those of Q sgl_sample_khop calls;
+ * a most-recent and a uniform 2-hop query of at most 32768 root slots and
+ * fanout <= 16 run side by side in one kernel launch.  The workspace is
+ * sgl_sample_khop_multi_workspace_bytes(S0, layers, largest fanout, Q). */
+size_t  sgl_sample_khop_multi_workspace_bytes(int64_t S0, int32_t layers,
+                                              int32_t fanout, int32_t Q);
+int32_t sgl_sample_khop_multi(const sgl_tcsr* g,
+                              int64_t R, const int64_t* roots, const int64_t* ts_ptr,
+                              int64_t S_pos, const int64_t* root_ts,
+                              int64_t N_neg, const int64_t* neg_roots,
+                              const int64_t* neg_ts,
+                              int32_t layers, int32_t Q, const sgl_sample_params* p,
+                              int64_t* slot_node0, int64_t* slot_ts0,
+                              const sgl_hop_out* outs,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------ unique / compaction */
 #define SGL_UNIQUE_SORTED  0 /* all arrays form one group: == np.unique(return_inverse) */
 #define SGL_UNIQUE_GROUPED 1 /* per array: ids new to the epoch, ascending, appended    */

@@ -345,6 +345,32 @@ int32_t sglo_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* roots,
     return SGL_OK;
 }
 
+/* Several k-hop calls over the same roots: by definition the calls one after
+ * the other (the reference submits one query per policy, graph.py:274-293). */
+size_t sglo_sample_khop_multi_workspace_bytes(int64_t S0, int32_t layers, int32_t fanout, int32_t Q) {
+    (void)S0; (void)layers; (void)fanout; (void)Q;
+    return 0;
+}
+
+int32_t sglo_sample_khop_multi(const sgl_tcsr* g, int64_t R, const int64_t* roots,
+                               const int64_t* ts_ptr, int64_t S_pos,
+                               const int64_t* root_ts, int64_t N_neg,
+                               const int64_t* neg_roots, const int64_t* neg_ts,
+                               int32_t layers, int32_t Q, const sgl_sample_params* p,
+                               int64_t* slot_node0, int64_t* slot_ts0,
+                               const sgl_hop_out* outs, void* ws, size_t ws_bytes,
+                               void* stream) {
+    if (Q < 0 || layers < 1 || (Q > 0 && (!p || !outs)))
+        return fail(SGL_EINVAL, "sample_khop_multi: bad Q, layers or NULL argument");
+    for (int32_t q = 0; q < Q; ++q) {
+        int32_t rc = sglo_sample_khop(g, R, roots, ts_ptr, S_pos, root_ts, N_neg, neg_roots, neg_ts,
+                                      layers, &p[q], slot_node0, slot_ts0,
+                                      outs + (size_t)q * layers, ws, ws_bytes, stream);
+        if (rc != SGL_OK) return rc;
+    }
+    return SGL_OK;
+}
+
 /* ----------------------------------------------------- unique / compaction */
 
 /* state layout: int64 header[3] = {epoch, id_count, universe}; then

@@ -668,10 +668,13 @@ struct Fused2Args {
     unsigned long long* desc;   // [gridDim] zeroed by fused_clear_kernel
 };
 
-__global__ void fused_clear_kernel(unsigned long long* desc, int n, int64_t* counts1) {
+__global__ void fused_clear_kernel(unsigned long long* desc, int n, int64_t* counts1, int64_t* counts1_b) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) desc[i] = 0ull;
-    if (i == 0) counts1[2] = 0;
+    if (i == 0) {
+        counts1[2] = 0;
+        if (counts1_b != nullptr) counts1_b[2] = 0;
+    }
 }
 
 // First index in [lo, hi) with ts[idx] >= key, by one lane.  (Wider searches - 8-ary per lane,
@@ -685,11 +688,13 @@ __device__ __forceinline__ int64_t lane_lower_bound(const int64_t* __restrict__ 
     return lo;
 }
 
-template <bool UNIFORM>
-__global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
+// `b` of `nb`: the block's index among the blocks of this call (set by the kernels below)
+// PRE: hop-2 slots of a most-recent call whose edges are loaded while the block waits for the
+// totals of the blocks before it (6 registers per slot).  s_pick: k * BLOCK entries of dynamic LDS
+// (uniform only): the draws of a hop-2 slot are made by the slot's lane; its k picks live there, pick-major.
+template <bool UNIFORM, int PRE>
+__device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b, const int64_t nb, int64_t* s_pick) {
     const HopArgs& a = f.h;
-    // uniform: the draws of a hop-2 slot are made by the slot's lane; its k picks live here, pick-major
-    __shared__ int64_t s_pick[UNIFORM ? FG * BLOCK : 1];
     __shared__ uint64_t s_grp[FSPB];
     __shared__ uint64_t s_red[NWAVE];
     __shared__ int s_gave[NWAVE];
@@ -698,7 +703,7 @@ __global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
     const int gshift = wlane / FG * FG, gbase = wlane - lig;
     const int32_t k = a.k;
     const int64_t S = a.S_max;
-    const int64_t slot = (int64_t)blockIdx.x * FSPB + gib;
+    const int64_t slot = b * FSPB + gib;
     const bool in_range = slot < S;
     int64_t v = 0, t = 0;
     if (in_range) load_slot(a, slot, &v, &t);
@@ -805,13 +810,12 @@ __global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
     }
     // ---- totals of all earlier blocks: publish this block's, then add up theirs as they appear
     // (every block publishes right after its searches, so nobody waits for a chain of blocks)
-    const int64_t b = blockIdx.x;
     if (threadIdx.x == 0)
         __hip_atomic_store(&f.desc[b], ST_AGG | btotal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // recent: what a hop-2 slot copies is known before its output place is, so the loads are issued
     // now (after the block has published) and are in flight while it waits for the totals of the blocks before it
-    constexpr int PRE = 8;     // slots preloaded (registers: 6 per slot); the rest is loaded afterwards
-    int64_t pre_ts[UNIFORM ? 1 : PRE], pre_col[UNIFORM ? 1 : PRE], pre_eid[UNIFORM ? 1 : PRE];
+    constexpr int NPRE = (UNIFORM || PRE == 0) ? 1 : PRE;
+    int64_t pre_ts[NPRE], pre_col[NPRE], pre_eid[NPRE];
     if constexpr (!UNIFORM) {
 #pragma unroll
         for (int j = 0; j < PRE; ++j) {
@@ -860,7 +864,7 @@ __global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
     }
     if (threadIdx.x == 0) {
         if (gave_up) a.counts[2] = INT64_MAX;         // poisoned: reading the result reports an error
-        if (b == (int64_t)gridDim.x - 1) {            // totals of the call
+        if (b == nb - 1) {            // totals of the call
             const uint64_t tot = prefix + btotal;
             const int64_t E0 = (int64_t)((tot >> SH_E0) & M_E0), E1 = (int64_t)(tot & M_E1);
             a.counts[0] = S;
@@ -1007,6 +1011,25 @@ __global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
     }
 }
 
+template <bool UNIFORM>
+__global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
+    extern __shared__ int64_t s_dyn[];
+    fused2_body<UNIFORM, 8>(f, blockIdx.x, gridDim.x, s_dyn);
+}
+
+// Two calls over the same roots in one launch, a most-recent one (even blocks) and a uniform one (odd
+// blocks): each call's blocks keep their order, so the wait of a block is still only for blocks
+// that were dispatched before it.  Either call alone is a chain of dependent loads that leaves most
+// of the chip idle; side by side they take little longer than one.
+__global__ __launch_bounds__(BLOCK) void fused2_pair_kernel(Fused2Args fr, Fused2Args fu) {
+    extern __shared__ int64_t s_dyn[];
+    const int64_t b = blockIdx.x >> 1, nb = gridDim.x >> 1;
+    if (blockIdx.x & 1)
+        fused2_body<true, 0>(fu, b, nb, s_dyn);
+    else
+        fused2_body<false, 0>(fr, b, nb, s_dyn);
+}
+
 struct RootSpec {  // hop-0 slot source of the k-hop driver
     int64_t R, S_pos;
     const int64_t *roots, *ts_ptr, *root_ts, *neg_roots, *neg_ts;
@@ -1049,11 +1072,8 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
 }
 
 
-int32_t run_fused2(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, const sgl_sample_params* p,
-                   const sgl_hop_out* outs, void* ws, size_t ws_bytes, hipStream_t st) {
-    if (ws_bytes < hop_workspace_bytes(S0) || !ws)
-        return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, hop_workspace_bytes(S0));
-    Arena ar(ws, ws_bytes);
+Fused2Args fused2_args(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, const sgl_sample_params* p,
+                       const sgl_hop_out* outs, unsigned long long* desc) {
     Fused2Args f{};
     HopArgs& a = f.h;
     a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid;
@@ -1073,16 +1093,53 @@ int32_t run_fused2(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, const sg
     f.rsp1 = outs[1].root_start_ptr; f.rep1 = outs[1].root_end_ptr;
     f.nbr1 = outs[1].neighbors; f.nbr_ts1 = outs[1].neighbors_ts; f.nbr_eid1 = outs[1].neighbors_eid;
     f.nbr_dt1 = outs[1].neighbors_dt; f.counts1 = outs[1].counts;
+    f.desc = desc;
+    return f;
+}
+
+size_t pick_lds_bytes(int32_t k) { return (size_t)k * BLOCK * sizeof(int64_t); }
+
+bool fused2_fits(int32_t layers, const sgl_sample_params* p, int64_t S0) {
+    return layers == 2 && p->fanout >= 1 && p->fanout <= FG && S0 >= 1 && S0 <= FUSED_MAX_SLOTS;
+}
+
+int32_t run_fused2(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, const sgl_sample_params* p,
+                   const sgl_hop_out* outs, void* ws, size_t ws_bytes, hipStream_t st) {
+    if (ws_bytes < hop_workspace_bytes(S0) || !ws)
+        return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, hop_workspace_bytes(S0));
+    Arena ar(ws, ws_bytes);
     const int blocks = (int)ceil_div<int64_t>(S0, FSPB);
-    f.desc = reinterpret_cast<unsigned long long*>(ar.take<int64_t>(blocks));
+    unsigned long long* desc = reinterpret_cast<unsigned long long*>(ar.take<int64_t>(blocks));
     if (!ar.ok()) return fail(SGL_ENOMEM, "sample: workspace too small");
+    const Fused2Args f = fused2_args(g, spec, S0, p, outs, desc);
     hipLaunchKernelGGL(fused_clear_kernel, dim3((unsigned)ceil_div<int>(blocks, BLOCK)), dim3(BLOCK), 0, st, f.desc, blocks,
-                       f.counts1);
+                       f.counts1, (int64_t*)nullptr);
     SGL_LAUNCH_CHECK();
     if (p->type == SGL_SAMPLE_UNIFORM)
-        hipLaunchKernelGGL(fused2_kernel<true>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, f);
+        hipLaunchKernelGGL(fused2_kernel<true>, dim3((unsigned)blocks), dim3(BLOCK), pick_lds_bytes(p->fanout), st, f);
     else
         hipLaunchKernelGGL(fused2_kernel<false>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, f);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}
+
+// a most-recent and a uniform call over the same roots: one launch (fused2_pair_kernel)
+int32_t run_fused2_pair(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, const sgl_sample_params* p_rec,
+                        const sgl_hop_out* outs_rec, const sgl_sample_params* p_uni, const sgl_hop_out* outs_uni,
+                        void* ws, size_t ws_bytes, hipStream_t st) {
+    if (ws_bytes < 2 * hop_workspace_bytes(S0) || !ws)
+        return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, 2 * hop_workspace_bytes(S0));
+    Arena ar(ws, ws_bytes);
+    const int blocks = (int)ceil_div<int64_t>(S0, FSPB);
+    unsigned long long* desc = reinterpret_cast<unsigned long long*>(ar.take<int64_t>(2 * (size_t)blocks));
+    if (!ar.ok()) return fail(SGL_ENOMEM, "sample: workspace too small");
+    const Fused2Args fr = fused2_args(g, spec, S0, p_rec, outs_rec, desc);
+    const Fused2Args fu = fused2_args(g, spec, S0, p_uni, outs_uni, desc + blocks);
+    hipLaunchKernelGGL(fused_clear_kernel, dim3((unsigned)ceil_div<int>(2 * blocks, BLOCK)), dim3(BLOCK), 0, st, desc,
+                       2 * blocks, fr.counts1, fu.counts1);
+    SGL_LAUNCH_CHECK();
+    hipLaunchKernelGGL(fused2_pair_kernel, dim3((unsigned)(2 * blocks)), dim3(BLOCK), pick_lds_bytes(p_uni->fanout), st,
+                       fr, fu);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }
@@ -1149,9 +1206,7 @@ extern "C" int32_t sgl_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* 
     }
     hipStream_t st = as_stream(stream);
     RootSpec spec{R, S_pos, roots, ts_ptr, root_ts, neg_roots, neg_ts, slot_node0, slot_ts0};
-    if (layers == 2 && p->fanout >= 1 && p->fanout <= FG && S0 >= 1 &&
-        S0 <= FUSED_MAX_SLOTS)
-        return run_fused2(g, &spec, S0, p, outs, ws, ws_bytes, st);
+    if (fused2_fits(layers, p, S0)) return run_fused2(g, &spec, S0, p, outs, ws, ws_bytes, st);
     const int64_t* sn = nullptr;
     const int64_t* stt = nullptr;
     const int64_t* S_dev = nullptr;
@@ -1164,6 +1219,47 @@ extern "C" int32_t sgl_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* 
         sn = outs[l].neighbors;
         stt = outs[l].neighbors_ts;
         S_dev = outs[l].counts + 1;
+    }
+    return SGL_OK;
+}
+
+extern "C" size_t sgl_sample_khop_multi_workspace_bytes(int64_t S0, int32_t layers, int32_t fanout, int32_t Q) {
+    return (size_t)(Q > 0 ? Q : 1) * sgl_sample_khop_workspace_bytes(S0, layers, fanout);
+}
+
+extern "C" int32_t sgl_sample_khop_multi(const sgl_tcsr* g, int64_t R, const int64_t* roots,
+                                         const int64_t* ts_ptr, int64_t S_pos, const int64_t* root_ts,
+                                         int64_t N_neg, const int64_t* neg_roots, const int64_t* neg_ts,
+                                         int32_t layers, int32_t Q, const sgl_sample_params* p,
+                                         int64_t* slot_node0, int64_t* slot_ts0, const sgl_hop_out* outs,
+                                         void* ws, size_t ws_bytes, void* stream) {
+    if (Q < 0 || (Q > 0 && (!p || !outs)) || layers < 1) return fail(SGL_EINVAL, "sample_khop_multi: bad Q, layers or NULL argument");
+    int32_t fan = 0;
+    for (int32_t q = 0; q < Q; ++q) fan = p[q].fanout > fan ? p[q].fanout : fan;
+    const int64_t S0 = (S_pos > 0 ? S_pos : 0) + (N_neg > 0 ? N_neg : 0);
+    const size_t per = sgl_sample_khop_workspace_bytes(S0, layers, fan);
+    if (Q > 0 && (!ws || ws_bytes < (size_t)Q * per))
+        return fail(SGL_ENOMEM, "sample_khop_multi: workspace %zu < %zu bytes", ws_bytes, (size_t)Q * per);
+    // one most-recent and one uniform 2-hop call of the single-launch size share a launch
+    if (Q == 2 && p[0].type != p[1].type && fused2_fits(layers, &p[0], S0) && fused2_fits(layers, &p[1], S0) &&
+        R >= 0 && S_pos >= 0 && N_neg >= 0 && slot_node0 && slot_ts0 &&
+        (S_pos == 0 || (R > 0 && roots && ts_ptr && root_ts)) && (N_neg == 0 || (neg_roots && neg_ts))) {
+        int32_t rc;
+        if ((rc = check_graph(g)) != SGL_OK) return rc;
+        for (int32_t q = 0; q < 2; ++q) {
+            if ((rc = check_params(&p[q])) != SGL_OK) return rc;
+            for (int32_t l = 0; l < 2; ++l)
+                if ((rc = check_out(&outs[q * 2 + l], worst_slots(S0, l, p[q].fanout), p[q].fanout)) != SGL_OK) return rc;
+        }
+        const int r = p[0].type == SGL_SAMPLE_RECENT ? 0 : 1, u = 1 - r;
+        RootSpec spec{R, S_pos, roots, ts_ptr, root_ts, neg_roots, neg_ts, slot_node0, slot_ts0};
+        return run_fused2_pair(g, &spec, S0, &p[r], &outs[r * 2], &p[u], &outs[u * 2], ws, ws_bytes, as_stream(stream));
+    }
+    for (int32_t q = 0; q < Q; ++q) {
+        const int32_t rc = sgl_sample_khop(g, R, roots, ts_ptr, S_pos, root_ts, N_neg, neg_roots, neg_ts, layers, &p[q],
+                                           slot_node0, slot_ts0, outs + (size_t)q * layers,
+                                           static_cast<char*>(ws) + (size_t)q * per, per, stream);
+        if (rc != SGL_OK) return rc;
     }
     return SGL_OK;
 }

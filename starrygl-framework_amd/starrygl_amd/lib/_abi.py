@@ -66,6 +66,9 @@ PROTOTYPES = {
     "sample_khop_workspace_bytes": (sz, [i64, i32, i32]),
     "sample_khop": (i32, [P(TCSR), i64, vp, vp, i64, vp, i64, vp, vp, i32,
                           P(SampleParams), vp, vp, P(HopOut), vp, sz, vp]),
+    "sample_khop_multi_workspace_bytes": (sz, [i64, i32, i32, i32]),
+    "sample_khop_multi": (i32, [P(TCSR), i64, vp, vp, i64, vp, i64, vp, vp, i32, i32,
+                                P(SampleParams), vp, vp, P(HopOut), vp, sz, vp]),
     "remap_state_bytes": (sz, [i64]),
     "remap_init": (i32, [vp, sz, i64, vp]),
     "unique_workspace_bytes": (sz, [i64, i32, P(i64)]),

@@ -202,6 +202,31 @@ class HotPath:
         res.S0_live = S0
         return res.finalize() if finalize else res
 
+    def sample_khop_multi(self, g, roots, ts_ptr, root_ts, neg_roots, neg_ts, layers, params, outs):
+        """Several k-hop calls (params[q] -> outs[q], buffers of khop_buffers) over the same roots
+        in one library call; a most-recent and a uniform 2-hop call share one launch.  The results
+        are not finalized; they share the hop-0 slot arrays of outs[0]."""
+        be, Q = self.be, len(params)
+        R, S_pos, N_neg = int(roots.shape[0]), int(root_ts.shape[0]), int(neg_roots.shape[0])
+        S0 = S_pos + N_neg
+        fan = max(p.fanout for p in params)
+        for p, res in zip(params, outs):
+            if res.S0 < S0 or len(res.hops) != layers or res.fanout < p.fanout:
+                raise MemoryError("khop buffers are smaller than this call needs")
+        head = outs[0]
+        need = int(self.lib.sample_khop_multi_workspace_bytes(S0, layers, fan, Q))
+        if getattr(head, "ws_multi", None) is None or be.nbytes(head.ws_multi) < need:
+            head.ws_multi = be.empty(max(need, 256), "u8")
+        structs = (HopOut * max(Q * layers, 1))(*[o.struct for res in outs for o in res.hops])
+        pa = (_abi.SampleParams * max(Q, 1))(*params)
+        self._ck(self.lib.sample_khop_multi(C.byref(g.view), R, be.ptr(roots), be.ptr(ts_ptr), S_pos,
+                                            be.ptr(root_ts), N_neg, be.ptr(neg_roots), be.ptr(neg_ts),
+                                            layers, Q, pa, be.ptr(head.slot_node0), be.ptr(head.slot_ts0),
+                                            structs, be.ptr(head.ws_multi), be.nbytes(head.ws_multi), be.stream()))
+        for res in outs:
+            res.slot_node0, res.slot_ts0, res.S0_live = head.slot_node0, head.slot_ts0, S0
+        return outs
+
     # ------------------------------------------------------------- unique
     def remap_state(self, universe):
         nbytes = self.lib.remap_state_bytes(universe)

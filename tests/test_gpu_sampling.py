@@ -187,3 +187,58 @@ def test_two_hop_recent_single_launch_boundaries(oracle, hot, fanout):
         got, want = _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, neg, neg_ts, 2, sample_type="recent",
                               fanout=fanout, equal_root_time=bool(S0 % 2))
         assert got.hops[1].E == want.hops[1].E
+
+
+@pytest.mark.parametrize("fanout,layers,S0", [(10, 2, 1), (10, 2, 700), (16, 2, 4099), (17, 2, 300), (10, 1, 500), (5, 3, 200)])
+def test_several_policies_in_one_call(oracle, hot, fanout, layers, S0):
+    """sgl_sample_khop_multi: every query's result equals the oracle's for that policy.  A recent and a
+    uniform 2-hop query of the single-launch size share one kernel; other shapes (fanout 17, one or
+    three hops, three queries) run query by query."""
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 3_000, 90_000, 1.15, 10**6, 29, hub=20_000)
+    rng = np.random.default_rng(13)
+    n_neg = S0 // 3
+    roots = rng.integers(0, g.n, S0 - n_neg).astype(np.int64)
+    root_ts = rng.integers(0, 10**6, S0 - n_neg).astype(np.int64)
+    ts_ptr = np.arange(S0 - n_neg + 1, dtype=np.int64)
+    neg = rng.integers(0, g.n, n_neg).astype(np.int64)
+    neg_ts = rng.integers(0, 10**6, n_neg).astype(np.int64)
+    dev_args = [to_dev(hot, x) for x in (roots, ts_ptr, root_ts, neg, neg_ts)]
+    policies = [dict(sample_type="recent", fanout=fanout, equal_root_time=True),
+                dict(sample_type="uniform", fanout=fanout, seed=77, keep_root_time=True),
+                dict(sample_type="recent", fanout=max(fanout - 2, 1), allowed_offset=50_000)]
+    for sel in ([0, 1], [1, 0], [0, 1, 2], [1]):
+        kws = [policies[i] for i in sel]
+        outs = [hot.khop_buffers(S0, layers, kw["fanout"]) for kw in kws]
+        hot.sample_khop_multi(dg, *dev_args, layers, [hot.params(**kw) for kw in kws], outs)
+        for kw, res in zip(kws, outs):
+            want = oracle.sample_khop(g, roots, ts_ptr, root_ts, neg, neg_ts, layers, oracle.params(**kw))
+            got = res.finalize()
+            assert np.array_equal(np_of(got.slot_node0), want.slot_node0)
+            assert np.array_equal(np_of(got.slot_ts0), want.slot_ts0)
+            for l in range(layers):
+                assert_hop_equal(got.hops[l], want.hops[l], tag=f"hop{l} {kw} of {sel}")
+
+
+def test_several_policies_with_marks_feed_unique(oracle, hot):
+    """The recent query of a shared launch records its ids for the unique stage like a call of its own."""
+    from starrygl_amd.lib import _abi
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 5_000, 120_000, 1.1, 10**6, 31)
+    rng = np.random.default_rng(17)
+    b = synth.link_batch(src, dst, ts, 60_000, 60_400, g.n, 400, rng)
+    state = hot.remap_state(g.n)
+    p_rec = hot.marking(hot.params("recent", 10), state)
+    p_uni = hot.params("uniform", 10, seed=5)
+    outs = [hot.khop_buffers(1200, 2, 10), hot.khop_buffers(1200, 2, 10)]
+    for _ in range(2):          # twice: the second call starts from the state the first one left
+        hot.sample_khop_multi(dg, *[to_dev(hot, x) for x in b], 2, [p_rec, p_uni], outs)
+        r = outs[0]
+        lens = [r.counts[0:1], r.counts[1:2], r.counts[4:5]]
+        arrays = [r.slot_node0, r.hops[0].neighbors, r.hops[1].neighbors]
+        local, uniq, U = hot.unique_compact(arrays, _abi.UNIQUE_SORTED, state, True, lens_dev=lens, finalize=False,
+                                            premarked=True)
+        c = np_of(r.counts)
+        ids = np.concatenate([np_of(r.slot_node0), np_of(r.hops[0].neighbors)[: c[1]], np_of(r.hops[1].neighbors)[: c[4]]])
+        want_u, want_inv = np.unique(ids, return_inverse=True)
+        assert int(np_of(U)[0]) == want_u.size and np.array_equal(np_of(uniq)[: want_u.size], want_u)
+        got_inv = np.concatenate([np_of(local[0]), np_of(local[1])[: c[1]], np_of(local[2])[: c[4]]])
+        assert np.array_equal(got_inv, want_inv)
