@@ -216,7 +216,10 @@ int32_t sgl_remap_init(void* state, size_t state_bytes, int64_t universe,
  *   reset        1: start a new local-id epoch (numbering restarts at 0);
  *                0: continue the epoch of the previous call on `state`.
  *   unique_out   local -> global; entries [U_before, U_total) are written.
- *   U_dev        device int64[2] = {U_total, U_before}.
+ *   U_dev        device int64[2] = {U_total, U_before}.  U_total reads INT64_MAX
+ *                when a numbering pass of this or an earlier call on the state
+ *                gave up its bounded wait for another block: the result is void
+ *                and the state must be initialised again.
  * `state` != NULL selects the dense-universe path: `universe` must be the value
  * given to sgl_remap_init, ids outside [0, universe) map to -1.  `state` ==
  * NULL (universe ignored) selects the hash-set path, which accepts arbitrary

@@ -16,6 +16,10 @@
 //              last group's commit is done by one thread of the lookup launch);
 //   then one lookup launch rewrites every input array through the table.
 //   No sort, no hash probing; the result is deterministic.
+//   Up to SINGLE_PASS_MAX tiles, reduce and assign are one launch: every tile
+//   publishes its count in a descriptor kept in the state (tagged with the
+//   state's pass counter, so descriptors never need clearing) and adds up the
+//   descriptors of the tiles before it as they appear.
 //
 // Replaces Remapper::remapper / insert, mark_new_ids_kernel and
 // update_new_ids_kernel (csrc/include/starrygl/sample.cu.hpp:1719-1854).
@@ -38,17 +42,22 @@ constexpr int TILE = BLOCK;            // flag words (8 ids each) per block in r
 constexpr int SCAN_BLOCK = 1024;
 constexpr int MAX_GRID = 2048;         // grid cap of the per-id kernels (grid-stride loops)
 constexpr int FUSED_SCAN_MAX = 4096;   // up to this many tiles assign sums the preceding tiles itself
+constexpr int SINGLE_PASS_MAX = 2048;  // up to this many tiles the counts are exchanged inside the assign launch
+constexpr int SPIN_LIMIT = 1 << 20;    // polls of one descriptor before a lane gives up (the result is then poisoned)
 constexpr size_t HEADER_BYTES = REMAP_HEADER_BYTES;
 
 struct Header {
     uint64_t epoch;     // committed epoch (low 32 bits are stamped into the table)
     int64_t id_count;   // committed number of local ids handed out in this epoch
+    uint64_t pass;      // numbering passes committed so far (tags the tile descriptors)
+    int64_t poisoned;   // sticky: a tile once gave up waiting for an earlier tile's descriptor
 };
 
 struct State {
     Header* hdr;
     uint64_t* table;
     uint64_t* bitmap;   // the pending flags, one byte per id, addressed as 8-byte words by reduce/assign
+    uint64_t* desc;     // one descriptor per tile of flag words: pass tag << 32 | flags set in the tile
     int64_t universe, words;
     int32_t bytes;      // 1: a flag byte per id (8 ids per word), 0: a bit per id (64 ids per word)
 };
@@ -62,6 +71,7 @@ State carve(void* state, int64_t universe) {
     s.hdr = reinterpret_cast<Header*>(p);
     s.table = reinterpret_cast<uint64_t*>(p + HEADER_BYTES);
     s.bitmap = s.table + universe;
+    s.desc = s.bitmap + s.words;
     return s;
 }
 
@@ -79,6 +89,13 @@ __device__ __forceinline__ uint32_t eff_stamp(const State& s, int reset) {
     return (uint32_t)(eff_epoch(s, reset) & 0xFFFFFFFFull);
 }
 __device__ __forceinline__ int64_t eff_base(const State& s, int reset) { return reset ? 0 : s.hdr->id_count; }
+// Tag of the numbering pass in flight: never 0, the value of a descriptor nobody has written yet.
+__device__ __forceinline__ uint64_t next_pass(uint64_t pass) {
+    pass += 1;
+    if ((pass & 0xFFFFFFFFull) == 0) pass += 1;
+    return pass;
+}
+__device__ __forceinline__ uint32_t eff_tag(const State& s) { return (uint32_t)(next_pass(s.hdr->pass) & 0xFFFFFFFFull); }
 
 struct Arrays {
     int32_t G;
@@ -94,9 +111,12 @@ __global__ void init_state_kernel(State s) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = t; i < s.universe; i += stride) s.table[i] = 0;
     for (int64_t i = t; i < s.words; i += stride) s.bitmap[i] = 0;
+    for (int64_t i = t; i < ceil_div<int64_t>(s.words, TILE); i += stride) s.desc[i] = 0;
     if (t == 0) {
         s.hdr->epoch = 1;
         s.hdr->id_count = 0;
+        s.hdr->pass = 0;
+        s.hdr->poisoned = 0;
     }
 }
 
@@ -177,26 +197,19 @@ __global__ __launch_bounds__(SCAN_BLOCK) void scan_tiles_kernel(int64_t* tile_su
     if (threadIdx.x == SCAN_BLOCK - 1) tile_sum[nt] = s_part[SCAN_BLOCK - 1];  // grand total
 }
 
-// Numbers the set bits in ascending id order.  `scanned`: tile_sum already holds
-// exclusive offsets (+ total at [nt]); otherwise it holds raw sums and the block
-// adds up the tiles before it.
+// Numbers the set bits in ascending id order.
+// MODE 0: tile_sum holds raw sums and the block adds up the tiles before it, MODE 1: tile_sum
+// holds exclusive offsets (+ total at [nt]), MODE 2: no tile_sum - the tiles
+// exchange their counts through the state's descriptors inside this launch (a tile waits, bounded,
+// only for tiles with a smaller index, which the dispatcher started no later than itself).
+template <int MODE>
 __global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* tile_sum, int64_t nt,
-                                                       int scanned, int reset, int64_t* unique_out,
+                                                       int reset, int64_t* unique_out,
                                                        int64_t unique_capacity, int64_t* U_dev, uint32_t* stamp_ws) {
     __shared__ int64_t s_red[BLOCK / WAVE];
     __shared__ int32_t s_wave[BLOCK / WAVE];
+    __shared__ int s_gave[BLOCK / WAVE];
     const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
-    int64_t tile_off = 0;
-    if (scanned) {
-        tile_off = tile_sum[blockIdx.x];
-    } else {
-        int64_t part = 0;
-        for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += BLOCK) part += tile_sum[b];
-        for (int d = WAVE / 2; d > 0; d >>= 1) part += shfl_i64(part, lane ^ d);  // butterfly: all lanes hold the wave sum
-        if (lane == 0) s_red[wid] = part;
-        __syncthreads();
-        for (int q = 0; q < BLOCK / WAVE; ++q) tile_off += s_red[q];
-    }
     const int64_t base = eff_base(s, reset);
     const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
     uint64_t word = (w < s.words) ? s.bitmap[w] : 0ull;
@@ -213,10 +226,55 @@ __global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* t
         if (q < wid) wave_off += s_wave[q];
         block_total += s_wave[q];
     }
+    int64_t tile_off = 0;
+    int gave_up = 0;
+    if constexpr (MODE == 1) {
+        tile_off = tile_sum[blockIdx.x];
+    } else {
+        int64_t part = 0;
+        if constexpr (MODE == 0) {
+            for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += BLOCK) part += tile_sum[b];
+        } else {
+            const uint64_t tag = (uint64_t)eff_tag(s) << 32;
+            if (threadIdx.x == 0)
+                __hip_atomic_store(&s.desc[blockIdx.x], tag | (uint64_t)(uint32_t)block_total, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += BLOCK) {
+                uint64_t d;
+                int spins = 0;
+                while (((d = __hip_atomic_load(&s.desc[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) &
+                        0xFFFFFFFF00000000ull) != tag) {
+                    if (++spins > SPIN_LIMIT) {
+                        gave_up = 1;
+                        d = 0;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+                part += (int64_t)(d & 0xFFFFFFFFull);
+            }
+        }
+        for (int d = WAVE / 2; d > 0; d >>= 1) {   // butterfly: all lanes hold the wave sum
+            part += shfl_i64(part, lane ^ d);
+            gave_up |= __shfl(gave_up, lane ^ d);
+        }
+        if (lane == 0) {
+            s_red[wid] = part;
+            s_gave[wid] = gave_up;
+        }
+        __syncthreads();
+        gave_up = 0;
+        for (int q = 0; q < BLOCK / WAVE; ++q) {
+            tile_off += s_red[q];
+            gave_up |= s_gave[q];
+        }
+    }
     if (blockIdx.x == nt - 1 && threadIdx.x == 0) {  // publish the counts and the stamp of this call
         U_dev[0] = base + tile_off + block_total;
         stamp_ws[0] = eff_stamp(s, reset);
     }
+    // a tile that gave up waiting poisons the state: every later commit reports INT64_MAX ids
+    if (gave_up && threadIdx.x == 0) s.hdr->poisoned = 1;
     if (c == 0) return;
     int64_t local = base + tile_off + wave_off + (inc - c);
     const uint64_t stamp = (uint64_t)eff_stamp(s, reset) << 32;
@@ -241,7 +299,13 @@ __device__ __forceinline__ void commit(const State& s, int reset, int first, int
     if (first) U_dev[1] = base;
     if (!has_new) U_dev[0] = base;
     s.hdr->epoch = epoch;
-    s.hdr->id_count = U_dev[0];
+    s.hdr->pass = next_pass(s.hdr->pass);
+    if (s.hdr->poisoned) {        // numbers handed out by a pass that gave up are meaningless
+        s.hdr->id_count = 0;
+        U_dev[0] = INT64_MAX;
+    } else {
+        s.hdr->id_count = U_dev[0];
+    }
 }
 
 __global__ void commit_kernel(State s, int reset, int first, int has_new, int64_t* U_dev) {
@@ -289,7 +353,8 @@ using namespace sgl;
 
 extern "C" size_t sgl_remap_state_bytes(int64_t universe) {
     if (universe < 0) return 0;
-    return HEADER_BYTES + (size_t)universe * 8 + (size_t)ceil_div<int64_t>(universe, remap_byte_flags(universe) ? 8 : 64) * 8 + 8;
+    const int64_t words = ceil_div<int64_t>(universe, remap_byte_flags(universe) ? 8 : 64);
+    return HEADER_BYTES + (size_t)universe * 8 + (size_t)words * 8 + (size_t)ceil_div<int64_t>(words, TILE) * 8 + 8;
 }
 
 extern "C" int32_t sgl_remap_init(void* state, size_t state_bytes, int64_t universe, void* stream) {
@@ -388,16 +453,24 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
             hipLaunchKernelGGL(mark_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, sub, rst);
             SGL_LAUNCH_CHECK();
         }
-        hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
-        SGL_LAUNCH_CHECK();
-        const int scanned = nt > FUSED_SCAN_MAX ? 1 : 0;
-        if (scanned) {
-            hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, tile_sum, nt);
+        if (nt <= SINGLE_PASS_MAX) {
+            hipLaunchKernelGGL(assign_kernel<2>, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, rst,
+                               unique_out, unique_capacity, U_dev, stamp_ws);
+            SGL_LAUNCH_CHECK();
+        } else {
+            hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
+            SGL_LAUNCH_CHECK();
+            if (nt > FUSED_SCAN_MAX) {
+                hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, tile_sum, nt);
+                SGL_LAUNCH_CHECK();
+                hipLaunchKernelGGL(assign_kernel<1>, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, rst,
+                                   unique_out, unique_capacity, U_dev, stamp_ws);
+            } else {
+                hipLaunchKernelGGL(assign_kernel<0>, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, rst,
+                                   unique_out, unique_capacity, U_dev, stamp_ws);
+            }
             SGL_LAUNCH_CHECK();
         }
-        hipLaunchKernelGGL(assign_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, scanned, rst,
-                           unique_out, unique_capacity, U_dev, stamp_ws);
-        SGL_LAUNCH_CHECK();
         if (fold && r == n_run - 1) break;   // committed by the lookup launch below
         hipLaunchKernelGGL(commit_kernel, dim3(1), dim3(1), 0, st, s, rst, first, 1, U_dev);
         SGL_LAUNCH_CHECK();

@@ -18,6 +18,7 @@ import torch
 
 from ..graph.graph import Block
 from ..lib import _abi, hot_path
+from ..lib.driver import check_unique_total
 
 
 class MiniBatch:
@@ -34,6 +35,7 @@ class MiniBatch:
         p = self._p
         c = p.kr.counts.cpu().tolist()
         u_total = int(p.U[0].item())
+        check_unique_total(u_total)
         bad = sum(c[3 * l + 2] for l in range(p.layers))
         if bad:
             raise IndexError(f"sgl status {_abi.SGL_ERANGE}: {bad} sampling slots name a node outside [0,n)")

@@ -96,6 +96,13 @@ class HopResult:
         return self
 
 
+def check_unique_total(u_total):
+    """The id count of a unique_compact call is INT64_MAX when a numbering pass gave up waiting for
+    an earlier tile (bounded wait): the result is void and the remap state has to be re-initialised."""
+    if u_total == (1 << 63) - 1:
+        raise RuntimeError("unique_compact: a numbering pass gave up waiting; re-initialise the remap state")
+
+
 class HotPath:
     def __init__(self, lib, backend):
         self.lib, self.be = lib, backend
@@ -267,6 +274,7 @@ class HotPath:
         if not finalize:
             return out_arrays, unique, U
         u_total, u_before = be.tolist(U)
+        check_unique_total(u_total)
         return out_arrays, unique[:u_total], (u_total, u_before)
 
     # ------------------------------------------------------------- gather

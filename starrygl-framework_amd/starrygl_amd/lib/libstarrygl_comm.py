@@ -20,6 +20,7 @@ import threading
 import torch
 
 from . import _abi, hot_path
+from .driver import check_unique_total
 
 
 class TemporalRoot:
@@ -218,6 +219,7 @@ class CUDAGraph:
         vals = hp.be.tolist(live)
         kr.finalize(vals[: 3 * L])
         total, before = vals[3 * L], vals[3 * L + 1]
+        check_unique_total(total)
         self._unique = uniq[:total] if (reset or self._unique is None) else torch.cat([self._unique[:before],
                                                                                         uniq[before:total]])
         res = TemporalResult(TemporalRoot(local[0], roots.ts_ptr, roots.ts, roots.q_ptr, roots.q_eid),
