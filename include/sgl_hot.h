@@ -51,6 +51,15 @@ extern "C" {
 const char* sgl_last_error_string(void);
 int32_t     sgl_abi_version(void);
 
+/* Kernels whose blocks exchange totals inside one launch (the 2-hop sampler of
+ * small calls, the numbering pass of sgl_unique_compact on small universes)
+ * poll for an earlier block's descriptor at most `polls` times before they give
+ * up and poison the call's counts (see sgl_sample_khop, sgl_unique_compact).
+ * polls <= 0 restores the default (2^20).  No counterpart in the reference;
+ * meant for tests of that error path (a limit of 1 makes it reachable while
+ * every kernel still exits normally).  Returns the previous limit. */
+int32_t     sgl_set_wait_limit(int32_t polls);
+
 /* ------------------------------------------------------------------- T-CSR */
 /* Time-sorted CSR of one partition.  Row v occupies [row_ptr[v], row_ptr[v+1]);
  * inside a row edges ascend in (ts, eid).  Replaces the device arrays

@@ -45,6 +45,14 @@ static int32_t fail(int32_t code, const char* msg) {
 const char* sglo_last_error_string(void) { return g_err; }
 int32_t     sglo_abi_version(void) { return SGL_ABI_VERSION; }
 
+/* The oracle has no kernels that wait for each other: the limit is kept and returned only. */
+static int32_t g_wait_limit = 1 << 20;
+int32_t sglo_set_wait_limit(int32_t polls) {
+    int32_t prev = g_wait_limit;
+    g_wait_limit = polls > 0 ? polls : (1 << 20);
+    return prev;
+}
+
 /* Number of OpenMP threads the sampler loops use (1 = the scalar port).  The
  * reference runs its sampler loops under numba.prange
  * (prepare_sample.py:31,44,91) / at::parallel_for (graph.cpu.hpp:270,293). */

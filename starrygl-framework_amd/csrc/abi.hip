@@ -1,6 +1,8 @@
 // Status plumbing of libsgl_hot.so.
 #include <stdarg.h>
 
+#include <atomic>
+
 #include "common.hpp"
 
 namespace sgl {
@@ -18,7 +20,17 @@ int32_t fail(int32_t code, const char* fmt, ...) {
     return code;
 }
 
+namespace {
+std::atomic<int32_t> g_wait_limit{WAIT_LIMIT_DEFAULT};
+}
+
+int32_t wait_limit() { return g_wait_limit.load(std::memory_order_relaxed); }
+
 }  // namespace sgl
+
+extern "C" int32_t sgl_set_wait_limit(int32_t polls) {
+    return sgl::g_wait_limit.exchange(polls > 0 ? polls : sgl::WAIT_LIMIT_DEFAULT, std::memory_order_relaxed);
+}
 
 extern "C" const char* sgl_last_error_string(void) { return sgl::err_buf(); }
 extern "C" int32_t sgl_abi_version(void) { return SGL_ABI_VERSION; }

@@ -56,6 +56,10 @@ struct Arena {
 // "pending" set: one flag byte per id for universes up to REMAP_BYTE_FLAGS_MAX ids (set by plain
 // stores), one bit per id beyond (set by atomicOr; sweeping a byte per id would cost more there
 // than the atomics do).  unique.hip owns the state; the sampler only sets flags.
+// polls of one descriptor before a waiting lane gives up (sgl_set_wait_limit)
+constexpr int32_t WAIT_LIMIT_DEFAULT = 1 << 20;
+int32_t wait_limit();
+
 constexpr size_t REMAP_HEADER_BYTES = 256;
 constexpr int64_t REMAP_BYTE_FLAGS_MAX = 1ll << 24;
 inline bool remap_byte_flags(int64_t universe) { return universe <= REMAP_BYTE_FLAGS_MAX; }

@@ -642,7 +642,7 @@ int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf) {
 // all earlier slots: the block publishes its totals in a 64-bit descriptor right after its
 // searches and adds up the descriptors of all blocks before it as they appear (a block waits
 // only for blocks with a smaller index, which the dispatcher started no later than itself,
-// and for nothing those blocks wait for).  The wait is bounded: after FUSED_SPIN_LIMIT polls
+// and for nothing those blocks wait for).  The wait is bounded: after `spin_limit` polls
 // a lane gives up and counts[2] of hop 0 is poisoned, so every wave exits whatever happens.  Then the group writes
 // hop 1 (one edge per lane) and copies each hop-2 slot's edges with all its lanes.
 //
@@ -651,7 +651,6 @@ int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf) {
 constexpr int FG = 16;
 constexpr int FSPB = BLOCK / FG;
 constexpr int64_t FUSED_MAX_SLOTS = 32768;
-constexpr int FUSED_SPIN_LIMIT = 1 << 20;
 constexpr uint64_t ST_AGG = 1ull << 62, ST_MASK = 3ull << 62;
 constexpr int SH_E0 = 24, SH_BAD = 46;
 constexpr uint64_t M_E1 = (1ull << 24) - 1, M_E0 = (1ull << 22) - 1, M_BAD = (1ull << 16) - 1;
@@ -666,6 +665,7 @@ struct Fused2Args {
     int64_t* nbr_dt1;
     int64_t* counts1;
     unsigned long long* desc;   // [gridDim] zeroed by fused_clear_kernel
+    int32_t spin_limit;         // polls of one descriptor before a lane gives up
 };
 
 __global__ void fused_clear_kernel(unsigned long long* desc, int n, int64_t* counts1, int64_t* counts1_b) {
@@ -838,7 +838,7 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
         uint64_t d;
         int spins = 0;
         while (((d = __hip_atomic_load(&f.desc[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) & ST_MASK) == 0) {
-            if (++spins > FUSED_SPIN_LIMIT) {
+            if (++spins > f.spin_limit) {
                 gave_up = 1;
                 break;
             }
@@ -1094,6 +1094,7 @@ Fused2Args fused2_args(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, cons
     f.nbr1 = outs[1].neighbors; f.nbr_ts1 = outs[1].neighbors_ts; f.nbr_eid1 = outs[1].neighbors_eid;
     f.nbr_dt1 = outs[1].neighbors_dt; f.counts1 = outs[1].counts;
     f.desc = desc;
+    f.spin_limit = wait_limit();
     return f;
 }
 

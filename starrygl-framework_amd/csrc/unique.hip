@@ -43,7 +43,6 @@ constexpr int SCAN_BLOCK = 1024;
 constexpr int MAX_GRID = 2048;         // grid cap of the per-id kernels (grid-stride loops)
 constexpr int FUSED_SCAN_MAX = 4096;   // up to this many tiles assign sums the preceding tiles itself
 constexpr int SINGLE_PASS_MAX = 2048;  // up to this many tiles the counts are exchanged inside the assign launch
-constexpr int SPIN_LIMIT = 1 << 20;    // polls of one descriptor before a lane gives up (the result is then poisoned)
 constexpr size_t HEADER_BYTES = REMAP_HEADER_BYTES;
 
 struct Header {
@@ -205,7 +204,8 @@ __global__ __launch_bounds__(SCAN_BLOCK) void scan_tiles_kernel(int64_t* tile_su
 template <int MODE>
 __global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* tile_sum, int64_t nt,
                                                        int reset, int64_t* unique_out,
-                                                       int64_t unique_capacity, int64_t* U_dev, uint32_t* stamp_ws) {
+                                                       int64_t unique_capacity, int64_t* U_dev, uint32_t* stamp_ws,
+                                                       int32_t spin_limit) {
     __shared__ int64_t s_red[BLOCK / WAVE];
     __shared__ int32_t s_wave[BLOCK / WAVE];
     __shared__ int s_gave[BLOCK / WAVE];
@@ -244,7 +244,7 @@ __global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* t
                 int spins = 0;
                 while (((d = __hip_atomic_load(&s.desc[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) &
                         0xFFFFFFFF00000000ull) != tag) {
-                    if (++spins > SPIN_LIMIT) {
+                    if (++spins > spin_limit) {
                         gave_up = 1;
                         d = 0;
                         break;
@@ -455,7 +455,7 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
         }
         if (nt <= SINGLE_PASS_MAX) {
             hipLaunchKernelGGL(assign_kernel<2>, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, rst,
-                               unique_out, unique_capacity, U_dev, stamp_ws);
+                               unique_out, unique_capacity, U_dev, stamp_ws, wait_limit());
             SGL_LAUNCH_CHECK();
         } else {
             hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
@@ -464,10 +464,10 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
                 hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, tile_sum, nt);
                 SGL_LAUNCH_CHECK();
                 hipLaunchKernelGGL(assign_kernel<1>, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, rst,
-                                   unique_out, unique_capacity, U_dev, stamp_ws);
+                                   unique_out, unique_capacity, U_dev, stamp_ws, wait_limit());
             } else {
                 hipLaunchKernelGGL(assign_kernel<0>, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, rst,
-                                   unique_out, unique_capacity, U_dev, stamp_ws);
+                                   unique_out, unique_capacity, U_dev, stamp_ws, wait_limit());
             }
             SGL_LAUNCH_CHECK();
         }

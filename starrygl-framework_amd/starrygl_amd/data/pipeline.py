@@ -18,7 +18,7 @@ import torch
 
 from ..graph.graph import Block
 from ..lib import _abi, hot_path
-from ..lib.driver import check_unique_total
+from ..lib.driver import check_sample_bad, check_unique_total
 
 
 class MiniBatch:
@@ -36,9 +36,8 @@ class MiniBatch:
         c = p.kr.counts.cpu().tolist()
         u_total = int(p.U[0].item())
         check_unique_total(u_total)
-        bad = sum(c[3 * l + 2] for l in range(p.layers))
-        if bad:
-            raise IndexError(f"sgl status {_abi.SGL_ERANGE}: {bad} sampling slots name a node outside [0,n)")
+        check_sample_bad(max(c[3 * l + 2] for l in range(p.layers)))
+        check_sample_bad(sum(c[3 * l + 2] for l in range(p.layers)))
         self.S = [c[3 * l] for l in range(p.layers)]
         self.E = [c[3 * l + 1] for l in range(p.layers)]
         self.num_unique = u_total

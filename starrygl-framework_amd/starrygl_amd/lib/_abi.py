@@ -58,6 +58,7 @@ P = C.POINTER
 PROTOTYPES = {
     "last_error_string": (C.c_char_p, []),
     "abi_version": (i32, []),
+    "set_wait_limit": (i32, [i32]),
     "tcsr_build_workspace_bytes": (sz, [i64, i64]),
     "tcsr_build": (i32, [i64, i64, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]),
     "tcsr_validate": (i32, [P(TCSR), vp, sz, vp]),

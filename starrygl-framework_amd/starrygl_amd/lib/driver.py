@@ -86,14 +86,22 @@ class HopResult:
         self.S = self.E = None
 
     def finalize(self, S, E, bad=0):
-        if bad:
-            raise IndexError(f"sgl status {_abi.SGL_ERANGE}: {bad} sampling slots name a node outside [0,n)")
+        check_sample_bad(bad)
         self.S, self.E = int(S), int(E)
         self.root_start_ptr = self.root_start_ptr[: self.S + 1]
         self.root_end_ptr = self.root_end_ptr[: self.S + 1]
         for f in self.FIELDS:
             setattr(self, f, getattr(self, f)[: self.E])
         return self
+
+
+def check_sample_bad(bad):
+    """counts[2] of a hop: slots whose node lies outside [0,n); INT64_MAX when a block of the
+    single-launch 2-hop sampler gave up its bounded wait (the call's outputs are void)."""
+    if bad >= (1 << 63) - 1:
+        raise RuntimeError("sample_khop: a block gave up waiting for the edge totals of an earlier block")
+    if bad:
+        raise IndexError(f"sgl status {_abi.SGL_ERANGE}: {bad} sampling slots name a node outside [0,n)")
 
 
 def check_unique_total(u_total):
@@ -153,6 +161,11 @@ class HotPath:
         return SampleParams(int(sample_type), int(fanout), int(allowed_offset),
                             int(bool(equal_root_time)), int(bool(keep_root_time)),
                             int(bool(replace)), int(hop), int(seed) & (2**64 - 1), None, 0)
+
+    def set_wait_limit(self, polls):
+        """Polls before a block that waits for another block's totals gives up (<= 0: default);
+        returns the previous limit.  For tests of that error path."""
+        return int(self.lib.set_wait_limit(int(polls)))
 
     def marking(self, p, state):
         """Copy of the sampling parameters `p` that makes the sampler record every id it
