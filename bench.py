@@ -687,7 +687,8 @@ def main():
         cpu = {"value": round(edges_cpu / t_cpu, 1), "unit": "sampled edges/s (2-hop recent 10x10)", "cores": threads,
                "kind": "port", "sample": f"{nb_cpu} batches of {S0} roots, {edges_cpu} edges in {t_cpu:.2f}s",
                "cpu_model": cpu_model, "one_thread_value": round(edges_one / t_one, 1),
-               "gpu_over_cpu_sampler": round(stages["sample_recent_2hop"]["edges_per_s"] / (edges_cpu / t_cpu), 1)}
+               "gpu_over_cpu_sampler": round(stages["sample_recent_2hop"]["edges_per_s"] / (edges_cpu / t_cpu), 1),
+               "gpu_over_cpu_one_thread": round(stages["sample_recent_2hop"]["edges_per_s"] / (edges_one / t_one), 1)}
 
     extra = {}
     has_edge_feat = edge_cache is not None
