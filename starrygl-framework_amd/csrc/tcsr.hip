@@ -81,15 +81,16 @@ __global__ __launch_bounds__(BLOCK) void stats_kernel(int64_t n, int64_t m, cons
                                                       const int64_t* __restrict__ eid, BuildStats* st) {
     __shared__ long long s_min[BLOCK / WAVE], s_max[BLOCK / WAVE], s_emax[BLOCK / WAVE];
     __shared__ int32_t s_flags[BLOCK / WAVE];
-    const int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
     long long tmin = INT64_MAX, tmax = INT64_MIN, emax = 0;
     int32_t f = 0;
-    if (i < m) {
+    // grid-stride: a block ends with four atomics on the same four words, so there must be few blocks
+    for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < m; i += (int64_t)gridDim.x * BLOCK) {
         const int64_t s = src[i], d = dst[i], t = ts[i], e = eid ? eid[i] : i;
         if (s < 0 || s >= n || d < 0 || d >= n) f |= 1;
         if (e < 0) f |= 16;
-        tmin = tmax = t;
-        emax = e;
+        tmin = t < tmin ? t : tmin;
+        tmax = t > tmax ? t : tmax;
+        emax = e > emax ? e : emax;
         if (i > 0) {
             const int64_t ps = src[i - 1], pt = ts[i - 1], pe = eid ? eid[i - 1] : i - 1;
             const bool te_le = (pt < t) || (pt == t && pe <= e);
@@ -198,7 +199,7 @@ extern "C" int32_t sgl_tcsr_build(int64_t n, int64_t m, const int64_t* src, cons
     hipLaunchKernelGGL(stats_init_kernel, dim3(1), dim3(1), 0, st, d_stats);
     SGL_LAUNCH_CHECK();
     if (m > 0) {
-        hipLaunchKernelGGL(stats_kernel, dim3(eb), dim3(BLOCK), 0, st, n, m, src, dst, ts, eid, d_stats);
+        hipLaunchKernelGGL(stats_kernel, dim3(eb < 4096u ? eb : 4096u), dim3(BLOCK), 0, st, n, m, src, dst, ts, eid, d_stats);
         SGL_LAUNCH_CHECK();
     }
     BuildStats h;
