@@ -302,3 +302,32 @@ def test_segment_max_and_mailbox(oracle, hot):
     idx = torch.tensor([7, 7, 9]).cuda()
     mb.set_mailbox_local(idx, torch.arange(60, dtype=torch.float32).reshape(3, 20).cuda(), torch.tensor([1.0, 5.0, 2.0]).cuda(), "max")
     assert np_of(mb.mailbox)[7, 0, 0] == 20 and np_of(mb.mailbox_ts)[7, 0] == 5 and np_of(mb.mailbox)[9, 0, 0] == 40
+
+
+@pytest.mark.parametrize("n,t_max", [(1, 50), (1023, 400), (1025, 400), (5000, 3000)])
+def test_seeds_heavy_windows_and_tile_boundaries(oracle, hot, n, t_max):
+    """Seed extraction against the oracle where one node holds most of every window (walked by a whole
+    wavefront, 64 events per step), timestamps repeat a lot, and the candidate count sits on either side
+    of the 1024-candidate tile; windows from empty to the whole history, chunk lists in any order."""
+    rng = np.random.default_rng(n)
+    m, C = 40_000, 5
+    src = rng.integers(0, n, m).astype(np.int64)
+    src[rng.random(m) < 0.6] = n // 2                  # the hub
+    dst = rng.integers(0, n, m).astype(np.int64)
+    ts = np.sort(rng.integers(0, t_max, m)).astype(np.int64)   # m >> t_max: long runs of equal timestamps
+    eid = np.arange(m, dtype=np.int64)
+    hg = host_graph(oracle, n, src, dst, ts, eid)
+    from util import mirror_graph
+    dg = mirror_graph(hot, hg)
+    chunk_of = rng.integers(0, C, n).astype(np.int64)
+    cp, cn = oracle.chunk_index(n, C, chunk_of)
+    dcp, dcn = hot.chunk_index(n, C, to_dev(hot, chunk_of))
+    assert np.array_equal(np_of(dcp), cp) and np.array_equal(np_of(dcn), cn)
+    for chunks in ([0, 1, 2, 3, 4], [3, 0], [int(chunk_of[n // 2])], []):
+        ch = np.asarray(chunks, dtype=np.int64)
+        off = np.concatenate([[0], np.cumsum(cp[ch + 1] - cp[ch])]).astype(np.int64)
+        for t0, t1 in ((0, t_max), (t_max // 3, t_max // 3 + 1), (t_max // 2, t_max // 2 + 7), (5, 5), (t_max, t_max + 9)):
+            want = oracle.seeds(hg, cp, cn, ch, off, int(off[-1]), t0, t1)
+            got = hot.seeds(dg, dcp, dcn, to_dev(hot, ch), to_dev(hot, off), int(off[-1]), t0, t1)
+            for f, a, b in zip(("roots", "ts_ptr", "ts", "q_ptr", "q_eid"), got, want):
+                assert np.array_equal(np_of(a), b), (f, chunks, t0, t1)
