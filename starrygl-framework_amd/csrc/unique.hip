@@ -16,7 +16,12 @@
 //              last group's commit is done by one thread of the lookup launch);
 //   then one lookup launch rewrites every input array through the table.
 //   No sort, no hash probing; the result is deterministic.
-//   Up to SINGLE_PASS_MAX tiles, reduce and assign are one launch: every tile
+//   Grouped mode (per array: the ids new to the epoch, ascending, appended) is
+//   one numbering pass as well when the flags are bytes: array g sets flags in
+//   plane g of the pending set, an id belongs to the first plane that has it,
+//   and the offsets of all (group, tile) buckets are one exclusive scan over
+//   the group-major counts.  With a bitmap the arrays are numbered one by one.
+//   Up to SINGLE_PASS_MAX tiles, reduce and assign of the sorted mode are one launch: every tile
 //   publishes its count in a descriptor kept in the state (tagged with the
 //   state's pass counter, so descriptors never need clearing) and adds up the
 //   descriptors of the tiles before it as they appear.
@@ -59,6 +64,7 @@ struct State {
     uint64_t* desc;     // one descriptor per tile of flag words: pass tag << 32 | flags set in the tile
     int64_t universe, words;
     int32_t bytes;      // 1: a flag byte per id (8 ids per word), 0: a bit per id (64 ids per word)
+    int32_t planes;     // copies of the pending set (one per array of a grouped call)
 };
 
 State carve(void* state, int64_t universe) {
@@ -69,8 +75,9 @@ State carve(void* state, int64_t universe) {
     s.words = ceil_div<int64_t>(universe, s.bytes ? 8 : 64);
     s.hdr = reinterpret_cast<Header*>(p);
     s.table = reinterpret_cast<uint64_t*>(p + HEADER_BYTES);
-    s.bitmap = s.table + universe;
-    s.desc = s.bitmap + s.words;
+    s.bitmap = s.table + universe;           // s.planes planes of s.words words each; plane 0 first
+    s.planes = s.bytes ? MAXG : 1;           // (a bitmap state numbers the arrays of a grouped call one by one)
+    s.desc = s.bitmap + (int64_t)s.planes * s.words;
     return s;
 }
 
@@ -109,7 +116,7 @@ __global__ void init_state_kernel(State s) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = t; i < s.universe; i += stride) s.table[i] = 0;
-    for (int64_t i = t; i < s.words; i += stride) s.bitmap[i] = 0;
+    for (int64_t i = t; i < (int64_t)s.planes * s.words; i += stride) s.bitmap[i] = 0;
     for (int64_t i = t; i < ceil_div<int64_t>(s.words, TILE); i += stride) s.desc[i] = 0;
     if (t == 0) {
         s.hdr->epoch = 1;
@@ -126,7 +133,7 @@ __global__ void init_state_kernel(State s) {
 // sweeping a byte per id in reduce/assign costs more than the atomics.  Testing
 // the flag first, or folding the block's ids through an LDS hash set first,
 // lengthens the dependent chain and runs 2-3x slower in both layouts.)
-__global__ __launch_bounds__(BLOCK) void mark_kernel(State s, Arrays a, int reset) {
+__global__ __launch_bounds__(BLOCK) void mark_kernel(State s, Arrays a, int reset, int grouped) {
     const uint32_t stamp = eff_stamp(s, reset);
     // Index i is processed for every array at once (loads of the different arrays are
     // independent and issue together: one dependent chain id -> table -> atomic per
@@ -151,8 +158,8 @@ __global__ __launch_bounds__(BLOCK) void mark_kernel(State s, Arrays a, int rese
         }
 #pragma unroll
         for (int g = 0; g < MAXG; ++g)
-            if ((uint32_t)(e[g] >> 32) != stamp)
-                remap_set_pending(s.bitmap, s.bytes, id[g]);
+            if ((uint32_t)(e[g] >> 32) != stamp)      // grouped: array g has plane g of the pending set
+                remap_set_pending(s.bitmap + (grouped ? (int64_t)g * s.words : 0), s.bytes, id[g]);
     }
 }
 
@@ -291,6 +298,110 @@ __global__ __launch_bounds__(BLOCK) void assign_kernel(State s, const int64_t* t
     s.bitmap[w] = 0;
 }
 
+// Grouped mode, counting: tile_cnt[g * nt + tile] = ids of the tile whose first plane is g.
+__global__ __launch_bounds__(BLOCK) void reduce_groups_kernel(State s, int G, int64_t nt, int64_t* tile_cnt) {
+    __shared__ int32_t s_w[MAXG][BLOCK / WAVE];
+    const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
+    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    uint64_t seen = 0;
+#pragma unroll
+    for (int g = 0; g < MAXG; ++g) {
+        int32_t c = 0;
+        if (g < G) {
+            const uint64_t m = (w < s.words) ? s.bitmap[(int64_t)g * s.words + w] : 0ull;
+            c = __popcll(m & ~seen);
+            seen |= m;
+        }
+        for (int d = WAVE / 2; d > 0; d >>= 1) c += __shfl_down(c, d);
+        if (lane == 0) s_w[g][wid] = c;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < G) {
+        int64_t sum = 0;
+        for (int q = 0; q < BLOCK / WAVE; ++q) sum += s_w[threadIdx.x][q];
+        tile_cnt[(int64_t)threadIdx.x * nt + blockIdx.x] = sum;
+    }
+}
+
+// Grouped mode, numbering.  The local id of an id of group g in tile t is
+//   base + (ids of groups < g, all tiles) + (ids of group g, tiles < t) + rank inside the tile,
+// and the two middle terms are the exclusive prefix of tile_cnt at g * nt + t (group-major order).
+// `scanned`: tile_cnt already holds that prefix (+ the grand total at [G * nt]); otherwise raw counts.
+__global__ __launch_bounds__(BLOCK) void assign_groups_kernel(State s, int G, const int64_t* tile_cnt, int64_t nt,
+                                                              int scanned, int reset, int64_t* unique_out,
+                                                              int64_t unique_capacity, int64_t* U_dev, uint32_t* stamp_ws) {
+    __shared__ int64_t s_red[MAXG + 1][BLOCK / WAVE];
+    __shared__ int32_t s_wave[BLOCK / WAVE];
+    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    const int64_t flat = (int64_t)G * nt;
+    int64_t off[MAXG], total = 0;
+    if (scanned) {
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) off[g] = g < G ? tile_cnt[(int64_t)g * nt + blockIdx.x] : 0;
+        total = tile_cnt[flat];
+    } else {
+        int64_t part[MAXG + 1];
+#pragma unroll
+        for (int g = 0; g <= MAXG; ++g) part[g] = 0;
+        for (int64_t i = threadIdx.x; i < flat; i += BLOCK) {
+            const int64_t v = tile_cnt[i];
+            part[MAXG] += v;
+#pragma unroll
+            for (int g = 0; g < MAXG; ++g)
+                if (g < G && i < (int64_t)g * nt + blockIdx.x) part[g] += v;
+        }
+#pragma unroll
+        for (int g = 0; g <= MAXG; ++g) {
+            int64_t x = part[g];
+            for (int d = WAVE / 2; d > 0; d >>= 1) x += shfl_i64(x, lane ^ d);
+            if (lane == 0) s_red[g][wid] = x;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) {
+            off[g] = 0;
+            for (int q = 0; q < BLOCK / WAVE; ++q) off[g] += s_red[g][q];
+        }
+        for (int q = 0; q < BLOCK / WAVE; ++q) total += s_red[MAXG][q];
+    }
+    const int64_t base = eff_base(s, reset);
+    if (blockIdx.x == nt - 1 && threadIdx.x == 0) {  // publish the counts and the stamp of this call
+        U_dev[0] = base + total;
+        stamp_ws[0] = eff_stamp(s, reset);
+    }
+    const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
+    const uint64_t stamp = (uint64_t)eff_stamp(s, reset) << 32;
+    const int64_t id0 = w * (s.bytes ? 8 : 64);
+    const int shift = s.bytes ? 3 : 0;
+    uint64_t seen = 0;
+    for (int g = 0; g < G; ++g) {
+        const uint64_t m = (w < s.words) ? s.bitmap[(int64_t)g * s.words + w] : 0ull;
+        uint64_t word = m & ~seen;
+        seen |= m;
+        const int32_t c = __popcll(word);
+        int32_t inc = c;
+        for (int d = 1; d < WAVE; d <<= 1) {
+            const int32_t x = __shfl_up(inc, d);
+            if (lane >= d) inc += x;
+        }
+        __syncthreads();
+        if (lane == WAVE - 1) s_wave[wid] = inc;
+        __syncthreads();
+        int32_t wave_off = 0;
+        for (int q = 0; q < wid; ++q) wave_off += s_wave[q];
+        int64_t local = base + off[g] + wave_off + (inc - c);
+        while (word) {
+            const int bit = __ffsll((unsigned long long)word) - 1;
+            word &= word - 1;
+            const int64_t id = id0 + (bit >> shift);
+            s.table[id] = stamp | (uint64_t)(uint32_t)local;
+            if (local < unique_capacity) unique_out[local] = id;
+            ++local;
+        }
+        if (m != 0) s.bitmap[(int64_t)g * s.words + w] = 0;
+    }
+}
+
 // Makes the call's epoch and id count the committed ones.  `first`: U_dev[1]
 // (ids numbered before this call) is recorded.  `has_new` == 0: no assign ran.
 __device__ __forceinline__ void commit(const State& s, int reset, int first, int has_new, int64_t* U_dev) {
@@ -343,7 +454,7 @@ __global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a, int fo
 
 size_t dense_workspace_bytes(int64_t universe) {
     const int64_t words = ceil_div<int64_t>(universe, remap_byte_flags(universe) ? 8 : 64);
-    return align_up((size_t)(ceil_div<int64_t>(words, TILE) + 2) * 8) + 512;
+    return align_up((size_t)(MAXG * ceil_div<int64_t>(words, TILE) + 2) * 8) + 512;
 }
 
 }  // namespace
@@ -354,7 +465,8 @@ using namespace sgl;
 extern "C" size_t sgl_remap_state_bytes(int64_t universe) {
     if (universe < 0) return 0;
     const int64_t words = ceil_div<int64_t>(universe, remap_byte_flags(universe) ? 8 : 64);
-    return HEADER_BYTES + (size_t)universe * 8 + (size_t)words * 8 + (size_t)ceil_div<int64_t>(words, TILE) * 8 + 8;
+    const size_t planes = remap_byte_flags(universe) ? MAXG : 1;
+    return HEADER_BYTES + (size_t)universe * 8 + planes * (size_t)words * 8 + (size_t)ceil_div<int64_t>(words, TILE) * 8 + 8;
 }
 
 extern "C" int32_t sgl_remap_init(void* state, size_t state_bytes, int64_t universe, void* stream) {
@@ -422,15 +534,21 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
     const int64_t total = all.start[MAXG];
     if (ceil_div<int64_t>(total, BLOCK) > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "unique_compact: too many ids");
 
-    int64_t* tile_sum = ar.take<int64_t>(nt + 2);
+    // Grouped mode over a byte-flag state: one numbering pass for all arrays (array g marks plane g).
+    // Over a bitmap state the arrays are numbered one after the other: there the marks are atomics,
+    // and an id that an earlier array has already numbered is skipped by the later array's marking
+    // pass - popular ids come back thousands of times in the deeper hops, and that many atomics on
+    // one word cost more (906 us against 262 us for 14.7M ids) than the extra passes.
+    const bool planes = mode == SGL_UNIQUE_GROUPED && s.bytes;
+    int64_t* tile_sum = ar.take<int64_t>((planes ? (int64_t)G : 1) * nt + 2);
     uint32_t* stamp_ws = ar.take<uint32_t>(4);
     if (!ar.ok()) return fail(SGL_ENOMEM, "unique_compact: workspace too small");
-    const int n_groups = (mode == SGL_UNIQUE_SORTED) ? (G > 0 ? 1 : 0) : G;
+    const int n_groups = (mode == SGL_UNIQUE_SORTED || planes) ? (G > 0 ? 1 : 0) : G;
     // groups that have anything to number; the commit of the last one is folded into the
     // lookup launch (one launch less per call), the others commit with a kernel of their own
     int runnable[MAXG], n_run = 0;
     for (int grp = 0; grp < n_groups; ++grp) {
-        const int64_t sub_total = (mode == SGL_UNIQUE_GROUPED) ? all.len_max[grp] : total;
+        const int64_t sub_total = (mode == SGL_UNIQUE_GROUPED && !planes) ? all.len_max[grp] : total;
         if (sub_total > 0 && universe > 0) runnable[n_run++] = grp;
     }
     const bool fold = n_run > 0 && total > 0;
@@ -438,7 +556,7 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
     for (int r = 0; r < n_run; ++r) {
         const int grp = runnable[r];
         Arrays sub = all;
-        if (mode == SGL_UNIQUE_GROUPED) {  // only array `grp`
+        if (mode == SGL_UNIQUE_GROUPED && !planes) {  // only array `grp`
             sub.G = 1;
             sub.ids[0] = all.ids[grp]; sub.out[0] = all.out[grp];
             sub.len_dev[0] = all.len_dev[grp]; sub.len_max[0] = all.len_max[grp];
@@ -450,10 +568,21 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
         int64_t mb = ceil_div<int64_t>(longest, BLOCK);
         if (mb > MAX_GRID) mb = MAX_GRID;
         if (!premarked) {
-            hipLaunchKernelGGL(mark_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, sub, rst);
+            hipLaunchKernelGGL(mark_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, sub, rst, planes ? 1 : 0);
             SGL_LAUNCH_CHECK();
         }
-        if (nt <= SINGLE_PASS_MAX) {
+        if (planes) {
+            hipLaunchKernelGGL(reduce_groups_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, (int)G, nt, tile_sum);
+            SGL_LAUNCH_CHECK();
+            const int scanned = (int64_t)G * nt > FUSED_SCAN_MAX ? 1 : 0;
+            if (scanned) {
+                hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, tile_sum, (int64_t)G * nt);
+                SGL_LAUNCH_CHECK();
+            }
+            hipLaunchKernelGGL(assign_groups_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, (int)G, tile_sum, nt, scanned,
+                               rst, unique_out, unique_capacity, U_dev, stamp_ws);
+            SGL_LAUNCH_CHECK();
+        } else if (nt <= SINGLE_PASS_MAX) {
             hipLaunchKernelGGL(assign_kernel<2>, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, rst,
                                unique_out, unique_capacity, U_dev, stamp_ws, wait_limit());
             SGL_LAUNCH_CHECK();

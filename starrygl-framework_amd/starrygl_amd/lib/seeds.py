@@ -30,10 +30,22 @@ def _candidates(graph, chunks):
     C = chunk_ptr_h.shape[0] - 1
     if chunks_h.size and (chunks_h.min() < 0 or chunks_h.max() >= C):
         raise IndexError("chunk id outside [0, chunk_size)")
+    # training loops ask for the same few chunk lists over and over: their device copies are kept
+    # (two small host-to-device copies cost more host time than the whole query costs GPU time)
+    cache = graph.__dict__.setdefault("_cand_cache", {})
+    key = chunks_h.tobytes()
+    hit = cache.get(key)
+    if hit is not None:
+        return hit
     sizes = chunk_ptr_h[chunks_h + 1] - chunk_ptr_h[chunks_h] if chunks_h.size else np.zeros(0, np.int64)
     cand_off = np.zeros(chunks_h.size + 1, dtype=np.int64)
     np.cumsum(sizes, out=cand_off[1:])
-    return torch.from_numpy(chunks_h.copy()).to(dev), torch.from_numpy(cand_off).to(dev), int(cand_off[-1])
+    packed = torch.from_numpy(np.concatenate([chunks_h, cand_off])).to(dev)      # one copy for both
+    out = (packed[: chunks_h.size], packed[chunks_h.size:], int(cand_off[-1]))
+    if len(cache) >= 64:
+        cache.clear()
+    cache[key] = out
+    return out
 
 
 def seeds_in_chunks(graph, chunks, t_begin, t_end, full_timestamps=False):
