@@ -77,9 +77,18 @@ class pyGraph:
     def slice_by_chunk_ts(self, chunk_list: torch.Tensor, time_begin: float, time_end: float):
         return self.g.slice_by_chunk_ts(chunk_list, time_begin, time_end)
 
-    def sample_src_in_chunks_khop(self, postive_root, negative_root, k: int, layers: int, allowed_offset=-1,
+    def sample_src_in_chunks_khop(self, postive_root, negative_root, k=None, layers=None, allowed_offset=-1,
                                   equal_root_time=False, keep_root_time=False, sample_type="recent"):
-        """Bound signature of the native method (export.cu:194-201)."""
+        """Bound signature of the native method (export.cu:194-201).  The reference's wrapper of the same
+        name passes (chunk_list, k, layers, time_begin, time_end) to it (graph.py:124-135), which the
+        native method does not accept; that form is served here as what it spells: the seeds of the
+        chunks in [time_begin, time_end), then k most recent neighbours per hop (`layers`: a hop count
+        or one entry per hop), no negatives."""
+        if isinstance(postive_root, torch.Tensor):
+            chunk_list, fanout, hops, time_begin, time_end = postive_root, negative_root, k, layers, allowed_offset
+            hops = len(hops) if isinstance(hops, (list, tuple)) else int(hops)
+            roots = self.g.get_seeds_in_chunks(chunk_list, int(time_begin), int(time_end))
+            return self.g.sample_src_in_chunks_khop(roots, None, int(fanout), hops, -1, False, False, "recent")
         return self.g.sample_src_in_chunks_khop(postive_root, negative_root, k, layers, allowed_offset,
                                                 equal_root_time, keep_root_time, sample_type)
 

@@ -143,6 +143,16 @@ def test_direct_khop_and_errors(oracle, world):
         pg.async_sample(0, 1, torch.tensor([0]), dict(sample_type="recent", layers=1), {}, op="r")
     with pytest.raises(TypeError):
         pg.async_sample(0, 1, [0], pol)
+    # the wrapper's own call form (graph.py:124-135): chunk list, fanout, hops, window
+    res = pg.sample_src_in_chunks_khop(torch.tensor([2, 6]), 4, [4, 4], 50_000, 51_000)
+    ch = np.array([2, 6], dtype=np.int64)
+    off = np.concatenate([[0], np.cumsum(world["cp"][ch + 1] - world["cp"][ch])]).astype(np.int64)
+    r, tp, t, _, _ = oracle.seeds(world["hg"], world["cp"], world["cn"], ch, off, int(off[-1]), 50_000, 51_000)
+    e = np.zeros(0, np.int64)
+    want = oracle.sample_khop(world["hg"], r, tp, t, e, e, 2, oracle.params("recent", 4))
+    assert len(res.neighbors_list) == 2 and res.roots.root_num == r.shape[0] > 0
+    for layer, h in zip(res.neighbors_list, want.hops):
+        assert np.array_equal(np_of(layer.neighbors), h.neighbors) and np.array_equal(np_of(layer.neighbors_eid), h.neighbors_eid)
 
 
 @pytest.mark.parametrize("full", [False, True])
