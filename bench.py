@@ -115,7 +115,8 @@ def workload_cache_stress(hot, torch, np, synth, rows=50_000_000, dim=128, n_req
     return res
 
 
-def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=2000, k=10, remote=0.30, steps=30):
+def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=2000, k=10, remote=0.30, steps=30,
+                      streams=None):
     """configs[4]: one GPU's share of a partitioned TGN step: 1-hop recent-10 sampling, gather of
     memory (+ int64 last update), node and edge features, cos time encoding to 100 dims.  30 % of
     the node rows (memory, node features) are served from pinned host memory; edge features are
@@ -163,59 +164,80 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     ts_ptr = D(bt[0][1])
     S0 = 3 * B
     p = hot.params("recent", k)
-    kr = hot.khop_buffers(S0, 1, k)
-    state = hot.remap_state(n)
-    local = [hot.be.empty(S0), hot.be.empty(S0 * k)]
-    ubuf, U = hot.be.empty(S0 + S0 * k), hot.be.zeros(2)
     S0_dev = D(np.array([S0], dtype=np.int64))
-    o_mem = torch.empty((S0 + S0 * k, 100), device=dev)
-    o_ts = hot.be.empty(S0 + S0 * k)
-    o_nf = torch.empty((S0 + S0 * k, 100), device=dev)
-    o_ef = torch.empty((S0 * k, 172), device=dev)
     w = torch.from_numpy((1.0 / 10 ** np.linspace(0, 9, 100, dtype=np.float32)).astype(np.float32)).to(dev)
     bias = torch.zeros(100, device=dev)
-    o_te = torch.empty((S0 * k, 100), device=dev)
-    s_in = [torch.empty_like(x[0]) for x in (roots, root_ts, neg, neg_ts)]
-    hot._workspace(hot.lib.unique_workspace_bytes(n, 2, (_abi.i64 * 2)(S0, S0 * k)))
-    E = kr.hops[0].counts[1:2]
-    acc = torch.zeros(2, dtype=torch.int64, device=dev)
-    plan = hot.gather_plan([(c_mem, ubuf, o_mem, o_ts, U[0:1]), (c_nf, ubuf, o_nf, None, U[0:1]),
-                            (c_ef, kr.hops[0].neighbors_eid, o_ef, None, E)])
+    packed = torch.cat([roots, root_ts, neg, neg_ts], dim=1).contiguous()
 
-    def body():
-        hot.sample_khop(dg, s_in[0], ts_ptr, s_in[1], s_in[2], s_in[3], 1, p, finalize=False, out=kr)
-        hot.unique_compact([kr.slot_node0, kr.hops[0].neighbors], _abi.UNIQUE_SORTED, state, True,
-                           lens_dev=[S0_dev, E], out_arrays=local, finalize=False, unique_out=ubuf, U_out=U)
-        hot.gather_multi(plan)
-        hot.time_encode(kr.hops[0].neighbors_dt, w, bias, out=o_te, N_dev=E)
-        acc[0:1].add_(E); acc[1:2].add_(U[0:1])
+    def make_pipeline(stream):
+        """One copy of the step: own buffers, remap state, HIP graph, on `stream`."""
+        P = type("Pipeline", (), {})()
+        P.kr = hot.khop_buffers(S0, 1, k)
+        P.state = hot.remap_state(n)
+        P.local = [hot.be.empty(S0), hot.be.empty(S0 * k)]
+        P.ubuf, P.U = hot.be.empty(S0 + S0 * k), hot.be.zeros(2)
+        P.o_mem = torch.empty((S0 + S0 * k, 100), device=dev)
+        P.o_ts = hot.be.empty(S0 + S0 * k)
+        P.o_nf = torch.empty((S0 + S0 * k, 100), device=dev)
+        P.o_ef = torch.empty((S0 * k, 172), device=dev)
+        P.o_te = torch.empty((S0 * k, 100), device=dev)
+        P.s_all = torch.empty_like(packed[0])
+        P.s_in = torch.split(P.s_all, [roots.shape[1], root_ts.shape[1], neg.shape[1], neg_ts.shape[1]])
+        P.E = P.kr.hops[0].counts[1:2]
+        P.acc = torch.zeros(2, dtype=torch.int64, device=dev)
+        P.plan = hot.gather_plan([(c_mem, P.ubuf, P.o_mem, P.o_ts, P.U[0:1]), (c_nf, P.ubuf, P.o_nf, None, P.U[0:1]),
+                                  (c_ef, P.kr.hops[0].neighbors_eid, P.o_ef, None, P.E)])
 
-    def stage(b):
-        for dst_, src_ in zip(s_in, (roots, root_ts, neg, neg_ts)):
-            dst_.copy_(src_[b])
+        def body():
+            hot.sample_khop(dg, P.s_in[0], ts_ptr, P.s_in[1], P.s_in[2], P.s_in[3], 1, p, finalize=False, out=P.kr)
+            hot.unique_compact([P.kr.slot_node0, P.kr.hops[0].neighbors], _abi.UNIQUE_SORTED, P.state, True,
+                               lens_dev=[S0_dev, P.E], out_arrays=P.local, finalize=False, unique_out=P.ubuf, U_out=P.U)
+            hot.gather_multi(P.plan)
+            hot.time_encode(P.kr.hops[0].neighbors_dt, w, bias, out=P.o_te, N_dev=P.E)
+            P.acc[0:1].add_(P.E); P.acc[1:2].add_(P.U[0:1])
+        P.body = body
+        with torch.cuda.stream(stream):
+            P.s_all.copy_(packed[0]); body(); stream.synchronize()
+            P.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(P.graph, stream=stream):
+                body()
 
-    stage(0); body(); torch.cuda.synchronize()
-    side = torch.cuda.Stream(); side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        body()
-    torch.cuda.current_stream().wait_stream(side); torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        body()
-    for i in range(3):
-        stage(i % NB); graph.replay()
-    torch.cuda.synchronize(); acc.zero_(); torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    for i in range(steps):
-        stage(i % NB); graph.replay()
+        def run(b):
+            with torch.cuda.stream(stream):
+                P.s_all.copy_(packed[b], non_blocking=True)
+                P.graph.replay()
+        P.run = run
+        return P
+
+    streams = streams if streams else [torch.cuda.Stream()]
+    pipes = [make_pipeline(st_) for st_ in streams]
+
+    def timed(np_):
+        for i in range(6):
+            pipes[i % np_].run(i % NB)
+        torch.cuda.synchronize()
+        for P in pipes:
+            P.acc.zero_()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(steps):
+            pipes[i % np_].run(i % NB)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t1, sum(P.acc for P in pipes).cpu().tolist()
+
+    wall1, _ = timed(1)
+    wall, (e_tot, u_tot) = timed(len(pipes))
+    P0 = pipes[0]
+    kr, ubuf, U, E, plan, s_in = P0.kr, P0.ubuf, P0.U, P0.E, P0.plan, P0.s_in
+    o_mem, o_ts, o_ef, o_te = P0.o_mem, P0.o_ts, P0.o_ef, P0.o_te
+    with torch.cuda.stream(streams[0]):
+        P0.s_all.copy_(packed[0]); P0.body()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t1
-    e_tot, u_tot = acc.cpu().tolist()
-    # stage timings (eager, back to back)
-    stage(0); body(); torch.cuda.synchronize()
     e1, u1 = int(E.item()), int(U[0].item())
     res = {"nodes": n, "edges": m, "roots_per_batch": S0, "remote_row_fraction": remote, "steps": steps,
-           "ms_per_step": round(wall / steps * 1e3, 4), "sampled_edges_per_s": round(e_tot / wall, 1),
+           "batches_in_flight": len(pipes), "ms_per_step": round(wall / steps * 1e3, 4),
+           "ms_per_step_one_batch_in_flight": round(wall1 / steps * 1e3, 4),
+           "sampled_edges_per_s": round(e_tot / wall, 1),
            "edges_per_step": e_tot / steps, "unique_nodes_per_step": u_tot / steps}
     ms = _time_launches(torch, lambda: hot.time_encode(kr.hops[0].neighbors_dt, w, bias, out=o_te, N_dev=E))
     res["time_encode"] = {"ms": round(ms, 4), "rows": e1, "GBps": round(e1 * 408 / ms / 1e6, 1)}
@@ -818,7 +840,7 @@ def main():
         torch.cuda.empty_cache()
     for name, fn in (("configs[2] cache stress", lambda: workload_cache_stress(hot, torch, np, synth)),
                      ("configs[3] large partition", lambda: workload_large_partition(hot, torch, np, synth, _abi)),
-                     ("configs[4] tgn step", lambda: workload_tgn_step(hot, torch, np, synth, _abi))):
+                     ("configs[4] tgn step", lambda: workload_tgn_step(hot, torch, np, synth, _abi, streams=pipe_streams))):
         key = {"configs[2]": "c3", "configs[3]": "c4", "configs[4]": "c5"}[name[:10]]
         if args.workload not in (key, "all"):
             continue
