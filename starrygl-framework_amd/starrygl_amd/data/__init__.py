@@ -1,1 +1,1 @@
-from .pipeline import MiniBatch, MiniBatchPipeline  # noqa: F401
+from .pipeline import MiniBatch, MiniBatchPipeline, MiniBatchPipelinePool  # noqa: F401

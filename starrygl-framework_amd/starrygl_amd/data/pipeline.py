@@ -33,6 +33,8 @@ class MiniBatch:
         if self.final:
             return self
         p = self._p
+        if p._done is not None:      # the batch ran on the pipeline's own stream
+            p._done.synchronize()
         c = p.kr.counts.cpu().tolist()
         u_total = int(p.U[0].item())
         check_unique_total(u_total)
@@ -92,13 +94,16 @@ class MiniBatch:
 class MiniBatchPipeline:
     def __init__(self, graph, num_pos_slots, num_neg, layers, fanout, sample_type="recent", node_tables=None,
                  edge_tables=None, time_encoder=None, allowed_offset=-1, equal_root_time=False,
-                 keep_root_time=False, seed=0, use_graph=True):
+                 keep_root_time=False, seed=0, use_graph=True, stream=None):
         """graph: the native graph object (`pyGraph.g`, i.e. `CUDAGraph`).
         num_pos_slots / num_neg: positive root timestamps and negatives per batch
         (fixed, they size every buffer).  node_tables / edge_tables: name ->
         `sgl_cache` (from `HotPath.cache`) gathered for the unique nodes / the
         sampled edge ids; a node table with timestamps also yields node_ts[name].
-        time_encoder: (w, b) fp32 device tensors, or a TimeEncoder module."""
+        time_encoder: (w, b) fp32 device tensors, or a TimeEncoder module.
+        stream: run every batch on this stream instead of the caller's current one (see
+        MiniBatchPipelinePool); inputs handed to run() must then be complete on the host side
+        or long-lived, and results are read through MiniBatch.finalize(), which waits for it."""
         self.g = graph
         self.hp = hp = graph._hp
         self.dev = hp.be.device
@@ -144,6 +149,8 @@ class MiniBatchPipeline:
                                                     (_abi.i64 * (1 + self.layers))(*caps)))
         self.use_graph, self._graph = use_graph, None
         self._plans, self._slow = None, []
+        self.stream = stream
+        self._done = torch.cuda.Event() if stream is not None else None
 
     def view(self, name, dtype):
         """Reinterpret the byte output buffers of table `name` as rows of `dtype`."""
@@ -187,6 +194,14 @@ class MiniBatchPipeline:
             raise ValueError(f"this pipeline was planned for {self.S_pos} positive slots")
         if self.N_neg and (neg_roots is None or neg_roots.numel() != self.N_neg or neg_ts.numel() != self.N_neg):
             raise ValueError(f"this pipeline was planned for {self.N_neg} negatives")
+        if self.stream is not None:
+            with torch.cuda.stream(self.stream):
+                out = self._run(roots, root_ts, neg_roots, neg_ts)
+                self._done.record(self.stream)
+            return out
+        return self._run(roots, root_ts, neg_roots, neg_ts)
+
+    def _run(self, roots, root_ts, neg_roots, neg_ts):
         self.in_roots.copy_(roots, non_blocking=True)
         self.in_ts.copy_(root_ts, non_blocking=True)
         if self.N_neg:
@@ -211,3 +226,34 @@ class MiniBatchPipeline:
         else:
             self._graph.replay()
         return MiniBatch(self)
+
+
+def bound_streams(n, device):
+    """n streams, each used once: a HIP stream gets its hardware queue at first use, and streams that
+    share a queue take turns instead of overlapping.  Call this before other streams are created."""
+    streams = [torch.cuda.Stream(device) for _ in range(n)]
+    for st in streams:
+        with torch.cuda.stream(st):
+            torch.zeros(1, device=device).add_(1)
+    torch.cuda.synchronize(device)
+    return streams
+
+
+class MiniBatchPipelinePool:
+    """`n` MiniBatchPipeline objects on streams of their own; run() hands the batches to them in
+    turn, so that up to `n` batches are in flight: the latency-bound sampling of one batch overlaps
+    the bandwidth-bound gathers of another (configs of 12 000 roots, 2 hops: 0.105 ms per batch with
+    three in flight against 0.127 ms one at a time).  A MiniBatch stays valid until the `n`-th
+    following run().  Create the pool before any other stream of the process."""
+
+    def __init__(self, n, graph, *args, **kwargs):
+        if n < 1:
+            raise ValueError("a pool needs at least one pipeline")
+        dev = graph._hp.be.device
+        self.pipes = [MiniBatchPipeline(graph, *args, stream=st, **kwargs) for st in bound_streams(n, dev)]
+        self._next = 0
+
+    def run(self, roots, root_ts, neg_roots=None, neg_ts=None):
+        p = self.pipes[self._next]
+        self._next = (self._next + 1) % len(self.pipes)
+        return p.run(roots, root_ts, neg_roots, neg_ts)

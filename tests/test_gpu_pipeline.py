@@ -58,3 +58,33 @@ def test_pipeline_matches_oracle(oracle, hot, use_graph, sample_type):
         assert np.array_equal(uniq[np_of(outer.srcdata["nid"])[-mb.E[1]:]], want.hops[1].neighbors)
     with pytest.raises(ValueError):
         pipe.run(to_dev(hot, roots[:5]), to_dev(hot, root_ts[:5]), to_dev(hot, neg), to_dev(hot, neg_ts))
+
+
+def test_pipeline_pool_keeps_batches_in_flight(oracle, hot):
+    """Three pipelines on streams of their own: batches are enqueued back to back and only read afterwards;
+    each must equal the oracle's result for its own roots (no pipeline sees another one's buffers)."""
+    from starrygl_amd.data import MiniBatchPipelinePool
+    from starrygl_amd.lib.libstarrygl_comm import from_edge_index
+    n, m, B = 4000, 80_000, 300
+    src, dst, ts, eid = synth.graph_stream(n, m, 1.15, 500_000, 23)
+    hg = host_graph(oracle, n, src, dst, ts, eid)
+    g = from_edge_index(n, 1, *(torch.from_numpy(x) for x in (src, dst, ts, eid)))
+    rng = np.random.default_rng(4)
+    feat = rng.standard_normal((n, 100)).astype(np.float32)
+    c_nf = hot.cache(400, to_dev(hot, feat, "f32"))
+    pool = MiniBatchPipelinePool(3, g, 2 * B, B, 2, 5, "recent", node_tables={"x": c_nf})
+    for p in pool.pipes:
+        p.view("x", torch.float32)
+    for rnd in range(3):
+        batches = [synth.link_batch(src, dst, ts, lo, lo + B, n, B, rng) for lo in (10_000 + 7_000 * rnd, 40_000, 79_000)]
+        inflight = [pool.run(to_dev(hot, b[0]), to_dev(hot, b[2]), to_dev(hot, b[3]), to_dev(hot, b[4])) for b in batches]
+        for b, mb in zip(batches, inflight):
+            mb.finalize()
+            want = oracle.sample_khop(hg, *b, 2, oracle.params("recent", 5))
+            arrays = [want.slot_node0] + [h.neighbors for h in want.hops]
+            loc, uniq, _ = oracle.unique_compact(arrays, _abi.UNIQUE_SORTED, None, True)
+            assert mb.E == [h.E for h in want.hops] and np.array_equal(np_of(mb.nid_mapper), uniq)
+            assert np.array_equal(np_of(mb.node_data["x"]), feat[uniq])
+            for l, h in enumerate(want.hops):
+                assert np.array_equal(np_of(mb.hops[l]["neighbors_local"]), loc[1 + l])
+                assert np.array_equal(np_of(mb.hops[l]["neighbors_eid"]), h.neighbors_eid)
