@@ -242,3 +242,44 @@ def test_several_policies_with_marks_feed_unique(oracle, hot):
         assert int(np_of(U)[0]) == want_u.size and np.array_equal(np_of(uniq)[: want_u.size], want_u)
         got_inv = np.concatenate([np_of(local[0]), np_of(local[1])[: c[1]], np_of(local[2])[: c[4]]])
         assert np.array_equal(got_inv, want_inv)
+
+
+@pytest.mark.parametrize("replace", [False, True])
+@pytest.mark.parametrize("layers", [1, 2])
+def test_uniform_invariants_and_chi_square_on_the_gpu(hot, replace, layers):
+    """The uniform sampler judged on its own output, without the oracle: sampled edges lie strictly
+    before the root's time, at most `fanout` per slot and distinct without replacement, (neighbour, ts,
+    eid) belong to one edge of the row, and every candidate position is drawn with probability k/cnt
+    (chi-square at the 0.999 quantile).  One hop goes through the count/fill kernels, two hops through
+    the single-launch kernel (its second hop is tested: a chain 1 -> 0 -> 37 candidates)."""
+    import scipy.stats as sps
+    cnt, k, trials = 37, 10, 20_000
+    # node 0 owns `cnt` edges at times 0..cnt-1 to node 2; node 1 owns one edge to node 0 at time cnt + 1
+    src = np.concatenate([np.zeros(cnt, np.int64), [1]])
+    dst = np.concatenate([np.full(cnt, 2, np.int64), [0]])
+    ts = np.concatenate([np.arange(cnt), [cnt + 1]]).astype(np.int64)
+    eid = np.arange(cnt + 1, dtype=np.int64)
+    dg = hot.tcsr_build(3, to_dev(hot, src), to_dev(hot, dst), to_dev(hot, ts), to_dev(hot, eid))
+    p = hot.params("uniform", k, replace=replace, seed=4242)
+    empty = to_dev(hot, np.zeros(0, np.int64))
+    if layers == 1:
+        roots, t_root = np.zeros(trials, np.int64), np.full(trials, cnt + 5, np.int64)
+    else:     # hop 1 of root 1 at time cnt + 3 is its only edge (to node 0, ts cnt + 1); hop 2 samples node 0 before cnt + 1
+        roots, t_root = np.ones(trials, np.int64), np.full(trials, cnt + 3, np.int64)
+    res = hot.sample_khop(dg, to_dev(hot, roots), to_dev(hot, np.arange(trials + 1)), to_dev(hot, t_root), empty, empty, layers, p)
+    h = res.hops[layers - 1]
+    assert h.S == trials and h.E == trials * k
+    start, end = np_of(h.root_start_ptr), np_of(h.root_end_ptr)
+    assert np.array_equal(end[:-1] - start[:-1], np.full(trials, k))
+    e, nb, nts, ndt = np_of(h.neighbors_eid), np_of(h.neighbors), np_of(h.neighbors_ts), np_of(h.neighbors_dt)
+    t_slot = cnt + 5 if layers == 1 else cnt + 1
+    assert (e >= 0).all() and (e < cnt).all() and (nb == 2).all()          # edges of row 0 only: eid <-> dst mapping
+    assert np.array_equal(nts, e) and (nts < t_slot).all() and np.array_equal(ndt, nts - t_slot)
+    per_slot = e.reshape(trials, k)
+    if not replace:
+        s = np.sort(per_slot, axis=1)
+        assert (s[:, 1:] > s[:, :-1]).all() and np.array_equal(s, per_slot)  # distinct, ascending position
+    freq = np.bincount(e, minlength=cnt).astype(np.float64)
+    expect = trials * k / cnt
+    chi2 = ((freq - expect) ** 2 / expect).sum()
+    assert chi2 < sps.chi2.ppf(0.999, cnt - 1), chi2
