@@ -54,6 +54,13 @@ class NumpyBackend:
     def stream(self):
         return None
 
+    def check(self, a, dtype, name):
+        if a.dtype != self._dt[dtype]:
+            raise TypeError(f"{name} must be {dtype}, got {a.dtype}")
+        if not a.flags["C_CONTIGUOUS"]:
+            raise ValueError(f"{name} must be contiguous")
+        return a
+
     def tolist(self, a):
         return a.tolist()
 

@@ -19,6 +19,7 @@ class TorchBackend:
         import torch
         self.torch = torch
         self.device = torch.device(device)
+        self._one_gpu = self.device.type == "cuda" and torch.cuda.device_count() == 1
         self._dt = {"i64": torch.int64, "i32": torch.int32, "f32": torch.float32,
                     "u8": torch.uint8, "bf16": torch.bfloat16, "f16": torch.float16}
 
@@ -47,9 +48,14 @@ class TorchBackend:
         return a.numel() * a.element_size()
 
     def check(self, a, dtype, name):
+        """The ABI takes raw pointers: an array of another dtype, a strided view or pageable host
+        memory would be read as something it is not."""
+        if a.dtype is self._dt[dtype] and a.is_cuda and a.is_contiguous() and self._one_gpu:
+            return a                 # the common case, kept cheap: this runs on every call
         if a.dtype != self._dt[dtype]:
             raise TypeError(f"{name} must be {dtype}, got {a.dtype}")
-        if a.device != self.device and not (a.device.type == "cpu" and a.is_pinned()):
+        here = a.device.type == self.device.type and (self.device.index is None or a.device.index == self.device.index)
+        if not here and not (a.device.type == "cpu" and a.is_pinned()):
             raise ValueError(f"{name} must live on {self.device}, got {a.device}")
         if not a.is_contiguous():
             raise ValueError(f"{name} must be contiguous")
@@ -129,11 +135,18 @@ class HotPath:
             ws = self._ws[key] = self.be.empty(nbytes, "u8")
         return ws, self.be.nbytes(ws)
 
+    def _chk(self, dtype, **arrays):
+        """Validate the arrays handed to a call (dtype, placement, contiguity); None entries pass."""
+        for name, a in arrays.items():
+            if a is not None:
+                self.be.check(a, dtype, name)
+
     def _ck(self, rc):
         check(self.lib, rc)
 
     # -------------------------------------------------------------- T-CSR
     def tcsr_build(self, n, src, dst, ts, eid=None):
+        self._chk("i64", src=src, dst=dst, ts=ts, eid=eid)
         be, m = self.be, int(src.shape[0])
         row_ptr, col, cts, ceid = be.empty(n + 1), be.empty(m), be.empty(m), be.empty(m)
         ws, wsb = self._workspace(self.lib.tcsr_build_workspace_bytes(n, m))
@@ -143,6 +156,7 @@ class HotPath:
         return TCSRArrays(be, n, row_ptr, col, cts, ceid)
 
     def tcsr_from_sorted(self, n, row_ptr, col, ts, eid, validate=True):
+        self._chk("i64", row_ptr=row_ptr, col=col, ts=ts, eid=eid)
         g = TCSRArrays(self.be, n, row_ptr, col, ts, eid)
         if validate:
             ws, wsb = self._workspace(256)
@@ -177,6 +191,7 @@ class HotPath:
         return q
 
     def sample_hop(self, g, slot_node, slot_ts, p, S_dev=None, finalize=True):
+        self._chk("i64", slot_node=slot_node, slot_ts=slot_ts, S_dev=S_dev)
         be, S = self.be, int(slot_node.shape[0])
         out = HopResult(be, S, S * p.fanout)
         ws, wsb = self._workspace(self.lib.sample_hop_workspace_bytes(S))
@@ -208,6 +223,7 @@ class HotPath:
 
     def sample_khop(self, g, roots, ts_ptr, root_ts, neg_roots, neg_ts, layers, p,
                     finalize=True, out=None):
+        self._chk("i64", roots=roots, ts_ptr=ts_ptr, root_ts=root_ts, neg_roots=neg_roots, neg_ts=neg_ts)
         be = self.be
         R, S_pos, N_neg = int(roots.shape[0]), int(root_ts.shape[0]), int(neg_roots.shape[0])
         S0 = S_pos + N_neg
@@ -226,6 +242,7 @@ class HotPath:
         """Several k-hop calls (params[q] -> outs[q], buffers of khop_buffers) over the same roots
         in one library call; a most-recent and a uniform 2-hop call share one launch.  The results
         are not finalized; they share the hop-0 slot arrays of outs[0]."""
+        self._chk("i64", roots=roots, ts_ptr=ts_ptr, root_ts=root_ts, neg_roots=neg_roots, neg_ts=neg_ts)
         be, Q = self.be, len(params)
         R, S_pos, N_neg = int(roots.shape[0]), int(root_ts.shape[0]), int(neg_roots.shape[0])
         S0 = S_pos + N_neg
@@ -257,6 +274,7 @@ class HotPath:
     def unique_compact(self, arrays, mode=_abi.UNIQUE_SORTED, state=None, reset=True,
                        lens_dev=None, out_arrays=None, finalize=True, unique_out=None, U_out=None,
                        premarked=False):
+        self._chk("i64", **{f"arrays[{i}]": a for i, a in enumerate(arrays)})
         be, G = self.be, len(arrays)
         len_max = (i64 * max(G, 1))(*[int(a.shape[0]) for a in arrays])
         total = sum(len_max[:G])
@@ -304,6 +322,7 @@ class HotPath:
         return c
 
     def gather(self, cache, ids, out, out_ts=None, stats=None, N_dev=None):
+        self._chk("i64", ids=ids, out_ts=out_ts, stats=stats, N_dev=N_dev)
         be = self.be
         self._ck(self.lib.gather(C.byref(cache), be.ptr(ids), int(ids.shape[0]), be.ptr(N_dev),
                                  be.ptr(out), be.ptr(out_ts), be.ptr(stats), be.stream()))
@@ -324,6 +343,7 @@ class HotPath:
         self._ck(self.lib.gather_multi(len(plan), plan, self.be.stream()))
 
     def scatter_update(self, cache, hot_rw, cold_rw, ts_hot_rw, ts_cold_rw, ids, values, ts=None):
+        self._chk("i64", ids=ids, ts=ts)
         be = self.be
         self._ck(self.lib.scatter_update(C.byref(cache), be.ptr(hot_rw), be.ptr(cold_rw),
                                          be.ptr(ts_hot_rw), be.ptr(ts_cold_rw), be.ptr(ids),
@@ -333,6 +353,7 @@ class HotPath:
     # ------------------------------------------------------ chunks / seeds
     def chunk_index(self, n, num_chunks, node_chunk):
         """-> (chunk_ptr[num_chunks+1], chunk_nodes[n]) on the backend's device."""
+        self._chk("i64", node_chunk=node_chunk)
         be = self.be
         chunk_ptr, chunk_nodes = be.empty(num_chunks + 1), be.empty(max(n, 1))
         ws, wsb = self._workspace(self.lib.chunk_index_workspace_bytes(n))
@@ -343,6 +364,7 @@ class HotPath:
     def seeds(self, g, chunk_ptr, chunk_nodes, chunks, cand_off, n_cand, t_begin, t_end):
         """-> (roots, ts_ptr, ts, q_ptr, q_eid).  `cand_off` is the exclusive prefix
         of the selected chunks' sizes, `n_cand` its last entry (host int)."""
+        self._chk("i64", chunk_ptr=chunk_ptr, chunk_nodes=chunk_nodes, chunks=chunks, cand_off=cand_off)
         be = self.be
         q = SeedQuery(be.ptr(chunk_ptr), be.ptr(chunk_nodes), int(chunks.shape[0]), be.ptr(chunks),
                       be.ptr(cand_off), int(n_cand), int(t_begin), int(t_end))
@@ -359,6 +381,7 @@ class HotPath:
               full_timestamps=False):
         """Sub-graph of the selected chunks over [t_begin, t_end)
         -> (nodes, ts_ptr, ts, edge_ptr, col, col_ts, col_eid)."""
+        self._chk("i64", chunk_ptr=chunk_ptr, chunk_nodes=chunk_nodes, node_chunk=node_chunk, chunks=chunks, cand_off=cand_off)
         be = self.be
         q = SeedQuery(be.ptr(chunk_ptr), be.ptr(chunk_nodes), int(chunks.shape[0]), be.ptr(chunks),
                       be.ptr(cand_off), int(n_cand), int(t_begin), int(t_end))
@@ -388,6 +411,7 @@ class HotPath:
     def unique_pairs(self, ids, ts, N_dev=None):
         """-> (uniq_ids[U], uniq_ts[U], inverse[N]): np.unique over (id, ts) records with
         return_inverse (one synchronising read of U)."""
+        self._chk("i64", ids=ids, ts=ts, N_dev=N_dev)
         be, N = self.be, int(ids.shape[0])
         uid, uts, inv, U = be.empty(max(N, 1)), be.empty(max(N, 1)), be.empty(max(N, 1)), be.zeros(1)
         ws, wsb = self._workspace(self.lib.unique_pairs_workspace_bytes(N))
@@ -399,6 +423,7 @@ class HotPath:
 
     def csc_from_pairs(self, dst_local, ts, num_dst, E_dev=None):
         """-> (indptr[num_dst + 1], perm[E]): the stable (dst_local, ts) edge order."""
+        self._chk("i64", dst_local=dst_local, ts=ts, E_dev=E_dev)
         be, E = self.be, int(dst_local.shape[0])
         indptr, perm = be.empty(num_dst + 1), be.empty(max(E, 1))
         ws, wsb = self._workspace(self.lib.csc_from_pairs_workspace_bytes(E))
@@ -410,6 +435,7 @@ class HotPath:
     def segment_max_ts(self, local, ts, U, N_dev=None, U_dev=None):
         """-> (max_ts[U], arg[U]): per dense key the largest timestamp and the first
         event index attaining it."""
+        self._chk("i64", local=local, ts=ts, N_dev=N_dev, U_dev=U_dev)
         be = self.be
         max_ts, arg = be.empty(max(U, 1)), be.empty(max(U, 1))
         self._ck(self.lib.segment_max_ts(be.ptr(local), be.ptr(ts), int(local.shape[0]), be.ptr(N_dev), int(U),
@@ -418,6 +444,8 @@ class HotPath:
 
     # -------------------------------------------------------- time encode
     def time_encode(self, dt, w, b, dt_dtype=_abi.DT_I64, out=None, N_dev=None):
+        self._chk("i64" if dt_dtype == _abi.DT_I64 else "f32", dt=dt)
+        self._chk("f32", w=w, b=b, out=out)
         be, N, dim = self.be, int(dt.shape[0]), int(w.shape[0])
         if out is None:
             out = be.empty((N, dim), "f32")

@@ -32,6 +32,10 @@ class DistRouteIndex:
     """Packed id of a row somewhere in the partitioned graph: local index in the
     low 48 bits, owning partition in the next 14, bit 62 set for shared rows."""
 
+    LOC_MASK = (1 << _FIELDS["loc"][1]) - 1          # what sgl_cache.id_mask takes for packed ids
+    PART_SHIFT, PART_MASK = _FIELDS["part"][0], (1 << _FIELDS["part"][1]) - 1
+    SHARED_BIT = _FIELDS["shared"][0]
+
     def __init__(self, index: Tensor, part_ids: Optional[Tensor] = None) -> None:
         data = index.long()
         self._data = data if part_ids is None else _packed(data, part_ids.long().to(data.device))

@@ -283,3 +283,26 @@ def test_uniform_invariants_and_chi_square_on_the_gpu(hot, replace, layers):
     expect = trials * k / cnt
     chi2 = ((freq - expect) ** 2 / expect).sum()
     assert chi2 < sps.chi2.ppf(0.999, cnt - 1), chi2
+
+
+def test_driver_rejects_arrays_it_cannot_pass_as_pointers(oracle, hot):
+    """The ABI takes raw pointers; the array-level driver refuses what would be misread: another
+    dtype, a strided view, pageable host memory."""
+    import torch
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 500, 5_000, 1.1, 10**5, 43)
+    roots = to_dev(hot, np.arange(40))
+    tp, t = to_dev(hot, np.arange(41)), to_dev(hot, np.full(40, 9 * 10**4))
+    e = to_dev(hot, np.zeros(0, np.int64))
+    p = hot.params("recent", 5)
+    hot.sample_khop(dg, roots, tp, t, e, e, 1, p)                                   # the well-formed call
+    with pytest.raises(TypeError):
+        hot.sample_khop(dg, roots.int(), tp, t, e, e, 1, p)
+    with pytest.raises(ValueError):
+        hot.sample_khop(dg, to_dev(hot, np.arange(80))[::2], tp, t, e, e, 1, p)    # strided view
+    with pytest.raises(ValueError):
+        hot.sample_khop(dg, torch.arange(40), tp, t, e, e, 1, p)                    # pageable host memory
+    with pytest.raises(TypeError):
+        hot.unique_compact([roots.float()], 0, hot.remap_state(500), True)
+    with pytest.raises(TypeError):
+        hot.gather(hot.cache(16, torch.zeros((500, 4), device=roots.device)), roots.int(),
+                   torch.empty((40, 4), device=roots.device))
