@@ -262,6 +262,11 @@ def workload_large_partition(hot, torch, np, synth, _abi, n=100_000_000, m=1_000
     t0 = time.time()
     row_ptr, col, ts, eid, key = synth.graph_by_degree_device(torch, dev, n, m, 1.05, 1_000_000, T_BITS, 20243)
     g = hot.tcsr_from_sorted(n, row_ptr, col, ts, eid, validate=True)
+    torch.cuda.synchronize()
+    t_h = time.perf_counter()
+    hot.build_hop_hint(g)
+    torch.cuda.synchronize()
+    hint_s = time.perf_counter() - t_h
     gen = torch.Generator(device=dev).manual_seed(1)
     NB = 4
     roots = [key[torch.randint(0, m, (R,), device=dev, generator=gen)] >> T_BITS for _ in range(NB)]
@@ -279,7 +284,8 @@ def workload_large_partition(hot, torch, np, synth, _abi, n=100_000_000, m=1_000
     state = hot.remap_state(n)
     R_dev = torch.tensor([R], device=dev)
     hot._workspace(hot.lib.unique_workspace_bytes(n, 3, (_abi.i64 * 3)(*caps)))
-    res = {"nodes": n, "edges": m, "roots_per_batch": R, "fanout": [k, k], "max_degree": max_deg}
+    res = {"nodes": n, "edges": m, "roots_per_batch": R, "fanout": [k, k], "max_degree": max_deg,
+           "next_hop_index_build_s": round(hint_s, 3)}
 
     def sample(b):
         hot.sample_khop(g, roots[b], ts_ptr, root_ts[b], empty, empty, 2, p, finalize=False, out=kr)
@@ -352,6 +358,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE readings can be scaled")
     ap.add_argument("--no-fused-mark", action="store_true",
                     help="unique runs its own marking pass instead of the sampler recording the ids it emits")
+    ap.add_argument("--no-hop-hint", action="store_true",
+                    help="sample without the graph's next-hop index (every slot of hops >= 1 searches its window)")
     ap.add_argument("--pipelines", type=int, default=3,
                     help="independent copies of the step (own buffers, graph and stream) that take the batches of the "
                          "timed region in turn, as a loader with that many batches in flight does; 1 = one batch at a time")
@@ -388,6 +396,12 @@ def main():
     log(f"[setup] graph n={n} m={m} generated in {time.time() - t0:.1f}s, max degree {int(np.diff(row_ptr).max())}")
     D = lambda a, dt="i64": hot.be.asarray(a, dt)
     dg = hot.tcsr_from_sorted(n, D(row_ptr), D(dst), D(ts), D(eid), validate=True)
+    if not args.no_hop_hint:     # the graph's next-hop index: hops >= 1 find their windows without searching
+        torch.cuda.synchronize()
+        t_h = time.perf_counter()
+        hot.build_hop_hint(dg)
+        torch.cuda.synchronize()
+        log(f"[setup] next-hop index of {m} edges built in {(time.perf_counter() - t_h) * 1e3:.1f} ms")
     gen = torch.Generator(device=dev).manual_seed(20242)
     node_feat = torch.randn((n, 100), device=dev, generator=gen)
     edge_feat = None

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define SGL_ABI_VERSION 2
+#define SGL_ABI_VERSION 3
 
 /* ------------------------------------------------------------------ status */
 #define SGL_OK        0
@@ -71,7 +71,20 @@ typedef struct sgl_tcsr {
     const int64_t* col;     /* [m]   device: destination node   */
     const int64_t* ts;      /* [m]   device: edge timestamp     */
     const int64_t* eid;     /* [m]   device: edge id            */
+    /* Optional (NULL = absent) next-hop index of sgl_tcsr_hop_hint_build: for the
+     * edge at position e, hop_hint[e] is the position in row col[e] of the first
+     * edge whose timestamp is >= ts[e], i.e. where the window of the next hop's
+     * slot (col[e], ts[e]) ends.  With it the sampler needs no search for the
+     * slots of hops >= 1 (strictly-before windows, slot time = edge time). */
+    const int64_t* hop_hint;/* [m]   device, or NULL            */
 } sgl_tcsr;
+
+/* Fill hop_hint[0..m) for the T-CSR `g` (whose own hop_hint field is ignored):
+ * one lower-bound search per edge, done once per graph.  -1 for an edge whose
+ * destination lies outside [0,n).  No counterpart in the reference, which
+ * searches the neighbour's row for every sampled edge of every batch
+ * (find_time_range, sample.cu.hpp:264-295). */
+int32_t sgl_tcsr_hop_hint_build(const sgl_tcsr* g, int64_t* hop_hint, void* stream);
 
 /* Build a T-CSR from a COO edge list (replaces from_edge_index / Graph::Graph,
  * export.cu:229-250, sample.cu.hpp:985-1185).  `eid` may be NULL (= 0..m-1).

@@ -148,6 +148,22 @@ static int64_t lower_bound_ts(const int64_t* ts, int64_t lo, int64_t hi, int64_t
     return lo;
 }
 
+/* The next-hop index is an accelerator of the kernels; the oracle samples by
+ * searching (hop_hint of the graph is ignored) and only restates the index's
+ * definition so that the built array can be checked. */
+int32_t sglo_tcsr_hop_hint_build(const sgl_tcsr* g, int64_t* hop_hint, void* stream) {
+    (void)stream;
+    if (!g || g->n < 0 || g->m < 0 || !g->row_ptr) return fail(SGL_EINVAL, "tcsr_hop_hint_build: null");
+    if (g->m > 0 && (!g->col || !g->ts || !hop_hint)) return fail(SGL_EINVAL, "tcsr_hop_hint_build: null array");
+    for (int64_t e = 0; e < g->m; ++e) {
+        int64_t v = g->col[e], p = -1;
+        if (v >= 0 && v < g->n) p = lower_bound_ts(g->ts, g->row_ptr[v], g->row_ptr[v + 1], g->ts[e]);
+        hop_hint[e] = p;
+    }
+    return SGL_OK;
+}
+
+
 /* Candidate window of a slot.  Reference: find_time_range
  * (sample.cu.hpp:264-295) called with (ts - allowed_offset or 0,
  * ts + equal_root_time) at :723-724; numba cut_idx/start_idx

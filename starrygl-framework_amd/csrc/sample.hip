@@ -46,6 +46,10 @@ struct HopArgs {
     const int64_t* col;
     const int64_t* ts;
     const int64_t* eid;
+    const int64_t* hint; // next-hop index of the graph (sgl_tcsr.hop_hint), or nullptr
+    const int64_t* slot_hint;  // per explicit slot: where its window ends (the index entry of the edge the slot
+                               // came from), or nullptr: search
+    int64_t* hint_out;   // per emitted edge: its index entry, for the next hop's slots; or nullptr
     // slots: explicit (slot_node/slot_ts), or - when roots != nullptr - derived from
     // R positive roots over ts_ptr/root_ts followed by N_neg negatives, and then
     // written to slot_node_out/slot_ts_out
@@ -213,7 +217,15 @@ __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
             re = a.row_ptr[v + 1];
         }
         const int64_t t_hi = t + (a.equal_root_time ? 1 : 0);
-        const int64_t hi = group_lower_bound<G>(a.ts, rs, re, t_hi, lig, gshift, active);
+        int64_t hi;
+        if (a.slot_hint != nullptr) {     // kernel argument: uniform across the wave
+            // the slot is (destination, time) of an edge whose index entry says where the window ends;
+            // an entry of -1 belongs to a destination outside [0,n), which is a bad slot anyway
+            const int64_t h = active ? a.slot_hint[slot] : 0;
+            hi = h >= rs ? h : rs;
+        } else {
+            hi = group_lower_bound<G>(a.ts, rs, re, t_hi, lig, gshift, active);
+        }
         int64_t lo = rs;
         if (a.allowed_offset >= 0)  // kernel argument: uniform across the wave
             lo = group_lower_bound<G>(a.ts, rs, hi, t - a.allowed_offset, lig, gshift, active);
@@ -456,6 +468,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
                             ets[r] = a.ts[e];
                             dst[r] = a.col[e];
                             id[r] = a.eid[e];
+                            if (a.hint_out != nullptr) a.hint_out[off + j] = a.hint[e];
                         }
                     }
 #pragma unroll
@@ -513,6 +526,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
                 a.nbr_ts[off + rank] = a.keep_root_time ? t : ets;
                 a.nbr_eid[off + rank] = a.eid[e];
                 a.nbr_dt[off + rank] = ets - t;
+                if (a.hint_out != nullptr) a.hint_out[off + rank] = a.hint[e];
             }
         }
     }
@@ -769,11 +783,12 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
         }
         pos = lo + sel;
     }
-    int64_t nbr = 0, ets = 0, id = 0;
+    int64_t nbr = 0, ets = 0, id = 0, hint = -1;
     if (e_on) {
         nbr = a.col[pos];
         ets = a.ts[pos];
         id = a.eid[pos];
+        if (a.hint != nullptr) hint = a.hint[pos];
     }
     // ---- hop 2: lane j counts the slot (neighbour j, its timestamp - or the root's, keep_root_time)
     const int64_t t2 = (UNIFORM && a.keep_root_time) ? t : ets;
@@ -781,8 +796,12 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
     int32_t c2 = 0;
     if (e_on) {
         if (nbr >= 0 && nbr < a.n) {
-            const int64_t rs2 = a.row_ptr[nbr], re2 = a.row_ptr[nbr + 1];
-            const int64_t hi2 = lane_lower_bound(a.ts, rs2, re2, t2 + eq);
+            // the window of (neighbour, its edge's time) ends where the graph's next-hop index says:
+            // no search (strictly-before windows only; a uniform call that keeps the root's time asks
+            // about another time and searches)
+            const bool hinted = hint >= 0 && eq == 0 && t2 == ets;
+            const int64_t rs2 = a.row_ptr[nbr];
+            const int64_t hi2 = hinted ? hint : lane_lower_bound(a.ts, rs2, a.row_ptr[nbr + 1], t2 + eq);
             int64_t lo2 = rs2;
             if (a.allowed_offset >= 0) lo2 = lane_lower_bound(a.ts, rs2, hi2, t2 - a.allowed_offset);
             len2 = hi2 - lo2;
@@ -1038,14 +1057,15 @@ struct RootSpec {  // hop-0 slot source of the k-hop driver
 
 int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot_ts, const RootSpec* derive,
                 int64_t S_max, const int64_t* S_dev, const sgl_sample_params* p, const sgl_hop_out* out, void* ws,
-                size_t ws_bytes, hipStream_t st) {
+                size_t ws_bytes, hipStream_t st, const int64_t* slot_hint = nullptr, int64_t* hint_out = nullptr) {
     if (!derive && S_max > 0 && (!slot_node || !slot_ts)) return fail(SGL_EINVAL, "sample: slot array is NULL");
     if (ws_bytes < hop_workspace_bytes(S_max) || !ws)
         return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, hop_workspace_bytes(S_max));
     Arena ar(ws, ws_bytes);
     HopArgs a{};
-    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid;
+    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint;
     a.slot_node = slot_node; a.slot_ts = slot_ts; a.S_max = S_max; a.S_dev = S_dev;
+    a.slot_hint = slot_hint; a.hint_out = hint_out;
     a.derive = derive ? 1 : 0;
     if (derive) {
         a.R = derive->R; a.S_pos = derive->S_pos; a.roots = derive->roots; a.ts_ptr = derive->ts_ptr;
@@ -1076,7 +1096,7 @@ Fused2Args fused2_args(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, cons
                        const sgl_hop_out* outs, unsigned long long* desc) {
     Fused2Args f{};
     HopArgs& a = f.h;
-    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid;
+    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint;
     a.S_max = S0; a.derive = 1;
     a.R = spec->R; a.S_pos = spec->S_pos; a.roots = spec->roots; a.ts_ptr = spec->ts_ptr;
     a.root_ts = spec->root_ts; a.neg_roots = spec->neg_roots; a.neg_ts = spec->neg_ts;
@@ -1174,6 +1194,9 @@ static int64_t worst_slots(int64_t S0, int32_t layer, int32_t k) {
     return s;
 }
 
+// the two arrays through which a hop hands the index entries of its edges to the next hop's slots
+static size_t hint_carry_bytes(int64_t worst) { return 2 * align_up((size_t)(worst + 1) * 8); }
+
 extern "C" size_t sgl_sample_khop_workspace_bytes(int64_t S0, int32_t layers, int32_t fanout) {
     if (S0 < 0 || layers <= 0 || fanout < 0) return hop_workspace_bytes(0);
     int64_t worst = S0;
@@ -1181,7 +1204,7 @@ extern "C" size_t sgl_sample_khop_workspace_bytes(int64_t S0, int32_t layers, in
         const int64_t s = worst_slots(S0, l, fanout);
         if (s > worst) worst = s;
     }
-    return hop_workspace_bytes(worst);
+    return hop_workspace_bytes(worst) + (layers > 1 ? hint_carry_bytes(worst) : 0);
 }
 
 extern "C" int32_t sgl_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* roots,
@@ -1211,11 +1234,26 @@ extern "C" int32_t sgl_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* 
     const int64_t* sn = nullptr;
     const int64_t* stt = nullptr;
     const int64_t* S_dev = nullptr;
+    // With the graph's next-hop index the slots of hops >= 1 need no search: hop l stores the index
+    // entry of every edge it emits, hop l+1 reads it as the end of that slot's window.  (Only for
+    // strictly-before windows whose slot time is the edge's own time.)
+    int64_t worst = S0;
+    for (int32_t l = 0; l < layers; ++l) worst = worst_slots(S0, l, p->fanout) > worst ? worst_slots(S0, l, p->fanout) : worst;
+    const size_t hop_ws = hop_workspace_bytes(worst);
+    const bool carry = layers > 1 && g->hop_hint != nullptr && !p->equal_root_time &&
+                       !(p->type == SGL_SAMPLE_UNIFORM && p->keep_root_time) && ws != nullptr &&
+                       ws_bytes >= hop_ws + hint_carry_bytes(worst);
+    int64_t* carry_buf[2] = {nullptr, nullptr};
+    if (carry) {
+        carry_buf[0] = reinterpret_cast<int64_t*>(static_cast<char*>(ws) + hop_ws);
+        carry_buf[1] = reinterpret_cast<int64_t*>(static_cast<char*>(ws) + hop_ws + align_up((size_t)(worst + 1) * 8));
+    }
     for (int32_t l = 0; l < layers; ++l) {
         sgl_sample_params pl = *p;
         pl.hop = l;
         const int64_t s_max = worst_slots(S0, l, p->fanout);
-        rc = run_hop(g, sn, stt, l == 0 ? &spec : nullptr, s_max, S_dev, &pl, &outs[l], ws, ws_bytes, st);
+        rc = run_hop(g, sn, stt, l == 0 ? &spec : nullptr, s_max, S_dev, &pl, &outs[l], ws, carry ? hop_ws : ws_bytes, st,
+                     (carry && l > 0) ? carry_buf[(l - 1) & 1] : nullptr, (carry && l + 1 < layers) ? carry_buf[l & 1] : nullptr);
         if (rc != SGL_OK) return rc;
         sn = outs[l].neighbors;
         stt = outs[l].neighbors_ts;

@@ -307,3 +307,37 @@ extern "C" int32_t sgl_chunk_index_build(int64_t n, int64_t num_chunks, const in
     SGL_HIP_TRY(hipStreamSynchronize(st));
     return SGL_OK;
 }
+
+namespace sgl {
+namespace {
+
+// hop_hint[e] = first position in row col[e] whose timestamp is >= ts[e]
+__global__ __launch_bounds__(BLOCK) void hop_hint_kernel(sgl_tcsr g, int64_t* __restrict__ hint) {
+    for (int64_t e = (int64_t)blockIdx.x * BLOCK + threadIdx.x; e < g.m; e += (int64_t)gridDim.x * BLOCK) {
+        const int64_t v = g.col[e], t = g.ts[e];
+        int64_t lo = -1;
+        if (v >= 0 && v < g.n) {
+            lo = g.row_ptr[v];
+            int64_t hi = g.row_ptr[v + 1];
+            while (lo < hi) {
+                const int64_t mid = lo + ((hi - lo) >> 1);
+                if (g.ts[mid] < t) lo = mid + 1; else hi = mid;
+            }
+        }
+        hint[e] = lo;
+    }
+}
+
+}  // namespace
+}  // namespace sgl
+
+extern "C" int32_t sgl_tcsr_hop_hint_build(const sgl_tcsr* g, int64_t* hop_hint, void* stream) {
+    if (!g || g->n < 0 || g->m < 0 || !g->row_ptr) return fail(SGL_EINVAL, "tcsr_hop_hint_build: NULL graph");
+    if (g->m == 0) return SGL_OK;
+    if (!g->col || !g->ts || !hop_hint) return fail(SGL_EINVAL, "tcsr_hop_hint_build: NULL array");
+    int64_t blocks = ceil_div<int64_t>(g->m, BLOCK);
+    if (blocks > (1 << 20)) blocks = 1 << 20;
+    hipLaunchKernelGGL(hop_hint_kernel, dim3((unsigned)blocks), dim3(BLOCK), 0, as_stream(stream), *g, hop_hint);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}

@@ -5,7 +5,7 @@ header declares.  The product library exports them as ``sgl_*``.
 """
 import ctypes as C
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
@@ -19,7 +19,7 @@ i32, i64, u64, vp, sz = C.c_int32, C.c_int64, C.c_uint64, C.c_void_p, C.c_size_t
 
 
 class TCSR(C.Structure):
-    _fields_ = [("n", i64), ("m", i64), ("row_ptr", vp), ("col", vp), ("ts", vp), ("eid", vp)]
+    _fields_ = [("n", i64), ("m", i64), ("row_ptr", vp), ("col", vp), ("ts", vp), ("eid", vp), ("hop_hint", vp)]
 
 
 class SampleParams(C.Structure):
@@ -62,6 +62,7 @@ PROTOTYPES = {
     "tcsr_build_workspace_bytes": (sz, [i64, i64]),
     "tcsr_build": (i32, [i64, i64, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]),
     "tcsr_validate": (i32, [P(TCSR), vp, sz, vp]),
+    "tcsr_hop_hint_build": (i32, [P(TCSR), vp, vp]),
     "sample_hop_workspace_bytes": (sz, [i64]),
     "sample_hop": (i32, [P(TCSR), vp, vp, i64, vp, P(SampleParams), P(HopOut), vp, sz, vp]),
     "sample_khop_workspace_bytes": (sz, [i64, i32, i32]),

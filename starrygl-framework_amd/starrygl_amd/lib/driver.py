@@ -65,11 +65,11 @@ class TorchBackend:
 class TCSRArrays:
     """Owner of the four T-CSR arrays plus the ABI view of them."""
 
-    def __init__(self, backend, n, row_ptr, col, ts, eid):
+    def __init__(self, backend, n, row_ptr, col, ts, eid, hop_hint=None):
         self.n, self.m = int(n), int(col.shape[0])
-        self.row_ptr, self.col, self.ts, self.eid = row_ptr, col, ts, eid
+        self.row_ptr, self.col, self.ts, self.eid, self.hop_hint = row_ptr, col, ts, eid, hop_hint
         self.view = TCSR(self.n, self.m, backend.ptr(row_ptr), backend.ptr(col),
-                         backend.ptr(ts), backend.ptr(eid))
+                         backend.ptr(ts), backend.ptr(eid), backend.ptr(hop_hint))
 
 
 class HopResult:
@@ -161,6 +161,15 @@ class HotPath:
         if validate:
             ws, wsb = self._workspace(256)
             self._ck(self.lib.tcsr_validate(C.byref(g.view), self.be.ptr(ws), wsb, self.be.stream()))
+        return g
+
+    def build_hop_hint(self, g):
+        """Attach the next-hop index to the T-CSR `g` (8 bytes per edge, one search per edge, once):
+        the sampler then finds the windows of the slots of hops >= 1 without searching."""
+        hint = self.be.empty(g.m)
+        self._ck(self.lib.tcsr_hop_hint_build(C.byref(g.view), self.be.ptr(hint), self.be.stream()))
+        g.hop_hint = hint
+        g.view.hop_hint = self.be.ptr(hint)
         return g
 
     # ----------------------------------------------------------- sampling

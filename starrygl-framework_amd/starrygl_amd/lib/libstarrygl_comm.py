@@ -277,10 +277,11 @@ class _Future:
         return self._val
 
 
-def from_edge_index(n, chunk_size, src, dst, ts, eid, mapper=None, stream=0, rank=0):
+def from_edge_index(n, chunk_size, src, dst, ts, eid, mapper=None, stream=0, rank=0, hop_hint=True):
     """Build the T-CSR on device `rank` (export.cu:229-250).  Raises
     RuntimeError-family exceptions for non-int64 input and out-of-range ids
-    (sample.cu.hpp:1001-1020, 1043-1062)."""
+    (sample.cu.hpp:1001-1020, 1043-1062).  `hop_hint` (not in the reference): also build the
+    next-hop index (8 bytes per edge) that spares the sampler the searches of hops >= 1."""
     device = torch.device("cuda", int(rank))
     hp = hot_path(device)
     n, chunk_size = int(n), int(chunk_size)
@@ -295,4 +296,6 @@ def from_edge_index(n, chunk_size, src, dst, ts, eid, mapper=None, stream=0, ran
             raise IndexError("row_chunk_mapper names a chunk outside [0, chunk_size)")   # sample.cu.hpp:1059-1062
     with torch.cuda.device(device):
         g = hp.tcsr_build(n, src, dst, ts, eid)
+        if hop_hint:
+            hp.build_hop_hint(g)
     return CUDAGraph(hp, g, chunk_size, mapper, stream if isinstance(stream, torch.cuda.Stream) else None)

@@ -31,6 +31,9 @@ def _one_case(seed, oracle, hot):
     for f in ("row_ptr", "col", "ts", "eid"):
         assert np.array_equal(np_of(getattr(dgb, f)), getattr(g, f)), ("tcsr_build", f)
     dg = mirror_graph(hot, g)
+    if seed % 2:        # every other case samples with the graph's next-hop index attached
+        hot.build_hop_hint(dg)
+        assert np.array_equal(np_of(dg.hop_hint), oracle.build_hop_hint(g).hop_hint), "hop_hint"
     # sampling
     S_pos = int(rng.choice([0, 1, 5, 200, 3000, 20000]))
     N_neg = int(rng.choice([0, 1, 77, 2000]))

@@ -306,3 +306,27 @@ def test_driver_rejects_arrays_it_cannot_pass_as_pointers(oracle, hot):
     with pytest.raises(TypeError):
         hot.gather(hot.cache(16, torch.zeros((500, 4), device=roots.device)), roots.int(),
                    torch.empty((40, 4), device=roots.device))
+
+
+@pytest.mark.parametrize("sample_type", ["recent", "uniform"])
+def test_next_hop_index_gives_the_same_samples(oracle, hot, sample_type):
+    """With sgl_tcsr.hop_hint the slots of hops >= 1 take the end of their window from the index instead
+    of searching.  The index itself equals its definition (first position in row col[e] with ts >= ts[e],
+    restated by a linear scan); sampling with it equals the oracle in the single-launch kernel, in the
+    multi-launch path over two and three hops, and for the parameter sets that must ignore it
+    (windows that include the slot's time, uniform slots that keep the root's time)."""
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 3_000, 90_000, 1.15, 5_000, 47, hub=20_000)   # 5000 times: many ties
+    hot.build_hop_hint(dg)
+    assert np.array_equal(np_of(dg.hop_hint), oracle.build_hop_hint(g).hop_hint)
+    rng = np.random.default_rng(21)
+    for S0, layers, fanout in ((700, 2, 10), (40_000, 2, 5), (3_000, 3, 6), (300, 2, 17), (5, 3, 3)):
+        n_neg = S0 // 3
+        roots = rng.integers(0, g.n, S0 - n_neg).astype(np.int64)
+        root_ts = rng.integers(0, 5_000, S0 - n_neg).astype(np.int64)
+        ts_ptr = np.arange(S0 - n_neg + 1, dtype=np.int64)
+        neg = rng.integers(0, g.n, n_neg).astype(np.int64)
+        neg_ts = rng.integers(0, 5_000, n_neg).astype(np.int64)
+        for kw in (dict(), dict(allowed_offset=300), dict(equal_root_time=True), dict(keep_root_time=True),
+                   dict(replace=True)):
+            _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, neg, neg_ts, layers, sample_type=sample_type,
+                      fanout=fanout, seed=5, **kw)

@@ -284,3 +284,21 @@ def test_time_encode_closed_form(oracle):
     # a fused multiply-add would give different bits somewhere on this input
     fused = np.cos((w[None, :].astype(np.float64) * x[:, None].astype(np.float64) + b[None, :]).astype(np.float32).astype(np.float64)).astype(np.float32)
     assert not np.array_equal(fused, y)
+
+
+def test_next_hop_index_is_searchsorted_per_edge(oracle):
+    """hop_hint[e] = first position in row col[e] with ts >= ts[e] (numpy's searchsorted on the row slice),
+    -1 where the destination is no node; the samples do not depend on it."""
+    rng = np.random.default_rng(5)
+    n, m = 60, 3000
+    src, dst, ts = rng.integers(0, n, m), rng.integers(0, n, m), rng.integers(0, 40, m)    # many equal timestamps
+    g = host_graph(oracle, n, src, dst, ts)
+    before = oracle.sample_khop(g, np.arange(n), np.arange(n + 1), np.full(n, 25), np.zeros(0, np.int64),
+                                np.zeros(0, np.int64), 2, oracle.params("recent", 4))
+    oracle.build_hop_hint(g)
+    want = np.array([g.row_ptr[v] + np.searchsorted(g.ts[g.row_ptr[v]: g.row_ptr[v + 1]], t, side="left")
+                     for v, t in zip(g.col, g.ts)])
+    assert np.array_equal(g.hop_hint, want)
+    after = oracle.sample_khop(g, np.arange(n), np.arange(n + 1), np.full(n, 25), np.zeros(0, np.int64),
+                               np.zeros(0, np.int64), 2, oracle.params("recent", 4))
+    assert np.array_equal(before.hops[1].neighbors_eid, after.hops[1].neighbors_eid)
