@@ -22,6 +22,8 @@ constexpr int UNROLL = 4;
 // device value, and launching the worst-case number of blocks costs ~0.2 ns per dead
 // block (10 us for 50 000 of them), more than the whole copy of a small batch.
 constexpr int MAX_GRID = 4096;
+// gather_multi writes its rows past the caches from this many output bytes (worst case) on
+constexpr int64_t NT_STORE_MIN_BYTES = 64ll << 20;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -134,6 +136,12 @@ struct MultiArgs {
 
 // Several gathers in one launch: every block walks its grid-stride share of the
 // tiles of segment 0, then of segment 1, ...  16-byte chunks only.
+// NT_STORE: the output rows are written with non-temporal stores.  The kernel itself runs as
+// fast either way (5.5 TB/s on 257 MB); what changes is that ~130 MB of rows nobody reads
+// again soon do not displace the graph arrays from the last-level cache: the sampler and
+// unique kernels of the neighbouring batches finish sooner (whole step -4 % with one batch
+// in flight, -8 % with three).
+template <bool NT_STORE>
 __global__ __launch_bounds__(BLOCK) void gather_multi_kernel(MultiArgs m) {
     extern __shared__ const char* s_src[];
 #pragma unroll 1
@@ -170,7 +178,10 @@ __global__ __launch_bounds__(BLOCK) void gather_multi_kernel(MultiArgs m) {
 #pragma unroll
                 for (int u = 0; u < UNROLL; ++u) {
                     const int32_t lc = base + u * BLOCK + threadIdx.x;
-                    if (lc < total) dst[lc] = val[u];
+                    if (lc < total) {
+                        if (NT_STORE) __builtin_nontemporal_store(val[u], dst + lc);
+                        else dst[lc] = val[u];
+                    }
                 }
             }
         }
@@ -298,7 +309,7 @@ extern "C" int32_t sgl_gather_multi(int32_t T, const sgl_gather_seg* segs, void*
     if (T > SGL_GATHER_MAX_SEGMENTS) return fail(SGL_ENOTSUP, "gather_multi: more than %d segments", SGL_GATHER_MAX_SEGMENTS);
     MultiArgs m;
     m.T = 0;
-    int64_t max_rpb = 1, want_blocks = 1;
+    int64_t max_rpb = 1, want_blocks = 1, out_bytes = 0;
     for (int32_t t = 0; t < T; ++t) {
         const sgl_gather_seg& g = segs[t];
         int32_t rc;
@@ -318,10 +329,12 @@ extern "C" int32_t sgl_gather_multi(int32_t T, const sgl_gather_seg* segs, void*
         max_rpb = rpb > max_rpb ? rpb : max_rpb;
         const int64_t b = ceil_div<int64_t>(g.N_max, rpb);
         want_blocks = b > want_blocks ? b : want_blocks;
+        out_bytes += g.N_max * g.cache->row_bytes;
     }
     if (m.T == 0) return SGL_OK;
     if (want_blocks > MAX_GRID) want_blocks = MAX_GRID;
-    hipLaunchKernelGGL(gather_multi_kernel, dim3((unsigned)want_blocks), dim3(BLOCK), (size_t)max_rpb * sizeof(char*),
+    auto kern = out_bytes >= NT_STORE_MIN_BYTES ? gather_multi_kernel<true> : gather_multi_kernel<false>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)want_blocks), dim3(BLOCK), (size_t)max_rpb * sizeof(char*),
                        as_stream(stream), m);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
