@@ -170,3 +170,29 @@ def test_gather_multi_equals_single_gathers(oracle, hot):
     bad = hot.gather_plan([(c3, d_ids[2], torch.zeros((7, 3), device="cuda"), None, None)])
     with pytest.raises(RuntimeError):
         hot.gather_multi(bad)
+
+
+def test_gather_multi_large_output(hot):
+    """Outputs of 64 MB and more take the multi gather's streaming-store path: same bytes as
+    torch.index_select, a device-side count still bounds a segment, and the rows are visible to a
+    kernel that reads them right after on the same stream."""
+    g = torch.Generator(device="cuda").manual_seed(5)
+    t_edge = torch.randn((200_000, 172), device="cuda", generator=g)
+    t_node = torch.randn((50_000, 100), device="cuda", generator=g)
+    ids_e = torch.randint(0, 200_000, (120_000,), device="cuda", generator=g)      # 120 000 x 688 B = 82.6 MB
+    ids_n = torch.randint(0, 50_000, (30_000,), device="cuda", generator=g)
+    live_n = torch.tensor([17_003], dtype=torch.int64, device="cuda")
+    out_e = torch.empty((120_000, 172), device="cuda")
+    out_n = torch.zeros((30_000, 100), device="cuda")
+    plan = hot.gather_plan([(hot.cache(400, t_node), ids_n, out_n, None, live_n),
+                            (hot.cache(688, t_edge), ids_e, out_e, None, None)])
+    for _ in range(2):      # the second launch overwrites rows that the first one streamed out
+        hot.gather_multi(plan)
+        total = out_e.sum(dtype=torch.float64) + out_n.sum(dtype=torch.float64)       # reads the rows right away
+        assert torch.equal(out_e, t_edge.index_select(0, ids_e))
+        assert torch.equal(out_n[:17_003], t_node.index_select(0, ids_n[:17_003])) and not out_n[17_003:].any()
+        want = t_edge.index_select(0, ids_e).sum(dtype=torch.float64) + t_node.index_select(0, ids_n[:17_003]).sum(dtype=torch.float64)
+        assert float(total) == float(want)
+        ids_e = ids_e.flip(0).contiguous()
+        plan = hot.gather_plan([(hot.cache(400, t_node), ids_n, out_n, None, live_n),
+                                (hot.cache(688, t_edge), ids_e, out_e, None, None)])
