@@ -682,11 +682,17 @@ struct Fused2Args {
     int32_t spin_limit;         // polls of one descriptor before a lane gives up
 };
 
-__global__ void fused_clear_kernel(unsigned long long* desc, int n, int64_t* counts1, int64_t* counts1_b) {
+// Zeroes the block descriptors and the two error counts of a call (of both calls of a pair):
+// counts0[2] takes atomic maxima (bad root slots from the last block, the poison value from any
+// block that gave up its wait - in either order the poison stays), counts1[2] atomic adds.
+__global__ void fused_clear_kernel(unsigned long long* desc, int n, int64_t* counts0, int64_t* counts1,
+                                   int64_t* counts0_b, int64_t* counts1_b) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) desc[i] = 0ull;
     if (i == 0) {
+        counts0[2] = 0;
         counts1[2] = 0;
+        if (counts0_b != nullptr) counts0_b[2] = 0;
         if (counts1_b != nullptr) counts1_b[2] = 0;
     }
 }
@@ -882,13 +888,15 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
         gave_up |= s_gave[q];
     }
     if (threadIdx.x == 0) {
-        if (gave_up) a.counts[2] = INT64_MAX;         // poisoned: reading the result reports an error
+        // poisoned: reading the result reports an error (a maximum, so that the last block's count
+        // of bad slots cannot replace it, whichever block writes first)
+        if (gave_up) atomicMax(reinterpret_cast<long long*>(&a.counts[2]), (long long)INT64_MAX);
         if (b == nb - 1) {            // totals of the call
             const uint64_t tot = prefix + btotal;
             const int64_t E0 = (int64_t)((tot >> SH_E0) & M_E0), E1 = (int64_t)(tot & M_E1);
             a.counts[0] = S;
             a.counts[1] = E0;
-            if (!gave_up) a.counts[2] = (int64_t)((tot >> SH_BAD) & M_BAD);
+            atomicMax(reinterpret_cast<long long*>(&a.counts[2]), (long long)((tot >> SH_BAD) & M_BAD));
             a.root_start_ptr[S] = E0;
             a.root_end_ptr[S] = E0;
             f.counts1[0] = E0;
@@ -1134,7 +1142,7 @@ int32_t run_fused2(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, const sg
     if (!ar.ok()) return fail(SGL_ENOMEM, "sample: workspace too small");
     const Fused2Args f = fused2_args(g, spec, S0, p, outs, desc);
     hipLaunchKernelGGL(fused_clear_kernel, dim3((unsigned)ceil_div<int>(blocks, BLOCK)), dim3(BLOCK), 0, st, f.desc, blocks,
-                       f.counts1, (int64_t*)nullptr);
+                       f.h.counts, f.counts1, (int64_t*)nullptr, (int64_t*)nullptr);
     SGL_LAUNCH_CHECK();
     if (p->type == SGL_SAMPLE_UNIFORM)
         hipLaunchKernelGGL(fused2_kernel<true>, dim3((unsigned)blocks), dim3(BLOCK), pick_lds_bytes(p->fanout), st, f);
@@ -1157,7 +1165,7 @@ int32_t run_fused2_pair(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, con
     const Fused2Args fr = fused2_args(g, spec, S0, p_rec, outs_rec, desc);
     const Fused2Args fu = fused2_args(g, spec, S0, p_uni, outs_uni, desc + blocks);
     hipLaunchKernelGGL(fused_clear_kernel, dim3((unsigned)ceil_div<int>(2 * blocks, BLOCK)), dim3(BLOCK), 0, st, desc,
-                       2 * blocks, fr.counts1, fu.counts1);
+                       2 * blocks, fr.h.counts, fr.counts1, fu.h.counts, fu.counts1);
     SGL_LAUNCH_CHECK();
     hipLaunchKernelGGL(fused2_pair_kernel, dim3((unsigned)(2 * blocks)), dim3(BLOCK), pick_lds_bytes(p_uni->fanout), st,
                        fr, fu);
