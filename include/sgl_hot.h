@@ -179,7 +179,11 @@ int32_t sgl_sample_hop(const sgl_tcsr* g,
  * ([S_pos + N_neg] each).  Hop l+1 slots are hop l's (neighbors, neighbors_ts),
  * one slot per sampled edge, no dedup between hops.  p->hop is ignored; hop l
  * draws from RNG stream l.  outs[l].capacity_slots must be >= the worst-case
- * slot count of hop l ((S_pos+N_neg) * fanout^l). */
+ * slot count of hop l ((S_pos+N_neg) * fanout^l).
+ * Two-hop calls of up to 32768 root slots and fanout <= 16 run as one launch
+ * whose blocks wait (bounded, sgl_set_wait_limit) for the edge totals of the
+ * blocks before them; should a block ever give up, outs[0].counts[2] reads
+ * INT64_MAX and the outputs of the call are void. */
 size_t  sgl_sample_khop_workspace_bytes(int64_t S0, int32_t layers,
                                         int32_t fanout);
 int32_t sgl_sample_khop(const sgl_tcsr* g,
