@@ -360,6 +360,8 @@ def main():
                     help="unique runs its own marking pass instead of the sampler recording the ids it emits")
     ap.add_argument("--no-hop-hint", action="store_true",
                     help="sample without the graph's next-hop index (every slot of hops >= 1 searches its window)")
+    ap.add_argument("--no-root-hint", action="store_true",
+                    help="batches do not carry the window ends of their positive roots (every root is searched)")
     ap.add_argument("--pipelines", type=int, default=3,
                     help="independent copies of the step (own buffers, graph and stream) that take the batches of the "
                          "timed region in turn, as a loader with that many batches in flight does; 1 = one batch at a time")
@@ -429,6 +431,17 @@ def main():
 
     p_rec = hot.params("recent", k)
     p_uni = hot.params("uniform", k, seed=20242)
+    # the loader's part of the root hints: where the window of every positive root (an endpoint of a
+    # batch event, at the event's time) ends, looked up once for the whole stream of batches; a batch
+    # then carries its 2B values beside its roots and the sampler searches for the negatives only
+    use_root_hint = not args.no_root_hint
+    torch.cuda.synchronize()
+    t_h = time.perf_counter()
+    root_hint = (hot.window_end(dg, roots.reshape(-1), root_ts.reshape(-1)).view(NB, -1) if use_root_hint
+                 else torch.zeros((NB, 0), dtype=torch.int64, device=dev))
+    torch.cuda.synchronize()
+    if use_root_hint:
+        log(f"[setup] root hints of {root_hint.numel()} batch roots looked up in {(time.perf_counter() - t_h) * 1e3:.2f} ms")
     # every device-side count of a step lives in one array, so that one add accumulates them all
     live = torch.zeros(14, dtype=torch.int64, device=dev)     # recent S,E,bad x2 | uniform S,E,bad x2 | U_total, U_before
     kr, ku = hot.khop_buffers(S0, 2, k, counts=live[0:6]), hot.khop_buffers(S0, 2, k, counts=live[6:12])
@@ -445,9 +458,14 @@ def main():
 
     # static input buffer: a step copies its batch here (one D2D copy of the packed roots, root
     # times, negatives and their times), the stages read views of it
-    packed = torch.cat([roots, root_ts, neg, neg_ts], dim=1).contiguous()
+    packed = torch.cat([roots, root_ts, neg, neg_ts, root_hint], dim=1).contiguous()
     s_all = torch.empty_like(packed[0])
-    s_roots, s_root_ts, s_neg, s_neg_ts = torch.split(s_all, [roots.shape[1], root_ts.shape[1], neg.shape[1], neg_ts.shape[1]])
+    split_sizes = [roots.shape[1], root_ts.shape[1], neg.shape[1], neg_ts.shape[1], root_hint.shape[1]]
+    s_roots, s_root_ts, s_neg, s_neg_ts, s_hint = torch.split(s_all, split_sizes)
+    if use_root_hint:
+        p_rec, p_uni_in = hot.with_root_hint(p_rec, s_hint), hot.with_root_hint(p_uni, s_hint)
+    else:
+        p_uni_in = p_uni
     acc = torch.zeros(14, dtype=torch.int64, device=dev)  # running sums of `live`
     ACC = [1, 4, 7, 10, 12]                               # E0, E1 (recent), E0, E1 (uniform), U
 
@@ -479,10 +497,10 @@ def main():
             hot.gather(edge_cache, kr.hops[1].neighbors_eid, e_out[1], N_dev=kr.hops[1].counts[1:2])
 
     def st_uniform():
-        hot.sample_khop(dg, s_roots, ts_ptr, s_root_ts, s_neg, s_neg_ts, 2, p_uni, finalize=False, out=ku)
+        hot.sample_khop(dg, s_roots, ts_ptr, s_root_ts, s_neg, s_neg_ts, 2, p_uni_in, finalize=False, out=ku)
 
     def st_samplers():      # both 2-hop samplers of the step in one library call (one launch)
-        hot.sample_khop_multi(dg, s_roots, ts_ptr, s_root_ts, s_neg, s_neg_ts, 2, [p_rec_mark, p_uni], [kr, ku])
+        hot.sample_khop_multi(dg, s_roots, ts_ptr, s_root_ts, s_neg, s_neg_ts, 2, [p_rec_mark, p_uni_in], [kr, ku])
 
     def st_account():
         acc.add_(live)
@@ -523,15 +541,16 @@ def main():
         P.node_out = torch.empty((min(total_ids, n), 100), device=dev)
         P.e_out = [torch.empty((S0 * k, 172), device=dev), torch.empty((S0 * k * k, 172), device=dev)]
         P.s_all = torch.empty_like(packed[0])
-        v = torch.split(P.s_all, [roots.shape[1], root_ts.shape[1], neg.shape[1], neg_ts.shape[1]])
-        P.p_rec = hot.marking(p_rec, P.state)
+        v = torch.split(P.s_all, split_sizes)
+        P.p_rec = hot.marking(hot.with_root_hint(p_rec, v[4]) if use_root_hint else p_rec, P.state)
+        P.p_uni = hot.with_root_hint(p_uni, v[4]) if use_root_hint else p_uni
         P.multi = hot.gather_plan([(node_cache, P.ubuf, P.node_out, None, P.U[0:1]),
                                    (edge_cache, P.kr.hops[0].neighbors_eid, P.e_out[0], None, P.kr.hops[0].counts[1:2]),
                                    (edge_cache, P.kr.hops[1].neighbors_eid, P.e_out[1], None, P.kr.hops[1].counts[1:2])])
         P.stream = stream
 
         def step():
-            hot.sample_khop_multi(dg, v[0], ts_ptr, v[1], v[2], v[3], 2, [P.p_rec, p_uni], [P.kr, P.ku])
+            hot.sample_khop_multi(dg, v[0], ts_ptr, v[1], v[2], v[3], 2, [P.p_rec, P.p_uni], [P.kr, P.ku])
             hot.unique_compact([P.kr.slot_node0, P.kr.hops[0].neighbors, P.kr.hops[1].neighbors], _abi.UNIQUE_SORTED,
                                P.state, True, lens_dev=[S0_dev, P.kr.hops[0].counts[1:2], P.kr.hops[1].counts[1:2]],
                                out_arrays=P.local, finalize=False, unique_out=P.ubuf, U_out=P.U, premarked=True)
@@ -546,13 +565,14 @@ def main():
             with torch.cuda.graph(P.graph, stream=P.stream):
                 step()
 
-        def run(b):
-            with torch.cuda.stream(P.stream):
-                P.s_all.copy_(packed[b], non_blocking=True)
-                P.graph.replay()
+        def run(b):          # (set_stream, not the context manager: the host's share of a step is what bounds
+            torch.cuda.set_stream(P.stream)      # the loop once the GPU needs less than ~0.07 ms per step)
+            P.s_all.copy_(batch_rows[b], non_blocking=True)
+            P.graph.replay()
         P.run = run
         return P
 
+    batch_rows = list(packed.unbind(0))
     K, W = args.steps, args.warmup
     stage_inputs(0)
     body()
@@ -624,8 +644,10 @@ def main():
             stage_inputs(b)
             run_step()
 
+    main_stream = torch.cuda.current_stream()
     for i in range(W):
         run_batch(i, i % NB)
+    torch.cuda.set_stream(main_stream)
     torch.cuda.synchronize()
     acc.zero_()
     for P in pipes:
@@ -638,6 +660,7 @@ def main():
     host_submit = time.perf_counter() - t_start      # the host's share: K batch copies + K graph launches enqueued
     torch.cuda.synchronize()
     wall = time.perf_counter() - t_start
+    torch.cuda.set_stream(main_stream)
     tot = (sum(P.acc for P in pipes) if pipes else acc).cpu().numpy()[ACC].astype(np.float64)
     one_in_flight = None
     if pipes:                  # the same K steps with one batch in flight at a time, for comparison
@@ -833,25 +856,28 @@ def main():
     # sampler throughput when several mini-batches are sampled by one call (what a loader with a
     # prefetch queue, or an AsyncGraphBlob of several windows, can do): same graph, same batches
     scaling = []
+    p_plain = hot.params("recent", k)
     REPS = 8                # calls per measurement, each over different batches (a repeated batch would find its rows in L2)
     cap = torch.cuda.Stream()
     for mult in (1, 4, 16, 64):
         ins = []
         for rep in range(REPS):
             idx = [(W + rep * mult + i) % NB for i in range(mult)]
-            ins.append((torch.cat([roots[i] for i in idx]), torch.cat([root_ts[i] for i in idx]),
-                        torch.cat([neg[i] for i in idx]), torch.cat([neg_ts[i] for i in idx])))
+            r_ = torch.cat([roots[i] for i in idx])
+            ins.append((r_, torch.cat([root_ts[i] for i in idx]),
+                        torch.cat([neg[i] for i in idx]), torch.cat([neg_ts[i] for i in idx]),
+                        hot.with_root_hint(p_plain, torch.cat([root_hint[i] for i in idx])) if use_root_hint else p_plain))
         tp_ = torch.arange(ins[0][0].numel() + 1, dtype=torch.int64, device=dev)
         kb = hot.khop_buffers(S0 * mult, 2, k)
         e_ = 0.0
-        for r_, rt_, n_, nt_ in ins:             # untimed: the edges each call samples
-            hot.sample_khop(dg, r_, tp_, rt_, n_, nt_, 2, p_rec, finalize=False, out=kb)
+        for r_, rt_, n_, nt_, pp_ in ins:        # untimed: the edges each call samples
+            hot.sample_khop(dg, r_, tp_, rt_, n_, nt_, 2, pp_, finalize=False, out=kb)
             cnt = kb.counts.cpu().numpy()
             e_ += float(cnt[1] + cnt[4]) / REPS
 
         def calls():
-            for r_, rt_, n_, nt_ in ins:
-                hot.sample_khop(dg, r_, tp_, rt_, n_, nt_, 2, p_rec, finalize=False, out=kb)
+            for r_, rt_, n_, nt_, pp_ in ins:
+                hot.sample_khop(dg, r_, tp_, rt_, n_, nt_, 2, pp_, finalize=False, out=kb)
         ms_eager = _time_launches(torch, calls, reps=1, warm=1) / REPS      # launched from the host, call by call
         # the same calls as one HIP graph: the GPU's time per call, without the host's launch cost
         cap.wait_stream(torch.cuda.current_stream())
@@ -904,7 +930,8 @@ def main():
         "config": {"workload": "configs[1]: 1M nodes / 20M edges Zipf(1.1) out-degree, batches of 4000 events + 4000 "
                                "negatives (12000 roots): 2-hop recent 10x10 + unique + node/edge gather + 2-hop uniform 10x10",
                    "nodes": n, "edges": m, "roots_per_batch": S0, "fanout": [k, k],
-                   "node_feat": "100xfp32", "edge_feat": "172xfp32" if has_edge_feat else None},
+                   "node_feat": "100xfp32", "edge_feat": "172xfp32" if has_edge_feat else None,
+                   "next_hop_index": not args.no_hop_hint, "root_hints_in_batch": use_root_hint},
         "edges_per_step": {"recent": float(np.mean(e_rec)), "uniform": float(np.mean(e_uni))},
         "mean_rows_per_step": {"gather_node_feat": float(np.mean(cl[:, 4])), "gather_edge_feat_hop1": float(np.mean(cl[:, 0])),
                                "gather_edge_feat_hop2": float(np.mean(cl[:, 1]))},

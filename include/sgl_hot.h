@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define SGL_ABI_VERSION 3
+#define SGL_ABI_VERSION 4
 
 /* ------------------------------------------------------------------ status */
 #define SGL_OK        0
@@ -86,6 +86,17 @@ typedef struct sgl_tcsr {
  * (find_time_range, sample.cu.hpp:264-295). */
 int32_t sgl_tcsr_hop_hint_build(const sgl_tcsr* g, int64_t* hop_hint, void* stream);
 
+/* out[i] = position in row node[i] of the first edge whose timestamp is >= t[i]
+ * (row_ptr[node[i]+1] if there is none, -1 for a node outside [0,n)), i < N:
+ * where the strictly-before window of the slot (node[i], t[i]) ends.  The same
+ * search as find_time_range's upper end (sample.cu.hpp:264-295), as a batch:
+ * a loader runs it once over the event stream it is going to train on -
+ * (src, ts) and (dst, ts) of every event - and hands the values of a batch's
+ * roots to the sampler (sgl_sample_params.root_hint), which then searches for
+ * the negatives only. */
+int32_t sgl_window_end(const sgl_tcsr* g, const int64_t* node, const int64_t* t,
+                       int64_t N, int64_t* out, void* stream);
+
 /* Build a T-CSR from a COO edge list (replaces from_edge_index / Graph::Graph,
  * export.cu:229-250, sample.cu.hpp:985-1185).  `eid` may be NULL (= 0..m-1).
  * Output order is the stable sort by (src, ts, eid).  Synchronous: returns
@@ -135,6 +146,13 @@ typedef struct sgl_sample_params {
      * arrays, with reset = 1 and mode SGL_UNIQUE_SORTED | SGL_UNIQUE_PREMARKED. */
     void*    mark_state;      /* NULL: off                                     */
     int64_t  mark_universe;
+    /* Optional, sgl_sample_khop / sgl_sample_khop_multi only (no counterpart in
+     * the reference): root_hint[s], s < S_pos, is where the window of positive
+     * slot s ends - the value sgl_window_end gives for (root of s, root_ts[s]) -
+     * or -1 (search).  Used when equal_root_time == 0; values are clamped to the
+     * root's row, so a wrong hint gives a wrong sample, never a stray access.
+     * Negative roots are always searched. */
+    const int64_t* root_hint; /* device int64[S_pos], or NULL                  */
 } sgl_sample_params;
 
 /* One hop's result, caller-allocated (replaces TemporalNeighbor,

@@ -163,6 +163,19 @@ int32_t sglo_tcsr_hop_hint_build(const sgl_tcsr* g, int64_t* hop_hint, void* str
     return SGL_OK;
 }
 
+/* Where the strictly-before window of (node[i], t[i]) ends: the upper end of
+ * find_time_range (sample.cu.hpp:264-295) for a batch of slots. */
+int32_t sglo_window_end(const sgl_tcsr* g, const int64_t* node, const int64_t* t, int64_t N, int64_t* out,
+                        void* stream) {
+    (void)stream;
+    if (!g || g->n < 0 || g->m < 0 || !g->row_ptr || N < 0) return fail(SGL_EINVAL, "window_end: null/negative");
+    if (N > 0 && (!node || !t || !out || (g->m > 0 && !g->ts))) return fail(SGL_EINVAL, "window_end: null array");
+    for (int64_t i = 0; i < N; ++i) {
+        int64_t v = node[i];
+        out[i] = (v >= 0 && v < g->n) ? lower_bound_ts(g->ts, g->row_ptr[v], g->row_ptr[v + 1], t[i]) : -1;
+    }
+    return SGL_OK;
+}
 
 /* Candidate window of a slot.  Reference: find_time_range
  * (sample.cu.hpp:264-295) called with (ts - allowed_offset or 0,
@@ -358,6 +371,15 @@ int32_t sglo_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* roots,
     for (int64_t i = 0; i < N_neg; ++i) {
         slot_node0[S_pos + i] = neg_roots[i]; slot_ts0[S_pos + i] = neg_ts[i];
     }
+    /* root_hint is an accelerator of the kernels: the oracle searches, and as the checker it
+     * refuses a hint that is not the window end it finds itself */
+    if (p->root_hint && !p->equal_root_time)
+        for (int64_t s = 0; s < S_pos; ++s) {
+            int64_t v = slot_node0[s], h = p->root_hint[s];
+            if (h < 0 || v < 0 || v >= g->n) continue;
+            if (h != lower_bound_ts(g->ts, g->row_ptr[v], g->row_ptr[v + 1], slot_ts0[s]))
+                return fail(SGL_EINVAL, "sample_khop: a root_hint entry is not the window end");
+        }
     const int64_t* sn = slot_node0; const int64_t* st = slot_ts0;
     int64_t S = S_pos + N_neg;
     for (int32_t l = 0; l < layers; ++l) {

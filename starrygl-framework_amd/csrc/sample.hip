@@ -50,6 +50,8 @@ struct HopArgs {
     const int64_t* slot_hint;  // per explicit slot: where its window ends (the index entry of the edge the slot
                                // came from), or nullptr: search
     int64_t* hint_out;   // per emitted edge: its index entry, for the next hop's slots; or nullptr
+    const int64_t* root_hint;  // derived slots only: per positive slot, where its window ends according to the
+                               // caller (sgl_sample_params.root_hint; -1: search), or nullptr
     // slots: explicit (slot_node/slot_ts), or - when roots != nullptr - derived from
     // R positive roots over ts_ptr/root_ts followed by N_neg negatives, and then
     // written to slot_node_out/slot_ts_out
@@ -181,6 +183,16 @@ __device__ __forceinline__ void load_slot(const HopArgs& a, int64_t s, int64_t* 
     *v = a.roots[lo];
 }
 
+// Where the window of derived slot s ends according to the caller, or -1 (search)
+__device__ __forceinline__ int64_t root_hint_of(const HopArgs& a, int64_t s) {
+    return (a.root_hint != nullptr && s < a.S_pos) ? a.root_hint[s] : -1;
+}
+
+// A caller's window end, kept inside the row [rs, re]
+__device__ __forceinline__ int64_t clamp_to_row(int64_t h, int64_t rs, int64_t re) {
+    return h < rs ? rs : (h > re ? re : h);
+}
+
 template <int G>
 __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
     constexpr int SPB = BLOCK / G;  // slots per block iteration
@@ -194,9 +206,12 @@ __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
     // count is: the slot can be loaded before the live count has arrived (one dependent
     // memory round trip less).  Slots in [S, S_max) are allocated, their content is unused.
     const bool fixed = a.align == SPB && (int64_t)gridDim.x * SPB >= a.S_max;
-    int64_t v0 = 0, t0 = 0;
+    int64_t v0 = 0, t0 = 0, h0 = -1;
     const int64_t slot0 = (int64_t)blockIdx.x * SPB + gib;
-    if (fixed && slot0 < a.S_max) load_slot(a, slot0, &v0, &t0);
+    if (fixed && slot0 < a.S_max) {
+        load_slot(a, slot0, &v0, &t0);
+        h0 = root_hint_of(a, slot0);
+    }
     const int64_t S = live_count(a.S_dev, a.S_max);
     int64_t first, run;
     block_run(S, a.align, &first, &run);
@@ -204,10 +219,14 @@ __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
     for (int64_t it = first; it < first + run && it < S; it += SPB) {
         const int64_t slot = it + gib;
         bool active = slot < S;
-        int64_t v = v0, t = t0;
+        int64_t v = v0, t = t0, rh = h0;
         if (!fixed || it != first) {
             v = t = 0;
-            if (active) load_slot(a, slot, &v, &t);
+            rh = -1;
+            if (active) {
+                load_slot(a, slot, &v, &t);
+                rh = root_hint_of(a, slot);
+            }
         }
         const bool bad = active && (v < 0 || v >= a.n);
         active = active && !bad;
@@ -224,7 +243,10 @@ __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
             const int64_t h = active ? a.slot_hint[slot] : 0;
             hi = h >= rs ? h : rs;
         } else {
-            hi = group_lower_bound<G>(a.ts, rs, re, t_hi, lig, gshift, active);
+            // positive roots whose window end the caller knows are not searched
+            const bool told = active && rh >= 0;
+            hi = group_lower_bound<G>(a.ts, rs, re, t_hi, lig, gshift, active && !told);
+            if (told) hi = clamp_to_row(rh, rs, re);
         }
         int64_t lo = rs;
         if (a.allowed_offset >= 0)  // kernel argument: uniform across the wave
@@ -725,8 +747,11 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
     const int64_t S = a.S_max;
     const int64_t slot = b * FSPB + gib;
     const bool in_range = slot < S;
-    int64_t v = 0, t = 0;
-    if (in_range) load_slot(a, slot, &v, &t);
+    int64_t v = 0, t = 0, rh = -1;
+    if (in_range) {
+        load_slot(a, slot, &v, &t);
+        rh = root_hint_of(a, slot);
+    }
     const bool bad = in_range && (v < 0 || v >= a.n);
     const bool active = in_range && !bad;
     if (in_range && lig == 0) {
@@ -741,7 +766,10 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
         re = a.row_ptr[v + 1];
     }
     const int64_t eq = a.equal_root_time ? 1 : 0;
-    const int64_t hi = group_lower_bound<FG>(a.ts, rs, re, t + eq, lig, gshift, active);
+    // positive roots whose window end the caller knows are not searched
+    const bool told = active && rh >= 0;
+    int64_t hi = group_lower_bound<FG>(a.ts, rs, re, t + eq, lig, gshift, active && !told);
+    if (told) hi = clamp_to_row(rh, rs, re);
     int64_t lo = rs;
     if (a.allowed_offset >= 0) lo = group_lower_bound<FG>(a.ts, rs, hi, t - a.allowed_offset, lig, gshift, active);
     const int64_t len = hi - lo;
@@ -1074,6 +1102,7 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
     a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint;
     a.slot_node = slot_node; a.slot_ts = slot_ts; a.S_max = S_max; a.S_dev = S_dev;
     a.slot_hint = slot_hint; a.hint_out = hint_out;
+    a.root_hint = (derive && !p->equal_root_time) ? p->root_hint : nullptr;
     a.derive = derive ? 1 : 0;
     if (derive) {
         a.R = derive->R; a.S_pos = derive->S_pos; a.roots = derive->roots; a.ts_ptr = derive->ts_ptr;
@@ -1106,6 +1135,7 @@ Fused2Args fused2_args(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, cons
     HopArgs& a = f.h;
     a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint;
     a.S_max = S0; a.derive = 1;
+    a.root_hint = p->equal_root_time ? nullptr : p->root_hint;
     a.R = spec->R; a.S_pos = spec->S_pos; a.roots = spec->roots; a.ts_ptr = spec->ts_ptr;
     a.root_ts = spec->root_ts; a.neg_roots = spec->neg_roots; a.neg_ts = spec->neg_ts;
     a.slot_node_out = spec->slot_node_out; a.slot_ts_out = spec->slot_ts_out;

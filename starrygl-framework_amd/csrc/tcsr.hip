@@ -311,10 +311,13 @@ extern "C" int32_t sgl_chunk_index_build(int64_t n, int64_t num_chunks, const in
 namespace sgl {
 namespace {
 
-// hop_hint[e] = first position in row col[e] whose timestamp is >= ts[e]
-__global__ __launch_bounds__(BLOCK) void hop_hint_kernel(sgl_tcsr g, int64_t* __restrict__ hint) {
-    for (int64_t e = (int64_t)blockIdx.x * BLOCK + threadIdx.x; e < g.m; e += (int64_t)gridDim.x * BLOCK) {
-        const int64_t v = g.col[e], t = g.ts[e];
+// out[i] = first position in row node[i] whose timestamp is >= t[i] (-1: node outside [0,n)).
+// With node = col and t = ts (N = m) this is the next-hop index.
+__global__ __launch_bounds__(BLOCK) void window_end_kernel(sgl_tcsr g, const int64_t* __restrict__ node,
+                                                           const int64_t* __restrict__ t_of, int64_t N,
+                                                           int64_t* __restrict__ out) {
+    for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < N; i += (int64_t)gridDim.x * BLOCK) {
+        const int64_t v = node[i], t = t_of[i];
         int64_t lo = -1;
         if (v >= 0 && v < g.n) {
             lo = g.row_ptr[v];
@@ -324,8 +327,17 @@ __global__ __launch_bounds__(BLOCK) void hop_hint_kernel(sgl_tcsr g, int64_t* __
                 if (g.ts[mid] < t) lo = mid + 1; else hi = mid;
             }
         }
-        hint[e] = lo;
+        out[i] = lo;
     }
+}
+
+int32_t launch_window_end(const sgl_tcsr* g, const int64_t* node, const int64_t* t, int64_t N, int64_t* out,
+                          void* stream) {
+    int64_t blocks = ceil_div<int64_t>(N, BLOCK);
+    if (blocks > (1 << 20)) blocks = 1 << 20;
+    hipLaunchKernelGGL(window_end_kernel, dim3((unsigned)blocks), dim3(BLOCK), 0, as_stream(stream), *g, node, t, N, out);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
 }
 
 }  // namespace
@@ -335,9 +347,14 @@ extern "C" int32_t sgl_tcsr_hop_hint_build(const sgl_tcsr* g, int64_t* hop_hint,
     if (!g || g->n < 0 || g->m < 0 || !g->row_ptr) return fail(SGL_EINVAL, "tcsr_hop_hint_build: NULL graph");
     if (g->m == 0) return SGL_OK;
     if (!g->col || !g->ts || !hop_hint) return fail(SGL_EINVAL, "tcsr_hop_hint_build: NULL array");
-    int64_t blocks = ceil_div<int64_t>(g->m, BLOCK);
-    if (blocks > (1 << 20)) blocks = 1 << 20;
-    hipLaunchKernelGGL(hop_hint_kernel, dim3((unsigned)blocks), dim3(BLOCK), 0, as_stream(stream), *g, hop_hint);
-    SGL_LAUNCH_CHECK();
-    return SGL_OK;
+    return launch_window_end(g, g->col, g->ts, g->m, hop_hint, stream);
+}
+
+extern "C" int32_t sgl_window_end(const sgl_tcsr* g, const int64_t* node, const int64_t* t, int64_t N,
+                                  int64_t* out, void* stream) {
+    if (!g || g->n < 0 || g->m < 0 || !g->row_ptr) return fail(SGL_EINVAL, "window_end: NULL graph");
+    if (N < 0) return fail(SGL_EINVAL, "window_end: N < 0");
+    if (N == 0) return SGL_OK;
+    if (!node || !t || !out || (g->m > 0 && !g->ts)) return fail(SGL_EINVAL, "window_end: NULL array");
+    return launch_window_end(g, node, t, N, out, stream);
 }

@@ -5,7 +5,7 @@ header declares.  The product library exports them as ``sgl_*``.
 """
 import ctypes as C
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
@@ -26,7 +26,7 @@ class SampleParams(C.Structure):
     _fields_ = [("type", i32), ("fanout", i32), ("allowed_offset", i64),
                 ("equal_root_time", i32), ("keep_root_time", i32),
                 ("replace", i32), ("hop", i32), ("seed", u64),
-                ("mark_state", vp), ("mark_universe", i64)]
+                ("mark_state", vp), ("mark_universe", i64), ("root_hint", vp)]
 
 
 class HopOut(C.Structure):
@@ -63,6 +63,7 @@ PROTOTYPES = {
     "tcsr_build": (i32, [i64, i64, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]),
     "tcsr_validate": (i32, [P(TCSR), vp, sz, vp]),
     "tcsr_hop_hint_build": (i32, [P(TCSR), vp, vp]),
+    "window_end": (i32, [P(TCSR), vp, vp, i64, vp, vp]),
     "sample_hop_workspace_bytes": (sz, [i64]),
     "sample_hop": (i32, [P(TCSR), vp, vp, i64, vp, P(SampleParams), P(HopOut), vp, sz, vp]),
     "sample_khop_workspace_bytes": (sz, [i64, i32, i32]),

@@ -110,6 +110,11 @@ def check_sample_bad(bad):
         raise IndexError(f"sgl status {_abi.SGL_ERANGE}: {bad} sampling slots name a node outside [0,n)")
 
 
+def _check_root_hint(p, S_pos):
+    if getattr(p, "_root_hint_len", S_pos) < S_pos:
+        raise ValueError(f"root_hint has {p._root_hint_len} entries for {S_pos} positive root slots")
+
+
 def check_unique_total(u_total):
     """The id count of a unique_compact call is INT64_MAX when a numbering pass gave up waiting for
     an earlier tile (bounded wait): the result is void and the remap state has to be re-initialised."""
@@ -172,6 +177,29 @@ class HotPath:
         g.view.hop_hint = self.be.ptr(hint)
         return g
 
+    def window_end(self, g, node, t):
+        """out[i] = position in row node[i] of the first edge with timestamp >= t[i] (-1 for a node
+        outside [0,n)): where the strictly-before window of the slot (node[i], t[i]) ends.  A loader
+        computes it once for the events it will train on and passes a batch's values as `root_hint`."""
+        self._chk("i64", node=node, t=t)
+        if node.shape[0] != t.shape[0]:
+            raise ValueError("window_end: node and t differ in length")
+        out = self.be.empty(int(node.shape[0]))
+        self._ck(self.lib.window_end(C.byref(g.view), self.be.ptr(node), self.be.ptr(t), int(node.shape[0]),
+                                     self.be.ptr(out), self.be.stream()))
+        return out
+
+    def with_root_hint(self, p, root_hint):
+        """Copy of the sampling parameters `p` that hands the k-hop sampler the window ends of the
+        positive root slots (`window_end` of (root, root_ts) per slot, -1 = search): those slots are
+        then sampled without a search."""
+        self._chk("i64", root_hint=root_hint)
+        q = SampleParams.from_buffer_copy(p)
+        q.root_hint = self.be.ptr(root_hint)
+        q._keep = (getattr(p, "_keep", None), root_hint)
+        q._root_hint_len = int(root_hint.shape[0])
+        return q
+
     # ----------------------------------------------------------- sampling
     @staticmethod
     def params(sample_type, fanout, allowed_offset=-1, equal_root_time=False,
@@ -183,7 +211,7 @@ class HotPath:
             sample_type = _abi.SAMPLE_TYPES[sample_type]
         return SampleParams(int(sample_type), int(fanout), int(allowed_offset),
                             int(bool(equal_root_time)), int(bool(keep_root_time)),
-                            int(bool(replace)), int(hop), int(seed) & (2**64 - 1), None, 0)
+                            int(bool(replace)), int(hop), int(seed) & (2**64 - 1), None, 0, None)
 
     def set_wait_limit(self, polls):
         """Polls before a block that waits for another block's totals gives up (<= 0: default);
@@ -196,7 +224,7 @@ class HotPath:
         reset=True, premarked=True)` over the sampled arrays then skips its first pass."""
         q = SampleParams.from_buffer_copy(p)
         q.mark_state, q.mark_universe = self.be.ptr(state.buf), state.universe
-        q._keep = state
+        q._keep = (getattr(p, "_keep", None), state)
         return q
 
     def sample_hop(self, g, slot_node, slot_ts, p, S_dev=None, finalize=True):
@@ -236,6 +264,7 @@ class HotPath:
         be = self.be
         R, S_pos, N_neg = int(roots.shape[0]), int(root_ts.shape[0]), int(neg_roots.shape[0])
         S0 = S_pos + N_neg
+        _check_root_hint(p, S_pos)
         res = out if out is not None else self.khop_buffers(S0, layers, p.fanout)
         if res.S0 < S0 or len(res.hops) != layers or res.fanout < p.fanout:
             raise MemoryError("khop buffers are smaller than this call needs")
@@ -257,6 +286,7 @@ class HotPath:
         S0 = S_pos + N_neg
         fan = max(p.fanout for p in params)
         for p, res in zip(params, outs):
+            _check_root_hint(p, S_pos)
             if res.S0 < S0 or len(res.hops) != layers or res.fanout < p.fanout:
                 raise MemoryError("khop buffers are smaller than this call needs")
         head = outs[0]

@@ -330,3 +330,47 @@ def test_next_hop_index_gives_the_same_samples(oracle, hot, sample_type):
                    dict(replace=True)):
             _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, neg, neg_ts, layers, sample_type=sample_type,
                       fanout=fanout, seed=5, **kw)
+
+
+@pytest.mark.parametrize("sample_type", ["recent", "uniform"])
+def test_root_hints_give_the_same_samples(oracle, hot, sample_type):
+    """sgl_window_end equals the oracle's; with its values as sgl_sample_params.root_hint (some entries -1 =
+    search, several timestamps per root, negatives behind the positives) the samples equal the oracle's
+    un-hinted ones in the single-launch kernel, the multi-launch path, the pair launch, with a lower window
+    bound, and when the hints must be ignored (windows that include the root's time)."""
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 3_000, 90_000, 1.15, 5_000, 53, hub=20_000)   # many ties
+    hot.build_hop_hint(dg)
+    rng = np.random.default_rng(22)
+    for S_pos, n_neg, layers, fanout in ((600, 300, 2, 10), (30_000, 10_000, 2, 5), (2_000, 0, 3, 6), (64, 7, 1, 17)):
+        R = max(1, S_pos // 2)
+        cuts = np.sort(rng.integers(0, S_pos + 1, R - 1))
+        ts_ptr = np.concatenate([[0], cuts, [S_pos]]).astype(np.int64)
+        roots = rng.integers(0, g.n, R).astype(np.int64)
+        roots[::5] = np.argmax(np.diff(g.row_ptr))                     # the hub: the longest searches
+        root_ts = rng.integers(0, 5_001, S_pos).astype(np.int64)
+        neg = rng.integers(0, g.n, n_neg).astype(np.int64)
+        neg_ts = rng.integers(0, 5_001, n_neg).astype(np.int64)
+        slot_node = np.repeat(roots, np.diff(ts_ptr))
+        hint = hot.window_end(dg, to_dev(hot, slot_node), to_dev(hot, root_ts))
+        assert np.array_equal(np_of(hint), oracle.window_end(g, slot_node, root_ts))
+        hint[::4] = -1
+        dev = [to_dev(hot, x) for x in (roots, ts_ptr, root_ts, neg, neg_ts)]
+        for kw in (dict(), dict(allowed_offset=300), dict(equal_root_time=True), dict(keep_root_time=True)):
+            kw = dict(sample_type=sample_type, fanout=fanout, seed=3, **kw)
+            want = oracle.sample_khop(g, roots, ts_ptr, root_ts, neg, neg_ts, layers, oracle.params(**kw))
+            got = hot.sample_khop(dg, *dev, layers, hot.with_root_hint(hot.params(**kw), hint))
+            for l in range(layers):
+                assert_hop_equal(got.hops[l], want.hops[l], tag=f"root hints, hop{l} {kw}")
+        if layers == 2 and fanout <= 16:                               # both strategies in one call
+            kws = [dict(sample_type=st_, fanout=fanout, seed=3) for st_ in ("recent", "uniform")]
+            outs = [hot.khop_buffers(S_pos + n_neg, 2, fanout) for _ in range(2)]
+            hot.sample_khop_multi(dg, *dev, 2, [hot.with_root_hint(hot.params(**k_), hint) for k_ in kws], outs)
+            for res, k_ in zip(outs, kws):
+                want = oracle.sample_khop(g, roots, ts_ptr, root_ts, neg, neg_ts, 2, oracle.params(**k_))
+                res.finalize()
+                for l in range(2):
+                    assert_hop_equal(res.hops[l], want.hops[l], tag=f"root hints, multi, hop{l} {k_}")
+    # hints outside the root's row are clamped to it: the call completes and stays inside its buffers
+    wild = to_dev(hot, rng.integers(-5, 2 * g.m, S_pos).astype(np.int64))
+    res = hot.sample_khop(dg, *dev, 1, hot.with_root_hint(hot.params(sample_type, 17), wild))
+    assert 0 <= res.hops[0].E <= (S_pos + n_neg) * 17

@@ -302,3 +302,35 @@ def test_next_hop_index_is_searchsorted_per_edge(oracle):
     after = oracle.sample_khop(g, np.arange(n), np.arange(n + 1), np.full(n, 25), np.zeros(0, np.int64),
                                np.zeros(0, np.int64), 2, oracle.params("recent", 4))
     assert np.array_equal(before.hops[1].neighbors_eid, after.hops[1].neighbors_eid)
+
+
+def test_window_end_is_searchsorted_and_root_hints_are_checked(oracle):
+    """window_end(node, t) = row start + numpy's searchsorted(side='left') on the row's timestamps, -1 for
+    ids that are no node; the oracle samples the same with the true values as root hints, and - being the
+    checker - refuses a hint that is not the window end."""
+    rng = np.random.default_rng(9)
+    n, m = 50, 2500
+    src, dst, ts = rng.integers(0, n, m), rng.integers(0, n, m), rng.integers(0, 30, m)
+    g = host_graph(oracle, n, src, dst, ts)
+    node = rng.integers(-2, n + 2, 400).astype(np.int64)
+    t = rng.integers(-1, 32, 400).astype(np.int64)
+    want = np.array([g.row_ptr[v] + np.searchsorted(g.ts[g.row_ptr[v]: g.row_ptr[v + 1]], tt, side="left")
+                     if 0 <= v < n else -1 for v, tt in zip(node, t)])
+    assert np.array_equal(oracle.window_end(g, node, t), want)
+    roots, root_ts = rng.integers(0, n, 120).astype(np.int64), rng.integers(0, 31, 120).astype(np.int64)
+    ts_ptr, none = np.arange(121, dtype=np.int64), np.zeros(0, np.int64)
+    p = oracle.params("recent", 4)
+    plain = oracle.sample_khop(g, roots, ts_ptr, root_ts, none, none, 2, p)
+    hint = oracle.window_end(g, roots, root_ts)
+    hint[::3] = -1                                   # "search"
+    told = oracle.sample_khop(g, roots, ts_ptr, root_ts, none, none, 2, oracle.with_root_hint(p, hint))
+    for a, b in zip(plain.hops, told.hops):
+        assert np.array_equal(a.neighbors_eid, b.neighbors_eid) and np.array_equal(a.root_start_ptr, b.root_start_ptr)
+    deg = np.diff(g.row_ptr)[roots]
+    bad = hint.copy()
+    i = int(np.flatnonzero((hint >= 0) & (deg > 0))[0])
+    bad[i] += 1 if hint[i] == g.row_ptr[roots[i]] else -1
+    with pytest.raises(Exception):
+        oracle.sample_khop(g, roots, ts_ptr, root_ts, none, none, 2, oracle.with_root_hint(p, bad))
+    with pytest.raises(ValueError):
+        oracle.sample_khop(g, roots, ts_ptr, root_ts, none, none, 2, oracle.with_root_hint(p, hint[:50].copy()))
