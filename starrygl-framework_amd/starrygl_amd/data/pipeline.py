@@ -94,13 +94,16 @@ class MiniBatch:
 class MiniBatchPipeline:
     def __init__(self, graph, num_pos_slots, num_neg, layers, fanout, sample_type="recent", node_tables=None,
                  edge_tables=None, time_encoder=None, allowed_offset=-1, equal_root_time=False,
-                 keep_root_time=False, seed=0, use_graph=True, stream=None):
+                 keep_root_time=False, seed=0, use_graph=True, stream=None, root_hints=False):
         """graph: the native graph object (`pyGraph.g`, i.e. `CUDAGraph`).
         num_pos_slots / num_neg: positive root timestamps and negatives per batch
         (fixed, they size every buffer).  node_tables / edge_tables: name ->
         `sgl_cache` (from `HotPath.cache`) gathered for the unique nodes / the
         sampled edge ids; a node table with timestamps also yields node_ts[name].
         time_encoder: (w, b) fp32 device tensors, or a TimeEncoder module.
+        root_hints: every run() also takes `root_hint`, the window ends of the positive slots
+        (`graph.window_end(roots, root_ts)`, which a loader looks up once for all the events it will
+        train on; -1 = search): those roots are then sampled without a search.
         stream: run every batch on this stream instead of the caller's current one (see
         MiniBatchPipelinePool); inputs handed to run() must then be complete on the host side
         or long-lived, and results are read through MiniBatch.finalize(), which waits for it."""
@@ -121,6 +124,9 @@ class MiniBatchPipeline:
         self.in_roots, self.in_ts = be.empty(self.S_pos), be.empty(self.S_pos)
         self.in_neg, self.in_neg_ts = be.empty(self.N_neg), be.empty(self.N_neg)
         self.ts_ptr = torch.arange(self.S_pos + 1, dtype=torch.int64, device=self.dev)
+        self.in_hint = be.empty(self.S_pos) if root_hints else None
+        if root_hints:
+            self.p = hp.with_root_hint(self.p, self.in_hint)
         # outputs
         self.kr = hp.khop_buffers(self.S0, self.layers, self.fanout)
         caps = [self.S0] + [self.S0 * self.fanout ** (l + 1) for l in range(self.layers)]
@@ -187,23 +193,28 @@ class MiniBatchPipeline:
             if self.te is not None:
                 hp.time_encode(h.neighbors_dt, self.te[0], self.te[1], out=self.te_out[l], N_dev=h.counts[1:2])
 
-    def run(self, roots, root_ts, neg_roots=None, neg_ts=None):
+    def run(self, roots, root_ts, neg_roots=None, neg_ts=None, root_hint=None):
         """Enqueue one batch (asynchronous).  `roots`/`root_ts`: S_pos ids and
-        timestamps (one timestamp per root); `neg_roots`/`neg_ts`: N_neg each."""
+        timestamps (one timestamp per root); `neg_roots`/`neg_ts`: N_neg each; `root_hint`: S_pos
+        window ends, for a pipeline built with root_hints=True."""
         if roots.numel() != self.S_pos or root_ts.numel() != self.S_pos:
             raise ValueError(f"this pipeline was planned for {self.S_pos} positive slots")
+        if (self.in_hint is None) != (root_hint is None) or (root_hint is not None and root_hint.numel() != self.S_pos):
+            raise ValueError("root_hint goes with a pipeline built with root_hints=True, one entry per positive slot")
         if self.N_neg and (neg_roots is None or neg_roots.numel() != self.N_neg or neg_ts.numel() != self.N_neg):
             raise ValueError(f"this pipeline was planned for {self.N_neg} negatives")
         if self.stream is not None:
             with torch.cuda.stream(self.stream):
-                out = self._run(roots, root_ts, neg_roots, neg_ts)
+                out = self._run(roots, root_ts, neg_roots, neg_ts, root_hint)
                 self._done.record(self.stream)
             return out
-        return self._run(roots, root_ts, neg_roots, neg_ts)
+        return self._run(roots, root_ts, neg_roots, neg_ts, root_hint)
 
-    def _run(self, roots, root_ts, neg_roots, neg_ts):
+    def _run(self, roots, root_ts, neg_roots, neg_ts, root_hint):
         self.in_roots.copy_(roots, non_blocking=True)
         self.in_ts.copy_(root_ts, non_blocking=True)
+        if root_hint is not None:
+            self.in_hint.copy_(root_hint, non_blocking=True)
         if self.N_neg:
             self.in_neg.copy_(neg_roots, non_blocking=True)
             self.in_neg_ts.copy_(neg_ts, non_blocking=True)
@@ -242,8 +253,8 @@ def bound_streams(n, device):
 class MiniBatchPipelinePool:
     """`n` MiniBatchPipeline objects on streams of their own; run() hands the batches to them in
     turn, so that up to `n` batches are in flight: the latency-bound sampling of one batch overlaps
-    the bandwidth-bound gathers of another (configs of 12 000 roots, 2 hops: 0.105 ms per batch with
-    three in flight against 0.127 ms one at a time).  A MiniBatch stays valid until the `n`-th
+    the bandwidth-bound gathers of another (configs of 12 000 roots, 2 hops: 0.09 ms per batch with
+    three in flight against 0.115 ms one at a time).  A MiniBatch stays valid until the `n`-th
     following run().  Create the pool before any other stream of the process."""
 
     def __init__(self, n, graph, *args, **kwargs):
@@ -253,7 +264,7 @@ class MiniBatchPipelinePool:
         self.pipes = [MiniBatchPipeline(graph, *args, stream=st, **kwargs) for st in bound_streams(n, dev)]
         self._next = 0
 
-    def run(self, roots, root_ts, neg_roots=None, neg_ts=None):
+    def run(self, roots, root_ts, neg_roots=None, neg_ts=None, root_hint=None):
         p = self.pipes[self._next]
         self._next = (self._next + 1) % len(self.pipes)
-        return p.run(roots, root_ts, neg_roots, neg_ts)
+        return p.run(roots, root_ts, neg_roots, neg_ts, root_hint)

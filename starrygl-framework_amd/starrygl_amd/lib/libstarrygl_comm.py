@@ -143,6 +143,13 @@ class CUDAGraph:
         return hp.sample_khop(self._g, postive_root.roots, postive_root.ts_ptr, postive_root.ts, neg.roots, neg.ts,
                               int(layers), p, finalize=False, out=out)
 
+    def window_end(self, node, t):
+        """Where the strictly-before window of every slot (node[i], t[i]) ends (not in the reference;
+        sgl_window_end): a loader looks this up once for the events it trains on and hands a batch's
+        values to MiniBatchPipeline.run(root_hint=...)."""
+        dev = self._hp.be.device
+        return self._hp.window_end(self._g, _i64(node, dev, "node"), _i64(t, dev, "t"))
+
     def get_seeds_in_chunks(self, chunks, time_begin, time_end, using_full_timestamp=False):
         from .seeds import seeds_in_chunks
         return seeds_in_chunks(self, chunks, int(time_begin), int(time_end), bool(using_full_timestamp))

@@ -88,3 +88,35 @@ def test_pipeline_pool_keeps_batches_in_flight(oracle, hot):
             for l, h in enumerate(want.hops):
                 assert np.array_equal(np_of(mb.hops[l]["neighbors_local"]), loc[1 + l])
                 assert np.array_equal(np_of(mb.hops[l]["neighbors_eid"]), h.neighbors_eid)
+
+
+@pytest.mark.parametrize("sample_type", ["recent", "uniform"])
+def test_pipeline_with_root_hints(oracle, hot, sample_type):
+    """A pool whose batches carry the window ends of their positive roots (looked up once for the whole
+    event stream, as a loader does) gives the oracle's result; a pipeline built for hints refuses a batch
+    without them and the other way round."""
+    from starrygl_amd.data import MiniBatchPipeline, MiniBatchPipelinePool
+    from starrygl_amd.lib.libstarrygl_comm import from_edge_index
+    n, m, B = 3000, 60_000, 250
+    src, dst, ts, eid = synth.graph_stream(n, m, 1.15, 40_000, 29)          # 40 000 times: ties inside rows
+    hg = host_graph(oracle, n, src, dst, ts, eid)
+    g = from_edge_index(n, 1, *(torch.from_numpy(x) for x in (src, dst, ts, eid)))
+    # the loader's one-off lookup: (src, ts) and (dst, ts) of every event
+    end_src, end_dst = g.window_end(torch.from_numpy(src), torch.from_numpy(ts)), g.window_end(torch.from_numpy(dst), torch.from_numpy(ts))
+    rng = np.random.default_rng(6)
+    pool = MiniBatchPipelinePool(2, g, 2 * B, B, 2, 6, sample_type, seed=9, root_hints=True)
+    for lo in (5_000, 31_000, 59_750):
+        b = synth.link_batch(src, dst, ts, lo, lo + B, n, B, rng)           # roots = [src; dst] of events lo..lo+B
+        assert np.array_equal(b[0], np.concatenate([src[lo: lo + B], dst[lo: lo + B]]))
+        hint = torch.cat([end_src[lo: lo + B], end_dst[lo: lo + B]])
+        mb = pool.run(to_dev(hot, b[0]), to_dev(hot, b[2]), to_dev(hot, b[3]), to_dev(hot, b[4]), root_hint=hint).finalize()
+        want = oracle.sample_khop(hg, *b, 2, oracle.params(sample_type, 6, seed=9))
+        assert mb.E == [h.E for h in want.hops]
+        for l, h in enumerate(want.hops):
+            assert np.array_equal(np_of(mb.hops[l]["neighbors_eid"]), h.neighbors_eid)
+            assert np.array_equal(np_of(mb.hops[l]["neighbors_dt"]), h.neighbors_dt)
+    with pytest.raises(ValueError):
+        pool.run(to_dev(hot, b[0]), to_dev(hot, b[2]), to_dev(hot, b[3]), to_dev(hot, b[4]))
+    plain = MiniBatchPipeline(g, 2 * B, B, 2, 6, sample_type)
+    with pytest.raises(ValueError):
+        plain.run(to_dev(hot, b[0]), to_dev(hot, b[2]), to_dev(hot, b[3]), to_dev(hot, b[4]), root_hint=hint)
