@@ -361,7 +361,11 @@ int32_t sgl_chunk_index_build(int64_t n, int64_t num_chunks,
  * (cand_off[num_chunks] = n_cand).  Two calls sharing one workspace:
  *   sgl_seeds_count -> totals[0..2] = {R roots, S timestamps, Q events};
  *   (caller allocates roots[R], ts_ptr[R+1], ts[S], q_ptr[S+1], q_eid[Q])
- *   sgl_seeds_fill. */
+ *   sgl_seeds_fill.
+ * window_end (optional, [S] or NULL; no counterpart in the reference): per
+ * (root, timestamp) the position of the root's first edge at that time, i.e.
+ * what sgl_window_end gives for it - the extraction walks those edges anyway -
+ * ready to be passed on as sgl_sample_params.root_hint. */
 typedef struct sgl_seed_query {
     const int64_t* chunk_ptr;   /* device [total chunks + 1]          */
     const int64_t* chunk_nodes; /* device [n]                          */
@@ -379,8 +383,8 @@ int32_t sgl_seeds_count(const sgl_tcsr* g, const sgl_seed_query* q,
 int32_t sgl_seeds_fill(const sgl_tcsr* g, const sgl_seed_query* q,
                        const int64_t* totals,
                        int64_t* roots, int64_t* ts_ptr, int64_t* ts,
-                       int64_t* q_ptr, int64_t* q_eid, void* workspace,
-                       size_t workspace_bytes, void* stream);
+                       int64_t* q_ptr, int64_t* q_eid, int64_t* window_end,
+                       void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------- sub-graph slice ("cluster" mode) */
 /* The sub-graph of a chunk set over a time window (replaces

@@ -689,7 +689,8 @@ size_t sglo_seeds_workspace_bytes(int64_t n_cand) { (void)n_cand; return 0; }
  * implemented for the window: t_begin <= ts < t_end (the early-exit tests of
  * find_time_range, :273, 279). */
 static int32_t seeds_walk(const sgl_tcsr* g, const sgl_seed_query* q, int64_t* totals,
-                          int64_t* roots, int64_t* ts_ptr, int64_t* ts, int64_t* q_ptr, int64_t* q_eid) {
+                          int64_t* roots, int64_t* ts_ptr, int64_t* ts, int64_t* q_ptr, int64_t* q_eid,
+                          int64_t* window_end) {
     int64_t R = 0, S = 0, Q = 0;
     for (int64_t p = 0; p < q->num_chunks; ++p) {
         const int64_t c = q->chunks[p];
@@ -706,6 +707,8 @@ static int32_t seeds_walk(const sgl_tcsr* g, const sgl_seed_query* q, int64_t* t
             for (int64_t e = lo; e < hi; ++e) {
                 if (e == lo || g->ts[e] != g->ts[e - 1]) {
                     if (roots) { ts[S] = g->ts[e]; q_ptr[S] = Q; }
+                    /* by definition, not by position: the first edge of the row with ts >= this time */
+                    if (roots && window_end) window_end[S] = lower_bound_ts(g->ts, rs, re, g->ts[e]);
                     ++S;
                 }
                 if (roots) q_eid[Q] = g->eid[e];
@@ -723,17 +726,17 @@ int32_t sglo_seeds_count(const sgl_tcsr* g, const sgl_seed_query* q, int64_t* to
                          size_t ws_bytes, void* stream) {
     (void)ws; (void)ws_bytes; (void)stream;
     if (!g || !q || !totals) return fail(SGL_EINVAL, "seeds_count: null");
-    return seeds_walk(g, q, totals, NULL, NULL, NULL, NULL, NULL);
+    return seeds_walk(g, q, totals, NULL, NULL, NULL, NULL, NULL, NULL);
 }
 
 int32_t sglo_seeds_fill(const sgl_tcsr* g, const sgl_seed_query* q, const int64_t* totals,
                         int64_t* roots, int64_t* ts_ptr, int64_t* ts, int64_t* q_ptr, int64_t* q_eid,
-                        void* ws, size_t ws_bytes, void* stream) {
+                        int64_t* window_end, void* ws, size_t ws_bytes, void* stream) {
     (void)ws; (void)ws_bytes; (void)stream; (void)totals;
     if (!g || !q || !ts_ptr || !q_ptr) return fail(SGL_EINVAL, "seeds_fill: null");
     int64_t dummy;
     if (!roots) roots = &dummy; /* R == 0 */
-    return seeds_walk(g, q, NULL, roots, ts_ptr, ts, q_ptr, q_eid);
+    return seeds_walk(g, q, NULL, roots, ts_ptr, ts, q_ptr, q_eid, window_end);
 }
 
 /* ------------------------------------------- sub-graph slice ("cluster" mode) */

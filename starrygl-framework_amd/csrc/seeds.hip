@@ -187,7 +187,8 @@ __global__ __launch_bounds__(SEED_SCAN_BLOCK) void seeds_scan_kernel(SeedWs w, i
 
 __global__ __launch_bounds__(BLOCK) void seeds_fill_kernel(sgl_tcsr g, sgl_seed_query q, SeedWs w,
                                                            const int64_t* totals, int64_t* roots, int64_t* ts_ptr,
-                                                           int64_t* ts, int64_t* q_ptr, int64_t* q_eid) {
+                                                           int64_t* ts, int64_t* q_ptr, int64_t* q_eid,
+                                                           int64_t* window_end) {
     __shared__ int64_t s_w[BLOCK / WAVE][3];
     const int lane = threadIdx.x % WAVE;
     if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -215,6 +216,8 @@ __global__ __launch_bounds__(BLOCK) void seeds_fill_kernel(sgl_tcsr g, sgl_seed_
                 if (e == lo || t != g.ts[e - 1]) {
                     ts[s] = t;
                     q_ptr[s] = q0 + (e - lo);
+                    // the first edge of the row at this time: where the window strictly before it ends
+                    if (window_end != nullptr) window_end[s] = e;
                     ++s;
                 }
                 q_eid[q0 + (e - lo)] = g.eid[e];
@@ -235,6 +238,7 @@ __global__ __launch_bounds__(BLOCK) void seeds_fill_kernel(sgl_tcsr g, sgl_seed_
                     const int64_t si = s + __popcll(hb & lt);
                     ts[si] = t;
                     q_ptr[si] = qb + (e - l);
+                    if (window_end != nullptr) window_end[si] = e;
                 }
                 if (in) q_eid[qb + (e - l)] = g.eid[e];
                 s += __popcll(hb);
@@ -314,7 +318,7 @@ extern "C" int32_t sgl_seeds_count(const sgl_tcsr* g, const sgl_seed_query* q, i
 
 extern "C" int32_t sgl_seeds_fill(const sgl_tcsr* g, const sgl_seed_query* q, const int64_t* totals,
                                   int64_t* roots, int64_t* ts_ptr, int64_t* ts, int64_t* q_ptr, int64_t* q_eid,
-                                  void* ws, size_t ws_bytes, void* stream) {
+                                  int64_t* window_end, void* ws, size_t ws_bytes, void* stream) {
     int32_t rc;
     if ((rc = check_query(g, q)) != SGL_OK) return rc;
     if (!totals || !ts_ptr || !q_ptr) return fail(SGL_EINVAL, "seeds_fill: totals/ts_ptr/q_ptr is NULL");
@@ -328,7 +332,7 @@ extern "C" int32_t sgl_seeds_fill(const sgl_tcsr* g, const sgl_seed_query* q, co
         return SGL_OK;
     }
     hipLaunchKernelGGL(seeds_fill_kernel, dim3((unsigned)w.nt), dim3(BLOCK), 0, st, *g, *q, w, totals, roots, ts_ptr, ts, q_ptr,
-                       q_eid);
+                       q_eid, window_end);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }

@@ -84,7 +84,7 @@ PROTOTYPES = {
     "chunk_index_build": (i32, [i64, i64, vp, vp, vp, vp, sz, vp]),
     "seeds_workspace_bytes": (sz, [i64]),
     "seeds_count": (i32, [P(TCSR), P(SeedQuery), vp, vp, sz, vp]),
-    "seeds_fill": (i32, [P(TCSR), P(SeedQuery), vp, vp, vp, vp, vp, vp, vp, sz, vp]),
+    "seeds_fill": (i32, [P(TCSR), P(SeedQuery), vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]),
     "unique_pairs_workspace_bytes": (sz, [i64]),
     "unique_pairs": (i32, [vp, vp, i64, vp, vp, vp, vp, vp, vp, sz, vp]),
     "csc_from_pairs_workspace_bytes": (sz, [i64]),

@@ -400,9 +400,11 @@ class HotPath:
                                             be.ptr(chunk_nodes), be.ptr(ws), wsb, be.stream()))
         return chunk_ptr, chunk_nodes[:n]
 
-    def seeds(self, g, chunk_ptr, chunk_nodes, chunks, cand_off, n_cand, t_begin, t_end):
+    def seeds(self, g, chunk_ptr, chunk_nodes, chunks, cand_off, n_cand, t_begin, t_end, with_window_end=False):
         """-> (roots, ts_ptr, ts, q_ptr, q_eid).  `cand_off` is the exclusive prefix
-        of the selected chunks' sizes, `n_cand` its last entry (host int)."""
+        of the selected chunks' sizes, `n_cand` its last entry (host int).  with_window_end: a sixth
+        array, per (root, timestamp) where the window strictly before it ends (the `root_hint` of
+        a sampling call over these roots)."""
         self._chk("i64", chunk_ptr=chunk_ptr, chunk_nodes=chunk_nodes, chunks=chunks, cand_off=cand_off)
         be = self.be
         q = SeedQuery(be.ptr(chunk_ptr), be.ptr(chunk_nodes), int(chunks.shape[0]), be.ptr(chunks),
@@ -412,9 +414,11 @@ class HotPath:
         self._ck(self.lib.seeds_count(C.byref(g.view), C.byref(q), be.ptr(totals), be.ptr(ws), wsb, be.stream()))
         R, S, Q = be.tolist(totals)
         roots, ts_ptr, ts, q_ptr, q_eid = be.empty(R), be.empty(R + 1), be.empty(S), be.empty(S + 1), be.empty(Q)
+        w_end = be.empty(S) if with_window_end else None
         self._ck(self.lib.seeds_fill(C.byref(g.view), C.byref(q), be.ptr(totals), be.ptr(roots), be.ptr(ts_ptr),
-                                     be.ptr(ts), be.ptr(q_ptr), be.ptr(q_eid), be.ptr(ws), wsb, be.stream()))
-        return roots, ts_ptr, ts, q_ptr, q_eid
+                                     be.ptr(ts), be.ptr(q_ptr), be.ptr(q_eid), be.ptr(w_end) if with_window_end else None,
+                                     be.ptr(ws), wsb, be.stream()))
+        return (roots, ts_ptr, ts, q_ptr, q_eid, w_end) if with_window_end else (roots, ts_ptr, ts, q_ptr, q_eid)
 
     def slice(self, g, chunk_ptr, chunk_nodes, node_chunk, chunks, cand_off, n_cand, t_begin, t_end,
               full_timestamps=False):

@@ -26,11 +26,14 @@ from .driver import check_unique_total
 class TemporalRoot:
     """export.cu:28-79 / sample.cu.hpp:849-871."""
 
-    def __init__(self, roots, ts_ptr, ts, q_ptr=None, q_eid=None):
+    def __init__(self, roots, ts_ptr, ts, q_ptr=None, q_eid=None, window_end=None):
         e = roots.new_empty(0)
         self.roots, self.ts_ptr, self.ts = roots, ts_ptr, ts
         self.q_ptr = e if q_ptr is None else q_ptr
         self.q_eid = e if q_eid is None else q_eid
+        # not in the reference: per (root, timestamp) where the window strictly before it ends; roots
+        # that come out of get_seeds_in_chunks carry it, and sampling them then needs no search
+        self.window_end = window_end
 
     @property
     def root_num(self):
@@ -133,6 +136,9 @@ class CUDAGraph:
         hp = self._hp
         p = hp.params(sample_type, k, allowed_offset, equal_root_time, keep_root_time,
                       seed=self._seed if seed is None else seed)
+        w_end = getattr(postive_root, "window_end", None)
+        if w_end is not None and w_end.numel() == postive_root.ts.numel():
+            p = hp.with_root_hint(p, w_end)
         neg = negative_root if negative_root is not None else self._empty_neg()
         if _defer is None:
             res = hp.sample_khop(self._g, postive_root.roots, postive_root.ts_ptr, postive_root.ts, neg.roots, neg.ts,

@@ -59,7 +59,8 @@ def seeds_in_chunks(graph, chunks, t_begin, t_end, full_timestamps=False):
         nodes, ts_ptr, ts, q_ptr, _, _, q_eid = graph._hp.slice(graph._g, chunk_ptr, chunk_nodes, None, d_chunks, d_off,
                                                                 n_cand, t_begin, t_end, True)
         return TemporalRoot(nodes, ts_ptr, ts, q_ptr, q_eid)
-    out = graph._hp.seeds(graph._g, chunk_ptr, chunk_nodes, d_chunks, d_off, n_cand, t_begin, t_end)
+    out = graph._hp.seeds(graph._g, chunk_ptr, chunk_nodes, d_chunks, d_off, n_cand, t_begin, t_end,
+                          with_window_end=True)
     return TemporalRoot(*out)
 
 

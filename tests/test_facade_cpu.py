@@ -80,10 +80,14 @@ def test_oracle_seeds_match_brute_force(oracle):
         ch = np.array(chunks, dtype=np.int64)
         sizes = chunk_ptr[ch + 1] - chunk_ptr[ch] if ch.size else np.zeros(0, np.int64)
         off = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
-        got = oracle.seeds(g, chunk_ptr, chunk_nodes, ch, off, int(off[-1]), t0, t1)
+        got = oracle.seeds(g, chunk_ptr, chunk_nodes, ch, off, int(off[-1]), t0, t1, with_window_end=True)
         want = _seed_brute(g, chunk_of, chunks, t0, t1)
         for a, b in zip(got, want):
             assert a.tolist() == [int(x) for x in b]
+        # window end of a (root, timestamp): number of the root's edges before that time, from the row's start
+        slot_root = np.repeat(got[0], np.diff(got[1]))
+        brute = [int(g.row_ptr[v] + (g.ts[g.row_ptr[v]: g.row_ptr[v + 1]] < t).sum()) for v, t in zip(slot_root, got[2])]
+        assert got[5].tolist() == brute
     with pytest.raises(IndexError):
         oracle.chunk_index(3, 2, np.array([0, 2, 1], dtype=np.int64))
 

@@ -337,7 +337,9 @@ def test_seeds_heavy_windows_and_tile_boundaries(oracle, hot, n, t_max):
         ch = np.asarray(chunks, dtype=np.int64)
         off = np.concatenate([[0], np.cumsum(cp[ch + 1] - cp[ch])]).astype(np.int64)
         for t0, t1 in ((0, t_max), (t_max // 3, t_max // 3 + 1), (t_max // 2, t_max // 2 + 7), (5, 5), (t_max, t_max + 9)):
-            want = oracle.seeds(hg, cp, cn, ch, off, int(off[-1]), t0, t1)
-            got = hot.seeds(dg, dcp, dcn, to_dev(hot, ch), to_dev(hot, off), int(off[-1]), t0, t1)
-            for f, a, b in zip(("roots", "ts_ptr", "ts", "q_ptr", "q_eid"), got, want):
+            want = oracle.seeds(hg, cp, cn, ch, off, int(off[-1]), t0, t1, with_window_end=True)
+            got = hot.seeds(dg, dcp, dcn, to_dev(hot, ch), to_dev(hot, off), int(off[-1]), t0, t1, with_window_end=True)
+            for f, a, b in zip(("roots", "ts_ptr", "ts", "q_ptr", "q_eid", "window_end"), got, want):
                 assert np.array_equal(np_of(a), b), (f, chunks, t0, t1)
+            # the sixth array is what a window-end lookup of every (root, timestamp) gives
+            assert np.array_equal(want[5], oracle.window_end(hg, np.repeat(want[0], np.diff(want[1])), want[2]))

@@ -91,9 +91,9 @@ def _one_case(seed, oracle, hot):
     off = np.concatenate([[0], np.cumsum(cp[ch + 1] - cp[ch])]).astype(np.int64)
     t0 = int(rng.integers(0, t_max + 1))
     t1 = t0 + int(rng.choice([0, 1, 7, t_max]))
-    ws = oracle.seeds(g, cp, cn, ch, off, int(off[-1]), t0, t1)
-    gs = hot.seeds(dg, dcp, dcn, to_dev(hot, ch), to_dev(hot, off), int(off[-1]), t0, t1)
-    for f, a, b in zip(("roots", "ts_ptr", "ts", "q_ptr", "q_eid"), gs, ws): assert np.array_equal(np_of(a), b), ("seeds", f)
+    ws = oracle.seeds(g, cp, cn, ch, off, int(off[-1]), t0, t1, with_window_end=True)
+    gs = hot.seeds(dg, dcp, dcn, to_dev(hot, ch), to_dev(hot, off), int(off[-1]), t0, t1, with_window_end=True)
+    for f, a, b in zip(("roots", "ts_ptr", "ts", "q_ptr", "q_eid", "window_end"), gs, ws): assert np.array_equal(np_of(a), b), ("seeds", f)
     if t1 - t0 <= 1000:
         full = bool(rng.integers(0, 2))
         wsl = oracle.slice(g, cp, cn, chunk_of, ch, off, int(off[-1]), t0, t1, full)
