@@ -374,3 +374,25 @@ def test_root_hints_give_the_same_samples(oracle, hot, sample_type):
     wild = to_dev(hot, rng.integers(-5, 2 * g.m, S_pos).astype(np.int64))
     res = hot.sample_khop(dg, *dev, 1, hot.with_root_hint(hot.params(sample_type, 17), wild))
     assert 0 <= res.hops[0].E <= (S_pos + n_neg) * 17
+
+
+def test_window_end_edge_cases(oracle, hot):
+    """No queries, ids that are no node (-1), nodes without edges (their row's start), times before the
+    first and after the last edge of a row, and a graph without edges."""
+    src = np.array([1, 1, 1, 4], dtype=np.int64)
+    dst = np.array([2, 3, 4, 1], dtype=np.int64)
+    ts = np.array([10, 10, 20, 5], dtype=np.int64)
+    g = host_graph(oracle, 6, src, dst, ts)
+    dg = mirror_graph(hot, g)
+    node = np.array([-1, 6, 0, 1, 1, 1, 1, 4, 5], dtype=np.int64)
+    t = np.array([0, 0, 7, 9, 10, 11, 99, 5, -3], dtype=np.int64)
+    want = oracle.window_end(g, node, t)
+    assert want.tolist() == [-1, -1, 0, 0, 0, 2, 3, 3, 4]
+    assert np.array_equal(np_of(hot.window_end(dg, to_dev(hot, node), to_dev(hot, t))), want)
+    e = np.zeros(0, np.int64)
+    assert hot.window_end(dg, to_dev(hot, e), to_dev(hot, e)).numel() == 0
+    g0 = host_graph(oracle, 3, e, e, e)
+    dg0 = mirror_graph(hot, g0)
+    assert np_of(hot.window_end(dg0, to_dev(hot, node[:3]), to_dev(hot, t[:3]))).tolist() == [-1, -1, 0]
+    with pytest.raises(ValueError):
+        hot.window_end(dg, to_dev(hot, node), to_dev(hot, t[:3]))
