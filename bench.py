@@ -895,6 +895,18 @@ def main():
                         "GBps": round((samp_bytes(S0 * mult, cnt[1]) + samp_bytes(cnt[1], cnt[4])) / ms / 1e6, 1)})
         del kb, gcalls, ins
     extra["sampler scaling (2-hop recent 10x10, several batches per call)"] = scaling
+    # time encoding at this config's scale: one row of cos(w * dt + b) per sampled edge of a batch at the
+    # worst case (S0*k + S0*k*k edges, dim 100): 8 bytes read and 400 written per row
+    te_rows, te_dim = S0 * k + S0 * k * k, 100
+    te_dt = torch.randint(0, 1 << 40, (te_rows,), dtype=torch.int64, device=dev)
+    te_w = (1.0 / 10 ** torch.linspace(0, 9, te_dim, dtype=torch.float32)).to(dev)
+    te_b = torch.zeros(te_dim, dtype=torch.float32, device=dev)
+    te_out = torch.empty((te_rows, te_dim), dtype=torch.float32, device=dev)
+    ms = _time_launches(torch, lambda: hot.time_encode(te_dt, te_w, te_b, out=te_out), reps=10)
+    te_gbps = te_rows * (8 + 4 * te_dim) / ms / 1e6
+    extra["time encode (1.32M rows x 100)"] = {"ms": round(ms, 4), "rows": te_rows, "GBps": round(te_gbps, 1),
+                                               "frac_of_hbm_peak": round(te_gbps / HBM_PEAK_GBPS, 3)}
+    del te_dt, te_out
     if cpu is not None:
         # GPU side: the GPU's time per 12000-root call, calls over different batches replayed back to back
         # from one HIP graph (as they run inside the step); then the same when one call samples several batches

@@ -36,14 +36,19 @@ struct TEArgs {
 // in double precision by multiples of pi (two-constant Cody-Waite, exact through
 // FMA) to r in [-pi/2, pi/2]; then cos(r) = 1 - 2 sin^2(r/2) with one odd
 // polynomial for sin on [-pi/4, pi/4] - no quadrant-dependent coefficients, so no
-// selects - and the sign (-1)^n is applied by a multiply.  About 20 fp64
+// selects - and the sign (-1)^n is applied to the sign bit of the result.  About 16 fp64
 // operations, all straight-line.  The library cosf takes ~2.5x as long (its
 // large-argument path is a Payne-Hanek reduction).  Arguments beyond 2^45 (not
 // reachable from int64 timestamps times w <= 1 in practice) take the library routine.
 __device__ __forceinline__ float cos_f32(float af) {
     if (!(__builtin_fabsf(af) < 3.5e13f)) return cosf(af);   // also NaN / inf
     const double x = (double)af;
-    const double n = __builtin_rint(x * 0.31830988618379067154);        // 1/pi
+    // n = nearest integer to x/pi without a rounding instruction: adding 1.5 * 2^52 leaves n in the low
+    // mantissa bits of the sum (|x/pi| < 2^44 here), whose lowest bit is the parity of n
+    constexpr double SHIFT = 6755399441055744.0;
+    const double t = __builtin_fma(x, 0.31830988618379067154, SHIFT);   // 1/pi
+    const uint32_t odd = (uint32_t)__double_as_longlong(t) & 1u;
+    const double n = t - SHIFT;
     double r = __builtin_fma(-n, 3.14159265358979311600e+00, x);        // pi, high part
     r = __builtin_fma(-n, 1.22464679914735317723e-16, r);               // pi, low part
     const double h = 0.5 * r, h2 = h * h;
@@ -54,11 +59,9 @@ __device__ __forceinline__ float cos_f32(float af) {
     p = __builtin_fma(p, h2, 8.333333333333333333e-03);                 //  1/5!
     p = __builtin_fma(p, h2, -1.666666666666666667e-01);                // -1/3!
     const double sn = __builtin_fma(p, h * h2, h);
-    const double c = __builtin_fma(-2.0 * sn, sn, 1.0);                 // cos(r)
-    // (-1)^n: n/2 has fraction 0 (even) or 1/2 (odd)
-    const double half = 0.5 * n;
-    const double frac = half - __builtin_floor(half);
-    return (float)(c * __builtin_fma(-4.0, frac, 1.0));
+    const float c = (float)__builtin_fma(-2.0 * sn, sn, 1.0);           // cos(r)
+    // (-1)^n: flip the sign bit of the rounded result
+    return __uint_as_float(__float_as_uint(c) ^ (odd << 31));
 }
 
 __device__ __forceinline__ float enc(float w, float x, float b) {
