@@ -50,6 +50,11 @@ extern "C" {
  * csrc/srcs/starrygl/export.cu:237-244 and sample.cu.hpp:1001-1062. */
 const char* sgl_last_error_string(void);
 int32_t     sgl_abi_version(void);
+/* sizeof of the ABI's structs as this library was compiled, so that a binding
+ * which mirrors them field by field (ctypes, cgo, JNI) can check its layout at
+ * load time: which = 0 sgl_tcsr, 1 sgl_sample_params, 2 sgl_hop_out,
+ * 3 sgl_cache, 4 sgl_gather_seg, 5 sgl_seed_query; 0 for any other index. */
+size_t      sgl_struct_bytes(int32_t which);
 
 /* Kernels whose blocks exchange totals inside one launch (the 2-hop sampler of
  * small calls, the numbering pass of sgl_unique_compact on small universes)

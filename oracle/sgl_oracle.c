@@ -44,6 +44,17 @@ static int32_t fail(int32_t code, const char* msg) {
 
 const char* sglo_last_error_string(void) { return g_err; }
 int32_t     sglo_abi_version(void) { return SGL_ABI_VERSION; }
+size_t      sglo_struct_bytes(int32_t which) {
+    switch (which) {
+        case 0: return sizeof(sgl_tcsr);
+        case 1: return sizeof(sgl_sample_params);
+        case 2: return sizeof(sgl_hop_out);
+        case 3: return sizeof(sgl_cache);
+        case 4: return sizeof(sgl_gather_seg);
+        case 5: return sizeof(sgl_seed_query);
+        default: return 0;
+    }
+}
 
 /* The oracle has no kernels that wait for each other: the limit is kept and returned only. */
 static int32_t g_wait_limit = 1 << 20;

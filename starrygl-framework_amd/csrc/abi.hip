@@ -34,3 +34,14 @@ extern "C" int32_t sgl_set_wait_limit(int32_t polls) {
 
 extern "C" const char* sgl_last_error_string(void) { return sgl::err_buf(); }
 extern "C" int32_t sgl_abi_version(void) { return SGL_ABI_VERSION; }
+extern "C" size_t sgl_struct_bytes(int32_t which) {
+    switch (which) {
+        case 0: return sizeof(sgl_tcsr);
+        case 1: return sizeof(sgl_sample_params);
+        case 2: return sizeof(sgl_hop_out);
+        case 3: return sizeof(sgl_cache);
+        case 4: return sizeof(sgl_gather_seg);
+        case 5: return sizeof(sgl_seed_query);
+        default: return 0;
+    }
+}

@@ -52,12 +52,17 @@ class SeedQuery(C.Structure):
                 ("cand_off", vp), ("n_cand", i64), ("t_begin", i64), ("t_end", i64)]
 
 
+# in the order of sgl_struct_bytes(which)
+STRUCTS = (TCSR, SampleParams, HopOut, Cache, GatherSeg, SeedQuery)
+
+
 P = C.POINTER
 
 # name -> (restype, argtypes); the order follows include/sgl_hot.h
 PROTOTYPES = {
     "last_error_string": (C.c_char_p, []),
     "abi_version": (i32, []),
+    "struct_bytes": (sz, [i32]),
     "set_wait_limit": (i32, [i32]),
     "tcsr_build_workspace_bytes": (sz, [i64, i64]),
     "tcsr_build": (i32, [i64, i64, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]),

@@ -127,6 +127,10 @@ class HotPath:
         self.lib, self.be = lib, backend
         if lib.abi_version() != _abi.ABI_VERSION:
             raise RuntimeError("sgl ABI version mismatch")
+        for which, mirror in enumerate(_abi.STRUCTS):     # the ctypes mirrors must have the library's layout
+            if int(lib.struct_bytes(which)) != C.sizeof(mirror):
+                raise RuntimeError(f"sgl ABI struct {mirror.__name__}: the library has {int(lib.struct_bytes(which))} "
+                                   f"bytes, the binding {C.sizeof(mirror)}")
         self._ws = {}
 
     # ------------------------------------------------------------ helpers

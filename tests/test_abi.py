@@ -27,6 +27,10 @@ def test_header_symbols_are_exported_and_bound():
 def test_abi_version_and_host_side_errors():
     lib = _abi.bind(C.CDLL(LIB_PATH))
     assert lib.abi_version() == _abi.ABI_VERSION
+    # the ctypes mirrors have the layout the library was compiled with
+    for which, mirror in enumerate(_abi.STRUCTS):
+        assert lib.struct_bytes(which) == C.sizeof(mirror), mirror.__name__
+    assert lib.struct_bytes(len(_abi.STRUCTS)) == 0 and lib.struct_bytes(-1) == 0
     # argument validation happens on the host, before any HIP call
     p = _abi.SampleParams(7, 3, -1, 0, 0, 0, 0, 0)
     g = _abi.TCSR(1, 0, 8, None, None, None)
