@@ -249,6 +249,17 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     res["gather_all_three_one_launch"] = {"ms": round(ms, 4), "GBps": round((u1 * (2 * 812 + 16) + e1 * 1384) / ms / 1e6, 1)}
     ms = _time_launches(torch, lambda: hot.sample_khop(dg, s_in[0], ts_ptr, s_in[1], s_in[2], s_in[3], 1, p, finalize=False, out=kr))
     res["sample_recent_1hop"] = {"ms": round(ms, 4), "edges_per_s": round(e1 / ms * 1e3, 1)}
+    # the write side of the step (last: it changes the tables): the 2B endpoints of the batch's events get new
+    # memory rows - latest event per node (unique + per-node maximum of the event times), then rows and times
+    # scattered into the two-tier table, 30 % of them over PCIe into pinned host memory
+    ends_, ends_ts = roots[0], root_ts[0]
+    loc_, uniq_, (u_n, _) = hot.unique_compact([ends_], _abi.UNIQUE_SORTED, None, True)
+    vals = torch.randn((u_n, 100), device=dev, generator=gen)
+    ms_red = _time_launches(torch, lambda: hot.segment_max_ts(loc_[0], ends_ts, u_n))
+    new_ts, _ = hot.segment_max_ts(loc_[0], ends_ts, u_n)
+    ms_upd = _time_launches(torch, lambda: hot.scatter_update(c_mem, mem_hot, mem_cold, ts_hot, ts_cold, uniq_, vals, new_ts))
+    res["memory_update"] = {"nodes": int(u_n), "latest_event_per_node_ms": round(ms_red, 4), "scatter_update_ms": round(ms_upd, 4),
+                            "GBps": round(u_n * (8 + 4 + 400 + 400 + 16) / ms_upd / 1e6, 1)}
     return res
 
 
