@@ -167,7 +167,9 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     S0_dev = D(np.array([S0], dtype=np.int64))
     w = torch.from_numpy((1.0 / 10 ** np.linspace(0, 9, 100, dtype=np.float32)).astype(np.float32)).to(dev)
     bias = torch.zeros(100, device=dev)
-    packed = torch.cat([roots, root_ts, neg, neg_ts], dim=1).contiguous()
+    # the loader's one-off lookup for the events of the stream: where the window of every positive root ends
+    root_hint = hot.window_end(dg, roots.reshape(-1), root_ts.reshape(-1)).view(NB, -1)
+    packed = torch.cat([roots, root_ts, neg, neg_ts, root_hint], dim=1).contiguous()
 
     def make_pipeline(stream):
         """One copy of the step: own buffers, remap state, HIP graph, on `stream`."""
@@ -182,16 +184,19 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
         P.o_ef = torch.empty((S0 * k, 172), device=dev)
         P.o_te = torch.empty((S0 * k, 100), device=dev)
         P.s_all = torch.empty_like(packed[0])
-        P.s_in = torch.split(P.s_all, [roots.shape[1], root_ts.shape[1], neg.shape[1], neg_ts.shape[1]])
+        P.s_in = torch.split(P.s_all, [roots.shape[1], root_ts.shape[1], neg.shape[1], neg_ts.shape[1], root_hint.shape[1]])
+        # the sampler takes the batch's root hints and records the ids it emits as pending for unique
+        P.p = hot.marking(hot.with_root_hint(p, P.s_in[4]), P.state)
         P.E = P.kr.hops[0].counts[1:2]
         P.acc = torch.zeros(2, dtype=torch.int64, device=dev)
         P.plan = hot.gather_plan([(c_mem, P.ubuf, P.o_mem, P.o_ts, P.U[0:1]), (c_nf, P.ubuf, P.o_nf, None, P.U[0:1]),
                                   (c_ef, P.kr.hops[0].neighbors_eid, P.o_ef, None, P.E)])
 
         def body():
-            hot.sample_khop(dg, P.s_in[0], ts_ptr, P.s_in[1], P.s_in[2], P.s_in[3], 1, p, finalize=False, out=P.kr)
+            hot.sample_khop(dg, P.s_in[0], ts_ptr, P.s_in[1], P.s_in[2], P.s_in[3], 1, P.p, finalize=False, out=P.kr)
             hot.unique_compact([P.kr.slot_node0, P.kr.hops[0].neighbors], _abi.UNIQUE_SORTED, P.state, True,
-                               lens_dev=[S0_dev, P.E], out_arrays=P.local, finalize=False, unique_out=P.ubuf, U_out=P.U)
+                               lens_dev=[S0_dev, P.E], out_arrays=P.local, finalize=False, unique_out=P.ubuf, U_out=P.U,
+                               premarked=True)
             hot.gather_multi(P.plan)
             hot.time_encode(P.kr.hops[0].neighbors_dt, w, bias, out=P.o_te, N_dev=P.E)
             P.acc[0:1].add_(P.E); P.acc[1:2].add_(P.U[0:1])
@@ -247,7 +252,8 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     res["gather_memory_30pct_host"] = {"ms": round(ms, 4), "rows": u1, "GBps": round(u1 * (8 + 4 + 800 + 16) / ms / 1e6, 1)}
     ms = _time_launches(torch, lambda: hot.gather_multi(plan))
     res["gather_all_three_one_launch"] = {"ms": round(ms, 4), "GBps": round((u1 * (2 * 812 + 16) + e1 * 1384) / ms / 1e6, 1)}
-    ms = _time_launches(torch, lambda: hot.sample_khop(dg, s_in[0], ts_ptr, s_in[1], s_in[2], s_in[3], 1, p, finalize=False, out=kr))
+    p_h = hot.with_root_hint(p, s_in[4])
+    ms = _time_launches(torch, lambda: hot.sample_khop(dg, s_in[0], ts_ptr, s_in[1], s_in[2], s_in[3], 1, p_h, finalize=False, out=kr))
     res["sample_recent_1hop"] = {"ms": round(ms, 4), "edges_per_s": round(e1 / ms * 1e3, 1)}
     # the write side of the step (last: it changes the tables): the 2B endpoints of the batch's events get new
     # memory rows - latest event per node (unique + per-node maximum of the event times), then rows and times
