@@ -211,13 +211,16 @@ class MiniBatchPipeline:
         return self._run(roots, root_ts, neg_roots, neg_ts, root_hint)
 
     def _run(self, roots, root_ts, neg_roots, neg_ts, root_hint):
-        self.in_roots.copy_(roots, non_blocking=True)
-        self.in_ts.copy_(root_ts, non_blocking=True)
+        dsts, srcs = [self.in_roots, self.in_ts], [roots, root_ts]
         if root_hint is not None:
-            self.in_hint.copy_(root_hint, non_blocking=True)
+            dsts.append(self.in_hint); srcs.append(root_hint)
         if self.N_neg:
-            self.in_neg.copy_(neg_roots, non_blocking=True)
-            self.in_neg_ts.copy_(neg_ts, non_blocking=True)
+            dsts += [self.in_neg, self.in_neg_ts]; srcs += [neg_roots, neg_ts]
+        if all(t.is_cuda and t.dtype == torch.int64 and t.is_contiguous() for t in srcs):
+            torch._foreach_copy_(dsts, [t.reshape(-1) for t in srcs], non_blocking=True)   # one launch for all inputs
+        else:
+            for d, t in zip(dsts, srcs):
+                d.copy_(t.reshape(-1), non_blocking=True)
         if not self.use_graph:
             self._chain()
         elif self._graph is None:
