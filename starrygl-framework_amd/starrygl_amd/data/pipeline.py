@@ -256,8 +256,8 @@ def bound_streams(n, device):
 class MiniBatchPipelinePool:
     """`n` MiniBatchPipeline objects on streams of their own; run() hands the batches to them in
     turn, so that up to `n` batches are in flight: the latency-bound sampling of one batch overlaps
-    the bandwidth-bound gathers of another (configs of 12 000 roots, 2 hops: 0.09 ms per batch with
-    three in flight against 0.115 ms one at a time).  A MiniBatch stays valid until the `n`-th
+    the bandwidth-bound gathers of another (12 000 roots, 2-hop recent 10x10, node and edge rows
+    of a 1M-node / 20M-edge graph: 0.071 ms per batch with three in flight against 0.094 ms one at a time).  A MiniBatch stays valid until the `n`-th
     following run().  Create the pool before any other stream of the process."""
 
     def __init__(self, n, graph, *args, **kwargs):
