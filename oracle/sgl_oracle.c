@@ -11,15 +11,20 @@
  * StarryGL tree).  Where the reference disagrees with itself the rule that is
  * implemented is written next to the citation.
  *
- * What pins each function (see tests/test_oracle_*.py):
+ * What pins each function (tests/test_oracle.py, tests/test_facade_cpu.py):
  *   window / recent      np.searchsorted + brute-force list comprehension
+ *   next-hop index,      np.searchsorted(side='left') on the row slice, a
+ *   window ends          brute-force count of the row's earlier edges
  *   uniform              Philox4x32-10 known-answer vectors (Random123),
  *                        subset invariants, chi-square over seeds
  *   unique               np.unique(return_inverse), np.setdiff1d per group
  *   gather / scatter     numpy fancy indexing
  *   time encode          float64 closed form
  *   t-csr build          np.lexsort((eid, ts, src)) + bincount/cumsum
- *   seeds / block        brute-force python loops on tiny graphs
+ *   seeds / block /      brute-force python loops on tiny graphs,
+ *   slice / chunk index  np.argsort(kind='stable')
+ *   pair unique / CSC    np.unique over (id, ts) records, np.lexsort((ts, dst))
+ *   latest event / node  per-key maximum and first arg-maximum in numpy
  *
  * Build:  make -C oracle      (gcc -O2 -fopenmp -ffp-contract=off)
  */
