@@ -359,8 +359,8 @@ def workload_large_partition(hot, torch, np, synth, _abi, n=100_000_000, m=1_000
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--nodes", type=int, default=1_000_000)
     ap.add_argument("--edges", type=int, default=20_000_000)
     ap.add_argument("--batch-edges", type=int, default=4000)
