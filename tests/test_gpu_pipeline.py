@@ -120,3 +120,45 @@ def test_pipeline_with_root_hints(oracle, hot, sample_type):
     plain = MiniBatchPipeline(g, 2 * B, B, 2, 6, sample_type)
     with pytest.raises(ValueError):
         plain.run(to_dev(hot, b[0]), to_dev(hot, b[2]), to_dev(hot, b[3]), to_dev(hot, b[4]), root_hint=hint)
+
+
+@pytest.mark.parametrize("prefetch", [1, 3])
+def test_event_batch_loader(oracle, hot, prefetch):
+    """The loader walks the event stream batch by batch with `prefetch` batches in flight and the window ends
+    of all event endpoints looked up once; every yielded batch equals the oracle's result for its own events
+    and the negatives it drew (read back from the batch), and is still intact while the next ones are in flight."""
+    from starrygl_amd.data import EventBatchLoader
+    from starrygl_amd.graph.graph import NegSamplingSet
+    from starrygl_amd.lib.libstarrygl_comm import from_edge_index
+    n, m, B, NEG = 2500, 50_000, 200, 150
+    src, dst, ts, eid = synth.graph_stream(n, m, 1.15, 30_000, 31)
+    order = np.argsort(ts, kind="stable")
+    src, dst, ts, eid = src[order], dst[order], ts[order], eid[order]       # the stream in time order
+    hg = host_graph(oracle, n, src, dst, ts, eid)
+    g = from_edge_index(n, 1, *(torch.from_numpy(x) for x in (src, dst, ts, eid)))
+    feat = np.random.default_rng(2).standard_normal((n, 100)).astype(np.float32)
+    lo_ev = 40_000                                                             # train on the last 10 000 events
+    sampler = NegSamplingSet(torch.arange(100, 2000, device="cuda"))
+    loader = EventBatchLoader(g, src[lo_ev:], dst[lo_ev:], ts[lo_ev:], B, NEG, 2, 5, "recent",
+                              node_tables={"x": hot.cache(400, to_dev(hot, feat, "f32"))}, prefetch=prefetch,
+                              negative_sampler=sampler)
+    for p in loader.pool.pipes:
+        p.view("x", torch.float32)
+    assert len(loader) == 10_000 // B
+    seen, held = 0, None
+    for i, mb in enumerate(loader):
+        lo = lo_ev + i * B
+        roots = np.concatenate([src[lo: lo + B], dst[lo: lo + B]])
+        root_ts = np.concatenate([ts[lo: lo + B], ts[lo: lo + B]])
+        neg, neg_ts = np_of(mb.slot_node)[2 * B:], np_of(mb.slot_ts)[2 * B:]
+        assert neg.shape[0] == NEG and (neg >= 100).all() and (neg < 2000).all()
+        assert np.array_equal(neg_ts, np.resize(ts[lo: lo + B], NEG))
+        want = oracle.sample_khop(hg, roots, np.arange(2 * B + 1, dtype=np.int64), root_ts, neg, neg_ts, 2,
+                                  oracle.params("recent", 5))
+        assert mb.E == [h.E for h in want.hops]
+        _, uniq, _ = oracle.unique_compact([want.slot_node0] + [h.neighbors for h in want.hops], _abi.UNIQUE_SORTED, None, True)
+        assert np.array_equal(np_of(mb.nid_mapper), uniq) and np.array_equal(np_of(mb.node_data["x"]), feat[uniq])
+        for l, h in enumerate(want.hops):
+            assert np.array_equal(np_of(mb.hops[l]["neighbors_eid"]), h.neighbors_eid)
+        seen += 1
+    assert seen == len(loader)
