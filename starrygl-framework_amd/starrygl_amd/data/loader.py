@@ -32,8 +32,16 @@ class EventBatchLoader:
         self.graph = graph
         self.negative_sampler = negative_sampler
         # one lookup per event endpoint for the whole stream (sgl_window_end)
-        self.end_src = graph.window_end(self.src, self.ts)
-        self.end_dst = graph.window_end(self.dst, self.ts)
+        end_src = graph.window_end(self.src, self.ts)
+        end_dst = graph.window_end(self.dst, self.ts)
+        # the inputs of every full batch, laid out once as rows: [sources; destinations] and their times and
+        # window ends, and the negatives' times (the batch's event times, repeated)
+        nb, B, n_neg = int(self.src.numel()) // self.B, self.B, self.num_neg
+        rows = lambda a, b_: torch.cat([a[: nb * B].view(nb, B), b_[: nb * B].view(nb, B)], dim=1).contiguous()
+        self._roots, self._root_ts, self._hint = rows(self.src, self.dst), rows(self.ts, self.ts), rows(end_src, end_dst)
+        t_rows = self.ts[: nb * B].view(nb, B)
+        self._neg_ts = t_rows.repeat(1, (n_neg + B - 1) // B)[:, :n_neg].contiguous() if n_neg else t_rows[:, :0]
+        self._neg_block, self._neg_at = None, 0
         self.pool = MiniBatchPipelinePool(max(1, int(prefetch)), graph, 2 * self.B, self.num_neg, layers, fanout,
                                           sample_type, node_tables=node_tables, edge_tables=edge_tables,
                                           time_encoder=time_encoder, root_hints=True, **pipeline_kwargs)
@@ -41,25 +49,23 @@ class EventBatchLoader:
     def __len__(self):
         return int(self.src.numel()) // self.B
 
-    def _negatives(self, lo):
+    NEG_BLOCK = 64      # negatives are drawn for this many batches at a time (one launch instead of 64)
+
+    def _negatives(self):
         n = self.num_neg
         if n == 0:
-            e = self.src.new_empty(0)
-            return e, e
-        if self.negative_sampler is not None:
-            neg = self.negative_sampler.sample(n, 1).reshape(-1).to(self.src.device)
-        else:
-            neg = torch.randint(0, self.graph._n, (n,), device=self.src.device)
-        t = self.ts[lo: lo + self.B]
-        return neg, t.repeat((n + self.B - 1) // self.B)[:n].contiguous()
+            return self.src.new_empty(0)
+        if self._neg_block is None or self._neg_at == self.NEG_BLOCK:
+            if self.negative_sampler is not None:
+                blk = self.negative_sampler.sample(self.NEG_BLOCK * n, 1).reshape(self.NEG_BLOCK, n)
+            else:
+                blk = torch.randint(0, self.graph._n, (self.NEG_BLOCK, n), device=self.src.device)
+            self._neg_block, self._neg_at = blk.to(self.src.device), 0
+        self._neg_at += 1
+        return self._neg_block[self._neg_at - 1]
 
     def _submit(self, i):
-        lo, hi = i * self.B, (i + 1) * self.B
-        roots = torch.cat([self.src[lo:hi], self.dst[lo:hi]])
-        root_ts = torch.cat([self.ts[lo:hi], self.ts[lo:hi]])
-        hint = torch.cat([self.end_src[lo:hi], self.end_dst[lo:hi]])
-        neg, neg_ts = self._negatives(lo)
-        return self.pool.run(roots, root_ts, neg, neg_ts, root_hint=hint)
+        return self.pool.run(self._roots[i], self._root_ts[i], self._negatives(), self._neg_ts[i], root_hint=self._hint[i])
 
     def __iter__(self):
         """Yields the finalized MiniBatch of every full batch, in order.  A MiniBatch is valid until

@@ -35,8 +35,8 @@ class MiniBatch:
         p = self._p
         if p._done is not None:      # the batch ran on the pipeline's own stream
             p._done.synchronize()
-        c = p.kr.counts.cpu().tolist()
-        u_total = int(p.U[0].item())
+        c = p.live.tolist()
+        u_total = int(c[3 * p.layers])
         check_unique_total(u_total)
         check_sample_bad(max(c[3 * l + 2] for l in range(p.layers)))
         check_sample_bad(sum(c[3 * l + 2] for l in range(p.layers)))
@@ -128,11 +128,13 @@ class MiniBatchPipeline:
         if root_hints:
             self.p = hp.with_root_hint(self.p, self.in_hint)
         # outputs
-        self.kr = hp.khop_buffers(self.S0, self.layers, self.fanout)
+        # every device-side count of a batch in one array: finalize() reads them with one copy
+        self.live = be.zeros(3 * self.layers + 2)
+        self.kr = hp.khop_buffers(self.S0, self.layers, self.fanout, counts=self.live[: 3 * self.layers])
         caps = [self.S0] + [self.S0 * self.fanout ** (l + 1) for l in range(self.layers)]
         self.local = [be.empty(c) for c in caps]
         self.ucap = min(sum(caps), graph._n)
-        self.ubuf, self.U = be.empty(max(self.ucap, 1)), be.zeros(2)
+        self.ubuf, self.U = be.empty(max(self.ucap, 1)), self.live[3 * self.layers:]
         self.state = hp.remap_state(graph._n)
         # the sampler records the ids it emits as pending in the remap state: unique skips its first pass
         self.p = hp.marking(self.p, self.state)
