@@ -67,7 +67,7 @@ __device__ __forceinline__ const char* resolve(const sgl_cache& c, int64_t id, i
 // NT: non-temporal loads and stores, for outputs much larger than the last-level
 // cache (measured: +5..13 % beyond ~0.5 GB, -15 % at 70 MB, so small calls keep
 // the cached path where repeated rows hit in L2).
-template <typename V, bool NT>
+template <typename V, bool NT, bool NT_STORE = NT>
 __global__ __launch_bounds__(BLOCK) void gather_kernel(GatherArgs a) {
     extern __shared__ const char* s_src[];  // [rpb]
     __shared__ int32_t s_tier[3];
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(BLOCK) void gather_kernel(GatherArgs a) {
             for (int u = 0; u < UNROLL; ++u) {
                 const int32_t lc = base + u * BLOCK + threadIdx.x;
                 if (lc < total) {
-                    if (NT) __builtin_nontemporal_store(val[u], dst + lc);
+                    if (NT_STORE) __builtin_nontemporal_store(val[u], dst + lc);
                     else dst[lc] = val[u];
                 }
             }
@@ -293,9 +293,14 @@ extern "C" int32_t sgl_gather(const sgl_cache* c, const int64_t* ids, int64_t N_
     if (blocks > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "gather: too many rows for one launch");
     const size_t shmem = (size_t)rpb * sizeof(char*);
     hipStream_t st = as_stream(stream);
-    const bool nt = (double)N_max * (double)c->row_bytes >= 256.0 * 1024 * 1024;
+    // host-known row count: loads and stores past the caches from 256 MB of output on; device-side count
+    // (the capacity says little about the live size): cached loads, streaming stores from 64 MB of capacity on
+    const double cap_bytes = (double)N_max * (double)c->row_bytes;
+    const bool nt = N_dev == nullptr && cap_bytes >= 256.0 * 1024 * 1024;
+    const bool nt_store = N_dev != nullptr && cap_bytes >= (double)NT_STORE_MIN_BYTES;
     const dim3 grid((unsigned)blocks), blk(BLOCK);
     if (vec == 16 && nt) hipLaunchKernelGGL((gather_kernel<u32x4, true>), grid, blk, shmem, st, a);
+    else if (vec == 16 && nt_store) hipLaunchKernelGGL((gather_kernel<u32x4, false, true>), grid, blk, shmem, st, a);
     else if (vec == 16) hipLaunchKernelGGL((gather_kernel<u32x4, false>), grid, blk, shmem, st, a);
     else if (vec == 8) hipLaunchKernelGGL((gather_kernel<u32x2, false>), grid, blk, shmem, st, a);
     else hipLaunchKernelGGL((gather_kernel<uint32_t, false>), grid, blk, shmem, st, a);
