@@ -195,6 +195,26 @@ int32_t sgl_sample_hop(const sgl_tcsr* g,
                        const sgl_sample_params* p, const sgl_hop_out* out,
                        void* workspace, size_t workspace_bytes, void* stream);
 
+/* sgl_sample_hop for callers that cannot allocate device memory and have no
+ * workspace to pass (code under HIP-graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and results as sgl_sample_hop, without the workspace: the
+ * hop's scratch (window starts / lengths per slot, per-block sums) is an array
+ * of sgl_sample_hop_workspace_bytes(SGL_STATIC_HOP_MAX_SLOTS) bytes (about
+ * 1.1 MB) inside the library image, one copy per GPU, held until the process
+ * ends.  S_max > SGL_STATIC_HOP_MAX_SLOTS is refused with SGL_ENOMEM.  The
+ * call allocates and frees nothing.  All calls on one GPU share that GPU's
+ * array: calls that overlap on one GPU (different streams, or host threads on
+ * different streams) race; order them on one stream or with events.  The
+ * first call on a device looks the array's address up (no allocation); make
+ * that call outside a stream capture. */
+#define SGL_STATIC_HOP_MAX_SLOTS 65536
+int32_t sgl_sample_hop_static(const sgl_tcsr* g,
+                              const int64_t* slot_node, const int64_t* slot_ts,
+                              int64_t S_max, const int64_t* S_dev,
+                              const sgl_sample_params* p, const sgl_hop_out* out,
+                              void* stream);
+
 /* k-hop driver (replaces Graph::sample_src_in_chunks_khop,
  * sample.cu.hpp:1532-1716).  Hop-0 slots are the positive roots expanded over
  * their timestamps (root r owns root_ts[ts_ptr[r]..ts_ptr[r+1])) followed by

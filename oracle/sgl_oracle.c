@@ -275,6 +275,7 @@ static void floyd_subset(uint64_t seed, int32_t hop, int64_t slot, int64_t cnt,
 
 size_t sglo_sample_hop_workspace_bytes(int64_t S_max) { (void)S_max; return 0; }
 
+
 /* One hop: count pass -> prefix sum -> fill pass, parallel over slots.
  * Reference: _jit_sample_kernel (prepare_sample.py:43-78 count, :80-82
  * prefix, :91-145 fill; recent :117-119, uniform :120-134);
@@ -356,6 +357,18 @@ int32_t sglo_sample_hop(const sgl_tcsr* g, const int64_t* slot_node,
     free(cnt); free(wlo); free(whi);
     return SGL_OK;
 }
+
+/* The workspace-free variant of the hop: the oracle never uses a workspace, so
+ * it is the same function (kept so that the oracle mirrors every entry point of
+ * include/sgl_hot.h; it has no counterpart in the reference). */
+int32_t sglo_sample_hop_static(const sgl_tcsr* g, const int64_t* slot_node,
+                               const int64_t* slot_ts, int64_t S_max,
+                               const int64_t* S_dev, const sgl_sample_params* p,
+                               const sgl_hop_out* out, void* stream) {
+    if (S_max > SGL_STATIC_HOP_MAX_SLOTS) return fail(SGL_ENOMEM, "sample_hop_static: slots exceed the limit");
+    return sglo_sample_hop(g, slot_node, slot_ts, S_max, S_dev, p, out, NULL, 0, stream);
+}
+
 
 size_t sglo_sample_khop_workspace_bytes(int64_t S0, int32_t layers, int32_t fanout) {
     (void)S0; (void)layers; (void)fanout;

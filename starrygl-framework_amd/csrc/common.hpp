@@ -33,7 +33,7 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 template <typename T>
 __host__ __device__ constexpr T ceil_div(T a, T b) { return (a + b - 1) / b; }
 
-inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
+constexpr size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
 
 // Bump allocator over a caller-provided workspace.
 struct Arena {

@@ -28,6 +28,8 @@
 // Replaces static_recent_neighbor_num / recent_sample_single_hop_kernel /
 // static_neighbor_num / uniform_sample_single_hop_kernel and the thrust calls
 // between them (csrc/include/starrygl/sample.cu.hpp:706-827, 1532-1716).
+#include <mutex>
+
 #include "common.hpp"
 
 namespace sgl {
@@ -579,7 +581,7 @@ int pick_search_group(int Gf, int64_t S_max) {
     return Gf;
 }
 
-size_t hop_workspace_bytes(int64_t S_max) {
+constexpr size_t hop_workspace_bytes(int64_t S_max) {
     size_t b = 0;
     b += align_up((size_t)(S_max + 1) * 8) * 2;
     b += align_up((size_t)MAX_BLOCKS * 8);
@@ -1221,6 +1223,52 @@ extern "C" int32_t sgl_sample_hop(const sgl_tcsr* g, const int64_t* slot_node, c
     if (S_max < 0) return fail(SGL_EINVAL, "sample_hop: S_max < 0");
     if ((rc = check_out(out, S_max, p->fanout)) != SGL_OK) return rc;
     return run_hop(g, slot_node, slot_ts, nullptr, S_max, S_dev, p, out, ws, ws_bytes, as_stream(stream));
+}
+
+// ---- sgl_sample_hop_static: the hop's scratch (window starts and lengths, block sums) lives in
+// device memory that belongs to the library image instead of a caller's workspace, for callers that
+// cannot allocate.  Each GPU holds its own copy of the array; host code never uses the array's name
+// as an address, only what hipGetSymbolAddress returned for the device that is current.
+constexpr size_t STATIC_SCRATCH_BYTES = hop_workspace_bytes(SGL_STATIC_HOP_MAX_SLOTS);
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int STATIC_MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[STATIC_MAX_DEVICES];   // per device, resolved at the first call on it
+
+int32_t static_scratch(void** out) {
+    int dev = -1;
+    SGL_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) return fail(SGL_ENOTSUP, "sample_hop_static: device %d not supported", dev);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        SGL_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (ptr == nullptr) return fail(SGL_EHIP, "sample_hop_static: no address for the scratch array on device %d", dev);
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return SGL_OK;
+}
+}  // namespace
+
+extern "C" int32_t sgl_sample_hop_static(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot_ts,
+                                         int64_t S_max, const int64_t* S_dev, const sgl_sample_params* p,
+                                         const sgl_hop_out* out, void* stream) {
+    int32_t rc;
+    if ((rc = check_graph(g)) != SGL_OK) return rc;
+    if ((rc = check_params(p)) != SGL_OK) return rc;
+    if (S_max < 0) return fail(SGL_EINVAL, "sample_hop_static: S_max < 0");
+    if (S_max > SGL_STATIC_HOP_MAX_SLOTS)
+        return fail(SGL_ENOMEM, "sample_hop_static: %lld slots exceed the limit of %lld (use sgl_sample_hop with a workspace)",
+                    (long long)S_max, (long long)SGL_STATIC_HOP_MAX_SLOTS);
+    if ((rc = check_out(out, S_max, p->fanout)) != SGL_OK) return rc;
+    void* ws = nullptr;
+    if ((rc = static_scratch(&ws)) != SGL_OK) return rc;
+    // every word of the scratch that a launch reads was written by an earlier launch of the same call
+    // (count_kernel writes the window arrays and block sums that scan/fill read): nothing to clear
+    return run_hop(g, slot_node, slot_ts, nullptr, S_max, S_dev, p, out, ws, STATIC_SCRATCH_BYTES, as_stream(stream));
 }
 
 static int64_t worst_slots(int64_t S0, int32_t layer, int32_t k) {

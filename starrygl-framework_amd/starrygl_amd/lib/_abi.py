@@ -10,6 +10,7 @@ ABI_VERSION = 4
 SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
 UNIFORM_MAX_FANOUT = 64
+STATIC_HOP_MAX_SLOTS = 65536
 UNIQUE_SORTED, UNIQUE_GROUPED, UNIQUE_PREMARKED = 0, 1, 0x100
 DT_I64, DT_F32 = 0, 1
 
@@ -71,6 +72,7 @@ PROTOTYPES = {
     "window_end": (i32, [P(TCSR), vp, vp, i64, vp, vp]),
     "sample_hop_workspace_bytes": (sz, [i64]),
     "sample_hop": (i32, [P(TCSR), vp, vp, i64, vp, P(SampleParams), P(HopOut), vp, sz, vp]),
+    "sample_hop_static": (i32, [P(TCSR), vp, vp, i64, vp, P(SampleParams), P(HopOut), vp]),
     "sample_khop_workspace_bytes": (sz, [i64, i32, i32]),
     "sample_khop": (i32, [P(TCSR), i64, vp, vp, i64, vp, i64, vp, vp, i32,
                           P(SampleParams), vp, vp, P(HopOut), vp, sz, vp]),

@@ -243,6 +243,16 @@ class HotPath:
             out.finalize(*be.tolist(out.counts))
         return out
 
+    def sample_hop_static(self, g, slot_node, slot_ts, p, out, S_dev=None):
+        """`sample_hop` into the caller's `out` (a HopResult) with the hop's scratch in the library's own
+        per-GPU array: the call allocates nothing.  At most STATIC_HOP_MAX_SLOTS slots; calls that overlap
+        on one GPU share the array and race.  The result is not finalized."""
+        self._chk("i64", slot_node=slot_node, slot_ts=slot_ts, S_dev=S_dev)
+        be = self.be
+        self._ck(self.lib.sample_hop_static(C.byref(g.view), be.ptr(slot_node), be.ptr(slot_ts), int(slot_node.shape[0]),
+                                            be.ptr(S_dev), C.byref(p), C.byref(out.struct), be.stream()))
+        return out
+
     def khop_buffers(self, S0, layers, fanout, counts=None):
         """Worst-case output buffers of a k-hop call; reusable across calls.  `counts`
         (int64[3 * layers], zeroed) may be a slice of a larger array of the caller's."""
