@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define SGL_ABI_VERSION 4
+#define SGL_ABI_VERSION 5
 
 /* ------------------------------------------------------------------ status */
 #define SGL_OK        0
@@ -291,8 +291,11 @@ int32_t sgl_remap_init(void* state, size_t state_bytes, int64_t universe,
  *                and the state must be initialised again.
  * `state` != NULL selects the dense-universe path: `universe` must be the value
  * given to sgl_remap_init, ids outside [0, universe) map to -1.  `state` ==
- * NULL (universe ignored) selects the hash-set path, which accepts arbitrary
- * non-negative ids but only reset = 1.  Negative ids always map to -1. */
+ * NULL (universe ignored) selects the one-shot hash-set path, which accepts
+ * arbitrary non-negative ids but only reset = 1 (its table lives in the
+ * workspace; sgl_unique_compact_hashed keeps one over several calls).
+ * Negative ids always map to -1.  Both paths are asynchronous, fixed launch
+ * sequences. */
 size_t  sgl_unique_workspace_bytes(int64_t universe, int32_t G,
                                    const int64_t* len_max);
 int32_t sgl_unique_compact(void* state, int64_t universe, int32_t reset,
@@ -304,6 +307,39 @@ int32_t sgl_unique_compact(void* state, int64_t universe, int32_t reset,
                            int64_t* U_dev,
                            void* workspace, size_t workspace_bytes,
                            void* stream);
+
+/* Persistent hash-set remap state for ids without a dense universe (arbitrary
+ * non-negative 63-bit values, e.g. DistRouteIndex-encoded ids): the same role
+ * as sgl_remap_init's state - Remapper's id_mapper and epoch counter
+ * (sample.cu.hpp:1752-1763), which the reference keeps per graph so that the
+ * queries of one AsyncGraphBlob share one numbering ('r' then 'f',
+ * graph.py:291) - with memory proportional to `capacity`, the largest number
+ * of distinct ids one epoch may hold (at most 2^31 - 256), instead of to the
+ * id range.  The caller allocates sgl_remap_hashed_state_bytes(capacity)
+ * device bytes (about 22 bytes per id) and calls sgl_remap_hashed_init once. */
+size_t  sgl_remap_hashed_state_bytes(int64_t capacity);
+int32_t sgl_remap_hashed_init(void* state, size_t state_bytes, int64_t capacity,
+                              void* stream);
+
+/* sgl_unique_compact over a hashed state: same arguments, modes and results
+ * (Remapper::insert, sample.cu.hpp:1825-1852), with `capacity` - the value
+ * given to sgl_remap_hashed_init - in place of the universe; reset = 0
+ * continues the epoch of the previous call on the state.  No host
+ * synchronisation.  When an epoch outgrows the capacity U_dev[0] reads
+ * INT64_MAX from then on: the result is void and the state must be
+ * initialised again (with a larger capacity). */
+size_t  sgl_unique_hashed_workspace_bytes(int64_t capacity, int32_t G,
+                                          const int64_t* len_max);
+int32_t sgl_unique_compact_hashed(void* state, int64_t capacity, int32_t reset,
+                                  int32_t mode, int32_t G,
+                                  const int64_t* const* ids,
+                                  const int64_t* len_max,
+                                  const int64_t* const* len_dev,
+                                  int64_t* const* local_out,
+                                  int64_t* unique_out, int64_t unique_capacity,
+                                  int64_t* U_dev,
+                                  void* workspace, size_t workspace_bytes,
+                                  void* stream);
 
 /* ------------------------------------------------------------ cache gather */
 /* Two-tier row store (replaces IDMapper.to_local + DistNodeState.__getitem__,

@@ -492,13 +492,12 @@ size_t sglo_unique_workspace_bytes(int64_t universe, int32_t G, const int64_t* l
  * restarts numbering, reset=0 continues it (the comment at
  * sample.cu.hpp:1874, and graph.py:291).  Ids that are negative, or outside
  * the state's universe, map to -1 and are never numbered. */
-int32_t sglo_unique_compact(void* state, int64_t universe_arg, int32_t reset, int32_t mode, int32_t G,
-                            const int64_t* const* ids, const int64_t* len_max,
-                            const int64_t* const* len_dev,
-                            int64_t* const* local_out, int64_t* unique_out,
-                            int64_t unique_capacity, int64_t* U_dev, void* ws,
-                            size_t ws_bytes, void* stream) {
-    (void)ws; (void)ws_bytes; (void)stream;
+static int32_t unique_core(void* state, int64_t universe_arg, seen_rec* known, int64_t* n_known_io, int64_t known_capacity,
+                           int32_t reset, int32_t mode, int32_t G,
+                           const int64_t* const* ids, const int64_t* len_max,
+                           const int64_t* const* len_dev,
+                           int64_t* const* local_out, int64_t* unique_out,
+                           int64_t unique_capacity, int64_t* U_dev) {
     if (G < 0 || (G > 0 && (!ids || !len_max || !local_out)) || !U_dev)
         return fail(SGL_EINVAL, "unique_compact: null");
     /* PREMARKED only tells the HIP library that the sampler already did its first pass; the
@@ -508,7 +507,7 @@ int32_t sglo_unique_compact(void* state, int64_t universe_arg, int32_t reset, in
     mode &= ~SGL_UNIQUE_PREMARKED;
     if (mode != SGL_UNIQUE_SORTED && mode != SGL_UNIQUE_GROUPED)
         return fail(SGL_EINVAL, "unique_compact: bad mode");
-    if (!state && !reset) return fail(SGL_ENOTSUP, "unique_compact: hash path needs reset=1");
+    if (!state && !known && !reset) return fail(SGL_ENOTSUP, "unique_compact: hash path needs reset=1");
     int64_t* hdr = (int64_t*)state;
     int64_t* table = state ? hdr + 3 : NULL;
     const int64_t universe = state ? hdr[2] : INT64_MAX;
@@ -526,6 +525,13 @@ int32_t sglo_unique_compact(void* state, int64_t universe_arg, int32_t reset, in
             for (int64_t i = 0; i < universe; ++i) table[i] = -1;
         }
         id_count = hdr[1];
+    }
+    /* hashed state: the ids of the epoch so far, sorted by id, with their local ids */
+    int64_t n_known = 0;
+    if (known) {
+        if (reset) *n_known_io = 0;
+        n_known = *n_known_io;
+        id_count = n_known;
     }
     const int64_t U_before = id_count;
     /* `seen` = ids numbered by this call, kept sorted by id. */
@@ -551,7 +557,13 @@ int32_t sglo_unique_compact(void* state, int64_t universe_arg, int32_t reset, in
             if (i > 0 && tmp[i] == tmp[i - 1]) continue;
             int64_t id = tmp[i];
             if (state && table[id] >= 0) continue;            /* earlier call, same epoch */
+            if (known && seen_find(known, n_known, id) >= 0) continue;
             if (seen_find(seen, n_prev, id) >= 0) continue;   /* earlier group, this call */
+            if (known && id_count >= known_capacity) {       /* the epoch outgrows the hashed state: void result */
+                U_dev[0] = INT64_MAX; U_dev[1] = U_before;
+                free(seen); free(tmp);
+                return SGL_OK;
+            }
             if (id_count >= unique_capacity) { free(seen); free(tmp); return fail(SGL_ENOMEM, "unique_out too small"); }
             seen[n_seen].id = id; seen[n_seen].local = id_count; n_seen++;
             unique_out[id_count] = id;
@@ -567,6 +579,7 @@ int32_t sglo_unique_compact(void* state, int64_t universe_arg, int32_t reset, in
             if (id >= 0 && id < universe) {
                 loc = seen_find(seen, n_seen, id);
                 if (loc < 0 && state) loc = table[id];
+                if (loc < 0 && known) loc = seen_find(known, n_known, id);
             }
             local_out[g][i] = loc;
         }
@@ -575,9 +588,64 @@ int32_t sglo_unique_compact(void* state, int64_t universe_arg, int32_t reset, in
         for (int64_t i = 0; i < n_seen; ++i) table[seen[i].id] = seen[i].local;
         hdr[1] = id_count;
     }
+    if (known) {
+        for (int64_t i = 0; i < n_seen; ++i) known[n_known + i] = seen[i];
+        *n_known_io = n_known + n_seen;
+        qsort(known, (size_t)*n_known_io, sizeof *known, seen_cmp);
+    }
     U_dev[0] = id_count; U_dev[1] = U_before;
     free(seen); free(tmp);
     return SGL_OK;
+}
+
+int32_t sglo_unique_compact(void* state, int64_t universe_arg, int32_t reset, int32_t mode, int32_t G,
+                            const int64_t* const* ids, const int64_t* len_max,
+                            const int64_t* const* len_dev,
+                            int64_t* const* local_out, int64_t* unique_out,
+                            int64_t unique_capacity, int64_t* U_dev, void* ws,
+                            size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    return unique_core(state, universe_arg, NULL, NULL, 0, reset, mode, G, ids, len_max, len_dev, local_out,
+                       unique_out, unique_capacity, U_dev);
+}
+
+/* Hashed state of the oracle: int64 header {capacity, ids of the epoch, void flag}, then the
+ * epoch's (id, local id) records sorted by id.  Same numbering rule as above
+ * (Remapper::insert, sample.cu.hpp:1825-1852) for ids of any non-negative value. */
+size_t sglo_remap_hashed_state_bytes(int64_t capacity) {
+    return 3 * sizeof(int64_t) + (size_t)(capacity > 0 ? capacity : 0) * sizeof(seen_rec);
+}
+
+int32_t sglo_remap_hashed_init(void* state, size_t bytes, int64_t capacity, void* stream) {
+    (void)stream;
+    if (!state || capacity < 1 || bytes < sglo_remap_hashed_state_bytes(capacity))
+        return fail(SGL_EINVAL, "remap_hashed_init: bad state");
+    int64_t* h = (int64_t*)state;
+    h[0] = capacity; h[1] = 0; h[2] = 0;
+    return SGL_OK;
+}
+
+size_t sglo_unique_hashed_workspace_bytes(int64_t capacity, int32_t G, const int64_t* len_max) {
+    (void)capacity; (void)G; (void)len_max;
+    return 0;
+}
+
+int32_t sglo_unique_compact_hashed(void* state, int64_t capacity, int32_t reset, int32_t mode, int32_t G,
+                                   const int64_t* const* ids, const int64_t* len_max,
+                                   const int64_t* const* len_dev,
+                                   int64_t* const* local_out, int64_t* unique_out,
+                                   int64_t unique_capacity, int64_t* U_dev, void* ws,
+                                   size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (!state) return fail(SGL_EINVAL, "unique_compact_hashed: state is NULL");
+    int64_t* h = (int64_t*)state;
+    if (capacity != h[0]) return fail(SGL_EINVAL, "unique_compact_hashed: capacity differs from remap_hashed_init");
+    if (mode & SGL_UNIQUE_PREMARKED) return fail(SGL_EINVAL, "unique_compact_hashed: bad mode");
+    int32_t rc = unique_core(NULL, 0, (seen_rec*)(h + 3), &h[1], capacity, reset, mode, G, ids, len_max, len_dev,
+                             local_out, unique_out, unique_capacity, U_dev);
+    if (rc == SGL_OK && U_dev[0] == INT64_MAX) h[2] = 1;
+    if (rc == SGL_OK && h[2]) U_dev[0] = INT64_MAX;      /* sticky */
+    return rc;
 }
 
 /* ------------------------------------------------------------ cache gather */

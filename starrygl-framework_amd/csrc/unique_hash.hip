@@ -1,54 +1,151 @@
 // Hash-set unique + compaction for ids without a dense universe (gfx950).
 //
-// Used when the caller has no remap state (ids are arbitrary non-negative
-// 63-bit values, e.g. partition-encoded ids).  Per group of input arrays:
-//   insert  : a block folds its 1024 ids through an LDS open-addressing set, so
-//             an id that repeats inside the tile reaches the global table
-//             once; block-unique ids are claimed in the global table with
-//             atomicCAS; the ids a block wins are appended to the group's list
-//             with ONE global atomicAdd per block (same-address atomics cost
-//             ~11 ns each on MI355X, per-id appends would dominate);
-//   (one host read of the per-group counts and the largest id)
-//   sort    : the group's new ids are radix-sorted on the bits actually used;
-//   number  : rank r of the sorted list gets local id base + r, written into the
-//             table's value array and the local->global list;
-// then one lookup launch rewrites every input array.  Numbering is by ascending
-// id inside each group, so the result equals the dense path and the reference's
-// sort + unique (csrc/include/starrygl/sample.cu.hpp:1786-1811) bit for bit.
-// The call synchronises with the host once.
+// For ids that are arbitrary non-negative 63-bit values (partition-encoded ids,
+// say), where no table indexed by id can be kept.  The set is an open-addressing
+// table of 8-byte keys with a parallel array of 4-byte local ids; it lives
+// either in a persistent "hashed state" of a stated capacity (an epoch of local
+// ids can then continue over several calls, as with the dense state) or, for
+// one-shot calls, in the call's workspace.  A call is a fixed sequence of seven
+// launches on the caller's stream, sized on the host from the worst case and
+// driven by device-side counts - no host synchronisation, HIP-graph capturable:
+//
+//   prep    : empties the table (everything for a workspace table; for a
+//             persistent one only on reset, and then only the slots the last
+//             epoch used when those are few) and zeroes the bucket counters;
+//   insert  : a block folds its 2048 ids through an LDS set, so an id that
+//             repeats inside the tile reaches the global table once; the
+//             tile-unique ids probe the table (a plain load first: most ids of
+//             a sampled batch are repeats and end there; atomicCAS only on an
+//             empty slot).  Every input element remembers the table slot of its
+//             id (4 bytes), so nothing is ever probed twice.  The ids a block
+//             added are appended - id and slot - to the call's list with ONE
+//             returning atomic per block; OR and AND over them are kept;
+//   hist    : the new ids have to be numbered in ascending order.  The bits in
+//             which they differ at all (OR ^ AND) are squeezed together into a
+//             short key that keeps the order, and its top bits select one of up
+//             to 2^18 buckets (in grouped mode the array that owns the id is
+//             the top digit); bucket sizes are counted with spread atomics;
+//   scan    : one block turns counts into offsets and lists oversized buckets;
+//   scatter : ids move to their bucket's segment;
+//   number  : an id's rank = bucket offset + ids of its bucket that are smaller
+//             (a handful: the buckets hold ~8 ids); rank + ids numbered before
+//             = local id, written to the table and the local->global list.
+//             Oversized buckets (skewed id distributions) are sorted by a block
+//             each with a bitonic network in place;
+//   lookup  : out[i] = local id at the slot element i remembered.
+//
+// Numbering is by ascending id inside each group, so the result equals the dense
+// path and the reference's sort + unique (csrc/include/starrygl/sample.cu.hpp:
+// 1786-1852) bit for bit.
 #include "common.hpp"
-#include "radix.hpp"
 
 namespace sgl {
 namespace {
 
 constexpr int BLOCK = 256;
 constexpr int MAXG = 8;
-constexpr int IPT = 4;
-constexpr int TILE = BLOCK * IPT;        // ids per block
+constexpr int IPT = 8;
+constexpr int TILE = BLOCK * IPT;        // ids per block of insert
 constexpr int LDS_SLOTS = 2 * TILE;      // load <= 0.5
 constexpr unsigned long long EMPTY = ~0ull;
+constexpr uint32_t NONE = 0xFFFFFFFFu;   // slot of an element whose id is negative
+constexpr uint32_t UNNUMBERED = 0x7FFFFFFFu;  // value of a slot whose id has no local id yet
+constexpr uint32_t PENDING0 = 0x7FFFFFE0u;    // PENDING0 + g: not numbered yet, first seen in array g (grouped mode)
+constexpr int64_t MAX_CAPACITY = 0x7FFFFF00ll;
+constexpr int NB_MIN_LOG = 8, NB_MAX_LOG = 18;
+constexpr int SMALL_BUCKET = 512;        // buckets up to this size are ranked by counting
+constexpr int SCAN_BLOCK = 1024;
+constexpr int MAX_GRID = 4096;
 
-struct Counters {
-    long long count[MAXG];  // new ids of each group
-    long long max_id;
+struct Header {
+    unsigned long long total;     // ids numbered in the current epoch (committed by the last launch of a call)
+    unsigned long long appended;  // ids the running call has added (0 between calls)
+    unsigned long long or_mask;   // OR / AND over the ids the running call has added (0 / ~0 between calls)
+    unsigned long long and_mask;
+    unsigned long long overflow;  // sticky: more ids than the capacity, or no free slot
+    unsigned long long nbig;      // oversized buckets of the running call (0 between calls)
 };
+constexpr size_t HEADER_BYTES = 256;
+
+struct Table {
+    Header* hdr;
+    unsigned long long* keys;   // [slots]
+    uint32_t* vals;             // [slots] local id, UNNUMBERED or PENDING0 + g
+    uint32_t* used;             // [capacity] slot of the k-th id of the epoch
+    int64_t capacity, slots;
+};
+
+int64_t slots_of(int64_t capacity) { return capacity + capacity / 2 + 64; }
+
+size_t state_bytes(int64_t capacity) {
+    const int64_t s = slots_of(capacity);
+    return HEADER_BYTES + align_up((size_t)s * 8) + align_up((size_t)s * 4) + align_up((size_t)(capacity + 1) * 4);
+}
+
+Table carve(void* state, int64_t capacity) {
+    Table t;
+    char* p = static_cast<char*>(state);
+    t.capacity = capacity;
+    t.slots = slots_of(capacity);
+    t.hdr = reinterpret_cast<Header*>(p);
+    p += HEADER_BYTES;
+    t.keys = reinterpret_cast<unsigned long long*>(p);
+    p += align_up((size_t)t.slots * 8);
+    t.vals = reinterpret_cast<uint32_t*>(p);
+    p += align_up((size_t)t.slots * 4);
+    t.used = reinterpret_cast<uint32_t*>(p);
+    return t;
+}
+
+// Per-call scratch
+struct Scratch {
+    uint32_t* slot_of;          // [total] table slot of every input element (NONE: negative id)
+    unsigned long long* list_id;  // [ncap] ids added by this call, in the order of their appends
+    uint32_t* list_b;           // [ncap] their buckets
+    unsigned long long* part_id;  // [ncap] the same ids grouped by bucket
+    uint32_t* part_slot;        // [ncap]
+    uint32_t* part_b;           // [ncap]
+    uint32_t* cnt;              // [nb + 1] bucket sizes, later the scatter cursors
+    uint32_t* off;              // [nb + 1] bucket offsets
+    uint32_t* big;              // [ncap / SMALL_BUCKET + 1] oversized buckets
+    int64_t ncap;               // most ids one call can add
+    int32_t nb_log;             // log2 of the number of buckets
+};
+
+int nb_log_of(int64_t ncap) {
+    int l = NB_MIN_LOG;
+    while (l < NB_MAX_LOG && (8ll << l) < ncap) ++l;
+    return l;
+}
+
+size_t scratch_bytes(int64_t total, int64_t ncap) {
+    const int64_t nb = 1ll << nb_log_of(ncap);
+    return align_up((size_t)(total + 1) * 4) + 2 * align_up((size_t)(ncap + 1) * 8) + 3 * align_up((size_t)(ncap + 1) * 4) +
+           2 * align_up((size_t)(nb + 1) * 4) + align_up((size_t)(ncap / SMALL_BUCKET + 2) * 4) + 1024;
+}
+
+Scratch carve_scratch(Arena& ar, int64_t total, int64_t ncap) {
+    Scratch s;
+    s.ncap = ncap;
+    s.nb_log = nb_log_of(ncap);
+    const int64_t nb = 1ll << s.nb_log;
+    s.slot_of = ar.take<uint32_t>(total + 1);
+    s.list_id = ar.take<unsigned long long>(ncap + 1);
+    s.part_id = ar.take<unsigned long long>(ncap + 1);
+    s.list_b = ar.take<uint32_t>(ncap + 1);
+    s.part_slot = ar.take<uint32_t>(ncap + 1);
+    s.part_b = ar.take<uint32_t>(ncap + 1);
+    s.cnt = ar.take<uint32_t>(nb + 1);
+    s.off = ar.take<uint32_t>(nb + 1);
+    s.big = ar.take<uint32_t>(ncap / SMALL_BUCKET + 2);
+    return s;
+}
 
 __device__ __forceinline__ uint64_t mix(uint64_t x) {  // splitmix64 finaliser
     x ^= x >> 30; x *= 0xBF58476D1CE4E5B9ull;
     x ^= x >> 27; x *= 0x94D049BB133111EBull;
     x ^= x >> 31;
     return x;
-}
-
-__global__ void fill_empty_kernel(unsigned long long* keys, int64_t cap, Counters* c) {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = t; i < cap; i += stride) keys[i] = EMPTY;
-    if (t == 0) {
-        for (int g = 0; g < MAXG; ++g) c->count[g] = 0;
-        c->max_id = 0;
-    }
 }
 
 struct Arrays {
@@ -73,140 +170,424 @@ __device__ __forceinline__ bool locate(const Arrays& a, int64_t t, int* g_out, i
     return true;
 }
 
-__global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, unsigned long long* __restrict__ keys,
-                                                       int64_t cap_mask, int grp, Counters* c,
-                                                       int64_t* __restrict__ list) {
-    __shared__ unsigned long long s_set[LDS_SLOTS];
+// What a call works with: ids numbered before it and (from the hist launch on) ids it added.
+__device__ __forceinline__ int64_t ids_before(const Table& t, int reset) { return reset ? 0 : (int64_t)t.hdr->total; }
+__device__ __forceinline__ int64_t ids_added(const Table& t, const Scratch& s, int64_t before) {
+    int64_t n = (int64_t)t.hdr->appended;
+    const int64_t room = t.capacity - before;
+    if (n > room) n = room;
+    if (n > s.ncap) n = s.ncap;
+    return n < 0 ? 0 : n;
+}
+
+__global__ __launch_bounds__(BLOCK) void init_kernel(Table t) {
+    const int64_t tid = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    for (int64_t i = tid; i < t.slots; i += (int64_t)gridDim.x * BLOCK) {
+        t.keys[i] = EMPTY;
+        t.vals[i] = UNNUMBERED;
+    }
+    if (tid == 0) {
+        t.hdr->total = 0;
+        t.hdr->appended = 0;
+        t.hdr->or_mask = 0;
+        t.hdr->and_mask = ~0ull;
+        t.hdr->overflow = 0;
+        t.hdr->nbig = 0;
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void prep_kernel(Table t, Scratch s, int fresh, int reset) {
+    const int64_t tid = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * BLOCK;
+    // every block reads the header before anyone writes it: only a fresh (workspace) table's header is
+    // written here, and nobody reads that one
+    const int64_t prev = fresh ? 0 : (int64_t)t.hdr->total;
+    if (fresh || (reset && prev * 4 >= t.slots)) {
+        for (int64_t i = tid; i < t.slots; i += stride) {
+            t.keys[i] = EMPTY;
+            t.vals[i] = UNNUMBERED;
+        }
+    } else if (reset) {
+        for (int64_t k = tid; k < prev; k += stride) {
+            const uint32_t h = t.used[k];
+            t.keys[h] = EMPTY;
+            t.vals[h] = UNNUMBERED;
+        }
+    }
+    const int64_t nb = 1ll << s.nb_log;
+    for (int64_t i = tid; i <= nb; i += stride) s.cnt[i] = 0;
+    if (fresh && tid == 0) {
+        t.hdr->total = 0;
+        t.hdr->appended = 0;
+        t.hdr->or_mask = 0;
+        t.hdr->and_mask = ~0ull;
+        t.hdr->overflow = 0;
+        t.hdr->nbig = 0;
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratch s, int reset, int grouped) {
+    __shared__ unsigned long long s_key[LDS_SLOTS];
+    __shared__ uint32_t s_aux[LDS_SLOTS];       // first the smallest array index that holds the id, then its table slot
     __shared__ int32_t s_won;
-    __shared__ long long s_base, s_max;
-    for (int q = threadIdx.x; q < LDS_SLOTS; q += BLOCK) s_set[q] = EMPTY;
-    if (threadIdx.x == 0) { s_won = 0; s_max = 0; }
+    __shared__ long long s_base;
+    __shared__ unsigned long long s_or, s_and;
+    for (int q = threadIdx.x; q < LDS_SLOTS; q += BLOCK) {
+        s_key[q] = EMPTY;
+        s_aux[q] = MAXG;
+    }
+    if (threadIdx.x == 0) {
+        s_won = 0;
+        s_or = 0;
+        s_and = ~0ull;
+    }
     __syncthreads();
     const int64_t t0 = (int64_t)blockIdx.x * TILE + threadIdx.x;
+    int32_t ls[IPT];
 #pragma unroll
     for (int q = 0; q < IPT; ++q) {
+        ls[q] = -2;                       // -2: no element, -1: negative id
         int g;
         int64_t i;
         if (!locate(a, t0 + (int64_t)q * BLOCK, &g, &i)) continue;
         const int64_t id = a.ids[g][i];
+        ls[q] = -1;
         if (id < 0) continue;
         uint32_t h = (uint32_t)mix((uint64_t)id) & (LDS_SLOTS - 1);
         while (true) {
-            const unsigned long long prev = atomicCAS(&s_set[h], EMPTY, (unsigned long long)id);
+            const unsigned long long prev = atomicCAS(&s_key[h], EMPTY, (unsigned long long)id);
             if (prev == EMPTY || prev == (unsigned long long)id) break;
             h = (h + 1) & (LDS_SLOTS - 1);
         }
+        ls[q] = (int32_t)h;
+        if (grouped) atomicMin(&s_aux[h], (uint32_t)g);
     }
     __syncthreads();
-    // every occupied LDS slot is one block-unique id: claim it in the global table
+    // every occupied LDS slot is one tile-unique id: find or claim its table slot
+    const int64_t before = ids_before(t, reset);
     unsigned long long won[LDS_SLOTS / BLOCK];
+    uint32_t won_slot[LDS_SLOTS / BLOCK];
     int32_t pos[LDS_SLOTS / BLOCK];
-    long long mx = 0;
+    unsigned long long my_or = 0, my_and = ~0ull;
+    bool lost = false;
 #pragma unroll
     for (int q = 0; q < LDS_SLOTS / BLOCK; ++q) {
-        const unsigned long long id = s_set[q * BLOCK + threadIdx.x];
+        const int l = q * BLOCK + threadIdx.x;
+        const unsigned long long id = s_key[l];
         won[q] = EMPTY;
+        won_slot[q] = 0;
         pos[q] = 0;
         if (id == EMPTY) continue;
-        uint64_t h = mix(id) & (uint64_t)cap_mask;
-        while (true) {
-            const unsigned long long prev = atomicCAS(&keys[h], EMPTY, id);
-            if (prev == EMPTY) { won[q] = id; break; }
-            if (prev == id) break;
-            h = (h + 1) & (uint64_t)cap_mask;
+        const uint32_t grp = s_aux[l];
+        uint64_t h = __umul64hi(mix(id), (uint64_t)t.slots);
+        bool placed = false;
+        for (int64_t probes = 0; probes < t.slots; ++probes) {
+            unsigned long long k = t.keys[h];     // a slot never changes once it holds an id: a cached value is good
+            if (k == EMPTY) {
+                k = atomicCAS(&t.keys[h], EMPTY, id);
+                if (k == EMPTY) {
+                    won[q] = id;
+                    k = id;
+                }
+            }
+            if (k == id) {
+                placed = true;
+                break;
+            }
+            h = h + 1 == (uint64_t)t.slots ? 0 : h + 1;
         }
+        if (!placed) {          // the table is full
+            lost = true;
+            s_aux[l] = NONE;
+            continue;
+        }
+        s_aux[l] = (uint32_t)h;
+        // grouped: an id that has no local id yet belongs to the first array that holds it (a local id is
+        // smaller than every PENDING value, so ids of earlier calls keep theirs)
+        if (grouped) atomicMin(&t.vals[h], PENDING0 + grp);
         if (won[q] != EMPTY) {
+            won_slot[q] = (uint32_t)h;
             pos[q] = atomicAdd(&s_won, 1);
-            mx = (long long)id > mx ? (long long)id : mx;
+            my_or |= id;
+            my_and &= id;
         }
     }
-    if (mx > 0) atomicMax(&s_max, mx);
+    if (my_or != 0 || my_and != ~0ull) {
+        atomicOr(&s_or, my_or);
+        atomicAnd(&s_and, my_and);
+    }
+    if (lost) atomicOr(&t.hdr->overflow, 1ull);
     __syncthreads();
     if (threadIdx.x == 0 && s_won > 0) {
-        s_base = (long long)atomicAdd(reinterpret_cast<unsigned long long*>(&c->count[grp]), (unsigned long long)s_won);
-        atomicMax(&c->max_id, s_max);
+        s_base = (long long)atomicAdd(&t.hdr->appended, (unsigned long long)s_won);
+        atomicOr(&t.hdr->or_mask, s_or);
+        atomicAnd(&t.hdr->and_mask, s_and);
+        if (before + s_base + s_won > t.capacity || s_base + s_won > s.ncap) atomicOr(&t.hdr->overflow, 1ull);
     }
     __syncthreads();
 #pragma unroll
-    for (int q = 0; q < LDS_SLOTS / BLOCK; ++q)
-        if (won[q] != EMPTY) list[s_base + pos[q]] = (int64_t)won[q];
-}
-
-__device__ __forceinline__ int64_t find_slot(const unsigned long long* __restrict__ keys, int64_t cap_mask,
-                                             unsigned long long id) {
-    uint64_t h = mix(id) & (uint64_t)cap_mask;
-    while (true) {
-        const unsigned long long k = keys[h];
-        if (k == id) return (int64_t)h;
-        if (k == EMPTY) return -1;
-        h = (h + 1) & (uint64_t)cap_mask;
+    for (int q = 0; q < LDS_SLOTS / BLOCK; ++q) {
+        if (won[q] == EMPTY) continue;
+        const int64_t k = s_base + pos[q];
+        if (k < s.ncap && before + k < t.capacity) {
+            s.list_id[k] = won[q];
+            t.used[before + k] = won_slot[q];
+        }
     }
+#pragma unroll
+    for (int q = 0; q < IPT; ++q)
+        if (ls[q] != -2) s.slot_of[t0 + (int64_t)q * BLOCK] = ls[q] < 0 ? NONE : s_aux[ls[q]];
 }
 
-__global__ __launch_bounds__(BLOCK) void number_kernel(const uint64_t* __restrict__ sorted, int64_t count,
-                                                       int64_t base, const unsigned long long* __restrict__ keys,
-                                                       int64_t* __restrict__ vals, int64_t cap_mask,
-                                                       int64_t* __restrict__ unique_out, int64_t unique_capacity) {
-    const int64_t r = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
-    if (r >= count) return;
-    const unsigned long long id = sorted[r];
-    const int64_t slot = find_slot(keys, cap_mask, id);
-    if (slot >= 0) vals[slot] = base + r;
-    if (base + r < unique_capacity) unique_out[base + r] = (int64_t)id;
-}
+// The bits in which the new ids differ, squeezed into a key that keeps their order: up to three runs
+// of such bits from the top, then one span down to the lowest of them (it may hold bits that do not
+// differ; only the top bits of the key select the bucket).
+struct Codec {
+    int32_t sh[4], dst[4];
+    uint64_t mask[4];
+    int32_t nb;   // bits of the key
+};
 
-__global__ __launch_bounds__(BLOCK) void lookup_kernel(Arrays a, const unsigned long long* __restrict__ keys,
-                                                       const int64_t* __restrict__ vals, int64_t cap_mask) {
-    const int64_t t = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
-    int g;
-    int64_t i;
-    if (!locate(a, t, &g, &i)) return;
-    const int64_t id = a.ids[g][i];
-    int64_t local = -1;
-    if (id >= 0) {
-        const int64_t slot = find_slot(keys, cap_mask, (unsigned long long)id);
-        if (slot >= 0) local = vals[slot];
+__device__ inline Codec make_codec(uint64_t or_mask, uint64_t and_mask) {
+    Codec c;
+    uint64_t diff = (or_mask ^ and_mask) & 0x7FFFFFFFFFFFFFFFull;
+    int32_t width[4];
+    int n = 0;
+    for (; n < 4; ++n) {
+        c.sh[n] = 0;
+        c.mask[n] = 0;
+        width[n] = 0;
     }
-    a.out[g][i] = local;
-}
-
-__global__ void publish_kernel(int64_t* U_dev, int64_t total) {
-    U_dev[0] = total;
-    U_dev[1] = 0;
-}
-
-int64_t table_capacity(int64_t total) {
-    int64_t c = 1024;
-    while (c < 2 * total) c <<= 1;
+    n = 0;
+    while (diff != 0 && n < 4) {
+        const int top = 63 - __clzll((long long)diff);
+        int lo;
+        if (n < 3) {
+            // the run of ones that ends at `top`
+            const uint64_t below = ~diff & ((top == 63) ? ~0ull : ((2ull << top) - 1ull));   // zeros at or below top
+            lo = below == 0 ? 0 : 64 - __clzll((long long)below);                           // first zero below the run, + 1
+        } else {
+            lo = __ffsll((unsigned long long)diff) - 1;
+        }
+        const int w = top - lo + 1;
+        c.sh[n] = lo;
+        c.mask[n] = w >= 64 ? ~0ull : ((1ull << w) - 1ull);
+        width[n] = w;
+        diff &= (lo == 0) ? 0ull : ((1ull << lo) - 1ull);
+        ++n;
+    }
+    int nb = 0;
+    for (int r = 0; r < 4; ++r) nb += width[r];
+    c.nb = nb;
+    int acc = nb;
+    for (int r = 0; r < 4; ++r) {
+        acc -= width[r];
+        c.dst[r] = acc;
+    }
     return c;
 }
 
-int bits_of(uint64_t x) {
-    int b = 0;
-    while (x) { ++b; x >>= 1; }
-    return b;
+__device__ __forceinline__ uint64_t squeeze(const Codec& c, uint64_t id) {
+    uint64_t k = 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) k |= ((id >> c.sh[r]) & c.mask[r]) << c.dst[r];
+    return k;
 }
 
-}  // namespace
+// bucket of an id of array group g: g is the top digit (glog bits), the key's top bits the rest
+__device__ __forceinline__ uint32_t bucket_of(const Codec& c, uint64_t id, uint32_t g, int nb_log, int glog) {
+    const int kb = nb_log - glog;
+    const uint64_t key = squeeze(c, id);
+    const uint64_t top = c.nb > kb ? key >> (c.nb - kb) : key;
+    return (g << kb) | (uint32_t)top;
+}
 
-size_t hash_unique_workspace_bytes(int32_t G, const int64_t* len_max) {
-    int64_t total = 0, longest = 0;
-    for (int32_t g = 0; g < G && len_max; ++g) {
-        const int64_t l = len_max[g] > 0 ? len_max[g] : 0;
-        total += l;
+__global__ __launch_bounds__(BLOCK) void hist_kernel(Table t, Scratch s, int reset, int grouped, int glog) {
+    __shared__ Codec s_codec;
+    if (threadIdx.x == 0) s_codec = make_codec(t.hdr->or_mask, t.hdr->and_mask);
+    __syncthreads();
+    const Codec c = s_codec;
+    const int64_t before = ids_before(t, reset);
+    const int64_t n = ids_added(t, s, before);
+    for (int64_t k = (int64_t)blockIdx.x * BLOCK + threadIdx.x; k < n; k += (int64_t)gridDim.x * BLOCK) {
+        uint32_t g = 0;
+        if (grouped) {
+            g = t.vals[t.used[before + k]] - PENDING0;
+            if (g >= (uint32_t)MAXG) g = 0;
+        }
+        const uint32_t b = bucket_of(c, s.list_id[k], g, s.nb_log, glog);
+        s.list_b[k] = b;
+        atomicAdd(&s.cnt[b], 1u);
     }
-    longest = total;  // sorted mode sorts all ids as one group
-    const int64_t cap = table_capacity(total);
-    return 2 * align_up((size_t)cap * 8) + 3 * align_up((size_t)(total + 1) * 8) + align_up((size_t)(longest + 1) * 8) +
-           radix_sort_workspace_bytes(longest) + 8192;
 }
 
-int32_t hash_unique_compact(int32_t mode, int32_t G, const int64_t* const* ids, const int64_t* len_max,
-                            const int64_t* const* len_dev, int64_t* const* local_out,
-                            int64_t* unique_out, int64_t unique_capacity, int64_t* U_dev, void* ws,
-                            size_t ws_bytes, hipStream_t st) {
-    if (!ws || ws_bytes < hash_unique_workspace_bytes(G, len_max))
-        return fail(SGL_ENOMEM, "unique_compact: workspace %zu < %zu bytes", ws_bytes, hash_unique_workspace_bytes(G, len_max));
+// One block: exclusive prefix of the bucket sizes, cursors zeroed, oversized buckets listed.
+__global__ __launch_bounds__(SCAN_BLOCK) void scan_kernel(Table t, Scratch s) {
+    constexpr int NW = SCAN_BLOCK / WAVE;
+    __shared__ uint32_t s_w[NW];
+    __shared__ uint32_t s_carry;
+    __shared__ uint32_t s_nbig;
+    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    const int64_t nb = 1ll << s.nb_log;
+    if (threadIdx.x == 0) {
+        s_carry = 0;
+        s_nbig = 0;
+    }
+    __syncthreads();
+    // rounds of 4 * SCAN_BLOCK counters: thread t owns 4 consecutive ones (one 16-byte load)
+    for (int64_t base = 0; base < nb; base += 4 * SCAN_BLOCK) {
+        const int64_t i0 = base + 4 * (int64_t)threadIdx.x;
+        uint32_t v[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (i0 + q < nb) v[q] = s.cnt[i0 + q];
+        const uint32_t sum = v[0] + v[1] + v[2] + v[3];
+        uint32_t inc = sum;
+        for (int d = 1; d < WAVE; d <<= 1) {
+            const uint32_t y = __shfl_up(inc, d);
+            if (lane >= d) inc += y;
+        }
+        if (lane == WAVE - 1) s_w[wid] = inc;
+        __syncthreads();
+        uint32_t woff = 0, round_total = 0;
+#pragma unroll
+        for (int q = 0; q < NW; ++q) {
+            const uint32_t x = s_w[q];
+            if (q < wid) woff += x;
+            round_total += x;
+        }
+        uint32_t o = s_carry + woff + inc - sum;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (i0 + q < nb) {
+                s.off[i0 + q] = o;
+                s.cnt[i0 + q] = 0;
+                if (v[q] > (uint32_t)SMALL_BUCKET) s.big[atomicAdd(&s_nbig, 1u)] = (uint32_t)(i0 + q);
+                o += v[q];
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) s_carry += round_total;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        s.off[nb] = s_carry;
+        t.hdr->nbig = s_nbig;
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void scatter_kernel(Table t, Scratch s, int reset) {
+    const int64_t before = ids_before(t, reset);
+    const int64_t n = ids_added(t, s, before);
+    for (int64_t k = (int64_t)blockIdx.x * BLOCK + threadIdx.x; k < n; k += (int64_t)gridDim.x * BLOCK) {
+        const uint32_t b = s.list_b[k];
+        const uint32_t p = s.off[b] + atomicAdd(&s.cnt[b], 1u);
+        s.part_id[p] = s.list_id[k];
+        s.part_slot[p] = t.used[before + k];
+        s.part_b[p] = b;
+    }
+}
+
+// In-place ascending sort of ids[0..n) (all distinct) with their slots, by one block: a bitonic network
+// in which every comparator puts the smaller id at the lower index, so that the positions from n up to
+// the next power of two act as +infinity and their comparators are simply skipped.
+__device__ void block_sort(unsigned long long* ids, uint32_t* slots, int64_t n) {
+    int64_t p2 = 1;
+    while (p2 < n) p2 <<= 1;
+    for (int64_t k = 2; k <= p2; k <<= 1) {
+        for (int64_t j = k >> 1; j > 0; j >>= 1) {
+            for (int64_t c = threadIdx.x; c < p2 / 2; c += BLOCK) {
+                int64_t i, l;
+                if (j == (k >> 1)) {       // first step of a merge: mirror inside the block of k
+                    const int64_t blk = c / j, r = c % j;
+                    i = blk * k + r;
+                    l = blk * k + k - 1 - r;
+                } else {
+                    i = 2 * j * (c / j) + (c % j);
+                    l = i + j;
+                }
+                if (l < n) {
+                    const unsigned long long x = ids[i], y = ids[l];
+                    if (x > y) {
+                        ids[i] = y;
+                        ids[l] = x;
+                        const uint32_t sx = slots[i], sy = slots[l];
+                        slots[i] = sy;
+                        slots[l] = sx;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void number_kernel(Table t, Scratch s, int reset, int64_t* __restrict__ unique_out,
+                                                       int64_t unique_capacity) {
+    const int64_t before = ids_before(t, reset);
+    const int64_t n = ids_added(t, s, before);
+    for (int64_t p = (int64_t)blockIdx.x * BLOCK + threadIdx.x; p < n; p += (int64_t)gridDim.x * BLOCK) {
+        const uint32_t b = s.part_b[p];
+        const uint32_t lo = s.off[b], hi = s.off[b + 1];
+        if (hi - lo > (uint32_t)SMALL_BUCKET) continue;       // sorted below
+        const unsigned long long id = s.part_id[p];
+        uint32_t r = lo;
+        for (uint32_t q = lo; q < hi; ++q) r += s.part_id[q] < id ? 1u : 0u;
+        const int64_t local = before + r;
+        if (local < unique_capacity) unique_out[local] = (int64_t)id;
+        t.vals[s.part_slot[p]] = (uint32_t)local;
+    }
+    const int64_t nbig = (int64_t)t.hdr->nbig;
+    for (int64_t q = blockIdx.x; q < nbig; q += gridDim.x) {
+        const uint32_t b = s.big[q];
+        const int64_t lo = s.off[b], len = (int64_t)s.off[b + 1] - lo;
+        __syncthreads();
+        block_sort(s.part_id + lo, s.part_slot + lo, len);
+        for (int64_t j = threadIdx.x; j < len; j += BLOCK) {
+            const int64_t local = before + lo + j;
+            if (local < unique_capacity) unique_out[local] = (int64_t)s.part_id[lo + j];
+            t.vals[s.part_slot[lo + j]] = (uint32_t)local;
+        }
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void lookup_kernel(Arrays a, Table t, Scratch s, int reset, int64_t* U_dev) {
+    const int64_t i0 = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    // the call's totals, committed by one thread: no other thread of this launch reads the header
+    if (i0 == 0) {
+        const int64_t before = ids_before(t, reset);
+        const int64_t n = ids_added(t, s, before);
+        const bool void_result = t.hdr->overflow != 0;
+        U_dev[0] = void_result ? INT64_MAX : before + n;
+        U_dev[1] = before;
+        t.hdr->total = (unsigned long long)(before + n);
+        t.hdr->appended = 0;
+        t.hdr->or_mask = 0;
+        t.hdr->and_mask = ~0ull;
+        t.hdr->nbig = 0;
+    }
+    for (int64_t x = i0; x < a.start[a.G]; x += (int64_t)gridDim.x * BLOCK) {
+        int g;
+        int64_t i;
+        if (!locate(a, x, &g, &i)) continue;
+        const uint32_t h = s.slot_of[x];
+        int64_t local = -1;
+        if (h != NONE) {
+            const uint32_t v = t.vals[h];
+            if (v < PENDING0) local = (int64_t)v;
+        }
+        a.out[g][i] = local;
+    }
+}
+
+int32_t check_capacity(int64_t capacity) {
+    if (capacity < 0 || capacity > MAX_CAPACITY) return fail(SGL_EINVAL, "hashed remap state: capacity %lld outside [0, %lld]", (long long)capacity, (long long)MAX_CAPACITY);
+    return SGL_OK;
+}
+
+int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const int64_t* const* ids, const int64_t* len_max,
+            const int64_t* const* len_dev, int64_t* const* local_out, int64_t* unique_out, int64_t unique_capacity,
+            int64_t* U_dev, Arena& ar, hipStream_t st) {
     Arrays all;
     all.G = G;
     all.start[0] = 0;
@@ -219,68 +600,115 @@ int32_t hash_unique_compact(int32_t mode, int32_t G, const int64_t* const* ids, 
         all.start[g + 1] = all.start[g] + all.len_max[g];
     }
     const int64_t total = all.start[MAXG];
-    if (ceil_div<int64_t>(total, BLOCK) > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "unique_compact: too many ids");
-    const int64_t cap = table_capacity(total);
-    Arena ar(ws, ws_bytes);
-    Counters* d_cnt = ar.take<Counters>(1);
-    unsigned long long* keys = ar.take<unsigned long long>(cap);
-    int64_t* vals = ar.take<int64_t>(cap);
-    int64_t* list = ar.take<int64_t>(total + 1);    // group g's new ids start at all.start[g] (sorted mode: 0)
-    uint64_t* sort_b = ar.take<uint64_t>(total + 1);
-    int64_t* dummy_a = ar.take<int64_t>(total + 1);  // the sort carries a value array; it is not used
-    int64_t* dummy_b = ar.take<int64_t>(total + 1);
-    const size_t rws_bytes = radix_sort_workspace_bytes(total);
-    void* rws = ar.take<char>(rws_bytes);
+    if (total > MAX_CAPACITY) return fail(SGL_ENOTSUP, "unique_compact: too many ids");
+    const int64_t ncap = total < t.capacity ? total : t.capacity;
+    const Scratch s = carve_scratch(ar, total, ncap);
     if (!ar.ok()) return fail(SGL_ENOMEM, "unique_compact: workspace too small");
+    const int grouped = (mode == SGL_UNIQUE_GROUPED && G > 1) ? 1 : 0;
+    int glog = 0;
+    while (grouped && (1 << glog) < G) ++glog;
 
-    int64_t fb = ceil_div<int64_t>(cap, 1024);
-    if (fb > 65536) fb = 65536;
-    hipLaunchKernelGGL(fill_empty_kernel, dim3((unsigned)fb), dim3(256), 0, st, keys, cap, d_cnt);
+    auto grid = [](int64_t work, int per_block) {
+        int64_t b = ceil_div<int64_t>(work > 0 ? work : 1, per_block);
+        return dim3((unsigned)(b > MAX_GRID ? MAX_GRID : b));
+    };
+    const int64_t clear_work = (fresh || reset) ? t.slots : (1ll << s.nb_log);
+    hipLaunchKernelGGL(prep_kernel, grid(clear_work, 4 * BLOCK), dim3(BLOCK), 0, st, t, s, fresh ? 1 : 0, reset);
     SGL_LAUNCH_CHECK();
-    const int n_groups = (mode == SGL_UNIQUE_SORTED) ? (G > 0 ? 1 : 0) : G;
-    for (int grp = 0; grp < n_groups; ++grp) {
-        Arrays sub = all;
-        int64_t list_off = 0;
-        if (mode == SGL_UNIQUE_GROUPED) {
-            sub.G = 1;
-            sub.ids[0] = all.ids[grp]; sub.out[0] = all.out[grp];
-            sub.len_dev[0] = all.len_dev[grp]; sub.len_max[0] = all.len_max[grp];
-            sub.start[0] = 0;
-            for (int g = 1; g <= MAXG; ++g) sub.start[g] = sub.len_max[0];
-            list_off = all.start[grp];
-        }
-        const int64_t sub_total = sub.start[sub.G];
-        if (sub_total == 0) continue;
-        hipLaunchKernelGGL(insert_kernel, dim3((unsigned)ceil_div<int64_t>(sub_total, TILE)), dim3(BLOCK), 0, st, sub,
-                           keys, cap - 1, grp, d_cnt, list + list_off);
-        SGL_LAUNCH_CHECK();
-    }
-    Counters h;
-    SGL_HIP_TRY(hipMemcpyAsync(&h, d_cnt, sizeof h, hipMemcpyDeviceToHost, st));
-    SGL_HIP_TRY(hipStreamSynchronize(st));
-    const int bits = bits_of((uint64_t)h.max_id);
-    int64_t base = 0;
-    for (int grp = 0; grp < n_groups; ++grp) {
-        const int64_t cnt = h.count[grp];
-        if (cnt == 0) continue;
-        const int64_t list_off = (mode == SGL_UNIQUE_GROUPED) ? all.start[grp] : 0;
-        uint64_t* seg = reinterpret_cast<uint64_t*>(list + list_off);
-        int in_b = 0;
-        int32_t rc = radix_sort_pairs(seg, dummy_a, sort_b, dummy_b, cnt, nullptr, 0, bits, &in_b, rws, rws_bytes, st);
-        if (rc != SGL_OK) return rc;
-        hipLaunchKernelGGL(number_kernel, dim3((unsigned)ceil_div<int64_t>(cnt, BLOCK)), dim3(BLOCK), 0, st,
-                           in_b ? sort_b : seg, cnt, base, keys, vals, cap - 1, unique_out, unique_capacity);
-        SGL_LAUNCH_CHECK();
-        base += cnt;
-    }
     if (total > 0) {
-        hipLaunchKernelGGL(lookup_kernel, dim3((unsigned)ceil_div<int64_t>(total, BLOCK)), dim3(BLOCK), 0, st, all, keys,
-                           vals, cap - 1);
+        hipLaunchKernelGGL(insert_kernel, dim3((unsigned)ceil_div<int64_t>(total, TILE)), dim3(BLOCK), 0, st, all, t, s, reset, grouped);
+        SGL_LAUNCH_CHECK();
+        hipLaunchKernelGGL(hist_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, grouped, glog);
+        SGL_LAUNCH_CHECK();
+        hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, t, s);
+        SGL_LAUNCH_CHECK();
+        hipLaunchKernelGGL(scatter_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset);
+        SGL_LAUNCH_CHECK();
+        hipLaunchKernelGGL(number_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, unique_out, unique_capacity);
         SGL_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(publish_kernel, dim3(1), dim3(1), 0, st, U_dev, base);
+    hipLaunchKernelGGL(lookup_kernel, grid(total, BLOCK), dim3(BLOCK), 0, st, all, t, s, reset, U_dev);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }
 
+int64_t total_of(int32_t G, const int64_t* len_max) {
+    int64_t total = 0;
+    for (int32_t g = 0; g < G && len_max; ++g) total += len_max[g] > 0 ? len_max[g] : 0;
+    return total;
+}
+
+}  // namespace
+
+// ---- one-shot calls (sgl_unique_compact without a state): the table lives in the workspace ----
+size_t hash_unique_workspace_bytes(int32_t G, const int64_t* len_max) {
+    const int64_t total = total_of(G, len_max);
+    return state_bytes(total) + scratch_bytes(total, total) + 1024;
+}
+
+int32_t hash_unique_compact(int32_t mode, int32_t G, const int64_t* const* ids, const int64_t* len_max,
+                            const int64_t* const* len_dev, int64_t* const* local_out,
+                            int64_t* unique_out, int64_t unique_capacity, int64_t* U_dev, void* ws,
+                            size_t ws_bytes, hipStream_t st) {
+    if (!ws || ws_bytes < hash_unique_workspace_bytes(G, len_max))
+        return fail(SGL_ENOMEM, "unique_compact: workspace %zu < %zu bytes", ws_bytes, hash_unique_workspace_bytes(G, len_max));
+    const int64_t total = total_of(G, len_max);
+    if (total > MAX_CAPACITY) return fail(SGL_ENOTSUP, "unique_compact: too many ids");
+    Arena ar(ws, ws_bytes);
+    void* state = ar.take<char>(state_bytes(total));
+    return run(carve(state, total), true, 1, mode, G, ids, len_max, len_dev, local_out, unique_out, unique_capacity, U_dev, ar, st);
+}
+
 }  // namespace sgl
+
+using namespace sgl;
+
+extern "C" size_t sgl_remap_hashed_state_bytes(int64_t capacity) {
+    return state_bytes(capacity < 0 ? 0 : (capacity > MAX_CAPACITY ? MAX_CAPACITY : capacity));
+}
+
+extern "C" int32_t sgl_remap_hashed_init(void* state, size_t bytes, int64_t capacity, void* stream) {
+    int32_t rc;
+    if ((rc = check_capacity(capacity)) != SGL_OK) return rc;
+    if (!state || bytes < state_bytes(capacity)) return fail(SGL_EINVAL, "remap_hashed_init: state is NULL or smaller than %zu bytes", state_bytes(capacity));
+    if (capacity < 1) return fail(SGL_EINVAL, "remap_hashed_init: capacity < 1");
+    Table t = carve(state, capacity);
+    int64_t b = ceil_div<int64_t>(t.slots, 4 * BLOCK);
+    if (b > MAX_GRID) b = MAX_GRID;
+    hipLaunchKernelGGL(init_kernel, dim3((unsigned)b), dim3(BLOCK), 0, as_stream(stream), t);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}
+
+extern "C" size_t sgl_unique_hashed_workspace_bytes(int64_t capacity, int32_t G, const int64_t* len_max) {
+    const int64_t total = total_of(G, len_max);
+    const int64_t cap = capacity < 0 ? 0 : capacity;
+    return scratch_bytes(total, total < cap ? total : cap) + 1024;
+}
+
+extern "C" int32_t sgl_unique_compact_hashed(void* state, int64_t capacity, int32_t reset, int32_t mode, int32_t G,
+                                             const int64_t* const* ids, const int64_t* len_max,
+                                             const int64_t* const* len_dev, int64_t* const* local_out,
+                                             int64_t* unique_out, int64_t unique_capacity, int64_t* U_dev, void* ws,
+                                             size_t ws_bytes, void* stream) {
+    int32_t rc;
+    if (!state) return fail(SGL_EINVAL, "unique_compact_hashed: state is NULL");
+    if ((rc = check_capacity(capacity)) != SGL_OK) return rc;
+    if (capacity < 1) return fail(SGL_EINVAL, "unique_compact_hashed: capacity < 1");
+    if (G < 0 || (G > 0 && (!ids || !len_max || !local_out)) || !U_dev)
+        return fail(SGL_EINVAL, "unique_compact_hashed: NULL argument");
+    if (mode != SGL_UNIQUE_SORTED && mode != SGL_UNIQUE_GROUPED) return fail(SGL_EINVAL, "unique_compact_hashed: bad mode");
+    if (G > MAXG) return fail(SGL_ENOTSUP, "unique_compact_hashed: more than %d arrays", MAXG);
+    if (unique_capacity < 0 || (unique_capacity > 0 && !unique_out))
+        return fail(SGL_EINVAL, "unique_compact_hashed: unique_out is NULL");
+    for (int32_t g = 0; g < G; ++g) {
+        if (len_max[g] < 0) return fail(SGL_EINVAL, "unique_compact_hashed: negative length");
+        if (len_max[g] > 0 && (!ids[g] || !local_out[g])) return fail(SGL_EINVAL, "unique_compact_hashed: array %d is NULL", g);
+    }
+    if (!ws || ws_bytes < sgl_unique_hashed_workspace_bytes(capacity, G, len_max))
+        return fail(SGL_ENOMEM, "unique_compact_hashed: workspace %zu < %zu bytes", ws_bytes,
+                    sgl_unique_hashed_workspace_bytes(capacity, G, len_max));
+    Arena ar(ws, ws_bytes);
+    return run(carve(state, capacity), false, reset ? 1 : 0, mode, G, ids, len_max, len_dev, local_out, unique_out,
+               unique_capacity, U_dev, ar, as_stream(stream));
+}

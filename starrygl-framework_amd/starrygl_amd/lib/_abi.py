@@ -5,7 +5,7 @@ header declares.  The product library exports them as ``sgl_*``.
 """
 import ctypes as C
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
@@ -84,6 +84,11 @@ PROTOTYPES = {
     "unique_workspace_bytes": (sz, [i64, i32, P(i64)]),
     "unique_compact": (i32, [vp, i64, i32, i32, i32, P(vp), P(i64), P(vp), P(vp),
                              vp, i64, vp, vp, sz, vp]),
+    "remap_hashed_state_bytes": (sz, [i64]),
+    "remap_hashed_init": (i32, [vp, sz, i64, vp]),
+    "unique_hashed_workspace_bytes": (sz, [i64, i32, P(i64)]),
+    "unique_compact_hashed": (i32, [vp, i64, i32, i32, i32, P(vp), P(i64), P(vp), P(vp),
+                                    vp, i64, vp, vp, sz, vp]),
     "gather": (i32, [P(Cache), vp, i64, vp, vp, vp, vp, vp]),
     "gather_multi": (i32, [i32, P(GatherSeg), vp]),
     "scatter_update": (i32, [P(Cache), vp, vp, vp, vp, vp, i64, vp, vp, vp]),

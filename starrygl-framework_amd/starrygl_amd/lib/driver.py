@@ -119,7 +119,8 @@ def check_unique_total(u_total):
     """The id count of a unique_compact call is INT64_MAX when a numbering pass gave up waiting for
     an earlier tile (bounded wait): the result is void and the remap state has to be re-initialised."""
     if u_total == (1 << 63) - 1:
-        raise RuntimeError("unique_compact: a numbering pass gave up waiting; re-initialise the remap state")
+        raise RuntimeError("unique_compact: the result is void (a numbering pass gave up waiting, or a hashed state's "
+                           "capacity was exceeded); re-initialise the remap state")
 
 
 class HotPath:
@@ -324,9 +325,17 @@ class HotPath:
         self._ck(self.lib.remap_init(self.be.ptr(st), nbytes, universe, self.be.stream()))
         return RemapState(st, universe)
 
+    def remap_hashed_state(self, capacity):
+        """Persistent hash-set remap state for arbitrary non-negative ids: `capacity` is the largest
+        number of distinct ids one epoch may hold."""
+        nbytes = self.lib.remap_hashed_state_bytes(capacity)
+        st = self.be.empty(max(nbytes, 8), "u8")
+        self._ck(self.lib.remap_hashed_init(self.be.ptr(st), nbytes, capacity, self.be.stream()))
+        return HashedRemapState(st, capacity)
+
     def unique_compact(self, arrays, mode=_abi.UNIQUE_SORTED, state=None, reset=True,
                        lens_dev=None, out_arrays=None, finalize=True, unique_out=None, U_out=None,
-                       premarked=False):
+                       premarked=False, workspace=None):
         self._chk("i64", **{f"arrays[{i}]": a for i, a in enumerate(arrays)})
         be, G = self.be, len(arrays)
         len_max = (i64 * max(G, 1))(*[int(a.shape[0]) for a in arrays])
@@ -338,6 +347,9 @@ class HotPath:
         ldev = None
         if lens_dev is not None:
             ldev = (vp * max(G, 1))(*[be.ptr(a) for a in lens_dev])
+        hashed = isinstance(state, HashedRemapState)
+        if hashed and premarked:
+            raise ValueError("unique_compact: premarked needs a dense remap state")
         cap = total if state is None else min(total + state.count_bound, state.universe)
         if state is not None and reset:
             cap = min(total, state.universe)
@@ -347,12 +359,20 @@ class HotPath:
             unique = be.empty(max(cap, 1))
         U = be.zeros(2) if U_out is None else U_out
         universe = 0 if state is None else state.universe
-        ws, wsb = self._workspace(self.lib.unique_workspace_bytes(universe, G, len_max))
-        self._ck(self.lib.unique_compact(None if state is None else be.ptr(state.buf), universe,
-                                         int(bool(reset)), int(mode) | (_abi.UNIQUE_PREMARKED if premarked else 0),
-                                         G, ids, len_max, ldev, outs,
-                                         be.ptr(unique), cap, be.ptr(U), be.ptr(ws), wsb,
-                                         be.stream()))
+        if hashed:
+            need = self.lib.unique_hashed_workspace_bytes(universe, G, len_max)
+            ws, wsb = (workspace, be.nbytes(workspace)) if workspace is not None else self._workspace(need)
+            self._ck(self.lib.unique_compact_hashed(be.ptr(state.buf), universe, int(bool(reset)), int(mode),
+                                                    G, ids, len_max, ldev, outs, be.ptr(unique), cap, be.ptr(U),
+                                                    be.ptr(ws), wsb, be.stream()))
+        else:
+            need = self.lib.unique_workspace_bytes(universe, G, len_max)
+            ws, wsb = (workspace, be.nbytes(workspace)) if workspace is not None else self._workspace(need)
+            self._ck(self.lib.unique_compact(None if state is None else be.ptr(state.buf), universe,
+                                             int(bool(reset)), int(mode) | (_abi.UNIQUE_PREMARKED if premarked else 0),
+                                             G, ids, len_max, ldev, outs,
+                                             be.ptr(unique), cap, be.ptr(U), be.ptr(ws), wsb,
+                                             be.stream()))
         if state is not None:
             state.count_bound = cap
         if not finalize:
@@ -514,6 +534,14 @@ class HotPath:
 class RemapState:
     def __init__(self, buf, universe):
         self.buf, self.universe, self.count_bound = buf, int(universe), 0
+
+
+class HashedRemapState(RemapState):
+    """Hash-set remap state: `universe` holds its capacity in distinct ids (what bounds an epoch)."""
+
+    def __init__(self, buf, capacity):
+        super().__init__(buf, capacity)
+        self.capacity = int(capacity)
 
 
 class KHopResult:

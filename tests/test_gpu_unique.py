@@ -123,3 +123,98 @@ def test_hash_path_rejects_follow(hot):
     a = to_dev(hot, np.arange(10, dtype=np.int64))
     with pytest.raises(RuntimeError):
         hot.unique_compact([a], _abi.UNIQUE_SORTED, None, False)
+
+
+# ------------------------------------------------- persistent hash-set state
+def _encode(rng, n_parts, per_part, count):
+    """DistRouteIndex-style ids: partition << 48 | local index (partition_book.py:14-31)."""
+    return (rng.integers(0, n_parts, count) << 48) | rng.integers(0, per_part, count)
+
+
+@pytest.mark.parametrize("mode", [_abi.UNIQUE_SORTED, _abi.UNIQUE_GROUPED])
+@pytest.mark.parametrize("kind", ["encoded", "wide", "dense", "squares"])
+def test_hashed_state_epochs_reset_and_follow(oracle, hot, mode, kind):
+    """'r' then 'f' calls on a hashed state (Remapper::insert over the queries of a blob) against the oracle,
+    call by call; the id distributions include a skewed one whose buckets need the in-place sort."""
+    rng = np.random.default_rng(31)
+    draw = {"encoded": lambda n: _encode(rng, 8, 300_000, n),
+            "wide": lambda n: rng.integers(0, 2**62, n),
+            "dense": lambda n: rng.integers(0, 5000, n),
+            "squares": lambda n: rng.integers(0, 60_000, n) ** 2 + (1 << 40)}[kind]
+    cap = 400_000
+    so, sh = oracle.remap_hashed_state(cap), hot.remap_hashed_state(cap)
+    resets = [True, False, False, True, False, False]
+    sizes = [(500, 5000, 50_000), (3, 0, 2000), (40_000, 40_000, 100_000), (100_000, 7, 7), (1, 1, 1), (0, 90_000, 9)]
+    pool = draw(60_000).astype(np.int64)
+    for c, (reset, sz) in enumerate(zip(resets, sizes)):
+        arrs = [np.where(rng.random(n) < 0.7, pool[rng.integers(0, pool.shape[0], n)], draw(n)).astype(np.int64) for n in sz]
+        if arrs[0].shape[0] > 4:
+            arrs[0][3] = -9
+        lo, uo, (to_, bo) = oracle.unique_compact([a.copy() for a in arrs], mode, so, reset)
+        lh, uh, (th, bh) = hot.unique_compact([to_dev(hot, a) for a in arrs], mode, sh, reset)
+        assert (th, bh) == (to_, bo), f"call {c}"
+        assert np.array_equal(np_of(uh)[bh:th], uo[bo:to_]), f"call {c}: unique list differs"
+        for g in range(len(arrs)):
+            assert np.array_equal(np_of(lh[g]), lo[g]), f"call {c} array {g}: local ids differ"
+
+
+def test_hashed_state_oversized_buckets_are_sorted_in_place(oracle, hot):
+    """Ids crowded at the low end of a huge range (one id near 2^62 stretches the key): thousands of ids
+    share a bucket and go through the block-wide sort."""
+    rng = np.random.default_rng(8)
+    a = np.concatenate([rng.integers(0, 3000, 40_000), np.array([2**62 - 5]), rng.integers(2**30, 2**30 + 1500, 9000)]).astype(np.int64)
+    rng.shuffle(a)
+    sh = hot.remap_hashed_state(60_000)
+    lh, uh, (th, _) = hot.unique_compact([to_dev(hot, a)], _abi.UNIQUE_SORTED, sh, True)
+    u, inv = np.unique(a, return_inverse=True)
+    assert th == u.shape[0] and np.array_equal(np_of(uh), u) and np.array_equal(np_of(lh[0]), inv)
+
+
+def test_hashed_state_reports_an_outgrown_capacity(hot):
+    sh = hot.remap_hashed_state(1000)
+    a = to_dev(hot, np.arange(900, dtype=np.int64) * 7)
+    hot.unique_compact([a], _abi.UNIQUE_SORTED, sh, True)
+    with pytest.raises(RuntimeError, match="void"):
+        hot.unique_compact([to_dev(hot, np.arange(200, dtype=np.int64) * 7 + 1)], _abi.UNIQUE_SORTED, sh, False)
+    with pytest.raises(RuntimeError, match="void"):
+        hot.unique_compact([a], _abi.UNIQUE_SORTED, sh, True)
+    # a fresh state works again
+    lh, uh, (th, _) = hot.unique_compact([a], _abi.UNIQUE_SORTED, hot.remap_hashed_state(1000), True)
+    assert th == 900 and np.array_equal(np_of(lh[0]), np.arange(900))
+
+
+def test_hash_unique_is_captured_and_replayed_in_a_hip_graph(oracle, hot):
+    """The hash-set path is a fixed launch sequence without host synchronisation: captured once, replayed
+    over new ids of varying live length, with eager work and synchronisations between the replays."""
+    import torch
+    rng = np.random.default_rng(3)
+    n = 30_000
+    ids = torch.zeros(n, dtype=torch.int64, device="cuda")
+    live = torch.zeros(1, dtype=torch.int64, device="cuda")
+    out, uniq, U = torch.empty_like(ids), torch.empty(n, dtype=torch.int64, device="cuda"), torch.zeros(2, dtype=torch.int64, device="cuda")
+    state = hot.remap_hashed_state(n)
+    lens = (_abi.i64 * 1)(n)
+    ws = torch.empty(int(hot.lib.unique_hashed_workspace_bytes(n, 1, lens)), dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.Stream()
+
+    def call(st):
+        hot.unique_compact([ids], _abi.UNIQUE_SORTED, st, True, lens_dev=[live], out_arrays=[out], unique_out=uniq,
+                           U_out=U, finalize=False, workspace=ws)
+
+    with torch.cuda.stream(stream):
+        call(state)                      # warm-up outside the capture
+    stream.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        call(state)
+    for rep, m in enumerate((n, 17, 12_345, 0, n)):
+        a = _encode(rng, 4, 9000, n).astype(np.int64)
+        ids.copy_(torch.from_numpy(a))
+        live.fill_(m)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        u, inv = np.unique(a[:m], return_inverse=True)
+        tot = int(U[0])
+        assert tot == u.shape[0], f"replay {rep}"
+        assert np.array_equal(np_of(uniq)[:tot], u) and np.array_equal(np_of(out)[:m], inv), f"replay {rep}"

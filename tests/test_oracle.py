@@ -233,6 +233,39 @@ def test_unique_epochs(oracle):
         oracle.unique_compact([b], _abi.UNIQUE_SORTED, None, False)
 
 
+def test_unique_hashed_state_follows_epochs_like_the_dense_state(oracle):
+    """A hashed state numbers exactly as a dense state does (pinned above by np.unique / setdiff1d), call by
+    call over an epoch, for ids shifted far outside any dense universe; pinned independently by np.setdiff1d."""
+    rng = np.random.default_rng(12)
+    shift = (5 << 48) + 12345
+    for mode in (_abi.UNIQUE_SORTED, _abi.UNIQUE_GROUPED):
+        dense, hashed = oracle.remap_state(4000), oracle.remap_hashed_state(5000)
+        known = np.zeros(0, np.int64)
+        for call, reset in enumerate([True, False, False, True, False]):
+            arrs = [rng.integers(0, 4000, n).astype(np.int64) for n in (30, 400, 900)]
+            ld, ud, cd = oracle.unique_compact(arrs, mode, dense, reset)
+            lh, uh, ch = oracle.unique_compact([a + shift for a in arrs], mode, hashed, reset)
+            assert cd == ch and np.array_equal(ud[cd[1]:] + shift, uh[ch[1]:ch[0]])
+            assert all(np.array_equal(a, b) for a, b in zip(ld, lh))
+            if reset:
+                known = np.zeros(0, np.int64)
+            groups = [np.concatenate(arrs)] if mode == _abi.UNIQUE_SORTED else arrs
+            for x in groups:
+                known = np.concatenate([known, np.setdiff1d(np.unique(x), known)])
+            assert ch[0] == known.shape[0] and np.array_equal(uh[ch[1]:ch[0]], known[ch[1]:] + shift)
+            for a, l in zip(arrs, lh):
+                assert np.array_equal(known[l], a)
+
+
+def test_unique_hashed_state_reports_an_outgrown_capacity(oracle):
+    st = oracle.remap_hashed_state(10)
+    oracle.unique_compact([np.arange(8, dtype=np.int64) * 1000], _abi.UNIQUE_SORTED, st, True)
+    with pytest.raises(RuntimeError, match="void"):
+        oracle.unique_compact([np.arange(5, dtype=np.int64) * 1000 + 1], _abi.UNIQUE_SORTED, st, False)
+    with pytest.raises(RuntimeError, match="void"):          # sticky until the state is initialised again
+        oracle.unique_compact([np.arange(2, dtype=np.int64)], _abi.UNIQUE_SORTED, st, True)
+
+
 # ------------------------------------------------------------------ gather
 def test_gather_and_scatter_are_fancy_indexing(oracle):
     rng = np.random.default_rng(5)
