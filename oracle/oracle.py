@@ -85,5 +85,18 @@ def load():
         cdll.sglo_draw_bits.argtypes = [C.c_uint64, C.c_int32, C.c_int64, C.c_int32]
         cdll.sglo_bounded.restype = C.c_int64
         cdll.sglo_bounded.argtypes = [C.c_uint64, C.c_int64]
+        # the indexed CPU sampler (same prototype as sample_khop): the CPU side of an equal-work timing
+        cdll.sglo_sample_khop_indexed.restype = lib.sample_khop.restype
+        cdll.sglo_sample_khop_indexed.argtypes = lib.sample_khop.argtypes
         _cached = (HotPath(lib, NumpyBackend()), cdll)
     return _cached
+
+
+def sample_khop_indexed(hp, cdll, g, roots, ts_ptr, root_ts, neg_roots, neg_ts, layers, p):
+    """`hp.sample_khop` through sglo_sample_khop_indexed: the oracle's sampler given the next-hop index of
+    `g` (g.view.hop_hint) and the root hints of `p`, searching only what those leave open."""
+    plain, hp.lib.sample_khop = hp.lib.sample_khop, cdll.sglo_sample_khop_indexed
+    try:
+        return hp.sample_khop(g, roots, ts_ptr, root_ts, neg_roots, neg_ts, layers, p)
+    finally:
+        hp.lib.sample_khop = plain

@@ -282,12 +282,13 @@ size_t sglo_sample_hop_workspace_bytes(int64_t S_max) { (void)S_max; return 0; }
  * static_recent_neighbor_num / recent_sample_single_hop_kernel and
  * static_neighbor_num / uniform_sample_single_hop_kernel
  * (sample.cu.hpp:706-827); sample_kernel (graph.cpu.hpp:256-310). */
-int32_t sglo_sample_hop(const sgl_tcsr* g, const int64_t* slot_node,
+/* slot_hint / hint_out: only for the indexed CPU baseline (sglo_sample_khop_indexed below).  slot_hint[s] >= 0
+ * is taken as the end of slot s's strictly-before window instead of searching for it; hint_out receives the
+ * graph's next-hop index entry of every emitted edge. */
+static int32_t hop_impl(const sgl_tcsr* g, const int64_t* slot_node,
                         const int64_t* slot_ts, int64_t S_max,
                         const int64_t* S_dev, const sgl_sample_params* p,
-                        const sgl_hop_out* out, void* ws, size_t ws_bytes,
-                        void* stream) {
-    (void)ws; (void)ws_bytes; (void)stream;
+                        const sgl_hop_out* out, const int64_t* slot_hint, int64_t* hint_out) {
     if (!g || !p || !out || S_max < 0) return fail(SGL_EINVAL, "sample_hop: null/negative");
     if (p->type != SGL_SAMPLE_RECENT && p->type != SGL_SAMPLE_UNIFORM)
         return fail(SGL_ENOTSUP, "undefined sampling strategy");
@@ -310,7 +311,14 @@ int32_t sglo_sample_hop(const sgl_tcsr* g, const int64_t* slot_node,
         int64_t v = slot_node[s];
         if (v < 0 || v >= g->n) { cnt[s] = 0; wlo[s] = whi[s] = 0; bad++; continue; }
         int64_t lo, hi;
-        window(g, v, slot_ts[s], p->allowed_offset, p->equal_root_time, &lo, &hi);
+        if (slot_hint && slot_hint[s] >= 0 && !p->equal_root_time) {
+            const int64_t rs = g->row_ptr[v], re = g->row_ptr[v + 1];
+            hi = slot_hint[s] < rs ? rs : (slot_hint[s] > re ? re : slot_hint[s]);
+            lo = rs;
+            if (p->allowed_offset >= 0) lo = lower_bound_ts(g->ts, rs, hi, slot_ts[s] - p->allowed_offset);
+        } else {
+            window(g, v, slot_ts[s], p->allowed_offset, p->equal_root_time, &lo, &hi);
+        }
         wlo[s] = lo; whi[s] = hi;
         int64_t c = hi - lo;
         cnt[s] = c < k ? c : k;
@@ -335,6 +343,7 @@ int32_t sglo_sample_hop(const sgl_tcsr* g, const int64_t* slot_node,
                     (p->type == SGL_SAMPLE_UNIFORM && p->keep_root_time) ? t : g->ts[e];
                 out->neighbors_eid[off + j] = g->eid[e];
                 out->neighbors_dt[off + j] = g->ts[e] - t;
+                if (hint_out) hint_out[off + j] = g->hop_hint[e];
             }
         } else {
             int64_t sel[SGL_UNIFORM_MAX_FANOUT];
@@ -350,12 +359,22 @@ int32_t sglo_sample_hop(const sgl_tcsr* g, const int64_t* slot_node,
                 out->neighbors_ts[off + j] = p->keep_root_time ? t : g->ts[e];
                 out->neighbors_eid[off + j] = g->eid[e];
                 out->neighbors_dt[off + j] = g->ts[e] - t;
+                if (hint_out) hint_out[off + j] = g->hop_hint[e];
             }
         }
     }
     out->counts[0] = S; out->counts[1] = acc; out->counts[2] = bad;
     free(cnt); free(wlo); free(whi);
     return SGL_OK;
+}
+
+int32_t sglo_sample_hop(const sgl_tcsr* g, const int64_t* slot_node,
+                        const int64_t* slot_ts, int64_t S_max,
+                        const int64_t* S_dev, const sgl_sample_params* p,
+                        const sgl_hop_out* out, void* ws, size_t ws_bytes,
+                        void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    return hop_impl(g, slot_node, slot_ts, S_max, S_dev, p, out, NULL, NULL);
 }
 
 /* The workspace-free variant of the hop: the oracle never uses a workspace, so
@@ -417,6 +436,48 @@ int32_t sglo_sample_khop(const sgl_tcsr* g, int64_t R, const int64_t* roots,
         if (rc != SGL_OK) return rc;
         sn = outs[l].neighbors; st = outs[l].neighbors_ts; S = outs[l].counts[1];
     }
+    return SGL_OK;
+}
+
+/* The k-hop driver given the same two indexes as the HIP library's fastest route: positive roots
+ * take their window end from p->root_hint (negatives are searched), the slots of hops >= 1 from
+ * the graph's next-hop index (g->hop_hint) - no search for them.  NOT part of the checker (the
+ * oracle proper always searches): this is the CPU side of an equal-work timing, and the tests
+ * hold it against sglo_sample_khop on the same inputs.  Same arguments as sglo_sample_khop. */
+int32_t sglo_sample_khop_indexed(const sgl_tcsr* g, int64_t R, const int64_t* roots,
+                                 const int64_t* ts_ptr, int64_t S_pos,
+                                 const int64_t* root_ts, int64_t N_neg,
+                                 const int64_t* neg_roots, const int64_t* neg_ts,
+                                 int32_t layers, const sgl_sample_params* p,
+                                 int64_t* slot_node0, int64_t* slot_ts0,
+                                 const sgl_hop_out* outs, void* ws, size_t ws_bytes,
+                                 void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (!g || !p || !outs || R < 0 || S_pos < 0 || N_neg < 0 || layers < 1)
+        return fail(SGL_EINVAL, "sample_khop_indexed: null/negative");
+    for (int64_t r = 0; r < R; ++r)
+        for (int64_t s = ts_ptr[r]; s < ts_ptr[r + 1]; ++s) { slot_node0[s] = roots[r]; slot_ts0[s] = root_ts[s]; }
+    for (int64_t i = 0; i < N_neg; ++i) { slot_node0[S_pos + i] = neg_roots[i]; slot_ts0[S_pos + i] = neg_ts[i]; }
+    const int carry = g->hop_hint != NULL && !p->equal_root_time && !(p->type == SGL_SAMPLE_UNIFORM && p->keep_root_time);
+    int64_t S = S_pos + N_neg;
+    int64_t* hint = (int64_t*)malloc((size_t)(S + 1) * sizeof(int64_t));
+    if (!hint) return fail(SGL_ENOMEM, "malloc");
+    for (int64_t s = 0; s < S; ++s) hint[s] = (p->root_hint && s < S_pos) ? p->root_hint[s] : -1;
+    const int64_t* sn = slot_node0; const int64_t* st = slot_ts0;
+    for (int32_t l = 0; l < layers; ++l) {
+        sgl_sample_params pl = *p; pl.hop = l;
+        int64_t* next = NULL;
+        if (carry && l + 1 < layers) {
+            next = (int64_t*)malloc((size_t)(S * (int64_t)p->fanout + 1) * sizeof(int64_t));
+            if (!next) { free(hint); return fail(SGL_ENOMEM, "malloc"); }
+        }
+        int32_t rc = hop_impl(g, sn, st, S, NULL, &pl, &outs[l], hint, next);
+        free(hint);
+        hint = next;
+        if (rc != SGL_OK) { free(hint); return rc; }
+        sn = outs[l].neighbors; st = outs[l].neighbors_ts; S = outs[l].counts[1];
+    }
+    free(hint);
     return SGL_OK;
 }
 

@@ -5,67 +5,79 @@
 // table of 8-byte keys with a parallel array of 4-byte local ids; it lives
 // either in a persistent "hashed state" of a stated capacity (an epoch of local
 // ids can then continue over several calls, as with the dense state) or, for
-// one-shot calls, in the call's workspace.  A call is a fixed sequence of seven
+// one-shot calls, in the call's workspace.  A call is a fixed sequence of
 // launches on the caller's stream, sized on the host from the worst case and
 // driven by device-side counts - no host synchronisation, HIP-graph capturable:
 //
 //   prep    : empties the table (everything for a workspace table; for a
 //             persistent one only on reset, and then only the slots the last
 //             epoch used when those are few) and zeroes the bucket counters;
-//   insert  : a block folds its 2048 ids through an LDS set, so an id that
+//   insert  : a block folds its tile of ids through an LDS set, so an id that
 //             repeats inside the tile reaches the global table once; the
-//             tile-unique ids probe the table (a plain load first: most ids of
-//             a sampled batch are repeats and end there; atomicCAS only on an
-//             empty slot).  Every input element remembers the table slot of its
-//             id (4 bytes), so nothing is ever probed twice.  The ids a block
-//             added are appended - id and slot - to the call's list with ONE
-//             returning atomic per block; OR and AND over them are kept;
-//   hist    : the new ids have to be numbered in ascending order.  The bits in
+//             element that put an id into the LDS set probes the table for it
+//             (a plain load first: most ids of a sampled batch are repeats and
+//             end there; atomicCAS only on an empty slot).  Every input element
+//             remembers the table slot of its id (4 bytes), so nothing is ever
+//             probed twice.  The ids a block added are appended - id and slot -
+//             to the call's list with ONE returning atomic per block; OR and
+//             AND over them are kept;
+//   order   : the new ids have to be numbered in ascending order.  The bits in
 //             which they differ at all (OR ^ AND) are squeezed together into a
-//             short key that keeps the order, and its top bits select one of up
-//             to 2^18 buckets (in grouped mode the array that owns the id is
-//             the top digit); bucket sizes are counted with spread atomics;
-//   scan    : one block turns counts into offsets and lists oversized buckets;
-//   scatter : ids move to their bucket's segment;
-//   number  : an id's rank = bucket offset + ids of its bucket that are smaller
-//             (a handful: the buckets hold ~8 ids); rank + ids numbered before
-//             = local id, written to the table and the local->global list.
-//             Oversized buckets (skewed id distributions) are sorted by a block
-//             each with a bitonic network in place;
+//             short key that keeps the order (in grouped mode the array that
+//             owns the id is the top digit), and the top bits of that key cut
+//             the ids into buckets of a few ids each:
+//             - calls of up to 2^20 ids: hist (bucket sizes by spread atomics),
+//               scan (one block), scatter (ids move to their bucket's segment);
+//             - larger calls, where an atomic per id costs more than a pass
+//               over the data: three 8-bit passes of the library's radix sort
+//               on the top 24 bits of the key;
+//   number  : an id's rank = first place of its bucket + ids of the bucket
+//             that are smaller (a handful); rank + ids numbered before = local
+//             id, written to the table and the local->global list.  Oversized
+//             buckets (skewed id distributions) are sorted by a block each with
+//             a bitonic network in place;
 //   lookup  : out[i] = local id at the slot element i remembered.
 //
 // Numbering is by ascending id inside each group, so the result equals the dense
 // path and the reference's sort + unique (csrc/include/starrygl/sample.cu.hpp:
 // 1786-1852) bit for bit.
 #include "common.hpp"
+#include "radix.hpp"
 
 namespace sgl {
 namespace {
 
 constexpr int BLOCK = 256;
 constexpr int MAXG = 8;
-constexpr int IPT = 8;
-constexpr int TILE = BLOCK * IPT;        // ids per block of insert
-constexpr int LDS_SLOTS = 2 * TILE;      // load <= 0.5
 constexpr unsigned long long EMPTY = ~0ull;
 constexpr uint32_t NONE = 0xFFFFFFFFu;   // slot of an element whose id is negative
 constexpr uint32_t UNNUMBERED = 0x7FFFFFFFu;  // value of a slot whose id has no local id yet
 constexpr uint32_t PENDING0 = 0x7FFFFFE0u;    // PENDING0 + g: not numbered yet, first seen in array g (grouped mode)
 constexpr int64_t MAX_CAPACITY = 0x7FFFFF00ll;
-constexpr int NB_MIN_LOG = 8, NB_MAX_LOG = 18;
+constexpr int NB_MIN_LOG = 8, NB_MAX_LOG = 15;   // buckets of the atomic route: 32 consecutive counters per scan thread
+constexpr int64_t ATOMIC_ROUTE_MAX = 1ll << 20;  // most ids a call may add for the atomic route to be taken
+constexpr int SORT_KEY_LOG = 24;         // bucket bits of the radix route (three 8-bit passes)
+constexpr int SORT_KEY_SHIFT = 64 - SORT_KEY_LOG;
 constexpr int SMALL_BUCKET = 512;        // buckets up to this size are ranked by counting
 constexpr int SCAN_BLOCK = 1024;
 constexpr int MAX_GRID = 4096;
 
+// Every field that blocks of one launch hammer with atomics has a 128-byte line of its own: a line that
+// holds a contended counter serves nothing else at a useful rate.
 struct Header {
     unsigned long long total;     // ids numbered in the current epoch (committed by the last launch of a call)
+    unsigned long long nbig;      // oversized buckets of the running call (0 between calls)
+    unsigned long long pad0[14];
     unsigned long long appended;  // ids the running call has added (0 between calls)
+    unsigned long long pad1[15];
     unsigned long long or_mask;   // OR / AND over the ids the running call has added (0 / ~0 between calls)
     unsigned long long and_mask;
+    unsigned long long pad2[14];
     unsigned long long overflow;  // sticky: more ids than the capacity, or no free slot
-    unsigned long long nbig;      // oversized buckets of the running call (0 between calls)
+    unsigned long long pad3[15];
 };
-constexpr size_t HEADER_BYTES = 256;
+constexpr size_t HEADER_BYTES = 512;
+static_assert(sizeof(Header) == HEADER_BYTES, "hashed state header layout");
 
 struct Table {
     Header* hdr;
@@ -97,7 +109,8 @@ Table carve(void* state, int64_t capacity) {
     return t;
 }
 
-// Per-call scratch
+// Per-call scratch.  Atomic route: list_b, part_*, cnt, off.  Radix route: key_a/b (bucket << 40 | table
+// slot) with the ids as the sort's values (id_a/b), and the sort's own workspace.
 struct Scratch {
     uint32_t* slot_of;          // [total] table slot of every input element (NONE: negative id)
     unsigned long long* list_id;  // [ncap] ids added by this call, in the order of their appends
@@ -107,37 +120,60 @@ struct Scratch {
     uint32_t* part_b;           // [ncap]
     uint32_t* cnt;              // [nb + 1] bucket sizes, later the scatter cursors
     uint32_t* off;              // [nb + 1] bucket offsets
-    uint32_t* big;              // [ncap / SMALL_BUCKET + 1] oversized buckets
+    uint32_t* big;              // [ncap / SMALL_BUCKET + 2] oversized buckets (atomic route) / their first places (radix route)
+    uint64_t* key_a;            // [ncap] radix route
+    uint64_t* key_b;
+    int64_t* id_b;              // (id_a is list_id)
+    void* sort_ws;
+    size_t sort_ws_bytes;
     int64_t ncap;               // most ids one call can add
     int32_t nb_log;             // log2 of the number of buckets
+    int32_t radix;              // 1: radix route
 };
 
+bool radix_route(int64_t ncap) { return ncap > ATOMIC_ROUTE_MAX; }
+
 int nb_log_of(int64_t ncap) {
+    if (radix_route(ncap)) return SORT_KEY_LOG;
     int l = NB_MIN_LOG;
-    while (l < NB_MAX_LOG && (8ll << l) < ncap) ++l;
+    while (l < NB_MAX_LOG && (32ll << l) < ncap) ++l;     // ~32 ids per bucket when every id of the call is new
     return l;
 }
 
 size_t scratch_bytes(int64_t total, int64_t ncap) {
     const int64_t nb = 1ll << nb_log_of(ncap);
-    return align_up((size_t)(total + 1) * 4) + 2 * align_up((size_t)(ncap + 1) * 8) + 3 * align_up((size_t)(ncap + 1) * 4) +
-           2 * align_up((size_t)(nb + 1) * 4) + align_up((size_t)(ncap / SMALL_BUCKET + 2) * 4) + 1024;
+    size_t b = align_up((size_t)(total + 1) * 4) + align_up((size_t)(ncap + 1) * 8) +
+               align_up((size_t)(ncap / SMALL_BUCKET + 2) * 4) + 1024;
+    if (radix_route(ncap))
+        b += 3 * align_up((size_t)(ncap + 1) * 8) + radix_sort_workspace_bytes(ncap) + 256;
+    else
+        b += align_up((size_t)(ncap + 1) * 8) + 3 * align_up((size_t)(ncap + 1) * 4) + 2 * align_up((size_t)(nb + 1) * 4);
+    return b;
 }
 
 Scratch carve_scratch(Arena& ar, int64_t total, int64_t ncap) {
-    Scratch s;
+    Scratch s{};
     s.ncap = ncap;
     s.nb_log = nb_log_of(ncap);
+    s.radix = radix_route(ncap) ? 1 : 0;
     const int64_t nb = 1ll << s.nb_log;
     s.slot_of = ar.take<uint32_t>(total + 1);
     s.list_id = ar.take<unsigned long long>(ncap + 1);
-    s.part_id = ar.take<unsigned long long>(ncap + 1);
-    s.list_b = ar.take<uint32_t>(ncap + 1);
-    s.part_slot = ar.take<uint32_t>(ncap + 1);
-    s.part_b = ar.take<uint32_t>(ncap + 1);
-    s.cnt = ar.take<uint32_t>(nb + 1);
-    s.off = ar.take<uint32_t>(nb + 1);
     s.big = ar.take<uint32_t>(ncap / SMALL_BUCKET + 2);
+    if (s.radix) {
+        s.key_a = ar.take<uint64_t>(ncap + 1);
+        s.key_b = ar.take<uint64_t>(ncap + 1);
+        s.id_b = ar.take<int64_t>(ncap + 1);
+        s.sort_ws_bytes = radix_sort_workspace_bytes(ncap);
+        s.sort_ws = ar.take<char>(s.sort_ws_bytes);
+    } else {
+        s.part_id = ar.take<unsigned long long>(ncap + 1);
+        s.list_b = ar.take<uint32_t>(ncap + 1);
+        s.part_slot = ar.take<uint32_t>(ncap + 1);
+        s.part_b = ar.take<uint32_t>(ncap + 1);
+        s.cnt = ar.take<uint32_t>(nb + 1);
+        s.off = ar.take<uint32_t>(nb + 1);
+    }
     return s;
 }
 
@@ -170,7 +206,7 @@ __device__ __forceinline__ bool locate(const Arrays& a, int64_t t, int* g_out, i
     return true;
 }
 
-// What a call works with: ids numbered before it and (from the hist launch on) ids it added.
+// What a call works with: ids numbered before it and (from the order launches on) ids it added.
 __device__ __forceinline__ int64_t ids_before(const Table& t, int reset) { return reset ? 0 : (int64_t)t.hdr->total; }
 __device__ __forceinline__ int64_t ids_added(const Table& t, const Scratch& s, int64_t before) {
     int64_t n = (int64_t)t.hdr->appended;
@@ -214,8 +250,10 @@ __global__ __launch_bounds__(BLOCK) void prep_kernel(Table t, Scratch s, int fre
             t.vals[h] = UNNUMBERED;
         }
     }
-    const int64_t nb = 1ll << s.nb_log;
-    for (int64_t i = tid; i <= nb; i += stride) s.cnt[i] = 0;
+    if (!s.radix) {
+        const int64_t nb = 1ll << s.nb_log;
+        for (int64_t i = tid; i <= nb; i += stride) s.cnt[i] = 0;
+    }
     if (fresh && tid == 0) {
         t.hdr->total = 0;
         t.hdr->appended = 0;
@@ -226,90 +264,116 @@ __global__ __launch_bounds__(BLOCK) void prep_kernel(Table t, Scratch s, int fre
     }
 }
 
+// IPT ids per thread: a tile of 256 * IPT ids per block (small calls take small tiles so that the chip has
+// blocks to run; large ones take large tiles, which fold more repeats before the table is touched).
+template <int IPT>
 __global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratch s, int reset, int grouped) {
+    constexpr int TILE = BLOCK * IPT;
+    constexpr int LDS_SLOTS = 2 * TILE;      // load <= 0.5
     __shared__ unsigned long long s_key[LDS_SLOTS];
     __shared__ uint32_t s_aux[LDS_SLOTS];       // first the smallest array index that holds the id, then its table slot
     __shared__ int32_t s_won;
     __shared__ long long s_base;
     __shared__ unsigned long long s_or, s_and;
-    for (int q = threadIdx.x; q < LDS_SLOTS; q += BLOCK) {
-        s_key[q] = EMPTY;
-        s_aux[q] = MAXG;
+#pragma unroll
+    for (int q = 0; q < LDS_SLOTS / BLOCK; ++q) {
+        s_key[q * BLOCK + threadIdx.x] = EMPTY;
+        s_aux[q * BLOCK + threadIdx.x] = MAXG;
     }
     if (threadIdx.x == 0) {
         s_won = 0;
         s_or = 0;
         s_and = ~0ull;
     }
-    __syncthreads();
     const int64_t t0 = (int64_t)blockIdx.x * TILE + threadIdx.x;
-    int32_t ls[IPT];
+    // the tile's ids (every load issued before the first LDS probe)
+    int64_t id[IPT];
+    int32_t grp[IPT];
 #pragma unroll
     for (int q = 0; q < IPT; ++q) {
-        ls[q] = -2;                       // -2: no element, -1: negative id
+        id[q] = -1;
+        grp[q] = -1;                      // -1: no element
         int g;
         int64_t i;
-        if (!locate(a, t0 + (int64_t)q * BLOCK, &g, &i)) continue;
-        const int64_t id = a.ids[g][i];
+        if (locate(a, t0 + (int64_t)q * BLOCK, &g, &i)) {
+            id[q] = a.ids[g][i];
+            grp[q] = g;
+        }
+    }
+    __syncthreads();
+    int32_t ls[IPT];                      // LDS slot of the id; -1: negative id or no element
+    bool owner[IPT];                      // this element put the id into the LDS set
+#pragma unroll
+    for (int q = 0; q < IPT; ++q) {
         ls[q] = -1;
-        if (id < 0) continue;
-        uint32_t h = (uint32_t)mix((uint64_t)id) & (LDS_SLOTS - 1);
+        owner[q] = false;
+        if (id[q] < 0) continue;
+        uint32_t h = (uint32_t)mix((uint64_t)id[q]) & (LDS_SLOTS - 1);
         while (true) {
-            const unsigned long long prev = atomicCAS(&s_key[h], EMPTY, (unsigned long long)id);
-            if (prev == EMPTY || prev == (unsigned long long)id) break;
+            const unsigned long long prev = atomicCAS(&s_key[h], EMPTY, (unsigned long long)id[q]);
+            if (prev == EMPTY) owner[q] = true;
+            if (prev == EMPTY || prev == (unsigned long long)id[q]) break;
             h = (h + 1) & (LDS_SLOTS - 1);
         }
         ls[q] = (int32_t)h;
-        if (grouped) atomicMin(&s_aux[h], (uint32_t)g);
+        if (grouped) atomicMin(&s_aux[h], (uint32_t)grp[q]);
     }
-    __syncthreads();
-    // every occupied LDS slot is one tile-unique id: find or claim its table slot
+    if (grouped) __syncthreads();          // an owner needs the smallest array index of its id
+    // every owner finds or claims the table slot of its id: first probes of all its ids in flight together
     const int64_t before = ids_before(t, reset);
-    unsigned long long won[LDS_SLOTS / BLOCK];
-    uint32_t won_slot[LDS_SLOTS / BLOCK];
-    int32_t pos[LDS_SLOTS / BLOCK];
+    uint64_t h[IPT];
+    unsigned long long k0[IPT];
+#pragma unroll
+    for (int q = 0; q < IPT; ++q) {
+        h[q] = 0;
+        k0[q] = 0;
+        if (owner[q]) {
+            h[q] = __umul64hi(mix((uint64_t)id[q]), (uint64_t)t.slots);
+            k0[q] = t.keys[h[q]];       // a slot never changes once it holds an id: a cached value is good
+        }
+    }
+    bool won[IPT];
+    int32_t pos[IPT];
     unsigned long long my_or = 0, my_and = ~0ull;
     bool lost = false;
 #pragma unroll
-    for (int q = 0; q < LDS_SLOTS / BLOCK; ++q) {
-        const int l = q * BLOCK + threadIdx.x;
-        const unsigned long long id = s_key[l];
-        won[q] = EMPTY;
-        won_slot[q] = 0;
+    for (int q = 0; q < IPT; ++q) {
+        won[q] = false;
         pos[q] = 0;
-        if (id == EMPTY) continue;
-        const uint32_t grp = s_aux[l];
-        uint64_t h = __umul64hi(mix(id), (uint64_t)t.slots);
+        if (!owner[q]) continue;
+        const unsigned long long me = (unsigned long long)id[q];
+        const uint32_t g_min = s_aux[ls[q]];
+        unsigned long long k = k0[q];
         bool placed = false;
         for (int64_t probes = 0; probes < t.slots; ++probes) {
-            unsigned long long k = t.keys[h];     // a slot never changes once it holds an id: a cached value is good
+            if (probes > 0) k = t.keys[h[q]];
             if (k == EMPTY) {
-                k = atomicCAS(&t.keys[h], EMPTY, id);
+                k = atomicCAS(&t.keys[h[q]], EMPTY, me);
                 if (k == EMPTY) {
-                    won[q] = id;
-                    k = id;
+                    won[q] = true;
+                    k = me;
                 }
             }
-            if (k == id) {
+            if (k == me) {
                 placed = true;
                 break;
             }
-            h = h + 1 == (uint64_t)t.slots ? 0 : h + 1;
+            h[q] = h[q] + 1 == (uint64_t)t.slots ? 0 : h[q] + 1;
         }
         if (!placed) {          // the table is full
             lost = true;
-            s_aux[l] = NONE;
+            won[q] = false;
+            s_aux[ls[q]] = NONE;
             continue;
         }
-        s_aux[l] = (uint32_t)h;
+        s_aux[ls[q]] = (uint32_t)h[q];
         // grouped: an id that has no local id yet belongs to the first array that holds it (a local id is
         // smaller than every PENDING value, so ids of earlier calls keep theirs)
-        if (grouped) atomicMin(&t.vals[h], PENDING0 + grp);
-        if (won[q] != EMPTY) {
-            won_slot[q] = (uint32_t)h;
+        if (grouped) atomicMin(&t.vals[h[q]], PENDING0 + g_min);
+        if (won[q]) {
             pos[q] = atomicAdd(&s_won, 1);
-            my_or |= id;
-            my_and &= id;
+            my_or |= me;
+            my_and &= me;
         }
     }
     if (my_or != 0 || my_and != ~0ull) {
@@ -320,23 +384,24 @@ __global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratc
     __syncthreads();
     if (threadIdx.x == 0 && s_won > 0) {
         s_base = (long long)atomicAdd(&t.hdr->appended, (unsigned long long)s_won);
-        atomicOr(&t.hdr->or_mask, s_or);
-        atomicAnd(&t.hdr->and_mask, s_and);
+        // the two masks settle after the first few blocks: an atomic only when this block still changes them
+        // (they move one way only, so a stale reading costs a redundant atomic, never a missing one)
+        if (s_or & ~__hip_atomic_load(&t.hdr->or_mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicOr(&t.hdr->or_mask, s_or);
+        if (~s_and & __hip_atomic_load(&t.hdr->and_mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicAnd(&t.hdr->and_mask, s_and);
         if (before + s_base + s_won > t.capacity || s_base + s_won > s.ncap) atomicOr(&t.hdr->overflow, 1ull);
     }
     __syncthreads();
 #pragma unroll
-    for (int q = 0; q < LDS_SLOTS / BLOCK; ++q) {
-        if (won[q] == EMPTY) continue;
-        const int64_t k = s_base + pos[q];
-        if (k < s.ncap && before + k < t.capacity) {
-            s.list_id[k] = won[q];
-            t.used[before + k] = won_slot[q];
+    for (int q = 0; q < IPT; ++q) {
+        if (won[q]) {
+            const int64_t k = s_base + pos[q];
+            if (k < s.ncap && before + k < t.capacity) {
+                s.list_id[k] = (unsigned long long)id[q];
+                t.used[before + k] = (uint32_t)h[q];
+            }
         }
+        if (grp[q] >= 0) s.slot_of[t0 + (int64_t)q * BLOCK] = ls[q] < 0 ? NONE : s_aux[ls[q]];
     }
-#pragma unroll
-    for (int q = 0; q < IPT; ++q)
-        if (ls[q] != -2) s.slot_of[t0 + (int64_t)q * BLOCK] = ls[q] < 0 ? NONE : s_aux[ls[q]];
 }
 
 // The bits in which the new ids differ, squeezed into a key that keeps their order: up to three runs
@@ -352,34 +417,31 @@ __device__ inline Codec make_codec(uint64_t or_mask, uint64_t and_mask) {
     Codec c;
     uint64_t diff = (or_mask ^ and_mask) & 0x7FFFFFFFFFFFFFFFull;
     int32_t width[4];
-    int n = 0;
-    for (; n < 4; ++n) {
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
         c.sh[n] = 0;
         c.mask[n] = 0;
         width[n] = 0;
-    }
-    n = 0;
-    while (diff != 0 && n < 4) {
-        const int top = 63 - __clzll((long long)diff);
-        int lo;
-        if (n < 3) {
-            // the run of ones that ends at `top`
-            const uint64_t below = ~diff & ((top == 63) ? ~0ull : ((2ull << top) - 1ull));   // zeros at or below top
-            lo = below == 0 ? 0 : 64 - __clzll((long long)below);                           // first zero below the run, + 1
-        } else {
-            lo = __ffsll((unsigned long long)diff) - 1;
+        if (diff != 0) {
+            const int top = 63 - __clzll((long long)diff);
+            int lo;
+            if (n < 3) {
+                // the run of ones that ends at `top`
+                const uint64_t below = ~diff & ((2ull << top) - 1ull);          // zeros at or below top
+                lo = below == 0 ? 0 : 64 - __clzll((long long)below);        // first zero below the run, + 1
+            } else {
+                lo = __ffsll((unsigned long long)diff) - 1;
+            }
+            const int w = top - lo + 1;
+            c.sh[n] = lo;
+            c.mask[n] = (1ull << w) - 1ull;      // w <= 63
+            width[n] = w;
+            diff &= (lo == 0) ? 0ull : ((1ull << lo) - 1ull);
         }
-        const int w = top - lo + 1;
-        c.sh[n] = lo;
-        c.mask[n] = w >= 64 ? ~0ull : ((1ull << w) - 1ull);
-        width[n] = w;
-        diff &= (lo == 0) ? 0ull : ((1ull << lo) - 1ull);
-        ++n;
     }
-    int nb = 0;
-    for (int r = 0; r < 4; ++r) nb += width[r];
-    c.nb = nb;
-    int acc = nb;
+    c.nb = width[0] + width[1] + width[2] + width[3];
+    int acc = c.nb;
+#pragma unroll
     for (int r = 0; r < 4; ++r) {
         acc -= width[r];
         c.dst[r] = acc;
@@ -402,6 +464,13 @@ __device__ __forceinline__ uint32_t bucket_of(const Codec& c, uint64_t id, uint3
     return (g << kb) | (uint32_t)top;
 }
 
+__device__ __forceinline__ uint32_t group_of(const Table& t, uint32_t slot, int grouped) {
+    if (!grouped) return 0;
+    const uint32_t g = t.vals[slot] - PENDING0;
+    return g < (uint32_t)MAXG ? g : 0;
+}
+
+// ---- atomic route -------------------------------------------------------------------------------
 __global__ __launch_bounds__(BLOCK) void hist_kernel(Table t, Scratch s, int reset, int grouped, int glog) {
     __shared__ Codec s_codec;
     if (threadIdx.x == 0) s_codec = make_codec(t.hdr->or_mask, t.hdr->and_mask);
@@ -410,68 +479,78 @@ __global__ __launch_bounds__(BLOCK) void hist_kernel(Table t, Scratch s, int res
     const int64_t before = ids_before(t, reset);
     const int64_t n = ids_added(t, s, before);
     for (int64_t k = (int64_t)blockIdx.x * BLOCK + threadIdx.x; k < n; k += (int64_t)gridDim.x * BLOCK) {
-        uint32_t g = 0;
-        if (grouped) {
-            g = t.vals[t.used[before + k]] - PENDING0;
-            if (g >= (uint32_t)MAXG) g = 0;
-        }
+        const uint32_t g = grouped ? group_of(t, t.used[before + k], 1) : 0;
         const uint32_t b = bucket_of(c, s.list_id[k], g, s.nb_log, glog);
         s.list_b[k] = b;
         atomicAdd(&s.cnt[b], 1u);
     }
 }
 
-// One block: exclusive prefix of the bucket sizes, cursors zeroed, oversized buckets listed.
+// One block: exclusive prefix of the bucket sizes, cursors zeroed, oversized buckets listed.  The counters
+// are read with coalesced loads, all of them in flight before the first is used, and pass through LDS
+// in chunks of CHUNK so that thread t can scan CHUNK / SCAN_BLOCK consecutive ones.
 __global__ __launch_bounds__(SCAN_BLOCK) void scan_kernel(Table t, Scratch s) {
     constexpr int NW = SCAN_BLOCK / WAVE;
-    __shared__ uint32_t s_w[NW];
-    __shared__ uint32_t s_carry;
+    constexpr int RUN = 8;                          // consecutive counters per thread and chunk
+    constexpr int CHUNK = SCAN_BLOCK * RUN;
+    constexpr int NCHUNK = (1 << NB_MAX_LOG) / CHUNK;
+    __shared__ uint32_t s_c[CHUNK];
+    __shared__ uint32_t s_w[2][NW];
     __shared__ uint32_t s_nbig;
     const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
-    const int64_t nb = 1ll << s.nb_log;
-    if (threadIdx.x == 0) {
-        s_carry = 0;
-        s_nbig = 0;
-    }
-    __syncthreads();
-    // rounds of 4 * SCAN_BLOCK counters: thread t owns 4 consecutive ones (one 16-byte load)
-    for (int64_t base = 0; base < nb; base += 4 * SCAN_BLOCK) {
-        const int64_t i0 = base + 4 * (int64_t)threadIdx.x;
-        uint32_t v[4] = {0, 0, 0, 0};
+    const int nb = 1 << s.nb_log;
+    if (threadIdx.x == 0) s_nbig = 0;
+    uint32_t v[NCHUNK][RUN];
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-            if (i0 + q < nb) v[q] = s.cnt[i0 + q];
-        const uint32_t sum = v[0] + v[1] + v[2] + v[3];
+    for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+        for (int j = 0; j < RUN; ++j) {
+            const int i = c * CHUNK + j * SCAN_BLOCK + threadIdx.x;
+            v[c][j] = (c * CHUNK < nb && i < nb) ? s.cnt[i] : 0;
+        }
+    uint32_t carry = 0;
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+        if (c * CHUNK >= nb) break;                 // uniform
+#pragma unroll
+        for (int j = 0; j < RUN; ++j) s_c[j * SCAN_BLOCK + threadIdx.x] = v[c][j];
+        __syncthreads();
+        uint32_t w[RUN];
+        uint32_t sum = 0;
+#pragma unroll
+        for (int j = 0; j < RUN; ++j) {
+            w[j] = s_c[threadIdx.x * RUN + j];
+            sum += w[j];
+        }
         uint32_t inc = sum;
         for (int d = 1; d < WAVE; d <<= 1) {
             const uint32_t y = __shfl_up(inc, d);
             if (lane >= d) inc += y;
         }
-        if (lane == WAVE - 1) s_w[wid] = inc;
+        if (lane == WAVE - 1) s_w[c & 1][wid] = inc;
         __syncthreads();
-        uint32_t woff = 0, round_total = 0;
+        uint32_t o = carry + inc - sum, chunk_total = 0;
 #pragma unroll
         for (int q = 0; q < NW; ++q) {
-            const uint32_t x = s_w[q];
-            if (q < wid) woff += x;
-            round_total += x;
+            const uint32_t x = s_w[c & 1][q];
+            if (q < wid) o += x;
+            chunk_total += x;
         }
-        uint32_t o = s_carry + woff + inc - sum;
+        carry += chunk_total;
+        const int i0 = c * CHUNK + threadIdx.x * RUN;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            if (i0 + q < nb) {
-                s.off[i0 + q] = o;
-                s.cnt[i0 + q] = 0;
-                if (v[q] > (uint32_t)SMALL_BUCKET) s.big[atomicAdd(&s_nbig, 1u)] = (uint32_t)(i0 + q);
-                o += v[q];
+        for (int j = 0; j < RUN; ++j) {
+            if (i0 + j < nb) {
+                s.off[i0 + j] = o;
+                s.cnt[i0 + j] = 0;
+                if (w[j] > (uint32_t)SMALL_BUCKET) s.big[atomicAdd(&s_nbig, 1u)] = (uint32_t)(i0 + j);
+                o += w[j];
             }
         }
-        __syncthreads();
-        if (threadIdx.x == 0) s_carry += round_total;
-        __syncthreads();
     }
+    __syncthreads();
     if (threadIdx.x == 0) {
-        s.off[nb] = s_carry;
+        s.off[nb] = carry;
         t.hdr->nbig = s_nbig;
     }
 }
@@ -488,10 +567,11 @@ __global__ __launch_bounds__(BLOCK) void scatter_kernel(Table t, Scratch s, int 
     }
 }
 
-// In-place ascending sort of ids[0..n) (all distinct) with their slots, by one block: a bitonic network
-// in which every comparator puts the smaller id at the lower index, so that the positions from n up to
-// the next power of two act as +infinity and their comparators are simply skipped.
-__device__ void block_sort(unsigned long long* ids, uint32_t* slots, int64_t n) {
+// In-place ascending sort of ids[0..n) (all distinct) with a companion array, by one block: a bitonic
+// network in which every comparator puts the smaller id at the lower index, so that the positions from n
+// up to the next power of two act as +infinity and their comparators are simply skipped.
+template <typename IdT, typename PayloadT>
+__device__ void block_sort(IdT* ids, PayloadT* payload, int64_t n) {
     int64_t p2 = 1;
     while (p2 < n) p2 <<= 1;
     for (int64_t k = 2; k <= p2; k <<= 1) {
@@ -507,13 +587,13 @@ __device__ void block_sort(unsigned long long* ids, uint32_t* slots, int64_t n) 
                     l = i + j;
                 }
                 if (l < n) {
-                    const unsigned long long x = ids[i], y = ids[l];
+                    const IdT x = ids[i], y = ids[l];
                     if (x > y) {
                         ids[i] = y;
                         ids[l] = x;
-                        const uint32_t sx = slots[i], sy = slots[l];
-                        slots[i] = sy;
-                        slots[l] = sx;
+                        const PayloadT sx = payload[i], sy = payload[l];
+                        payload[i] = sy;
+                        payload[l] = sx;
                     }
                 }
             }
@@ -551,6 +631,89 @@ __global__ __launch_bounds__(BLOCK) void number_kernel(Table t, Scratch s, int r
     }
 }
 
+// ---- radix route --------------------------------------------------------------------------------
+// sort key of the k-th new id: bucket << 40 | table slot (the sort only looks at the bucket); value: the id
+__global__ __launch_bounds__(BLOCK) void sortkey_kernel(Table t, Scratch s, int reset, int grouped, int glog, int64_t* n_out) {
+    __shared__ Codec s_codec;
+    if (threadIdx.x == 0) s_codec = make_codec(t.hdr->or_mask, t.hdr->and_mask);
+    __syncthreads();
+    const Codec c = s_codec;
+    const int64_t before = ids_before(t, reset);
+    const int64_t n = ids_added(t, s, before);
+    if (blockIdx.x == 0 && threadIdx.x == 0) *n_out = n;      // the sort's live length
+    for (int64_t k = (int64_t)blockIdx.x * BLOCK + threadIdx.x; k < n; k += (int64_t)gridDim.x * BLOCK) {
+        const uint32_t slot = t.used[before + k];
+        const uint32_t b = bucket_of(c, s.list_id[k], group_of(t, slot, grouped), SORT_KEY_LOG, glog);
+        s.key_a[k] = ((uint64_t)b << SORT_KEY_SHIFT) | slot;
+    }
+}
+
+// keys/ids: the new ids ordered by bucket.  A bucket is a run of equal keys >> 40; a thread finds the ends of
+// its run by walking (runs hold tens of ids), counting the smaller ids on the way.  A run longer than
+// SMALL_BUCKET is left to sorted_runs_kernel: its first place is listed by the thread that stands there.
+__global__ __launch_bounds__(BLOCK) void rank_kernel(Table t, Scratch s, const uint64_t* __restrict__ keys,
+                                                     const int64_t* __restrict__ ids, int reset,
+                                                     int64_t* __restrict__ unique_out, int64_t unique_capacity) {
+    const int64_t before = ids_before(t, reset);
+    const int64_t n = ids_added(t, s, before);
+    for (int64_t p = (int64_t)blockIdx.x * BLOCK + threadIdx.x; p < n; p += (int64_t)gridDim.x * BLOCK) {
+        const uint64_t key = keys[p];
+        const uint64_t top = key >> SORT_KEY_SHIFT;
+        const int64_t id = ids[p];
+        int64_t smaller = 0, left = 0, right = 0;
+        bool open = false;
+        for (int64_t q = p - 1;; --q) {               // to the left
+            if (q < 0 || (keys[q] >> SORT_KEY_SHIFT) != top) break;
+            if (++left > SMALL_BUCKET) { open = true; break; }
+            smaller += ids[q] < id ? 1 : 0;
+        }
+        for (int64_t q = p + 1; !open; ++q) {         // to the right
+            if (q >= n || (keys[q] >> SORT_KEY_SHIFT) != top) break;
+            if (++right > SMALL_BUCKET) { open = true; break; }
+            smaller += ids[q] < id ? 1 : 0;
+        }
+        if (open || left + right + 1 > SMALL_BUCKET) {
+            if (left == 0) s.big[atomicAdd(&t.hdr->nbig, 1ull)] = (uint32_t)p;
+            continue;
+        }
+        const int64_t local = before + (p - left) + smaller;
+        if (local < unique_capacity) unique_out[local] = id;
+        t.vals[(uint32_t)key] = (uint32_t)local;
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void sorted_runs_kernel(Table t, Scratch s, uint64_t* keys, int64_t* ids, int reset,
+                                                            int64_t* __restrict__ unique_out, int64_t unique_capacity) {
+    __shared__ int64_t s_end;
+    const int64_t before = ids_before(t, reset);
+    const int64_t n = ids_added(t, s, before);
+    const int64_t nbig = (int64_t)t.hdr->nbig;
+    for (int64_t q = blockIdx.x; q < nbig; q += gridDim.x) {
+        const int64_t lo = s.big[q];
+        const uint64_t top = keys[lo] >> SORT_KEY_SHIFT;
+        // the run's end: the first place from lo on whose bucket differs
+        if (threadIdx.x == 0) s_end = n;
+        __syncthreads();
+        for (int64_t base = lo; base < n; base += BLOCK) {
+            const int64_t x = base + threadIdx.x;
+            if (x < n && (keys[x] >> SORT_KEY_SHIFT) != top) atomicMin(reinterpret_cast<unsigned long long*>(&s_end), (unsigned long long)x);
+            __syncthreads();
+            const int64_t e = s_end;
+            __syncthreads();              // (nobody writes s_end again before everybody has read it)
+            if (e < n) break;
+        }
+        const int64_t len = s_end - lo;
+        __syncthreads();
+        block_sort(ids + lo, keys + lo, len);
+        for (int64_t j = threadIdx.x; j < len; j += BLOCK) {
+            const int64_t local = before + lo + j;
+            if (local < unique_capacity) unique_out[local] = ids[lo + j];
+            t.vals[(uint32_t)keys[lo + j]] = (uint32_t)local;
+        }
+        __syncthreads();
+    }
+}
+
 __global__ __launch_bounds__(BLOCK) void lookup_kernel(Arrays a, Table t, Scratch s, int reset, int64_t* U_dev) {
     const int64_t i0 = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
     // the call's totals, committed by one thread: no other thread of this launch reads the header
@@ -581,9 +744,12 @@ __global__ __launch_bounds__(BLOCK) void lookup_kernel(Arrays a, Table t, Scratc
 }
 
 int32_t check_capacity(int64_t capacity) {
-    if (capacity < 0 || capacity > MAX_CAPACITY) return fail(SGL_EINVAL, "hashed remap state: capacity %lld outside [0, %lld]", (long long)capacity, (long long)MAX_CAPACITY);
+    if (capacity < 0 || capacity > MAX_CAPACITY)
+        return fail(SGL_EINVAL, "hashed remap state: capacity %lld outside [0, %lld]", (long long)capacity, (long long)MAX_CAPACITY);
     return SGL_OK;
 }
+
+using InsertKernel = void (*)(Arrays, Table, Scratch, int, int);
 
 int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const int64_t* const* ids, const int64_t* len_max,
             const int64_t* const* len_dev, int64_t* const* local_out, int64_t* unique_out, int64_t unique_capacity,
@@ -603,6 +769,7 @@ int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const i
     if (total > MAX_CAPACITY) return fail(SGL_ENOTSUP, "unique_compact: too many ids");
     const int64_t ncap = total < t.capacity ? total : t.capacity;
     const Scratch s = carve_scratch(ar, total, ncap);
+    int64_t* n_sort = ar.take<int64_t>(1);
     if (!ar.ok()) return fail(SGL_ENOMEM, "unique_compact: workspace too small");
     const int grouped = (mode == SGL_UNIQUE_GROUPED && G > 1) ? 1 : 0;
     int glog = 0;
@@ -612,20 +779,42 @@ int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const i
         int64_t b = ceil_div<int64_t>(work > 0 ? work : 1, per_block);
         return dim3((unsigned)(b > MAX_GRID ? MAX_GRID : b));
     };
-    const int64_t clear_work = (fresh || reset) ? t.slots : (1ll << s.nb_log);
+    const int64_t clear_work = (fresh || reset) ? t.slots : (s.radix ? 1 : (1ll << s.nb_log));
     hipLaunchKernelGGL(prep_kernel, grid(clear_work, 4 * BLOCK), dim3(BLOCK), 0, st, t, s, fresh ? 1 : 0, reset);
     SGL_LAUNCH_CHECK();
     if (total > 0) {
-        hipLaunchKernelGGL(insert_kernel, dim3((unsigned)ceil_div<int64_t>(total, TILE)), dim3(BLOCK), 0, st, all, t, s, reset, grouped);
+        // tile of the insert: 1024 ids per block (larger tiles fold more repeats before the table is touched but
+        // leave fewer waves per compute unit to hide the table's latency: 2048 ids per block is 10 % slower
+        // on 15.6M ids); small calls take smaller tiles so that the chip still has a few hundred blocks
+        int ipt = 4;
+        while (ipt > 1 && total / (BLOCK * ipt) < 256) ipt >>= 1;
+        const InsertKernel ins = ipt == 4 ? insert_kernel<4> : ipt == 2 ? insert_kernel<2> : insert_kernel<1>;
+        hipLaunchKernelGGL(ins, dim3((unsigned)ceil_div<int64_t>(total, BLOCK * ipt)), dim3(BLOCK), 0, st, all, t, s, reset, grouped);
         SGL_LAUNCH_CHECK();
-        hipLaunchKernelGGL(hist_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, grouped, glog);
-        SGL_LAUNCH_CHECK();
-        hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, t, s);
-        SGL_LAUNCH_CHECK();
-        hipLaunchKernelGGL(scatter_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset);
-        SGL_LAUNCH_CHECK();
-        hipLaunchKernelGGL(number_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, unique_out, unique_capacity);
-        SGL_LAUNCH_CHECK();
+        if (!s.radix) {
+            hipLaunchKernelGGL(hist_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, grouped, glog);
+            SGL_LAUNCH_CHECK();
+            hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, t, s);
+            SGL_LAUNCH_CHECK();
+            hipLaunchKernelGGL(scatter_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset);
+            SGL_LAUNCH_CHECK();
+            hipLaunchKernelGGL(number_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, unique_out, unique_capacity);
+            SGL_LAUNCH_CHECK();
+        } else {
+            hipLaunchKernelGGL(sortkey_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, grouped, glog, n_sort);
+            SGL_LAUNCH_CHECK();
+            int in_b = 0;
+            int64_t* id_a = reinterpret_cast<int64_t*>(s.list_id);
+            const int32_t rc = radix_sort_pairs(s.key_a, id_a, s.key_b, s.id_b, ncap, n_sort, SORT_KEY_SHIFT, 64, &in_b, s.sort_ws,
+                                                s.sort_ws_bytes, st);
+            if (rc != SGL_OK) return rc;
+            uint64_t* keys = in_b ? s.key_b : s.key_a;
+            int64_t* sorted_ids = in_b ? s.id_b : id_a;
+            hipLaunchKernelGGL(rank_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, keys, sorted_ids, reset, unique_out, unique_capacity);
+            SGL_LAUNCH_CHECK();
+            hipLaunchKernelGGL(sorted_runs_kernel, dim3(256), dim3(BLOCK), 0, st, t, s, keys, sorted_ids, reset, unique_out, unique_capacity);
+            SGL_LAUNCH_CHECK();
+        }
     }
     hipLaunchKernelGGL(lookup_kernel, grid(total, BLOCK), dim3(BLOCK), 0, st, all, t, s, reset, U_dev);
     SGL_LAUNCH_CHECK();
@@ -670,8 +859,9 @@ extern "C" size_t sgl_remap_hashed_state_bytes(int64_t capacity) {
 extern "C" int32_t sgl_remap_hashed_init(void* state, size_t bytes, int64_t capacity, void* stream) {
     int32_t rc;
     if ((rc = check_capacity(capacity)) != SGL_OK) return rc;
-    if (!state || bytes < state_bytes(capacity)) return fail(SGL_EINVAL, "remap_hashed_init: state is NULL or smaller than %zu bytes", state_bytes(capacity));
     if (capacity < 1) return fail(SGL_EINVAL, "remap_hashed_init: capacity < 1");
+    if (!state || bytes < state_bytes(capacity))
+        return fail(SGL_EINVAL, "remap_hashed_init: state is NULL or smaller than %zu bytes", state_bytes(capacity));
     Table t = carve(state, capacity);
     int64_t b = ceil_div<int64_t>(t.slots, 4 * BLOCK);
     if (b > MAX_GRID) b = MAX_GRID;

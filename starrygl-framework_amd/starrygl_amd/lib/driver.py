@@ -182,14 +182,19 @@ class HotPath:
         g.view.hop_hint = self.be.ptr(hint)
         return g
 
-    def window_end(self, g, node, t):
+    def window_end(self, g, node, t, out=None):
         """out[i] = position in row node[i] of the first edge with timestamp >= t[i] (-1 for a node
         outside [0,n)): where the strictly-before window of the slot (node[i], t[i]) ends.  A loader
         computes it once for the events it will train on and passes a batch's values as `root_hint`."""
         self._chk("i64", node=node, t=t)
         if node.shape[0] != t.shape[0]:
             raise ValueError("window_end: node and t differ in length")
-        out = self.be.empty(int(node.shape[0]))
+        if out is None:
+            out = self.be.empty(int(node.shape[0]))
+        else:
+            self._chk("i64", out=out)
+            if out.shape[0] < node.shape[0]:
+                raise ValueError("window_end: out is shorter than node")
         self._ck(self.lib.window_end(C.byref(g.view), self.be.ptr(node), self.be.ptr(t), int(node.shape[0]),
                                      self.be.ptr(out), self.be.stream()))
         return out

@@ -170,6 +170,39 @@ def test_hashed_state_oversized_buckets_are_sorted_in_place(oracle, hot):
     assert th == u.shape[0] and np.array_equal(np_of(uh), u) and np.array_equal(np_of(lh[0]), inv)
 
 
+@pytest.mark.parametrize("mode", [_abi.UNIQUE_SORTED, _abi.UNIQUE_GROUPED])
+@pytest.mark.parametrize("kind", ["encoded", "wide", "crowded"])
+def test_hash_path_of_large_calls_orders_by_radix_passes(oracle, hot, mode, kind):
+    """Calls that may add more than 2^20 ids order the new ids with two radix passes on the top bits of the
+    squeezed key and rank inside the runs; 'crowded' puts thousands of ids into one run (block-wide sort)."""
+    rng = np.random.default_rng(77)
+    sizes = (300_000, 900_000, 1_200_000)
+    if kind == "encoded":
+        pool = _encode(rng, 8, 2_000_000, 900_000)
+    elif kind == "wide":
+        pool = rng.integers(0, 2**62, 900_000)
+    else:
+        pool = np.concatenate([rng.integers(0, 40_000, 500_000), rng.integers(0, 2**62, 2000),
+                               rng.integers(2**61, 2**61 + 50_000, 400_000)])
+    arrs = [pool[rng.integers(0, pool.shape[0], s)].astype(np.int64) for s in sizes]
+    arrs[1][::11] = -1
+    so, sh = oracle.remap_hashed_state(2_500_000), hot.remap_hashed_state(2_500_000)
+    for c, reset in enumerate((True, False)):
+        if c == 1:
+            arrs = [np.where(rng.random(a.shape[0]) < 0.5, a, a + 1) for a in arrs]
+            arrs = [np.where(a == 0, -1, a) for a in arrs]
+        lo, uo, (to_, bo) = oracle.unique_compact([a.copy() for a in arrs], mode, so, reset)
+        lh, uh, (th, bh) = hot.unique_compact([to_dev(hot, a) for a in arrs], mode, sh, reset)
+        assert (th, bh) == (to_, bo), f"call {c}"
+        assert np.array_equal(np_of(uh)[bh:th], uo[bo:to_]), f"call {c}: unique list differs"
+        for g in range(len(arrs)):
+            assert np.array_equal(np_of(lh[g]), lo[g]), f"call {c} array {g}: local ids differ"
+    # the one-shot call takes the same route
+    lh, uh, (th, _) = hot.unique_compact([to_dev(hot, a) for a in arrs], mode, None, True)
+    lo, uo, (to_, _) = oracle.unique_compact([a.copy() for a in arrs], mode, None, True)
+    assert th == to_ and np.array_equal(np_of(uh), uo) and all(np.array_equal(np_of(a), b) for a, b in zip(lh, lo))
+
+
 def test_hashed_state_reports_an_outgrown_capacity(hot):
     sh = hot.remap_hashed_state(1000)
     a = to_dev(hot, np.arange(900, dtype=np.int64) * 7)
@@ -183,12 +216,13 @@ def test_hashed_state_reports_an_outgrown_capacity(hot):
     assert th == 900 and np.array_equal(np_of(lh[0]), np.arange(900))
 
 
-def test_hash_unique_is_captured_and_replayed_in_a_hip_graph(oracle, hot):
+@pytest.mark.parametrize("n", [30_000, 1_300_000])
+def test_hash_unique_is_captured_and_replayed_in_a_hip_graph(oracle, hot, n):
     """The hash-set path is a fixed launch sequence without host synchronisation: captured once, replayed
-    over new ids of varying live length, with eager work and synchronisations between the replays."""
+    over new ids of varying live length, with eager work and synchronisations between the replays (the
+    larger size takes the radix route)."""
     import torch
     rng = np.random.default_rng(3)
-    n = 30_000
     ids = torch.zeros(n, dtype=torch.int64, device="cuda")
     live = torch.zeros(1, dtype=torch.int64, device="cuda")
     out, uniq, U = torch.empty_like(ids), torch.empty(n, dtype=torch.int64, device="cuda"), torch.zeros(2, dtype=torch.int64, device="cuda")
@@ -208,7 +242,7 @@ def test_hash_unique_is_captured_and_replayed_in_a_hip_graph(oracle, hot):
     with torch.cuda.graph(g, stream=stream):
         call(state)
     for rep, m in enumerate((n, 17, 12_345, 0, n)):
-        a = _encode(rng, 4, 9000, n).astype(np.int64)
+        a = _encode(rng, 4, n // 3, n).astype(np.int64)
         ids.copy_(torch.from_numpy(a))
         live.fill_(m)
         torch.cuda.synchronize()

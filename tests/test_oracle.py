@@ -7,7 +7,7 @@ from scipy import stats as sps
 
 from starrygl_amd.lib import _abi
 from starrygl_amd.utils import synth
-from util import host_graph
+from util import assert_hop_equal, host_graph
 
 E = np.zeros(0, np.int64)
 
@@ -367,3 +367,26 @@ def test_window_end_is_searchsorted_and_root_hints_are_checked(oracle):
         oracle.sample_khop(g, roots, ts_ptr, root_ts, none, none, 2, oracle.with_root_hint(p, bad))
     with pytest.raises(ValueError):
         oracle.sample_khop(g, roots, ts_ptr, root_ts, none, none, 2, oracle.with_root_hint(p, hint[:50].copy()))
+
+
+@pytest.mark.parametrize("strategy", ["recent", "uniform"])
+def test_indexed_cpu_sampler_equals_the_searching_oracle(oracle, oracle_cdll, strategy):
+    """sglo_sample_khop_indexed (the CPU side of the benchmark's equal-work timing: window ends from the root
+    hints and the next-hop index instead of searches) returns what the searching oracle returns."""
+    from oracle import oracle as O
+    rng = np.random.default_rng(21)
+    n, m = 300, 20_000
+    src, dst, ts = rng.integers(0, n, m), rng.integers(0, n, m), rng.integers(0, 500, m)
+    g = host_graph(oracle, n, src, dst, ts)
+    oracle.build_hop_hint(g)
+    roots, root_ts = rng.integers(0, n, 200).astype(np.int64), rng.integers(0, 520, 200).astype(np.int64)
+    neg, neg_ts = rng.integers(0, n, 70).astype(np.int64), rng.integers(0, 520, 70).astype(np.int64)
+    ts_ptr = np.arange(201, dtype=np.int64)
+    for kw in ({}, {"allowed_offset": 60}, {"keep_root_time": True}, {"equal_root_time": True}):
+        p = oracle.params(strategy, 5, seed=4, **kw)
+        want = oracle.sample_khop(g, roots, ts_ptr, root_ts, neg, neg_ts, 3, p)
+        hint = oracle.window_end(g, roots, root_ts)
+        hint[::4] = -1
+        got = O.sample_khop_indexed(oracle, oracle_cdll, g, roots, ts_ptr, root_ts, neg, neg_ts, 3, oracle.with_root_hint(p, hint))
+        for a, b in zip(want.hops, got.hops):
+            assert_hop_equal(b, a, f"{strategy} {kw}")
