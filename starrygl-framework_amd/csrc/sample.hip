@@ -243,7 +243,7 @@ __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
             // the slot is (destination, time) of an edge whose index entry says where the window ends;
             // an entry of -1 belongs to a destination outside [0,n), which is a bad slot anyway
             const int64_t h = active ? a.slot_hint[slot] : 0;
-            hi = h >= rs ? h : rs;
+            hi = clamp_to_row(h, rs, re);     // an index that does not belong to this graph cannot lead outside the row
         } else {
             // positive roots whose window end the caller knows are not searched
             const bool told = active && rh >= 0;
@@ -836,8 +836,8 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
             // no search (strictly-before windows only; a uniform call that keeps the root's time asks
             // about another time and searches)
             const bool hinted = hint >= 0 && eq == 0 && t2 == ets;
-            const int64_t rs2 = a.row_ptr[nbr];
-            const int64_t hi2 = hinted ? hint : lane_lower_bound(a.ts, rs2, a.row_ptr[nbr + 1], t2 + eq);
+            const int64_t rs2 = a.row_ptr[nbr], re2 = a.row_ptr[nbr + 1];
+            const int64_t hi2 = hinted ? clamp_to_row(hint, rs2, re2) : lane_lower_bound(a.ts, rs2, re2, t2 + eq);
             int64_t lo2 = rs2;
             if (a.allowed_offset >= 0) lo2 = lane_lower_bound(a.ts, rs2, hi2, t2 - a.allowed_offset);
             len2 = hi2 - lo2;

@@ -99,10 +99,14 @@ class DistNodeState:
         self._hp.gather(self._c_ts, ids, out_ts)
         return out, out_ts
 
-    def update(self, gids: Tensor, values: Tensor, ts: Optional[Tensor] = None):
+    def update(self, gids: Tensor, values: Tensor, ts: Optional[Tensor] = None, check_unique: bool = False):
         """Overwrite the rows of the given ids (ids not stored here are skipped).
-        Ids must be unique within one call."""
+        Ids must be unique within one call: with a repeated id the row that wins is unspecified (the
+        reference's index_put keeps the last one); check_unique=True verifies it (one host synchronisation).
+        Rows of the HBM tier are written there only: `.data` / `.ts` show them after flush()."""
         ids = self._keys(gids)
+        if check_unique and torch.unique(ids).numel() != ids.numel():
+            raise ValueError("DistNodeState.update: ids repeat within one call")
         vals = values.to(self.gpu, torch.float32).contiguous()
         hot_rw = self.hot_data if self.hot_data is not None else (self.data if self.device.type == "cuda" else None)
         cold_rw = self.data if self.device.type == "cpu" else None
@@ -115,12 +119,24 @@ class DistNodeState:
         if self.device.type == "cpu":
             torch.cuda.current_stream(self.gpu).synchronize()   # host-visible before the caller reads .data
 
+    def flush(self):
+        """Fold the rows of the HBM tier back into `.data` / `.ts` (the tensors of the reference's layout, which
+        callers read and checkpoint): until then those tensors hold the hot rows as of the last flush."""
+        if self.hot_data is not None:
+            torch.cuda.current_stream(self.gpu).synchronize()
+            self.data[self._hot_ids] = self.hot_data.cpu()
+            self.ts[self._hot_ids] = self.hot_ts.cpu()
+        return self
+
+    def state_dict(self):
+        """{'data', 'ts'} with the HBM tier folded in."""
+        self.flush()
+        return {"data": self.data, "ts": self.ts}
+
     def to(self, device: Union[str, torch.device]):
         new_device = torch.device(device)
         if new_device != self.device:
-            if self.hot_data is not None:    # fold the HBM tier back before moving
-                self.data[self._hot_ids] = self.hot_data.cpu()
-                self.ts[self._hot_ids] = self.hot_ts.cpu()
+            self.flush()                     # fold the HBM tier back before moving
             self.data, self.ts = self.data.to(new_device), self.ts.to(new_device)
             if new_device.type == "cpu":
                 self.data, self.ts = self.data.pin_memory(), self.ts.pin_memory()

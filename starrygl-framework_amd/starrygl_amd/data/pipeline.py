@@ -153,8 +153,10 @@ class MiniBatchPipeline:
             dim = int(self.te[0].numel())
             self.te_out = [torch.empty((caps[l + 1], dim), dtype=f32, device=self.dev) for l in range(self.layers)]
         self._views = {}
-        hp._workspace(hp.lib.unique_workspace_bytes(graph._n, 1 + self.layers,
-                                                    (_abi.i64 * (1 + self.layers))(*caps)))
+        # the unique stage's scratch belongs to this pipeline: its pointer is baked into the pipeline's HIP
+        # graph, and graphs of different pipelines replay side by side on different streams
+        self.uws = be.empty(max(int(hp.lib.unique_workspace_bytes(graph._n, 1 + self.layers,
+                                                                  (_abi.i64 * (1 + self.layers))(*caps))), 256), "u8")
         self.use_graph, self._graph = use_graph, None
         self._plans, self._slow = None, []
         self.stream = stream
@@ -178,7 +180,7 @@ class MiniBatchPipeline:
         arrays = [kr.slot_node0] + [h.neighbors for h in kr.hops]
         lens = [self.S0_dev] + [h.counts[1:2] for h in kr.hops]
         hp.unique_compact(arrays, _abi.UNIQUE_SORTED, self.state, True, lens_dev=lens, out_arrays=self.local,
-                          finalize=False, unique_out=self.ubuf, U_out=self.U, premarked=True)
+                          finalize=False, unique_out=self.ubuf, U_out=self.U, premarked=True, workspace=self.uws)
         if self._plans is None:      # every gather of the batch in as few launches as possible
             segs = [(c, self.ubuf, self.node_out[name], self.node_ts_out.get(name), self.U[0:1])
                     for name, c in self.node_tables.items()]

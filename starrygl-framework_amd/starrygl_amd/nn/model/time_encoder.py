@@ -20,20 +20,25 @@ class _TimeEncode(torch.autograd.Function):
             dt, code = t.reshape(-1).float().contiguous(), _abi.DT_F32
         w = weight.detach().reshape(-1).contiguous()
         b = bias.detach().contiguous()
-        out = hp.time_encode(dt.to(weight.device), w, b, dt_dtype=code)
+        dt = dt.to(weight.device)          # the copy the kernel read is the one backward multiplies with
+        out = hp.time_encode(dt, w, b, dt_dtype=code)
         ctx.save_for_backward(dt, weight, bias)
+        ctx.t_shape, ctx.t_device, ctx.t_dtype = t.shape, t.device, t.dtype
         return out
 
     @staticmethod
     def backward(ctx, grad):
-        # d cos(a)/da = -sin(a), a = w * x + b; only w and b carry gradients
+        # d cos(a)/da = -sin(a), a = w * x + b
         dt, weight, bias = ctx.saved_tensors
         x = dt.float().reshape(-1, 1)
         a = x * weight.reshape(1, -1) + bias.reshape(1, -1)
         g = -torch.sin(a) * grad
         gw = (g * x).sum(0).reshape(weight.shape) if ctx.needs_input_grad[1] else None
         gb = g.sum(0) if ctx.needs_input_grad[2] else None
-        return None, gw, gb
+        gt = None
+        if ctx.needs_input_grad[0]:        # a floating-point t: d/dt cos(w t + b) summed over the frequencies
+            gt = (g * weight.reshape(1, -1)).sum(1).reshape(ctx.t_shape).to(device=ctx.t_device, dtype=ctx.t_dtype)
+        return gt, gw, gb
 
 
 class TimeEncoder(nn.Module):

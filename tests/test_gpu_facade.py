@@ -237,6 +237,11 @@ def test_dist_node_state(mode, tiered):
         d, tt = ns[absent]
         assert not d.any() and not tt.any()
         ns.update(absent, torch.ones(7, dim).cuda())
+    # the tensors of the reference's layout show the rows of the HBM tier after a flush (state_dict flushes)
+    sd = ns.state_dict()
+    assert torch.equal(sd["data"], ref_data) and torch.equal(sd["ts"], ref_ts)
+    with pytest.raises(ValueError, match="repeat"):
+        ns.update(q[:1].repeat(2), torch.ones(2, dim).cuda(), check_unique=True)
     ns.to("cuda:0")
     d, tt = ns[q]
     assert torch.equal(d.cpu(), ref_data[q_loc]) and torch.equal(tt.cpu(), ref_ts[q_loc])

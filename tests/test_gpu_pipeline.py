@@ -90,6 +90,37 @@ def test_pipeline_pool_keeps_batches_in_flight(oracle, hot):
                 assert np.array_equal(np_of(mb.hops[l]["neighbors_eid"]), h.neighbors_eid)
 
 
+def test_pipeline_pool_with_staggered_run_counts(oracle, hot):
+    """Rounds of one or two batches on a pool of three: the pipelines' replay counts drift apart (r+1, r, r),
+    so that graphs of different pipelines which shared any scratch - the unique stage's epoch stamp, its tile
+    sums - would hand each other stale values.  Every batch must still equal the oracle's result."""
+    from starrygl_amd.data import MiniBatchPipelinePool
+    from starrygl_amd.lib.libstarrygl_comm import from_edge_index
+    n, m, B = 6000, 120_000, 400
+    src, dst, ts, eid = synth.graph_stream(n, m, 1.15, 500_000, 41)
+    hg = host_graph(oracle, n, src, dst, ts, eid)
+    g = from_edge_index(n, 1, *(torch.from_numpy(x) for x in (src, dst, ts, eid)))
+    rng = np.random.default_rng(6)
+    pool = MiniBatchPipelinePool(3, g, 2 * B, B, 2, 5, "recent")
+    assert len({p.uws.data_ptr() for p in pool.pipes}) == 3          # a scratch buffer per pipeline
+    lo = 5000
+    for rnd, burst in enumerate([1, 2, 2, 1, 1, 2, 1, 2, 2, 1, 1, 1, 2]):
+        batches = []
+        for _ in range(burst):
+            batches.append(synth.link_batch(src, dst, ts, lo, lo + B, n, B, rng))
+            lo += 4321
+        inflight = [pool.run(to_dev(hot, b[0]), to_dev(hot, b[2]), to_dev(hot, b[3]), to_dev(hot, b[4])) for b in batches]
+        for b, mb in zip(batches, inflight):
+            mb.finalize()
+            want = oracle.sample_khop(hg, *b, 2, oracle.params("recent", 5))
+            arrays = [want.slot_node0] + [h.neighbors for h in want.hops]
+            loc, uniq, _ = oracle.unique_compact(arrays, _abi.UNIQUE_SORTED, None, True)
+            assert np.array_equal(np_of(mb.nid_mapper), uniq), f"round {rnd}"
+            assert np.array_equal(np_of(mb.slot_local), loc[0]), f"round {rnd}"
+            for l in range(2):
+                assert np.array_equal(np_of(mb.hops[l]["neighbors_local"]), loc[1 + l]), f"round {rnd} hop {l}"
+
+
 @pytest.mark.parametrize("sample_type", ["recent", "uniform"])
 def test_pipeline_with_root_hints(oracle, hot, sample_type):
     """A pool whose batches carry the window ends of their positive roots (looked up once for the whole

@@ -59,3 +59,26 @@ def test_time_encode_is_within_one_ulp_everywhere(oracle, hot):
     err = np.abs(got.astype(np.float64) - want.astype(np.float64))
     assert err.max() <= 1.2e-7, err.max()
     assert (got == want).mean() > 0.99
+
+
+def test_time_encoder_module_backward_with_host_and_float_inputs(hot):
+    """The module's gradients equal autograd's over cos(Linear(t)) (starrygl/nn/model/time_encoder.py:29-31):
+    for an int64 t kept on the host (the kernel reads a device copy, backward must use that copy) and for a
+    floating-point t that asks for its own gradient."""
+    import torch
+    from starrygl_amd.nn.model.time_encoder import TimeEncoder
+    torch.manual_seed(0)
+    enc = TimeEncoder(16).cuda()
+    t_host = torch.randint(0, 1000, (50,))
+    enc(t_host).sum().backward()                     # a host tensor: no device mismatch in backward
+    gw = enc.w.weight.grad.clone()
+    ref = torch.nn.Linear(1, 16).cuda()
+    ref.load_state_dict(enc.w.state_dict())
+    torch.cos(ref(t_host.cuda().float().reshape(-1, 1))).sum().backward()
+    assert torch.allclose(gw, ref.weight.grad, rtol=1e-4, atol=1e-3)
+    t = (torch.rand(40, device="cuda") * 100).requires_grad_()
+    t2 = t.detach().clone().requires_grad_()
+    g = torch.randn(40, 16, device="cuda")
+    (enc(t) * g).sum().backward()
+    (torch.cos(ref(t2.reshape(-1, 1))) * g).sum().backward()
+    assert t.grad is not None and torch.allclose(t.grad, t2.grad, rtol=1e-4, atol=1e-4)
