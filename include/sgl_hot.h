@@ -82,7 +82,19 @@ typedef struct sgl_tcsr {
      * slot (col[e], ts[e]) ends.  With it the sampler needs no search for the
      * slots of hops >= 1 (strictly-before windows, slot time = edge time). */
     const int64_t* hop_hint;/* [m]   device, or NULL            */
+    /* Optional (NULL = absent) interleaved copy of the edge arrays, filled by
+     * sgl_tcsr_records_build: rec[4*e .. 4*e+3] = {col[e], ts[e], eid[e],
+     * hop_hint[e] (-1 without the index)}, 32 bytes per edge.  The uniform
+     * strategy picks edges scattered over a window: from the separate arrays
+     * every pick costs one memory sector per array, from the records one per
+     * pick.  Searches always run on `ts`; results do not depend on it. */
+    const int64_t* rec;     /* [4*m] device, 32-byte aligned, or NULL */
 } sgl_tcsr;
+
+/* Fill rec[0 .. 4*m) for the T-CSR `g` (whose own rec field is ignored; its
+ * hop_hint field, when set, is copied into the records).  No counterpart in
+ * the reference. */
+int32_t sgl_tcsr_records_build(const sgl_tcsr* g, int64_t* rec, void* stream);
 
 /* Fill hop_hint[0..m) for the T-CSR `g` (whose own hop_hint field is ignored):
  * one lower-bound search per edge, done once per graph.  -1 for an edge whose
@@ -124,9 +136,11 @@ int32_t sgl_tcsr_validate(const sgl_tcsr* g, void* workspace,
 #define SGL_SAMPLE_RECENT  0 /* "recent"  : the last min(k,cnt) window edges  */
 #define SGL_SAMPLE_UNIFORM 1 /* "uniform" : k distinct window edges, uniform  */
 
-/* Largest fanout the uniform strategy accepts (one wavefront holds one slot's
- * draws).  The recent strategy has no limit. */
-#define SGL_UNIFORM_MAX_FANOUT 64
+/* Largest fanout the uniform strategy accepts (a slot's picks are kept in the
+ * registers of one wavefront up to 64, in its block's LDS beyond).  The recent
+ * strategy has no limit; the reference has none for either
+ * (uniform_sample_single_hop_kernel, sample.cu.hpp:783-827). */
+#define SGL_UNIFORM_MAX_FANOUT 1024
 
 /* Arguments of Graph::sample_src_in_chunks_khop (sample.cu.hpp:1532-1534,
  * export.cu:194-201).  Candidate window of a slot (v, t):

@@ -179,6 +179,19 @@ int32_t sglo_tcsr_hop_hint_build(const sgl_tcsr* g, int64_t* hop_hint, void* str
     return SGL_OK;
 }
 
+/* The interleaved records are an accelerator of the kernels as well: the oracle samples from the
+ * separate arrays and only restates the layout so that the built array can be checked. */
+int32_t sglo_tcsr_records_build(const sgl_tcsr* g, int64_t* rec, void* stream) {
+    (void)stream;
+    if (!g || g->n < 0 || g->m < 0) return fail(SGL_EINVAL, "tcsr_records_build: null");
+    if (g->m > 0 && (!g->col || !g->ts || !g->eid || !rec)) return fail(SGL_EINVAL, "tcsr_records_build: null array");
+    for (int64_t e = 0; e < g->m; ++e) {
+        rec[4 * e] = g->col[e]; rec[4 * e + 1] = g->ts[e]; rec[4 * e + 2] = g->eid[e];
+        rec[4 * e + 3] = g->hop_hint ? g->hop_hint[e] : -1;
+    }
+    return SGL_OK;
+}
+
 /* Where the strictly-before window of (node[i], t[i]) ends: the upper end of
  * find_time_range (sample.cu.hpp:264-295) for a batch of slots. */
 int32_t sglo_window_end(const sgl_tcsr* g, const int64_t* node, const int64_t* t, int64_t N, int64_t* out,
@@ -346,7 +359,7 @@ static int32_t hop_impl(const sgl_tcsr* g, const int64_t* slot_node,
                 if (hint_out) hint_out[off + j] = g->hop_hint[e];
             }
         } else {
-            int64_t sel[SGL_UNIFORM_MAX_FANOUT];
+            int64_t sel[SGL_UNIFORM_MAX_FANOUT];      /* 8 KB of stack per thread */
             if (p->replace) {
                 for (int32_t j = 0; j < k; ++j)
                     sel[j] = bounded(draw_bits(p->seed, p->hop, s, j), len);

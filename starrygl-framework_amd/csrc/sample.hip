@@ -49,6 +49,7 @@ struct HopArgs {
     const int64_t* ts;
     const int64_t* eid;
     const int64_t* hint; // next-hop index of the graph (sgl_tcsr.hop_hint), or nullptr
+    const int64_t* rec;  // interleaved edge records of the graph (sgl_tcsr.rec), or nullptr
     const int64_t* slot_hint;  // per explicit slot: where its window ends (the index entry of the edge the slot
                                // came from), or nullptr: search
     int64_t* hint_out;   // per emitted edge: its index entry, for the next hop's slots; or nullptr
@@ -137,6 +138,26 @@ __device__ __forceinline__ int64_t group_lower_bound(const int64_t* __restrict__
         }
     }
     return lo;
+}
+
+// One edge for the uniform strategy, whose picks are scattered over a window: from the graph's interleaved
+// records when it has them (one 32-byte access), else from the four arrays (a memory sector each).
+struct Edge {
+    int64_t col, ts, eid, hint;
+};
+__device__ __forceinline__ Edge load_picked_edge(const HopArgs& a, int64_t e) {
+    Edge r;
+    if (a.rec != nullptr) {     // kernel argument: uniform across the launch
+        const longlong2* p = reinterpret_cast<const longlong2*>(a.rec) + 2 * e;
+        const longlong2 x = p[0], y = p[1];
+        r.col = x.x; r.ts = x.y; r.eid = y.x; r.hint = y.y;
+    } else {
+        r.ts = a.ts[e];
+        r.col = a.col[e];
+        r.eid = a.eid[e];
+        r.hint = a.hint != nullptr ? a.hint[e] : -1;
+    }
+    return r;
 }
 
 // Records `id` as pending in the remap state (as unique.hip's mark pass does)
@@ -508,8 +529,58 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
                     }
                 }
             }
+        } else if (G == WAVE && k > G) {
+            // ---- uniform with a fanout beyond one wavefront (a wave per slot, picks in dynamic LDS) ----
+            // Block-uniform control flow (the loops run to k for every wave, idle waves skip the work),
+            // so that block barriers order the LDS accesses of the sequential subset construction.
+            extern __shared__ int64_t s_wide[];
+            int64_t* pk = s_wide + (size_t)wid * k;
+            const bool draw = active && len > k;
+            auto emit = [&](int64_t sel, int64_t place) {
+                const Edge ed = load_picked_edge(a, start + sel);
+                a.nbr[off + place] = ed.col;
+                if (a.mark != nullptr) mark_id(a, ed.col);
+                a.nbr_ts[off + place] = a.keep_root_time ? t : ed.ts;
+                a.nbr_eid[off + place] = ed.eid;
+                a.nbr_dt[off + place] = ed.ts - t;
+                if (a.hint_out != nullptr) a.hint_out[off + place] = ed.hint;
+            };
+            if (active && !draw)                      // the whole window, in storage order
+                for (int32_t j = lig; j < c; j += G) emit(j, j);
+            if (draw)
+                for (int32_t j = lig; j < k; j += G) {
+                    const uint64_t bits = draw_bits(a.seed, a.hop, slot, j);
+                    pk[j] = a.replace ? bounded(bits, len) : bounded(bits, len - k + j + 1);
+                }
+            __syncthreads();
+            if (a.replace) {                          // kernel argument: uniform; draw order is kept
+                if (draw)
+                    for (int32_t j = lig; j < k; j += G) emit(pk[j], j);
+            } else {
+                // Floyd: step j keeps its draw unless an earlier step holds the same value, then it takes len-k+j
+                for (int32_t j = 1; j < k; ++j) {
+                    bool dup = false;
+                    if (draw) {
+                        const int64_t cand = pk[j];
+                        for (int32_t i = lig; i < j; i += G) dup |= pk[i] == cand;
+                    }
+                    dup = __any(dup);
+                    __syncthreads();
+                    if (draw && dup && lig == 0) pk[j] = len - k + j;
+                    __syncthreads();
+                }
+                // ascending: the place of a pick is the number of smaller picks (all distinct)
+                if (draw)
+                    for (int32_t j = lig; j < k; j += G) {
+                        const int64_t mine = pk[j];
+                        int32_t r = 0;
+                        for (int32_t i = 0; i < k; ++i) r += pk[i] < mine ? 1 : 0;
+                        emit(mine, r);
+                    }
+            }
+            __syncthreads();                          // the picks are reused by the next iteration
         } else {
-            // ---- uniform: needs k <= G (checked on the host) ------------------------
+            // ---- uniform: k <= G ----------------------------------------------------
             const bool draw = active && len > k;  // uniform inside the group
             int64_t sel = lig;                    // offset inside the window; copy path: identity
             int32_t rank = lig;
@@ -543,14 +614,13 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
                 }
             }
             if (active && lig < c) {
-                const int64_t e = start + sel;
-                const int64_t ets = a.ts[e], dst = a.col[e];
-                a.nbr[off + rank] = dst;
-                if (a.mark != nullptr) mark_id(a, dst);
-                a.nbr_ts[off + rank] = a.keep_root_time ? t : ets;
-                a.nbr_eid[off + rank] = a.eid[e];
-                a.nbr_dt[off + rank] = ets - t;
-                if (a.hint_out != nullptr) a.hint_out[off + rank] = a.hint[e];
+                const Edge ed = load_picked_edge(a, start + sel);
+                a.nbr[off + rank] = ed.col;
+                if (a.mark != nullptr) mark_id(a, ed.col);
+                a.nbr_ts[off + rank] = a.keep_root_time ? t : ed.ts;
+                a.nbr_eid[off + rank] = ed.eid;
+                a.nbr_dt[off + rank] = ed.ts - t;
+                if (a.hint_out != nullptr) a.hint_out[off + rank] = ed.hint;
             }
         }
     }
@@ -662,7 +732,9 @@ int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf) {
         hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, a, (int)blocks);
         SGL_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(fill_fn(Gf, a.type == SGL_SAMPLE_UNIFORM), dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
+    // a uniform fanout beyond one wavefront keeps a slot's picks in LDS (one wave per slot)
+    const size_t wide_lds = (a.type == SGL_SAMPLE_UNIFORM && a.k > WAVE) ? (size_t)NWAVE * a.k * sizeof(int64_t) : 0;
+    hipLaunchKernelGGL(fill_fn(Gf, a.type == SGL_SAMPLE_UNIFORM), dim3((unsigned)blocks), dim3(BLOCK), wide_lds, st, a);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }
@@ -821,10 +893,16 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
     }
     int64_t nbr = 0, ets = 0, id = 0, hint = -1;
     if (e_on) {
-        nbr = a.col[pos];
-        ets = a.ts[pos];
-        id = a.eid[pos];
-        if (a.hint != nullptr) hint = a.hint[pos];
+        if constexpr (UNIFORM) {
+            const Edge ed = load_picked_edge(a, pos);
+            nbr = ed.col; ets = ed.ts; id = ed.eid;
+            if (a.hint != nullptr) hint = ed.hint;
+        } else {
+            nbr = a.col[pos];
+            ets = a.ts[pos];
+            id = a.eid[pos];
+            if (a.hint != nullptr) hint = a.hint[pos];
+        }
     }
     // ---- hop 2: lane j counts the slot (neighbour j, its timestamp - or the root's, keep_root_time)
     const int64_t t2 = (UNIFORM && a.keep_root_time) ? t : ets;
@@ -1048,11 +1126,17 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
             const int32_t cc = __shfl(c2, src);
             on[r] = j0 + r < c && lig < cc;
             if (on[r]) {
-                int64_t e = st2 + lig;
-                if constexpr (UNIFORM) e = st2 + s_pick[lig * BLOCK + (threadIdx.x - lig) + ((j0 + r) & (FG - 1))];
-                ets2[r] = a.ts[e];
-                dst2[r] = a.col[e];
-                id2[r] = a.eid[e];
+                if constexpr (UNIFORM) {
+                    const Edge ed = load_picked_edge(a, st2 + s_pick[lig * BLOCK + (threadIdx.x - lig) + ((j0 + r) & (FG - 1))]);
+                    ets2[r] = ed.ts;
+                    dst2[r] = ed.col;
+                    id2[r] = ed.eid;
+                } else {
+                    const int64_t e = st2 + lig;
+                    ets2[r] = a.ts[e];
+                    dst2[r] = a.col[e];
+                    id2[r] = a.eid[e];
+                }
             }
         }
 #pragma unroll
@@ -1101,7 +1185,7 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
         return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, hop_workspace_bytes(S_max));
     Arena ar(ws, ws_bytes);
     HopArgs a{};
-    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint;
+    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint; a.rec = g->rec;
     a.slot_node = slot_node; a.slot_ts = slot_ts; a.S_max = S_max; a.S_dev = S_dev;
     a.slot_hint = slot_hint; a.hint_out = hint_out;
     a.root_hint = (derive && !p->equal_root_time) ? p->root_hint : nullptr;
@@ -1135,7 +1219,7 @@ Fused2Args fused2_args(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, cons
                        const sgl_hop_out* outs, unsigned long long* desc) {
     Fused2Args f{};
     HopArgs& a = f.h;
-    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint;
+    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint; a.rec = g->rec;
     a.S_max = S0; a.derive = 1;
     a.root_hint = p->equal_root_time ? nullptr : p->root_hint;
     a.R = spec->R; a.S_pos = spec->S_pos; a.roots = spec->roots; a.ts_ptr = spec->ts_ptr;

@@ -343,6 +343,34 @@ int32_t launch_window_end(const sgl_tcsr* g, const int64_t* node, const int64_t*
 }  // namespace
 }  // namespace sgl
 
+namespace sgl {
+namespace {
+__global__ __launch_bounds__(BLOCK) void records_kernel(sgl_tcsr g, int64_t* __restrict__ rec) {
+    for (int64_t e = (int64_t)blockIdx.x * BLOCK + threadIdx.x; e < g.m; e += (int64_t)gridDim.x * BLOCK) {
+        longlong2 a, b;
+        a.x = g.col[e];
+        a.y = g.ts[e];
+        b.x = g.eid[e];
+        b.y = g.hop_hint != nullptr ? g.hop_hint[e] : -1;
+        reinterpret_cast<longlong2*>(rec)[2 * e] = a;
+        reinterpret_cast<longlong2*>(rec)[2 * e + 1] = b;
+    }
+}
+}  // namespace
+}  // namespace sgl
+
+extern "C" int32_t sgl_tcsr_records_build(const sgl_tcsr* g, int64_t* rec, void* stream) {
+    if (!g || g->n < 0 || g->m < 0) return fail(SGL_EINVAL, "tcsr_records_build: NULL graph");
+    if (g->m == 0) return SGL_OK;
+    if (!g->col || !g->ts || !g->eid || !rec) return fail(SGL_EINVAL, "tcsr_records_build: NULL array");
+    if (reinterpret_cast<uintptr_t>(rec) % 32 != 0) return fail(SGL_EINVAL, "tcsr_records_build: rec must be 32-byte aligned");
+    int64_t blocks = ceil_div<int64_t>(g->m, BLOCK);
+    if (blocks > (1 << 20)) blocks = 1 << 20;
+    hipLaunchKernelGGL(records_kernel, dim3((unsigned)blocks), dim3(BLOCK), 0, as_stream(stream), *g, rec);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}
+
 extern "C" int32_t sgl_tcsr_hop_hint_build(const sgl_tcsr* g, int64_t* hop_hint, void* stream) {
     if (!g || g->n < 0 || g->m < 0 || !g->row_ptr) return fail(SGL_EINVAL, "tcsr_hop_hint_build: NULL graph");
     if (g->m == 0) return SGL_OK;

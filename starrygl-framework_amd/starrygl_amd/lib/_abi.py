@@ -9,7 +9,7 @@ ABI_VERSION = 5
 
 SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
-UNIFORM_MAX_FANOUT = 64
+UNIFORM_MAX_FANOUT = 1024
 STATIC_HOP_MAX_SLOTS = 65536
 UNIQUE_SORTED, UNIQUE_GROUPED, UNIQUE_PREMARKED = 0, 1, 0x100
 DT_I64, DT_F32 = 0, 1
@@ -20,7 +20,8 @@ i32, i64, u64, vp, sz = C.c_int32, C.c_int64, C.c_uint64, C.c_void_p, C.c_size_t
 
 
 class TCSR(C.Structure):
-    _fields_ = [("n", i64), ("m", i64), ("row_ptr", vp), ("col", vp), ("ts", vp), ("eid", vp), ("hop_hint", vp)]
+    _fields_ = [("n", i64), ("m", i64), ("row_ptr", vp), ("col", vp), ("ts", vp), ("eid", vp), ("hop_hint", vp),
+                ("rec", vp)]
 
 
 class SampleParams(C.Structure):
@@ -69,6 +70,7 @@ PROTOTYPES = {
     "tcsr_build": (i32, [i64, i64, vp, vp, vp, vp, vp, vp, vp, vp, vp, sz, vp]),
     "tcsr_validate": (i32, [P(TCSR), vp, sz, vp]),
     "tcsr_hop_hint_build": (i32, [P(TCSR), vp, vp]),
+    "tcsr_records_build": (i32, [P(TCSR), vp, vp]),
     "window_end": (i32, [P(TCSR), vp, vp, i64, vp, vp]),
     "sample_hop_workspace_bytes": (sz, [i64]),
     "sample_hop": (i32, [P(TCSR), vp, vp, i64, vp, P(SampleParams), P(HopOut), vp, sz, vp]),

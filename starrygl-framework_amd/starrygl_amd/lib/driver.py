@@ -65,11 +65,11 @@ class TorchBackend:
 class TCSRArrays:
     """Owner of the four T-CSR arrays plus the ABI view of them."""
 
-    def __init__(self, backend, n, row_ptr, col, ts, eid, hop_hint=None):
+    def __init__(self, backend, n, row_ptr, col, ts, eid, hop_hint=None, rec=None):
         self.n, self.m = int(n), int(col.shape[0])
-        self.row_ptr, self.col, self.ts, self.eid, self.hop_hint = row_ptr, col, ts, eid, hop_hint
+        self.row_ptr, self.col, self.ts, self.eid, self.hop_hint, self.rec = row_ptr, col, ts, eid, hop_hint, rec
         self.view = TCSR(self.n, self.m, backend.ptr(row_ptr), backend.ptr(col),
-                         backend.ptr(ts), backend.ptr(eid), backend.ptr(hop_hint))
+                         backend.ptr(ts), backend.ptr(eid), backend.ptr(hop_hint), backend.ptr(rec))
 
 
 class HopResult:
@@ -180,6 +180,18 @@ class HotPath:
         self._ck(self.lib.tcsr_hop_hint_build(C.byref(g.view), self.be.ptr(hint), self.be.stream()))
         g.hop_hint = hint
         g.view.hop_hint = self.be.ptr(hint)
+        if g.rec is not None:        # the records carry a copy of the index
+            self.build_records(g)
+        return g
+
+    def build_records(self, g):
+        """Attach the interleaved edge records to the T-CSR `g` (32 bytes per edge: destination, time, edge id,
+        next-hop index entry): the uniform strategy then reads one memory sector per picked edge instead of
+        one per array.  Build the next-hop index first if it is wanted (it is copied into the records)."""
+        rec = self.be.empty(4 * g.m)
+        self._ck(self.lib.tcsr_records_build(C.byref(g.view), self.be.ptr(rec), self.be.stream()))
+        g.rec = rec
+        g.view.rec = self.be.ptr(rec)
         return g
 
     def window_end(self, g, node, t, out=None):

@@ -33,11 +33,11 @@ def test_abi_version_and_host_side_errors():
     assert lib.struct_bytes(len(_abi.STRUCTS)) == 0 and lib.struct_bytes(-1) == 0
     # argument validation happens on the host, before any HIP call
     p = _abi.SampleParams(7, 3, -1, 0, 0, 0, 0, 0)
-    g = _abi.TCSR(1, 0, 8, None, None, None)
+    g = _abi.TCSR(1, 0, 8, None, None, None, None, None)
     assert lib.sample_hop(C.byref(g), None, None, 0, None, C.byref(p), None, None, 0, None) == _abi.SGL_ENOTSUP
     assert b"undefined sampling strategy" in lib.last_error_string()
     assert lib.sample_hop(None, None, None, 0, None, C.byref(p), None, None, 0, None) == _abi.SGL_EINVAL
-    p.type, p.fanout = _abi.SAMPLE_UNIFORM, 65
+    p.type, p.fanout = _abi.SAMPLE_UNIFORM, _abi.UNIFORM_MAX_FANOUT + 1
     assert lib.sample_hop(C.byref(g), None, None, 0, None, C.byref(p), None, None, 0, None) == _abi.SGL_ENOTSUP
     c = _abi.Cache(10, 6, -1, None, 0, None, 8, 10, None, None, None)
     assert lib.gather(C.byref(c), 8, 1, None, 8, None, None, None) == _abi.SGL_EINVAL   # row_bytes % 4

@@ -52,9 +52,10 @@ def test_window_flags(oracle, hot, sample_type):
 
 
 @pytest.mark.parametrize("sample_type", ["recent", "uniform"])
-@pytest.mark.parametrize("fanout", [3, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize("fanout", [3, 16, 17, 32, 33, 64, 65, 200, 1024])
 def test_long_rows_and_wide_fanout(oracle, hot, sample_type, fanout):
-    """a 120k-edge row (5 search steps with 16 lanes) and every group width."""
+    """a 120k-edge row (5 search steps with 16 lanes) and every group width; beyond 64 the uniform
+    strategy keeps a slot's picks in LDS."""
     (src, dst, ts, _), g, dg = _graph(oracle, hot, 500, 150_000, 1.05, 10**12, 5, hub=120_000)
     rng = np.random.default_rng(3)
     roots = np.concatenate([np.full(200, 3), rng.integers(0, g.n, 300)]).astype(np.int64)
@@ -396,3 +397,51 @@ def test_window_end_edge_cases(oracle, hot):
     assert np_of(hot.window_end(dg0, to_dev(hot, node[:3]), to_dev(hot, t[:3]))).tolist() == [-1, -1, 0]
     with pytest.raises(ValueError):
         hot.window_end(dg, to_dev(hot, node), to_dev(hot, t[:3]))
+
+
+@pytest.mark.parametrize("index", [False, True])
+@pytest.mark.parametrize("layers,fanout,n_roots", [(1, 10, 700), (2, 10, 1800), (3, 4, 900), (2, 20, 40_000), (1, 33, 500)])
+def test_interleaved_records_give_the_same_samples(oracle, hot, index, layers, fanout, n_roots):
+    """With the graph's interleaved edge records (and, `index`, its next-hop index copied into them) the
+    uniform sampler reads its picks from the records: same result as the oracle, through the launch-per-hop
+    route, the single-launch 2-hop route and the recent + uniform pair launch; recent is unchanged."""
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 3_000, 120_000, 1.15, 400_000, 17)
+    if index:
+        hot.build_hop_hint(dg)
+    hot.build_records(dg)
+    rec = np_of(dg.rec).reshape(-1, 4)
+    assert np.array_equal(rec[:, 0], g.col) and np.array_equal(rec[:, 1], g.ts) and np.array_equal(rec[:, 2], g.eid)
+    assert np.array_equal(rec[:, 3], np_of(dg.hop_hint) if index else np.full(g.m, -1))
+    rng = np.random.default_rng(5)
+    roots = rng.integers(0, g.n, n_roots).astype(np.int64)
+    root_ts = rng.integers(0, 400_000, n_roots).astype(np.int64)
+    ts_ptr = np.arange(n_roots + 1, dtype=np.int64)
+    neg, neg_ts = rng.integers(0, g.n, n_roots // 3).astype(np.int64), rng.integers(0, 400_000, n_roots // 3).astype(np.int64)
+    for kw in (dict(), dict(keep_root_time=True), dict(replace=True), dict(allowed_offset=50_000)):
+        _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, neg, neg_ts, layers, sample_type="uniform", fanout=fanout, seed=3, **kw)
+    _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, neg, neg_ts, layers, sample_type="recent", fanout=fanout)
+    if layers == 2 and fanout <= 16:      # both policies in one launch
+        S0 = n_roots + n_roots // 3
+        outs = [hot.khop_buffers(S0, 2, fanout) for _ in range(2)]
+        ps = [hot.params("recent", fanout), hot.params("uniform", fanout, seed=3)]
+        hot.sample_khop_multi(dg, *[to_dev(hot, x) for x in (roots, ts_ptr, root_ts, neg, neg_ts)], 2, ps, outs)
+        for p, res in zip(ps, outs):
+            want = oracle.sample_khop(g, roots, ts_ptr, root_ts, neg, neg_ts, 2, p)
+            for l, h in enumerate(res.finalize().hops):
+                assert_hop_equal(h, want.hops[l], tag=f"pair hop{l}")
+
+
+def test_wide_uniform_fanout_over_two_hops_and_flags(oracle, hot):
+    """fanout 100 through the k-hop driver (windows shorter and longer than the fanout, with replacement,
+    root time kept, lower window bound), from the arrays and from the interleaved records."""
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 400, 90_000, 1.1, 300_000, 13)
+    rng = np.random.default_rng(9)
+    roots = rng.integers(0, g.n, 150).astype(np.int64)
+    root_ts = rng.integers(0, 300_000, 150).astype(np.int64)
+    ts_ptr, e = np.arange(151, dtype=np.int64), np.zeros(0, np.int64)
+    for records in (False, True):
+        if records:
+            hot.build_hop_hint(dg)
+            hot.build_records(dg)
+        for kw in (dict(), dict(replace=True), dict(keep_root_time=True), dict(allowed_offset=20_000)):
+            _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, e, e, 2, sample_type="uniform", fanout=100, seed=5, **kw)

@@ -186,7 +186,7 @@ def test_sampling_errors(oracle):
     with pytest.raises(RuntimeError, match="undefined sampling strategy"):
         oracle.sample_hop(g, np.array([0]), np.array([5]), p)
     with pytest.raises(RuntimeError):
-        oracle.sample_hop(g, np.array([0]), np.array([5]), oracle.params("uniform", 65))
+        oracle.sample_hop(g, np.array([0]), np.array([5]), oracle.params("uniform", _abi.UNIFORM_MAX_FANOUT + 1))
     with pytest.raises(IndexError):
         oracle.sample_hop(g, np.array([3]), np.array([5]), oracle.params("recent", 2))
 
@@ -390,3 +390,13 @@ def test_indexed_cpu_sampler_equals_the_searching_oracle(oracle, oracle_cdll, st
         got = O.sample_khop_indexed(oracle, oracle_cdll, g, roots, ts_ptr, root_ts, neg, neg_ts, 3, oracle.with_root_hint(p, hint))
         for a, b in zip(want.hops, got.hops):
             assert_hop_equal(b, a, f"{strategy} {kw}")
+
+
+def test_edge_records_are_the_four_arrays_side_by_side(oracle):
+    rng = np.random.default_rng(2)
+    n, m = 40, 900
+    g = host_graph(oracle, n, rng.integers(0, n, m), rng.integers(0, n, m), rng.integers(0, 100, m))
+    oracle.build_records(g)
+    assert np.array_equal(g.rec.reshape(-1, 4), np.stack([g.col, g.ts, g.eid, np.full(m, -1)], axis=1))
+    oracle.build_hop_hint(g)          # the records follow the index
+    assert np.array_equal(g.rec.reshape(-1, 4), np.stack([g.col, g.ts, g.eid, g.hop_hint], axis=1))
