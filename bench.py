@@ -335,6 +335,33 @@ def workload_large_partition(hot, torch, np, synth, _abi, n=100_000_000, m=1_000
     res["sample_recent_2hop"] = {"ms": round(ms, 4), "edges_per_batch": e_tot / NB,
                                  "edges_per_s": round(e_tot / NB / ms * 1e3, 1),
                                  "GBps": round((samp_bytes(R, E0) + samp_bytes(E0, E1)) / ms / 1e6, 1)}
+    # the uniform strategy over the same roots: picks scattered over each window, first from the four edge
+    # arrays (a memory sector per array and pick), then from the interleaved 32-byte records
+    p_u = hot.params("uniform", k, seed=11)
+    ku = hot.khop_buffers(R, 2, k)
+
+    def sample_uniform(b):
+        hot.sample_khop(g, roots[b], ts_ptr, root_ts[b], empty, empty, 2, p_u, finalize=False, out=ku)
+
+    for tag in ("sample_uniform_2hop_from_arrays", "sample_uniform_2hop_from_records"):
+        if tag.endswith("records"):
+            torch.cuda.synchronize()
+            t_r = time.perf_counter()
+            hot.build_records(g)
+            torch.cuda.synchronize()
+            res["edge_records_build_s"] = round(time.perf_counter() - t_r, 3)
+        ms_u, e_u = [], 0
+        for b in range(NB):
+            ms_u.append(_time_launches(torch, lambda: sample_uniform(b), reps=5, warm=1))
+            cu = ku.counts.cpu().numpy()
+            e_u += int(cu[1] + cu[4])
+        ms_m = float(np.mean(ms_u))
+        res[tag] = {"ms": round(ms_m, 4), "edges_per_batch": e_u / NB, "edges_per_s": round(e_u / NB / ms_m * 1e3, 1),
+                    "over_recent": round(ms_m / ms, 2)}
+    del ku
+    g.rec = None
+    g.view.rec = None
+    torch.cuda.empty_cache()
     ids_in = R + E0 + E1
     ms = _time_launches(torch, unique_dense, reps=5, warm=1)
     u = int(U[0].item())

@@ -172,7 +172,14 @@ typedef struct sgl_sample_params {
      * root's row, so a wrong hint gives a wrong sample, never a stray access.
      * Negative roots are always searched. */
     const int64_t* root_hint; /* device int64[S_pos], or NULL                  */
+    /* SGL_SAMPLE_MULTI_LAUNCH: sgl_sample_khop / _multi take the launch-per-hop
+     * route whatever the size of the call (no kernel of that route waits for
+     * another block).  What a caller re-issues a query with after a result
+     * whose counts[2] read INT64_MAX (see sgl_sample_khop). */
+    int32_t  flags;
+    int32_t  reserved;        /* 0 */
 } sgl_sample_params;
+#define SGL_SAMPLE_MULTI_LAUNCH 1
 
 /* One hop's result, caller-allocated (replaces TemporalNeighbor,
  * sample.cu.hpp:882-915).  With S slots and E = sum_s c_s sampled edges:
@@ -240,7 +247,10 @@ int32_t sgl_sample_hop_static(const sgl_tcsr* g,
  * Two-hop calls of up to 32768 root slots and fanout <= 16 run as one launch
  * whose blocks wait (bounded, sgl_set_wait_limit) for the edge totals of the
  * blocks before them; should a block ever give up, outs[0].counts[2] reads
- * INT64_MAX and the outputs of the call are void. */
+ * INT64_MAX and the outputs of the call are void (a remap state named by
+ * mark_state is then marked void as well: the next sgl_unique_compact on it
+ * reports INT64_MAX until sgl_remap_init).  The same call with
+ * SGL_SAMPLE_MULTI_LAUNCH in p->flags cannot give up. */
 size_t  sgl_sample_khop_workspace_bytes(int64_t S0, int32_t layers,
                                         int32_t fanout);
 int32_t sgl_sample_khop(const sgl_tcsr* g,
@@ -277,6 +287,9 @@ int32_t sgl_sample_khop_multi(const sgl_tcsr* g,
 /* ------------------------------------------------------ unique / compaction */
 #define SGL_UNIQUE_SORTED  0 /* all arrays form one group: == np.unique(return_inverse) */
 #define SGL_UNIQUE_GROUPED 1 /* per array: ids new to the epoch, ascending, appended    */
+#define SGL_UNIQUE_MULTI_LAUNCH 0x200 /* flag: the numbering pass of a dense state never exchanges counts
+                                      * inside one launch (no bounded wait); for re-issuing a call whose
+                                      * U_dev[0] read INT64_MAX, after sgl_remap_init                    */
 #define SGL_UNIQUE_PREMARKED 0x100 /* flag, with SGL_UNIQUE_SORTED, reset = 1 and a dense state:
                                     * the sampler has already recorded the arrays' ids as
                                     * pending (sgl_sample_params.mark_state)              */

@@ -576,6 +576,7 @@ static int32_t unique_core(void* state, int64_t universe_arg, seen_rec* known, i
         return fail(SGL_EINVAL, "unique_compact: null");
     /* PREMARKED only tells the HIP library that the sampler already did its first pass; the
      * result is defined by the arrays alone, so the restatement just numbers them. */
+    mode &= ~SGL_UNIQUE_MULTI_LAUNCH;      /* a launch-structure choice of the HIP library, no meaning here */
     if ((mode & SGL_UNIQUE_PREMARKED) && ((mode & ~SGL_UNIQUE_PREMARKED) != SGL_UNIQUE_SORTED || !reset || !state))
         return fail(SGL_EINVAL, "unique_compact: PREMARKED needs the dense state, SORTED mode and reset = 1");
     mode &= ~SGL_UNIQUE_PREMARKED;

@@ -66,6 +66,12 @@ inline bool remap_byte_flags(int64_t universe) { return universe <= REMAP_BYTE_F
 inline void* remap_flags(void* state, int64_t universe) {
     return static_cast<char*>(state) + REMAP_HEADER_BYTES + (size_t)universe * 8;
 }
+// Marks the remap state whose pending flags are `flags` as void (the sticky field of its header, see
+// unique.hip): what a sampler launch that gave up does to the state it was recording ids in.
+__device__ __forceinline__ void remap_poison(void* flags, int64_t universe) {
+    char* base = static_cast<char*>(flags) - REMAP_HEADER_BYTES - (size_t)universe * 8;
+    reinterpret_cast<int64_t*>(base)[3] = 1;
+}
 __device__ __forceinline__ void remap_set_pending(void* flags, int bytes, int64_t id) {
     if (bytes) {
         static_cast<uint8_t*>(flags)[id] = 1;

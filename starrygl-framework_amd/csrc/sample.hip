@@ -725,6 +725,10 @@ int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf) {
     a.align = BLOCK / (Gc < Gf ? Gc : Gf);
     int64_t blocks = ceil_div<int64_t>(a.S_max > 0 ? a.S_max : 1, a.align);
     if (blocks > MAX_BLOCKS) blocks = MAX_BLOCKS;
+    // a block counts the edges of its run of slots in 32 bits (count_kernel's partial sums, scan_kernel's staging)
+    const int64_t run = ceil_div<int64_t>(ceil_div<int64_t>(a.S_max > 0 ? a.S_max : 1, blocks), a.align) * a.align;
+    if (a.k > 0 && run > (int64_t)INT32_MAX / a.k)
+        return fail(SGL_ENOTSUP, "sample: %lld slots x fanout %d exceed what a block counts in 32 bits", (long long)a.S_max, a.k);
     a.scanned = blocks > FUSED_PREFIX_MAX ? 1 : 0;
     hipLaunchKernelGGL(count_fn(Gc), dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
     SGL_LAUNCH_CHECK();
@@ -998,7 +1002,10 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
     if (threadIdx.x == 0) {
         // poisoned: reading the result reports an error (a maximum, so that the last block's count
         // of bad slots cannot replace it, whichever block writes first)
-        if (gave_up) atomicMax(reinterpret_cast<long long*>(&a.counts[2]), (long long)INT64_MAX);
+        if (gave_up) {
+            atomicMax(reinterpret_cast<long long*>(&a.counts[2]), (long long)INT64_MAX);
+            if (a.mark != nullptr) remap_poison(a.mark, a.mark_universe);   // the ids recorded there are void too
+        }
         if (b == nb - 1) {            // totals of the call
             const uint64_t tot = prefix + btotal;
             const int64_t E0 = (int64_t)((tot >> SH_E0) & M_E0), E1 = (int64_t)(tot & M_E1);
@@ -1245,7 +1252,8 @@ Fused2Args fused2_args(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, cons
 size_t pick_lds_bytes(int32_t k) { return (size_t)k * BLOCK * sizeof(int64_t); }
 
 bool fused2_fits(int32_t layers, const sgl_sample_params* p, int64_t S0) {
-    return layers == 2 && p->fanout >= 1 && p->fanout <= FG && S0 >= 1 && S0 <= FUSED_MAX_SLOTS;
+    return layers == 2 && p->fanout >= 1 && p->fanout <= FG && S0 >= 1 && S0 <= FUSED_MAX_SLOTS &&
+           !(p->flags & SGL_SAMPLE_MULTI_LAUNCH);
 }
 
 int32_t run_fused2(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, const sgl_sample_params* p,

@@ -496,7 +496,8 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
     if (G < 0 || (G > 0 && (!ids || !len_max || !local_out)) || !U_dev)
         return fail(SGL_EINVAL, "unique_compact: NULL argument");
     const bool premarked = (mode & SGL_UNIQUE_PREMARKED) != 0;
-    mode &= ~SGL_UNIQUE_PREMARKED;
+    const bool multi_launch = (mode & SGL_UNIQUE_MULTI_LAUNCH) != 0;
+    mode &= ~(SGL_UNIQUE_PREMARKED | SGL_UNIQUE_MULTI_LAUNCH);
     if (mode != SGL_UNIQUE_SORTED && mode != SGL_UNIQUE_GROUPED) return fail(SGL_EINVAL, "unique_compact: bad mode");
     if (premarked && (mode != SGL_UNIQUE_SORTED || !reset || !state))
         return fail(SGL_EINVAL, "unique_compact: PREMARKED needs the dense state, SORTED mode and reset = 1");
@@ -582,7 +583,7 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
             hipLaunchKernelGGL(assign_groups_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, (int)G, tile_sum, nt, scanned,
                                rst, unique_out, unique_capacity, U_dev, stamp_ws);
             SGL_LAUNCH_CHECK();
-        } else if (nt <= SINGLE_PASS_MAX) {
+        } else if (nt <= SINGLE_PASS_MAX && !multi_launch) {
             hipLaunchKernelGGL(assign_kernel<2>, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, rst,
                                unique_out, unique_capacity, U_dev, stamp_ws, wait_limit());
             SGL_LAUNCH_CHECK();

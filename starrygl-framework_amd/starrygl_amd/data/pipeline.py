@@ -18,7 +18,7 @@ import torch
 
 from ..graph.graph import Block
 from ..lib import _abi, hot_path
-from ..lib.driver import check_sample_bad, check_unique_total
+from ..lib.driver import POISON, check_sample_bad, check_unique_total
 
 
 class MiniBatch:
@@ -37,6 +37,12 @@ class MiniBatch:
             p._done.synchronize()
         c = p.live.tolist()
         u_total = int(c[3 * p.layers])
+        if u_total == POISON or max(c[3 * l + 2] for l in range(p.layers)) >= POISON:
+            # a block of a single-launch kernel gave up its bounded wait: the batch (still in the pipeline's input
+            # buffers) is re-issued through the launch-per-stage routes, which have no such wait
+            p._recover()
+            c = p.live.tolist()
+            u_total = int(c[3 * p.layers])
         check_unique_total(u_total)
         check_sample_bad(max(c[3 * l + 2] for l in range(p.layers)))
         check_sample_bad(sum(c[3 * l + 2] for l in range(p.layers)))
@@ -173,14 +179,26 @@ class MiniBatchPipeline:
             self._views[key] = True
         return self
 
-    def _chain(self):
+    def _recover(self):
+        """Run the batch in the input buffers again, eagerly, with every kernel that exchanges totals inside one
+        launch replaced by its multi-launch route, after initialising the remap state again."""
+        hp = self.hp
+        cur = torch.cuda.current_stream(self.dev)
+        with torch.cuda.stream(self.stream if self.stream is not None else cur):
+            hp._reinit_marked(self.p)
+            self._chain(multi_launch=True)
+            torch.cuda.current_stream(self.dev).synchronize()
+        hp.recoveries += 1
+
+    def _chain(self, multi_launch=False):
         hp, kr = self.hp, self.kr
         hp.sample_khop(self.g._g, self.in_roots, self.ts_ptr, self.in_ts, self.in_neg, self.in_neg_ts, self.layers,
-                       self.p, finalize=False, out=kr)
+                       hp.multi_launch(self.p) if multi_launch else self.p, finalize=False, out=kr)
         arrays = [kr.slot_node0] + [h.neighbors for h in kr.hops]
         lens = [self.S0_dev] + [h.counts[1:2] for h in kr.hops]
-        hp.unique_compact(arrays, _abi.UNIQUE_SORTED, self.state, True, lens_dev=lens, out_arrays=self.local,
-                          finalize=False, unique_out=self.ubuf, U_out=self.U, premarked=True, workspace=self.uws)
+        hp.unique_compact(arrays, _abi.UNIQUE_SORTED | (_abi.UNIQUE_MULTI_LAUNCH if multi_launch else 0), self.state, True,
+                          lens_dev=lens, out_arrays=self.local, finalize=False, unique_out=self.ubuf, U_out=self.U,
+                          premarked=True, workspace=self.uws)
         if self._plans is None:      # every gather of the batch in as few launches as possible
             segs = [(c, self.ubuf, self.node_out[name], self.node_ts_out.get(name), self.U[0:1])
                     for name, c in self.node_tables.items()]

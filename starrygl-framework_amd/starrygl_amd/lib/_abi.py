@@ -11,7 +11,8 @@ SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
 UNIFORM_MAX_FANOUT = 1024
 STATIC_HOP_MAX_SLOTS = 65536
-UNIQUE_SORTED, UNIQUE_GROUPED, UNIQUE_PREMARKED = 0, 1, 0x100
+UNIQUE_SORTED, UNIQUE_GROUPED, UNIQUE_PREMARKED, UNIQUE_MULTI_LAUNCH = 0, 1, 0x100, 0x200
+SAMPLE_MULTI_LAUNCH = 1
 DT_I64, DT_F32 = 0, 1
 
 SAMPLE_TYPES = {"recent": SAMPLE_RECENT, "uniform": SAMPLE_UNIFORM}
@@ -28,7 +29,8 @@ class SampleParams(C.Structure):
     _fields_ = [("type", i32), ("fanout", i32), ("allowed_offset", i64),
                 ("equal_root_time", i32), ("keep_root_time", i32),
                 ("replace", i32), ("hop", i32), ("seed", u64),
-                ("mark_state", vp), ("mark_universe", i64), ("root_hint", vp)]
+                ("mark_state", vp), ("mark_universe", i64), ("root_hint", vp),
+                ("flags", i32), ("reserved", i32)]
 
 
 class HopOut(C.Structure):

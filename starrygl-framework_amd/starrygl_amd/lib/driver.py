@@ -101,6 +101,9 @@ class HopResult:
         return self
 
 
+POISON = (1 << 63) - 1
+
+
 def check_sample_bad(bad):
     """counts[2] of a hop: slots whose node lies outside [0,n); INT64_MAX when a block of the
     single-launch 2-hop sampler gave up its bounded wait (the call's outputs are void)."""
@@ -108,6 +111,16 @@ def check_sample_bad(bad):
         raise RuntimeError("sample_khop: a block gave up waiting for the edge totals of an earlier block")
     if bad:
         raise IndexError(f"sgl status {_abi.SGL_ERANGE}: {bad} sampling slots name a node outside [0,n)")
+
+
+def _marked_state(p):
+    """The RemapState a SampleParams made by HotPath.marking records ids in (None otherwise)."""
+    keep = getattr(p, "_keep", None)
+    while isinstance(keep, tuple):
+        if isinstance(keep[1], RemapState):
+            return keep[1]
+        keep = keep[0] if isinstance(keep[0], tuple) else None
+    return None
 
 
 def _check_root_hint(p, S_pos):
@@ -133,6 +146,7 @@ class HotPath:
                 raise RuntimeError(f"sgl ABI struct {mirror.__name__}: the library has {int(lib.struct_bytes(which))} "
                                    f"bytes, the binding {C.sizeof(mirror)}")
         self._ws = {}
+        self.recoveries = 0     # calls re-issued because a block had given up its bounded wait
 
     # ------------------------------------------------------------ helpers
     def _workspace(self, nbytes):
@@ -233,12 +247,28 @@ class HotPath:
             sample_type = _abi.SAMPLE_TYPES[sample_type]
         return SampleParams(int(sample_type), int(fanout), int(allowed_offset),
                             int(bool(equal_root_time)), int(bool(keep_root_time)),
-                            int(bool(replace)), int(hop), int(seed) & (2**64 - 1), None, 0, None)
+                            int(bool(replace)), int(hop), int(seed) & (2**64 - 1), None, 0, None, 0, 0)
 
     def set_wait_limit(self, polls):
         """Polls before a block that waits for another block's totals gives up (<= 0: default);
         returns the previous limit.  For tests of that error path."""
         return int(self.lib.set_wait_limit(int(polls)))
+
+    def multi_launch(self, p):
+        """Copy of the sampling parameters `p` that keeps a k-hop call off the single-launch route."""
+        q = SampleParams.from_buffer_copy(p)
+        q.flags |= _abi.SAMPLE_MULTI_LAUNCH
+        q._keep = getattr(p, "_keep", None)
+        if hasattr(p, "_root_hint_len"):
+            q._root_hint_len = p._root_hint_len
+        return q
+
+    def _reinit_marked(self, p):
+        """Initialise the remap state that the sampling parameters `p` record ids in (if any) again."""
+        st = _marked_state(p)
+        if st is not None:
+            self._ck(self.lib.remap_init(self.be.ptr(st.buf), self.be.nbytes(st.buf), st.universe, self.be.stream()))
+            st.count_bound = 0
 
     def marking(self, p, state):
         """Copy of the sampling parameters `p` that makes the sampler record every id it
@@ -301,11 +331,19 @@ class HotPath:
         if res.S0 < S0 or len(res.hops) != layers or res.fanout < p.fanout:
             raise MemoryError("khop buffers are smaller than this call needs")
         ws, wsb = res.ws, be.nbytes(res.ws)
-        self._ck(self.lib.sample_khop(C.byref(g.view), R, be.ptr(roots), be.ptr(ts_ptr), S_pos,
-                                      be.ptr(root_ts), N_neg, be.ptr(neg_roots), be.ptr(neg_ts),
-                                      layers, C.byref(p), be.ptr(res.slot_node0), be.ptr(res.slot_ts0),
-                                      res.structs, be.ptr(ws), wsb, be.stream()))
+
+        def launch(params):
+            self._ck(self.lib.sample_khop(C.byref(g.view), R, be.ptr(roots), be.ptr(ts_ptr), S_pos,
+                                          be.ptr(root_ts), N_neg, be.ptr(neg_roots), be.ptr(neg_ts),
+                                          layers, C.byref(params), be.ptr(res.slot_node0), be.ptr(res.slot_ts0),
+                                          res.structs, be.ptr(ws), wsb, be.stream()))
+
+        launch(p)
         res.S0_live = S0
+        # Should a block of the single-launch route have given up its bounded wait, reading the result
+        # re-issues the call through the launch-per-hop route (which has no such wait); a remap state the
+        # sampler was recording ids in is initialised again first.
+        res._recover = lambda: (self._reinit_marked(p), launch(self.multi_launch(p)))
         return res.finalize() if finalize else res
 
     def sample_khop_multi(self, g, roots, ts_ptr, root_ts, neg_roots, neg_ts, layers, params, outs):
@@ -352,7 +390,7 @@ class HotPath:
 
     def unique_compact(self, arrays, mode=_abi.UNIQUE_SORTED, state=None, reset=True,
                        lens_dev=None, out_arrays=None, finalize=True, unique_out=None, U_out=None,
-                       premarked=False, workspace=None):
+                       premarked=False, workspace=None, _retry=False):
         self._chk("i64", **{f"arrays[{i}]": a for i, a in enumerate(arrays)})
         be, G = self.be, len(arrays)
         len_max = (i64 * max(G, 1))(*[int(a.shape[0]) for a in arrays])
@@ -395,6 +433,15 @@ class HotPath:
         if not finalize:
             return out_arrays, unique, U
         u_total, u_before = be.tolist(U)
+        if (u_total == POISON and state is not None and not hashed and reset and not premarked and not _retry):
+            # a tile of the single-launch numbering pass gave up its bounded wait: the state is initialised
+            # again and the call re-issued with the numbering in separate launches (nothing there waits)
+            self._ck(self.lib.remap_init(be.ptr(state.buf), be.nbytes(state.buf), state.universe, be.stream()))
+            state.count_bound = 0
+            self.recoveries += 1
+            return self.unique_compact(arrays, int(mode) | _abi.UNIQUE_MULTI_LAUNCH, state, True, lens_dev=lens_dev,
+                                       out_arrays=out_arrays, unique_out=unique_out, U_out=U_out, workspace=workspace,
+                                       _retry=True)
         check_unique_total(u_total)
         return out_arrays, unique[:u_total], (u_total, u_before)
 
@@ -571,6 +618,11 @@ class KHopResult:
         already has them on the host) and narrow."""
         if not self.final:
             c = self.hp.be.tolist(self.counts) if counts_host is None else list(counts_host)
+            if self.hops and c[2] >= POISON and getattr(self, "_recover", None) is not None:
+                self._recover()                      # once: the launch-per-hop route cannot give up
+                self._recover = None
+                self.hp.recoveries += 1
+                c = self.hp.be.tolist(self.counts)
             for l, h in enumerate(self.hops):
                 h.finalize(*c[3 * l: 3 * l + 3])
             S0 = getattr(self, "S0_live", None)

@@ -20,7 +20,7 @@ import threading
 import torch
 
 from . import _abi, hot_path
-from .driver import check_unique_total
+from .driver import POISON, check_unique_total
 
 
 class TemporalRoot:
@@ -230,6 +230,18 @@ class CUDAGraph:
         local, uniq, _ = hp.unique_compact(arrays, _abi.UNIQUE_GROUPED, self._state, reset, lens_dev=lens,
                                            finalize=False, U_out=live[3 * L:])
         vals = hp.be.tolist(live)
+        if reset and (vals[3 * L] == POISON or (L and vals[2] >= POISON)):
+            # a block of a single-launch kernel gave up its bounded wait: the sampler call is re-issued through the
+            # launch-per-hop route and the numbering in separate launches, on a state initialised again.  Only a
+            # query that opens an epoch can afford that; one that continues an epoch raises below.
+            if getattr(kr, "_recover", None) is not None and vals[2] >= POISON:
+                kr._recover()
+                kr._recover = None
+            self._state = hp.remap_state(self._n)
+            hp.recoveries += 1
+            local, uniq, _ = hp.unique_compact(arrays, _abi.UNIQUE_GROUPED | _abi.UNIQUE_MULTI_LAUNCH, self._state, reset,
+                                               lens_dev=lens, finalize=False, U_out=live[3 * L:])
+            vals = hp.be.tolist(live)
         kr.finalize(vals[: 3 * L])
         total, before = vals[3 * L], vals[3 * L + 1]
         check_unique_total(total)

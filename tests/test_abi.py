@@ -32,7 +32,7 @@ def test_abi_version_and_host_side_errors():
         assert lib.struct_bytes(which) == C.sizeof(mirror), mirror.__name__
     assert lib.struct_bytes(len(_abi.STRUCTS)) == 0 and lib.struct_bytes(-1) == 0
     # argument validation happens on the host, before any HIP call
-    p = _abi.SampleParams(7, 3, -1, 0, 0, 0, 0, 0)
+    p = _abi.SampleParams(7, 3, -1, 0, 0, 0, 0, 0, None, 0, None, 0, 0)
     g = _abi.TCSR(1, 0, 8, None, None, None, None, None)
     assert lib.sample_hop(C.byref(g), None, None, 0, None, C.byref(p), None, None, 0, None) == _abi.SGL_ENOTSUP
     assert b"undefined sampling strategy" in lib.last_error_string()
