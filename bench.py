@@ -54,64 +54,61 @@ def _time_launches(torch, fn, reps=10, warm=2):
 
 
 def workload_cache_stress(hot, torch, np, synth, rows=50_000_000, dim=128, n_req=2_000_000, hot_frac=0.10):
-    """configs[2]: 50M x 128 bf16 table, hottest 10 % of rows (Zipf(1.1) access rank) in HBM,
-    the rest in pinned host memory, 2M Zipf(1.1) requests per batch."""
+    """configs[2]: 50M x 128 bf16 table, hottest 10 % of rows (by access rank) in HBM, every row in pinned host
+    memory, 2M requests per batch.  Two request mixes: Zipf(1.1) by access rank (about 80 % of the requests of a
+    batch repeat an earlier one, so the gather is helped by L2) and a Zipf whose exponent is set so that about
+    40 % do (the duplicate rate the config states).  Every output row is checked against the generating formula."""
     dev = hot.be.device
     row_bytes = dim * 2
     hot_rows = int(rows * hot_frac)
     t0 = time.time()
-    # access rank r -> row id through an affine permutation (odd multiplier mod 2^k would need a
-    # power-of-two table; a random offset rotation keeps hot rows non-contiguous in id space)
-    g = torch.Generator(device=dev).manual_seed(3)
-    rank_to_id = torch.randperm(rows, device=dev, generator=g)
-    hot_slot = torch.full((rows,), -1, dtype=torch.int32, device=dev)
-    hot_slot[rank_to_id[:hot_rows]] = torch.arange(hot_rows, dtype=torch.int32, device=dev)
-    # row content: bf16 bit pattern derived from the row id (any bit pattern is a valid payload)
-    def content(ids):
-        base = (ids * 2654435761 % 65521).to(torch.int32).unsqueeze(1)
-        return ((base + torch.arange(dim, device=dev, dtype=torch.int32)) & 0x7FFF).to(torch.int16)
-    hot_tab = torch.empty((hot_rows, dim), dtype=torch.int16, device=dev)
-    for lo in range(0, hot_rows, 1 << 20):
-        hot_tab[lo: lo + (1 << 20)] = content(rank_to_id[lo: min(lo + (1 << 20), hot_rows)])
-    cold = torch.empty((rows, dim), dtype=torch.int16, pin_memory=True)
-    for lo in range(0, rows, 1 << 22):
-        hi = min(lo + (1 << 22), rows)
-        cold[lo:hi].copy_(content(torch.arange(lo, hi, device=dev)))
-    torch.cuda.synchronize()
+    rank_to_id, hot_slot, hot_tab, cold = synth.two_tier_table(torch, dev, rows, dim, hot_frac, 3)
     log(f"[c3] tables ready in {time.time() - t0:.1f}s (hot {hot_rows * row_bytes / 1e9:.2f} GB HBM, cold {rows * row_bytes / 1e9:.1f} GB pinned)")
     cache = hot.cache(row_bytes, hot_tab, rows=rows, cold=cold, hot_slot=hot_slot)
-    ranks = torch.from_numpy(synth.zipf_requests(rows, n_req, 1.1, 5)).to(dev)
-    ids_mixed = rank_to_id[ranks]
-    ids_hit = rank_to_id[ranks[ranks < hot_rows]][: n_req]
-    if ids_hit.numel() < n_req:
-        ids_hit = ids_hit.repeat((n_req + ids_hit.numel() - 1) // ids_hit.numel())[:n_req]
-    miss_ranks = ranks[ranks >= hot_rows]
-    ids_miss = rank_to_id[miss_ranks]
     out = torch.empty((n_req, dim), dtype=torch.int16, device=dev)
-    stats = hot.be.zeros(3)
-    hot.gather(cache, ids_mixed, out, stats=stats)
-    n_hot, n_cold, n_abs = stats.cpu().tolist()
-    # byte-exact check of a sample against the generating formula
-    chk = torch.arange(0, n_req, 97, device=dev)
-    assert torch.equal(out[chk], content(ids_mixed[chk])), "cache stress gather: output differs from the table content"
-    dup = 1.0 - torch.unique(ids_mixed).numel() / n_req
     per_row = 8 + 4 + 2 * row_bytes          # id + index entry + row read + row written
-    res = {"rows": rows, "row_bytes": row_bytes, "requests": n_req, "hit_fraction": n_hot / n_req,
-           "duplicate_fraction": round(dup, 4)}
-    ms = _time_launches(torch, lambda: hot.gather(cache, ids_hit, out))
-    res["all_hit"] = {"ms": round(ms, 4), "GBps": round(n_req * per_row / ms / 1e6, 1),
-                      "frac_of_hbm_peak": round(n_req * per_row / ms / 1e6 / HBM_PEAK_GBPS, 4)}
-    ms = _time_launches(torch, lambda: hot.gather(cache, ids_mixed, out), reps=5)
-    res["mixed"] = {"ms": round(ms, 4), "GBps": round(n_req * per_row / ms / 1e6, 1)}
-    if ids_miss.numel() > 0:
-        om = out[: ids_miss.numel()]
-        ms = _time_launches(torch, lambda: hot.gather(cache, ids_miss, om), reps=5)
-        res["miss_only"] = {"rows": int(ids_miss.numel()), "ms": round(ms, 4),
-                            "host_read_GBps": round(ids_miss.numel() * row_bytes / ms / 1e6, 2)}
-        # the practical PCIe roof: one pinned -> device copy of the same number of bytes
-        nb = ids_miss.numel()
-        ms = _time_launches(torch, lambda: om.copy_(cold[:nb], non_blocking=True), reps=5)
-        res["miss_only"]["memcpy_h2d_same_bytes_GBps"] = round(nb * row_bytes / ms / 1e6, 2)
+    res = {"rows": rows, "row_bytes": row_bytes, "requests": n_req}
+
+    def checked_gather(ids):
+        stats = hot.be.zeros(3)
+        hot.gather(cache, ids, out[: ids.numel()], stats=stats)
+        for lo in range(0, ids.numel(), 1 << 19):
+            hi = min(lo + (1 << 19), ids.numel())
+            assert torch.equal(out[lo:hi], synth.row_content(torch, ids[lo:hi], dim)), "cache stress gather: output differs from the table content"
+        return stats.cpu().tolist()
+
+    a40 = synth.zipf_exponent_for_duplicates(rows, n_req, 0.40, 5)
+    a40_hot = synth.zipf_exponent_for_duplicates(hot_rows, n_req, 0.40, 5)
+    for tag, a_all, a_hot in (("zipf_1.1", 1.1, None), ("40pct_duplicates", a40, a40_hot)):
+        ranks = torch.from_numpy(synth.zipf_requests(rows, n_req, a_all, 5)).to(dev)
+        ids_mixed = rank_to_id[ranks]
+        if a_hot is None:      # the hits of the mixed stream, repeated up to the batch size
+            ids_hit = rank_to_id[ranks[ranks < hot_rows]][: n_req]
+            ids_hit = ids_hit.repeat((n_req + ids_hit.numel() - 1) // ids_hit.numel())[:n_req]
+        else:                  # requests over the hot rows only, at the same duplicate rate
+            ids_hit = rank_to_id[torch.from_numpy(synth.zipf_requests(hot_rows, n_req, a_hot, 6)).to(dev)]
+        n_hot, n_cold, n_abs = checked_gather(ids_mixed)
+        assert n_abs == 0 and checked_gather(ids_hit)[0] == n_req
+        r = {"zipf_exponent": round(a_all, 3), "hit_fraction": n_hot / n_req,
+             "duplicate_fraction": round(1.0 - torch.unique(ids_mixed).numel() / n_req, 4),
+             "duplicate_fraction_all_hit": round(1.0 - torch.unique(ids_hit).numel() / n_req, 4)}
+        ms = _time_launches(torch, lambda: hot.gather(cache, ids_hit, out))
+        r["all_hit"] = {"ms": round(ms, 4), "GBps": round(n_req * per_row / ms / 1e6, 1),
+                        "frac_of_hbm_peak": round(n_req * per_row / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        ms = _time_launches(torch, lambda: hot.gather(cache, ids_mixed, out), reps=3, warm=1)
+        r["mixed"] = {"ms": round(ms, 4), "GBps": round(n_req * per_row / ms / 1e6, 1)}
+        miss_ranks = ranks[ranks >= hot_rows]
+        if miss_ranks.numel() > 0:
+            ids_miss = rank_to_id[miss_ranks]
+            om = out[: ids_miss.numel()]
+            ms = _time_launches(torch, lambda: hot.gather(cache, ids_miss, om), reps=3, warm=1)
+            r["miss_only"] = {"rows": int(ids_miss.numel()), "ms": round(ms, 4),
+                              "host_read_GBps": round(ids_miss.numel() * row_bytes / ms / 1e6, 2)}
+            # the practical PCIe roof: one pinned -> device copy of the same number of bytes
+            nb = ids_miss.numel()
+            ms = _time_launches(torch, lambda: om.copy_(cold[:nb], non_blocking=True), reps=3, warm=1)
+            r["miss_only"]["memcpy_h2d_same_bytes_GBps"] = round(nb * row_bytes / ms / 1e6, 2)
+        res[tag] = r
     return res
 
 

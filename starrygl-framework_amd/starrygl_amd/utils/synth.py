@@ -138,3 +138,48 @@ def graph_by_degree_device(torch, device, n, m, a, max_deg, t_bits, seed, dst_by
         col = torch.randint(0, n, (m,), device=device, generator=gen)
     eid = torch.arange(m, device=device)
     return row_ptr, col, ts, eid, key
+
+
+def zipf_exponent_for_duplicates(rows, count, target_dup, seed, tol=0.01):
+    """The exponent a for which `count` requests drawn Zipf(a) over `rows` ranks (zipf_requests) repeat an
+    earlier request with probability ~ target_dup (found by bisection on the measured duplicate fraction;
+    Zipf(1.1) itself gives about 0.8 at 2M requests over 50M rows)."""
+    lo, hi = 0.0, 2.0
+    a = 1.0
+    for _ in range(24):
+        a = 0.5 * (lo + hi)
+        dup = 1.0 - np.unique(zipf_requests(rows, count, a, seed)).size / count
+        if abs(dup - target_dup) <= tol:
+            break
+        if dup < target_dup:
+            lo = a
+        else:
+            hi = a
+    return a
+
+
+def row_content(torch, ids, dim):
+    """int16 payload (any bit pattern is a valid bf16 row) of the rows `ids` of a synthetic table: a function of
+    the row id alone, so that a gathered row can be checked without keeping a second copy of the table."""
+    base = (ids * 2654435761 % 65521).to(torch.int32).unsqueeze(1)
+    return ((base + torch.arange(dim, device=ids.device, dtype=torch.int32)) & 0x7FFF).to(torch.int16)
+
+
+def two_tier_table(torch, device, rows, dim, hot_frac, seed):
+    """A rows x dim int16 table whose hottest hot_frac of rows by access rank live on `device` and all rows
+    in pinned host memory; rank r maps to row rank_to_id[r] (a random permutation), content = row_content.
+    Returns (rank_to_id, hot_slot[int32], hot_table, cold_table)."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    hot_rows = int(rows * hot_frac)
+    rank_to_id = torch.randperm(rows, device=device, generator=g)
+    hot_slot = torch.full((rows,), -1, dtype=torch.int32, device=device)
+    hot_slot[rank_to_id[:hot_rows]] = torch.arange(hot_rows, dtype=torch.int32, device=device)
+    hot_tab = torch.empty((hot_rows, dim), dtype=torch.int16, device=device)
+    for lo in range(0, hot_rows, 1 << 20):
+        hot_tab[lo: lo + (1 << 20)] = row_content(torch, rank_to_id[lo: min(lo + (1 << 20), hot_rows)], dim)
+    cold = torch.empty((rows, dim), dtype=torch.int16, pin_memory=True)
+    for lo in range(0, rows, 1 << 22):
+        hi = min(lo + (1 << 22), rows)
+        cold[lo:hi].copy_(row_content(torch, torch.arange(lo, hi, device=device), dim))
+    torch.cuda.synchronize(device)
+    return rank_to_id, hot_slot, hot_tab, cold
