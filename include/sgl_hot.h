@@ -53,7 +53,8 @@ int32_t     sgl_abi_version(void);
 /* sizeof of the ABI's structs as this library was compiled, so that a binding
  * which mirrors them field by field (ctypes, cgo, JNI) can check its layout at
  * load time: which = 0 sgl_tcsr, 1 sgl_sample_params, 2 sgl_hop_out,
- * 3 sgl_cache, 4 sgl_gather_seg, 5 sgl_seed_query; 0 for any other index. */
+ * 3 sgl_cache, 4 sgl_gather_seg, 5 sgl_seed_query, 6 sgl_window_params;
+ * 0 for any other index. */
 size_t      sgl_struct_bytes(int32_t which);
 
 /* Kernels whose blocks exchange totals inside one launch (the 2-hop sampler of
@@ -235,6 +236,37 @@ int32_t sgl_sample_hop_static(const sgl_tcsr* g,
                               int64_t S_max, const int64_t* S_dev,
                               const sgl_sample_params* p, const sgl_hop_out* out,
                               void* stream);
+
+/* Whole-window sampling: every edge of a slot's time window, or the first k,
+ * optionally only those carrying a given tag.  Replaces the 'full' and
+ * 'cluster' layer types and the discrete-time branch of the offline sampler
+ * (_jit_sample_kernel, prepare_sample.py:32-172; cut_idx / start_idx :50-55,
+ * continuous cluster/full :62, :112-113, :131-132; discrete :65-76, :147-170).
+ * Window of a slot (v, t): edges e of row v with
+ *   (bounded_below ? t + lo_offset : -inf) <= ts[e] < t + hi_offset,
+ * candidates: all of them, or those with edge_tag[e] == tag_value when
+ * edge_tag != NULL ([m] device, in T-CSR order); taken: the first
+ * min(first_k, candidates) in storage order (first_k < 0: all).
+ * neighbors_ts = t when keep_slot_time (discrete snapshots) else ts[e];
+ * neighbors_dt = ts[e] - t.  Result layout as sgl_hop_out.
+ * The edge count is not bounded beforehand: called with out->neighbors ==
+ * NULL the function only counts (root_start_ptr, root_end_ptr and counts are
+ * written; counts[1] = E); the caller then allocates E edges and calls again.
+ * Should capacity_edges of that second call be below E, counts[2] reads
+ * INT64_MAX and the edge arrays are void. */
+typedef struct sgl_window_params {
+    int64_t        lo_offset, hi_offset;
+    int32_t        bounded_below;
+    int32_t        keep_slot_time;
+    int64_t        first_k;
+    const int64_t* edge_tag;   /* device [m] or NULL */
+    int64_t        tag_value;
+} sgl_window_params;
+size_t  sgl_sample_window_workspace_bytes(int64_t S);
+int32_t sgl_sample_window(const sgl_tcsr* g, const int64_t* slot_node,
+                          const int64_t* slot_ts, int64_t S,
+                          const sgl_window_params* p, const sgl_hop_out* out,
+                          void* workspace, size_t workspace_bytes, void* stream);
 
 /* k-hop driver (replaces Graph::sample_src_in_chunks_khop,
  * sample.cu.hpp:1532-1716).  Hop-0 slots are the positive roots expanded over

@@ -57,6 +57,7 @@ size_t      sglo_struct_bytes(int32_t which) {
         case 3: return sizeof(sgl_cache);
         case 4: return sizeof(sgl_gather_seg);
         case 5: return sizeof(sgl_seed_query);
+        case 6: return sizeof(sgl_window_params);
         default: return 0;
     }
 }
@@ -401,6 +402,52 @@ int32_t sglo_sample_hop_static(const sgl_tcsr* g, const int64_t* slot_node,
     return sglo_sample_hop(g, slot_node, slot_ts, S_max, S_dev, p, out, NULL, 0, stream);
 }
 
+
+/* Whole-window sampling.  Reference: _jit_sample_kernel (prepare_sample.py:32-172): cut_idx / start_idx
+ * = np.searchsorted (side='left') of t + end_offset / t + start_offset on the target's time-sorted edges
+ * (:50-55), 'cluster' and 'full' of a continuous graph take [0, cut_idx) (:62, :112-113, :131-132); the
+ * discrete branch takes [start_idx, cut_idx): every edge ('full'), the first `fanout` ('uniform', :68-70,
+ * :159-170) or the edges of one cluster (:65-67, :148-158), and reports the target's time as the edge time. */
+size_t sglo_sample_window_workspace_bytes(int64_t S) { (void)S; return 0; }
+
+int32_t sglo_sample_window(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot_ts, int64_t S,
+                           const sgl_window_params* p, const sgl_hop_out* out, void* ws, size_t ws_bytes,
+                           void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (!g || !p || !out || S < 0) return fail(SGL_EINVAL, "sample_window: null/negative");
+    if (out->capacity_slots < S) return fail(SGL_EINVAL, "sample_window: capacity_slots < S");
+    const int fill = out->neighbors != NULL;
+    int64_t acc = 0, bad = 0, overflow = 0;
+    for (int64_t s = 0; s < S; ++s) {
+        out->root_start_ptr[s] = acc;
+        int64_t v = slot_node[s], t = slot_ts[s];
+        if (v < 0 || v >= g->n) { bad++; out->root_end_ptr[s] = acc; continue; }
+        int64_t rs = g->row_ptr[v], re = g->row_ptr[v + 1];
+        int64_t hi = lower_bound_ts(g->ts, rs, re, t + p->hi_offset);
+        int64_t lo = p->bounded_below ? lower_bound_ts(g->ts, rs, hi, t + p->lo_offset) : rs;
+        if (lo > hi) lo = hi;
+        int64_t taken = 0;
+        for (int64_t e = lo; e < hi; ++e) {
+            if (p->edge_tag && p->edge_tag[e] != p->tag_value) continue;
+            if (p->first_k >= 0 && taken >= p->first_k) break;
+            if (fill) {
+                if (acc + taken >= out->capacity_edges) { overflow = 1; }
+                else {
+                    out->neighbors[acc + taken] = g->col[e];
+                    out->neighbors_ts[acc + taken] = p->keep_slot_time ? t : g->ts[e];
+                    out->neighbors_eid[acc + taken] = g->eid[e];
+                    out->neighbors_dt[acc + taken] = g->ts[e] - t;
+                }
+            }
+            taken++;
+        }
+        acc += taken;
+        out->root_end_ptr[s] = acc;
+    }
+    out->root_start_ptr[S] = acc; out->root_end_ptr[S] = acc;
+    out->counts[0] = S; out->counts[1] = acc; out->counts[2] = overflow ? INT64_MAX : bad;
+    return SGL_OK;
+}
 
 size_t sglo_sample_khop_workspace_bytes(int64_t S0, int32_t layers, int32_t fanout) {
     (void)S0; (void)layers; (void)fanout;

@@ -42,6 +42,7 @@ extern "C" size_t sgl_struct_bytes(int32_t which) {
         case 3: return sizeof(sgl_cache);
         case 4: return sizeof(sgl_gather_seg);
         case 5: return sizeof(sgl_seed_query);
+        case 6: return sizeof(sgl_window_params);
         default: return 0;
     }
 }

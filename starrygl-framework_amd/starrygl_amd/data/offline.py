@@ -14,11 +14,21 @@ The sampling (most recent / uniform before t over the in-edges of each target),
 the (id, ts) pair unique and the (destination, time) edge order run in
 libsgl_hot.so; only concatenations and permutation indexing are torch glue.
 
+Layer types (prepare_sample.py:57-76, 105-170), with the window of a target
+(v, t) = its in-edges with ts < t + meta['end_offset'] (continuous graphs:
+from the first edge; discrete graphs, meta graph_type != 'c': from
+t + meta['start_offset']):
+  continuous  'recent'  the last `fanout` window edges     'uniform' `fanout` of them at random
+              'full', 'cluster'  every window edge
+  discrete    'uniform' the first `fanout` window edges    'full' every window edge
+              'cluster' the window edges whose event cluster ('cid' of the partition data) is `cluster_ids`
+              'recent'  as 'full' (the reference counts the whole window for it and then writes nothing,
+                        prepare_sample.py:75, 147-170: its output arrays stay uninitialised)
+              every edge of a discrete layer reports the target's time as its own (edge_ts = t).
+
 Differences from the reference
   * `comm_plan` entries are None: routing plans between partitions belong to
     the multi-GPU exchange, which this library does not build;
-  * only the 'recent' and 'uniform' layer types of a continuous-time graph
-    (meta graph_type 'c') are supported;
   * uniform draws come from the library's counter-based generator (the
     reference draws from numpy's unseeded global generator).
 
@@ -56,19 +66,40 @@ class MaterializedMultiLayerBuilder:
         with torch.cuda.device(dev):
             g = hp.tcsr_build(self.num_nodes, dst, src, ts, torch.arange(m, device=dev))
             self.g = TCSRArrays(hp.be, self.num_nodes, g.row_ptr, g.col, g.ts, eid[g.eid])
+            # the events' cluster ids in the same order (sorted_cluster, prepare_sample.py:183, 198)
+            cid = _dev_i64(partition_data["cid"], dev) if "cid" in partition_data else torch.zeros(m, dtype=torch.int64, device=dev)
+            self.edge_cluster = cid[g.eid].contiguous()
 
     # ---- one layer -----------------------------------------------------------
-    def _sample_layer(self, target_nodes, target_ts, fanout, sample_type, seed):
+    def _sample_layer(self, target_nodes, target_ts, fanout, sample_type, seed, meta=None, cluster_id=None):
         """-> (raw_src, raw_dst, raw_ts, raw_dt, raw_eid) or None when no target has an in-edge at all
-        (prepare_sample.py:248-265)."""
+        (prepare_sample.py:248-265; the kernel's branches :57-76, :105-170)."""
         hp, g = self.hp, self.g
+        meta = meta or {}
+        if sample_type not in ("recent", "uniform", "cluster", "full"):
+            sample_type = "recent"                  # the reference's .get(sample_type, 0)
         if target_nodes.numel() == 0 or not bool((g.row_ptr[target_nodes + 1] > g.row_ptr[target_nodes]).any()):
             return None
-        p = hp.params(sample_type, int(fanout), seed=seed)
-        hop = hp.sample_hop(g, target_nodes, target_ts, p)
+        start_off, end_off = int(meta.get("start_offset", 0)), int(meta.get("end_offset", 0))
+        discrete = meta.get("graph_type", "c") != "c"
+        if not discrete and sample_type in ("recent", "uniform"):
+            # the k-hop sampler's windows end strictly before the slot time: shift it by end_offset
+            p = hp.params(sample_type, int(fanout), seed=seed)
+            hop = hp.sample_hop(g, target_nodes, target_ts + end_off if end_off else target_ts, p)
+        elif not discrete:                           # 'cluster' and 'full': every edge before the cut
+            hop = hp.sample_window(g, target_nodes, target_ts, hi_offset=end_off)
+        elif sample_type == "cluster":
+            hop = hp.sample_window(g, target_nodes, target_ts, lo_offset=start_off, hi_offset=end_off, keep_slot_time=True,
+                                   edge_tag=self.edge_cluster, tag_value=-1 if cluster_id is None else int(cluster_id))
+        else:                                        # discrete 'uniform': the first `fanout`; 'full' / 'recent': all
+            hop = hp.sample_window(g, target_nodes, target_ts, lo_offset=start_off, hi_offset=end_off, keep_slot_time=True,
+                                   first_k=int(fanout) if sample_type == "uniform" else -1)
         counts = torch.tensor([hop.S, hop.E, 0], device=self.device)
         raw_dst = hp.block_build(hop.root_start_ptr, counts, hop.S, hop.E, 0, 0, with_edge_dst=True)[2]
-        raw_dt = (-hop.neighbors_dt).to(torch.float32)          # t_cut - ts, prepare_sample.py:130, 145
+        if not discrete and sample_type in ("recent", "uniform") and end_off:
+            raw_dt = (target_ts[raw_dst[: hop.E]] - hop.neighbors_ts).to(torch.float32)
+        else:
+            raw_dt = (-hop.neighbors_dt).to(torch.float32)      # t_cut - ts, prepare_sample.py:130, 145
         return hop.neighbors, raw_dst[: hop.E], hop.neighbors_ts, raw_dt, hop.neighbors_eid
 
     def build_aligned_batch(self, task_param, save_path, layer_configs, num_neg=1, global_dst_pool=None,
@@ -76,8 +107,6 @@ class MaterializedMultiLayerBuilder:
         hp, dev = self.hp, self.device
         task_type, task_nodes = task_param
         meta = layer_configs.get("meta", {})
-        if meta.get("graph_type", "c") != "c":
-            raise NotImplementedError("discrete-time (snapshot) sampling is not part of this builder")
         extra = {}
         if task_type == "link":
             task_src, task_dst, task_ts, task_label, task_eid = task_nodes
@@ -109,12 +138,10 @@ class MaterializedMultiLayerBuilder:
             routes = [None]
             last_inv = None
             for l, cfg in enumerate(layer_configs["layer"]):
-                if cfg["type"] not in ("recent", "uniform"):
-                    raise NotImplementedError(f"layer type {cfg['type']!r} is not part of this builder")
                 target_u = curr_uid if last_inv is None else curr_uid[last_inv]
                 target_t = curr_uts if last_inv is None else curr_uts[last_inv]
-                raw = self._sample_layer(target_u, target_t, cfg["fanout"], cfg["type"],
-                                         seed=self.seed + 104729 * self._calls + l)
+                raw = self._sample_layer(target_u, target_t, cfg.get("fanout", 10), cfg["type"],
+                                         seed=self.seed + 104729 * self._calls + l, meta=meta, cluster_id=cluster_ids)
                 if raw is None:
                     e = curr_uid.new_empty(0)
                     batch.append({"indptr": curr_uid.new_zeros(1), "indices": e, "eid": e, "edge_ts": e,

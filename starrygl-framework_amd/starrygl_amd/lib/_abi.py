@@ -56,8 +56,13 @@ class SeedQuery(C.Structure):
                 ("cand_off", vp), ("n_cand", i64), ("t_begin", i64), ("t_end", i64)]
 
 
+class WindowParams(C.Structure):
+    _fields_ = [("lo_offset", i64), ("hi_offset", i64), ("bounded_below", i32), ("keep_slot_time", i32),
+                ("first_k", i64), ("edge_tag", vp), ("tag_value", i64)]
+
+
 # in the order of sgl_struct_bytes(which)
-STRUCTS = (TCSR, SampleParams, HopOut, Cache, GatherSeg, SeedQuery)
+STRUCTS = (TCSR, SampleParams, HopOut, Cache, GatherSeg, SeedQuery, WindowParams)
 
 
 P = C.POINTER
@@ -77,6 +82,8 @@ PROTOTYPES = {
     "sample_hop_workspace_bytes": (sz, [i64]),
     "sample_hop": (i32, [P(TCSR), vp, vp, i64, vp, P(SampleParams), P(HopOut), vp, sz, vp]),
     "sample_hop_static": (i32, [P(TCSR), vp, vp, i64, vp, P(SampleParams), P(HopOut), vp]),
+    "sample_window_workspace_bytes": (sz, [i64]),
+    "sample_window": (i32, [P(TCSR), vp, vp, i64, P(WindowParams), P(HopOut), vp, sz, vp]),
     "sample_khop_workspace_bytes": (sz, [i64, i32, i32]),
     "sample_khop": (i32, [P(TCSR), i64, vp, vp, i64, vp, i64, vp, vp, i32,
                           P(SampleParams), vp, vp, P(HopOut), vp, sz, vp]),

@@ -9,7 +9,7 @@ library with the same ABI on host memory.
 import ctypes as C
 
 from . import _abi
-from ._abi import (TCSR, Cache, GatherSeg, HopOut, SampleParams, SeedQuery, check, i64, vp)
+from ._abi import (TCSR, Cache, GatherSeg, HopOut, SampleParams, SeedQuery, WindowParams, check, i64, vp)
 
 
 class TorchBackend:
@@ -300,6 +300,28 @@ class HotPath:
         self._ck(self.lib.sample_hop_static(C.byref(g.view), be.ptr(slot_node), be.ptr(slot_ts), int(slot_node.shape[0]),
                                             be.ptr(S_dev), C.byref(p), C.byref(out.struct), be.stream()))
         return out
+
+    def sample_window(self, g, slot_node, slot_ts, lo_offset=None, hi_offset=0, first_k=-1, edge_tag=None,
+                      tag_value=0, keep_slot_time=False):
+        """Every edge of each slot's window [t + lo_offset (None: unbounded), t + hi_offset), or the first
+        `first_k` of them, optionally only edges whose `edge_tag` (an [m] array in T-CSR order) equals
+        `tag_value`.  Two library calls: count, then fill into arrays of the counted size.  -> HopResult."""
+        self._chk("i64", slot_node=slot_node, slot_ts=slot_ts, edge_tag=edge_tag)
+        be, S = self.be, int(slot_node.shape[0])
+        p = WindowParams(int(lo_offset or 0), int(hi_offset), int(lo_offset is not None), int(bool(keep_slot_time)),
+                         int(first_k), be.ptr(edge_tag), int(tag_value))
+        ws, wsb = self._workspace(self.lib.sample_window_workspace_bytes(S))
+        out = HopResult(be, S, 0)
+        count_only = HopOut(S, 0, be.ptr(out.root_start_ptr), be.ptr(out.root_end_ptr), None, None, None, None,
+                            be.ptr(out.counts))
+        self._ck(self.lib.sample_window(C.byref(g.view), be.ptr(slot_node), be.ptr(slot_ts), S, C.byref(p),
+                                        C.byref(count_only), be.ptr(ws), wsb, be.stream()))
+        _, E, bad = be.tolist(out.counts)
+        check_sample_bad(bad)
+        full = HopResult(be, S, E, counts=out.counts)
+        self._ck(self.lib.sample_window(C.byref(g.view), be.ptr(slot_node), be.ptr(slot_ts), S, C.byref(p),
+                                        C.byref(full.struct), be.ptr(ws), wsb, be.stream()))
+        return full.finalize(*be.tolist(full.counts))
 
     def khop_buffers(self, S0, layers, fanout, counts=None):
         """Worst-case output buffers of a k-hop call; reusable across calls.  `counts`

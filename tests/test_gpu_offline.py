@@ -18,13 +18,35 @@ def _pairs(ids, ts):
     return c
 
 
-def _want_batch(oracle, hg, l0_nodes, l0_ts, layers):
-    """prepare_sample.py:310-371 with numpy: np.unique over (id, ts) records, np.lexsort((ts, dst))."""
+def _want_layer(oracle, hg, tu, tt, cfg, meta, edge_cluster, cluster_id):
+    """One layer as the numba kernel defines it (prepare_sample.py:57-76, 105-170), sampled with the oracle:
+    -> (src, edge_ts, eid, dt = t - ts, per-target counts)."""
+    st, fanout = cfg["type"], cfg.get("fanout", 10)
+    so, eo = meta.get("start_offset", 0), meta.get("end_offset", 0)
+    if meta.get("graph_type", "c") == "c":
+        if st in ("recent", "uniform"):
+            hop = oracle.sample_hop(hg, tu, tt + eo, oracle.params(st, fanout))
+        else:
+            hop = oracle.sample_window(hg, tu, tt, hi_offset=eo)
+    elif st == "cluster":
+        hop = oracle.sample_window(hg, tu, tt, lo_offset=so, hi_offset=eo, keep_slot_time=True, edge_tag=edge_cluster,
+                                   tag_value=-1 if cluster_id is None else cluster_id)
+    else:
+        hop = oracle.sample_window(hg, tu, tt, lo_offset=so, hi_offset=eo, keep_slot_time=True,
+                                   first_k=fanout if st == "uniform" else -1)
+    return hop
+
+
+def _want_batch(oracle, hg, l0_nodes, l0_ts, layers, meta=None, edge_cluster=None, cluster_id=None):
+    """prepare_sample.py:310-371 with numpy: np.unique over (id, ts) records, np.lexsort((ts, dst)).
+    layers: fanouts of 'recent' layers, or layer config dicts."""
+    meta = meta or {}
+    layers = [l if isinstance(l, dict) else {"type": "recent", "fanout": l} for l in layers]
     u, inv = np.unique(_pairs(l0_nodes, l0_ts), return_inverse=True)
     cur_id, cur_ts = u["id"].copy(), u["ts"].copy()
     out = [dict(gids=cur_id, ts=cur_ts, inv_map=inv)]
     last_inv = None
-    for fanout in layers:
+    for cfg in layers:
         tu = cur_id if last_inv is None else cur_id[last_inv]
         tt = cur_ts if last_inv is None else cur_ts[last_inv]
         if tu.size == 0 or not (hg.row_ptr[tu + 1] > hg.row_ptr[tu]).any():
@@ -32,9 +54,11 @@ def _want_batch(oracle, hg, l0_nodes, l0_ts, layers):
             out.append(dict(indptr=np.zeros(1, np.int64), indices=e, eid=e, edge_ts=e, edge_dt=np.zeros(0, np.float32),
                             gids=e, ts=e))
             break
-        hop = oracle.sample_hop(hg, tu, tt, oracle.params("recent", fanout))
+        hop = _want_layer(oracle, hg, tu, tt, cfg, meta, edge_cluster, cluster_id)
         raw_dst = np.repeat(np.arange(tu.size), np.diff(hop.root_start_ptr))
-        raw_dt = (tt[raw_dst] - hop.neighbors_ts).astype(np.float32)
+        # t_cut - ts of the edge (prepare_sample.py:130, 145, 157), t_cut the target's own time whatever the offsets
+        raw_dt = (tt[raw_dst] - (tt[raw_dst] + hop.neighbors_dt if meta.get("graph_type", "c") != "c" or cfg["type"] in ("full", "cluster")
+                                 else hop.neighbors_ts)).astype(np.float32)
         dst_m = raw_dst if last_inv is None else last_inv[raw_dst]
         allp = np.unique(np.concatenate([_pairs(cur_id, cur_ts), _pairs(hop.neighbors, hop.neighbors_ts)]))
         nxt_inv = np.searchsorted(allp, _pairs(hop.neighbors, hop.neighbors_ts))
@@ -128,3 +152,39 @@ def test_neg_and_node_tasks_and_empty_history(hot, tmp_path):
     assert len(node) == 2 and node[1]["indptr"].tolist() == [0] and node[1]["gids"].numel() == 0
     with pytest.raises(ValueError):
         b.build_aligned_batch(("graph", None), None, cfg)
+
+
+@pytest.mark.parametrize("graph_type,types,meta", [
+    ("c", ["full", "recent"], {}),
+    ("c", ["cluster"], {"end_offset": 40}),
+    ("c", ["recent", "full"], {"end_offset": -25}),
+    ("d", ["uniform", "full"], {"start_offset": -300, "end_offset": 1}),
+    ("d", ["cluster", "uniform"], {"start_offset": -900, "end_offset": 0}),
+    ("d", ["recent"], {"start_offset": -120, "end_offset": 5}),
+])
+def test_every_layer_type_of_both_graph_modes(oracle, hot, graph_type, types, meta):
+    """'full' / 'cluster' layers and the discrete-time branch of the offline sampler (prepare_sample.py:57-76,
+    105-170) against the numpy restatement of the builder that samples with the oracle."""
+    rng = np.random.default_rng(12)
+    n, m = 300, 12_000
+    src, dst = rng.integers(0, n, m), rng.integers(0, n - 10, m)
+    ts = np.sort(rng.integers(0, 2000, m))
+    cid = rng.integers(0, 6, m)
+    b = offline.MaterializedMultiLayerBuilder(dict(src=src, dst=dst, ts=ts, cid=cid), n, device=hot.be.device)
+    hg = host_graph(oracle, n, dst, src, ts, np.arange(m))
+    edge_cluster = cid[hg.eid].astype(np.int64)        # the events' clusters in the graph's edge order
+    meta = dict(meta, graph_type=graph_type)
+    layers = [{"type": t, "fanout": 4} for t in types]
+    lo = 9000
+    node, t_node = dst[lo: lo + 150], ts[lo: lo + 150]
+    task = tuple(torch.from_numpy(np.ascontiguousarray(x)) for x in (node, t_node, np.zeros(150, np.int64)))
+    got = b.build_aligned_batch(("node", task), None, {"layer": layers, "meta": meta}, cluster_ids=2)
+    want = _want_batch(oracle, hg, node, t_node, layers, meta, edge_cluster, 2)
+    assert len(got) == len(want)
+    for l, (g, w) in enumerate(zip(got, want)):
+        for k, v in w.items():
+            assert np.array_equal(np_of(g[k]), v), (l, k)
+    assert got[1]["indices"].numel() > 0
+    if graph_type == "d":      # a discrete layer reports the target's time as the edge time
+        deg = np.diff(np_of(got[1]["indptr"]))
+        assert np.array_equal(np_of(got[1]["edge_ts"]), np.repeat(np_of(got[0]["ts"]), deg))

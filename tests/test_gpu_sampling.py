@@ -445,3 +445,25 @@ def test_wide_uniform_fanout_over_two_hops_and_flags(oracle, hot):
             hot.build_records(dg)
         for kw in (dict(), dict(replace=True), dict(keep_root_time=True), dict(allowed_offset=20_000)):
             _run_both(oracle, hot, g, dg, roots, ts_ptr, root_ts, e, e, 2, sample_type="uniform", fanout=100, seed=5, **kw)
+
+
+def test_sample_window_parity(oracle, hot):
+    """Whole-window sampling (the offline sampler's 'full' / 'cluster' layers and its discrete branch) against
+    the oracle: hub rows of 100k edges, empty windows, tags, first-k, both time conventions."""
+    (src, dst, ts, _), g, dg = _graph(oracle, hot, 800, 200_000, 1.1, 50_000, 19, hub=100_000)
+    rng = np.random.default_rng(7)
+    tag = rng.integers(0, 5, g.m).astype(np.int64)
+    d_tag = to_dev(hot, tag)
+    node = np.concatenate([np.full(20, 3), rng.integers(0, g.n, 3000)]).astype(np.int64)
+    t = rng.integers(-5, 50_010, node.shape[0]).astype(np.int64)
+    for kw in (dict(), dict(first_k=7), dict(lo_offset=-3000), dict(lo_offset=-500, hi_offset=1, first_k=40, keep_slot_time=True),
+               dict(tag_value=3, tagged=True), dict(tag_value=0, tagged=True, lo_offset=-8000, first_k=9, keep_slot_time=True)):
+        kw = dict(kw)
+        tagged = kw.pop("tagged", False)
+        want = oracle.sample_window(g, node, t, edge_tag=tag if tagged else None, **kw)
+        got = hot.sample_window(dg, to_dev(hot, node), to_dev(hot, t), edge_tag=d_tag if tagged else None, **kw)
+        assert_hop_equal(got, want, tag=str(kw))
+    bad = hot.sample_window(dg, to_dev(hot, np.array([1, 2])), to_dev(hot, np.array([5, 5])))      # tiny call
+    assert bad.S == 2
+    with pytest.raises(IndexError):
+        hot.sample_window(dg, to_dev(hot, np.array([1, g.n])), to_dev(hot, np.array([5, 5])))

@@ -400,3 +400,34 @@ def test_edge_records_are_the_four_arrays_side_by_side(oracle):
     assert np.array_equal(g.rec.reshape(-1, 4), np.stack([g.col, g.ts, g.eid, np.full(m, -1)], axis=1))
     oracle.build_hop_hint(g)          # the records follow the index
     assert np.array_equal(g.rec.reshape(-1, 4), np.stack([g.col, g.ts, g.eid, g.hop_hint], axis=1))
+
+
+def test_sample_window_is_brute_force(oracle):
+    """sample_window against list comprehensions over each row (the numba kernel's searchsorted windows,
+    prepare_sample.py:50-55): all edges, the first k, the edges of one tag, with and without a lower bound."""
+    rng = np.random.default_rng(14)
+    n, m = 30, 1500
+    src, dst, ts = rng.integers(0, n, m), rng.integers(0, n, m), rng.integers(0, 60, m)
+    g = host_graph(oracle, n, src, dst, ts)
+    tag = rng.integers(0, 4, m).astype(np.int64)          # per edge, in T-CSR order
+    node = rng.integers(0, n, 80).astype(np.int64)
+    t = rng.integers(-2, 65, 80).astype(np.int64)
+    for kw in (dict(), dict(first_k=3), dict(lo_offset=-10), dict(lo_offset=-7, hi_offset=2, first_k=5),
+               dict(edge_tag=tag, tag_value=2), dict(edge_tag=tag, tag_value=1, lo_offset=-20, first_k=2, keep_slot_time=True)):
+        got = oracle.sample_window(g, node, t, **kw)
+        want_n, want_ts, want_eid, want_dt, ptr = [], [], [], [], [0]
+        for v, tt in zip(node, t):
+            rs, re = g.row_ptr[v], g.row_ptr[v + 1]
+            lo_t = tt + kw["lo_offset"] if "lo_offset" in kw else -10**18
+            hi_t = tt + kw.get("hi_offset", 0)
+            es = [e for e in range(rs, re) if lo_t <= g.ts[e] < hi_t and ("edge_tag" not in kw or tag[e] == kw["tag_value"])]
+            if kw.get("first_k", -1) >= 0:
+                es = es[: kw["first_k"]]
+            want_n += [g.col[e] for e in es]
+            want_ts += [tt if kw.get("keep_slot_time") else g.ts[e] for e in es]
+            want_eid += [g.eid[e] for e in es]
+            want_dt += [g.ts[e] - tt for e in es]
+            ptr.append(len(want_n))
+        assert got.root_start_ptr.tolist() == ptr and got.root_end_ptr.tolist() == ptr[1:] + [ptr[-1]]
+        assert got.neighbors.tolist() == want_n and got.neighbors_ts.tolist() == want_ts
+        assert got.neighbors_eid.tolist() == want_eid and got.neighbors_dt.tolist() == want_dt
