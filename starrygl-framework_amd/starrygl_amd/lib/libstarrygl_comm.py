@@ -324,3 +324,112 @@ def from_edge_index(n, chunk_size, src, dst, ts, eid, mapper=None, stream=0, ran
         if hop_hint:
             hp.build_hop_hint(g)
     return CUDAGraph(hp, g, chunk_size, mapper, stream if isinstance(stream, torch.cuda.Stream) else None)
+
+
+class ShardTensor:
+    """A logical [rows, ...] tensor made of shards appended in row order, each either in this GPU's memory
+    (`target_device` = the GPU's index) or in pinned host memory read in place by the gather kernel
+    (`target_device` < 0); `st[indices]` gathers rows into a new device tensor.  The interface of the
+    reference's ShardTensor (csrc/include/starrygl/feature.cu.hpp:236-297 append, :298-422 operator[],
+    :713-750 bindings) on one GPU: shards on other GPUs, IPC sharing and NCCL exchange are not part of it."""
+
+    def __init__(self, device, ctx=None):
+        self._device = int(device.index if isinstance(device, torch.device) else device)
+        self._hp = hot_path(torch.device("cuda", self._device))
+        self._shards, self._where = [], []
+        self._tail_shape, self._dtype, self._cache = None, None, None
+
+    def append(self, tensor, target_device):
+        if not isinstance(tensor, torch.Tensor) or tensor.is_cuda:
+            raise RuntimeError("ShardTensor.append expects a CPU tensor")        # CHECK_CPU, feature.cu.hpp:238
+        if target_device >= 0 and int(target_device) != self._device:
+            raise RuntimeError(f"this build serves one GPU: a shard can live on device {self._device} or on the host (-1)")
+        t = tensor.contiguous()
+        if self._tail_shape is None:
+            self._tail_shape, self._dtype = tuple(t.shape[1:]), t.dtype
+        elif tuple(t.shape[1:]) != self._tail_shape or t.dtype != self._dtype:
+            raise RuntimeError("ShardTensor.append: shards differ in row shape or dtype")
+        if (t.numel() // max(t.shape[0], 1)) * t.element_size() % 4 != 0:
+            raise RuntimeError("ShardTensor: the row size must be a multiple of 4 bytes")
+        self._shards.append(t.to(self._hp.be.device) if target_device >= 0 else (t if t.is_pinned() else t.pin_memory()))
+        self._where.append(int(target_device))
+        self._cache = None
+
+    def _build(self):
+        dev = self._hp.be.device
+        rows = [int(s.shape[0]) for s in self._shards]
+        total = sum(rows)
+        row_elems = 1
+        for d in self._tail_shape:
+            row_elems *= int(d)
+        host = [s.reshape(s.shape[0], row_elems) for s, w in zip(self._shards, self._where) if w < 0]
+        devs = [s.reshape(s.shape[0], row_elems) for s, w in zip(self._shards, self._where) if w >= 0]
+        n_host = sum(int(s.shape[0]) for s in host)
+        # local row space: host rows first (their rows of the cold table), then the device rows
+        g2l = torch.empty(total, dtype=torch.int64)
+        h_off, d_off, lo = 0, n_host, 0
+        for r, w in zip(rows, self._where):
+            if w < 0:
+                g2l[lo: lo + r] = torch.arange(h_off, h_off + r)
+                h_off += r
+            else:
+                g2l[lo: lo + r] = torch.arange(d_off, d_off + r)
+                d_off += r
+            lo += r
+        slot = torch.full((total,), -1, dtype=torch.int32)
+        slot[n_host:] = torch.arange(total - n_host, dtype=torch.int32)
+        cold = None
+        if host:
+            cold = host[0] if len(host) == 1 else torch.cat(host).pin_memory()
+        if not devs:      # (one placeholder row: the cache wants a device table)
+            hot = torch.zeros((1, row_elems), dtype=self._dtype, device=dev)
+        else:
+            hot = torch.cat(devs) if len(devs) != 1 else devs[0]
+        self._keep = (hot, cold)
+        self._cache = self._hp.cache(row_elems * self._shards[0].element_size(), hot, rows=total, cold=cold,
+                                     hot_slot=slot.to(dev) if cold is not None else None,
+                                     g2l=g2l.to(dev) if cold is not None else None)
+        self._rows, self._row_elems = total, row_elems
+
+    def __getitem__(self, indices):
+        if not self._shards:
+            raise RuntimeError("ShardTensor is empty")
+        if self._cache is None:
+            self._build()
+        ids = _i64(indices, self._hp.be.device, "indices").reshape(-1)
+        out = torch.empty((ids.numel(), self._row_elems), dtype=self._dtype, device=self._hp.be.device)
+        if ids.numel():
+            self._hp.gather(self._cache, ids, out)
+        return out.reshape((ids.numel(),) + self._tail_shape)
+
+    def shape(self):
+        return [sum(int(s.shape[0]) for s in self._shards)] + list(self._tail_shape or ())
+
+    def size(self, dim):
+        return self.shape()[dim]
+
+    def numel(self):
+        n = 1
+        for d in self.shape():
+            n *= d
+        return n
+
+    def stride(self, dim):
+        st = 1
+        for d in self.shape()[dim + 1:]:
+            st *= d
+        return st
+
+    def device(self):
+        return self._device
+
+    def device_count(self):
+        return len(self._shards)
+
+    def unregister(self, tensor=None):
+        """Drop the shards (the reference un-registers its zero-copy host mappings here)."""
+        self._shards, self._where, self._cache, self._keep = [], [], None, None
+
+    def share_ipc(self):
+        raise NotImplementedError("sharing shards between processes is part of the multi-GPU exchange, which this "
+                                  "one-GPU build does not contain")

@@ -348,3 +348,32 @@ def test_seeds_heavy_windows_and_tile_boundaries(oracle, hot, n, t_max):
                 assert np.array_equal(np_of(a), b), (f, chunks, t0, t1)
             # the sixth array is what a window-end lookup of every (root, timestamp) gives
             assert np.array_equal(want[5], oracle.window_end(hg, np.repeat(want[0], np.diff(want[1])), want[2]))
+
+
+def test_shard_tensor_gathers_rows_of_device_and_host_shards(hot):
+    """ShardTensor (feature.cu.hpp:236-422): shards appended in row order, some in HBM, some in pinned host
+    memory; st[indices] equals indexing the concatenation."""
+    from starrygl_amd.lib.libstarrygl_comm import ShardTensor
+    torch.manual_seed(0)
+    parts = [torch.randn(700, 25), torch.randn(1200, 25), torch.randn(300, 25), torch.randn(50, 25)]
+    full = torch.cat(parts)
+    for where in ([0, -1, 0, -1], [0, 0, 0, 0], [-1, -1, -1, -1], [-1, 0, -1, 0]):
+        st = ShardTensor(0)
+        for p, w in zip(parts, where):
+            st.append(p, w)
+        assert st.shape() == [2250, 25] and st.size(0) == 2250 and st.numel() == 2250 * 25 and st.stride(0) == 25
+        assert st.device() == 0 and st.device_count() == 4
+        idx = torch.randint(0, 2250, (5000,))
+        got = st[idx.cuda()]
+        assert got.is_cuda and torch.equal(got.cpu(), full[idx])
+        assert torch.equal(st[idx][:10].cpu(), full[idx][:10])          # host indices are moved over
+    st3 = ShardTensor(0)
+    st3.append(torch.arange(24, dtype=torch.float32).reshape(4, 2, 3), -1)     # rows of any trailing shape
+    assert torch.equal(st3[torch.tensor([3, 0])].cpu(), torch.arange(24, dtype=torch.float32).reshape(4, 2, 3)[[3, 0]])
+    with pytest.raises(RuntimeError):
+        st3.append(torch.zeros(2, 5), -1)
+    with pytest.raises(RuntimeError):
+        st3.append(torch.zeros(2, 2, 3), 1)                                    # another GPU
+    st3.unregister()
+    with pytest.raises(RuntimeError):
+        st3[torch.tensor([0])]
