@@ -20,7 +20,9 @@
 //             remembers the table slot of its id (4 bytes), so nothing is ever
 //             probed twice.  The ids a block added are appended - id and slot -
 //             to the call's list with ONE returning atomic per block; OR and
-//             AND over them are kept;
+//             AND over them are kept.  In grouped mode (an id belongs to the first
+//             array that holds it) the arrays are inserted by one launch each, in
+//             array order, so the ids an array adds are exactly those new to it;
 //   order   : the new ids have to be numbered in ascending order.  The bits in
 //             which they differ at all (OR ^ AND) are squeezed together into a
 //             short key that keeps the order (in grouped mode the array that
@@ -52,7 +54,6 @@ constexpr int MAXG = 8;
 constexpr unsigned long long EMPTY = ~0ull;
 constexpr uint32_t NONE = 0xFFFFFFFFu;   // slot of an element whose id is negative
 constexpr uint32_t UNNUMBERED = 0x7FFFFFFFu;  // value of a slot whose id has no local id yet
-constexpr uint32_t PENDING0 = 0x7FFFFFE0u;    // PENDING0 + g: not numbered yet, first seen in array g (grouped mode)
 constexpr int64_t MAX_CAPACITY = 0x7FFFFF00ll;
 constexpr int NB_MIN_LOG = 8, NB_MAX_LOG = 15;   // buckets of the atomic route: 32 consecutive counters per scan thread
 constexpr int64_t ATOMIC_ROUTE_MAX = 1ll << 20;  // most ids a call may add for the atomic route to be taken
@@ -68,21 +69,20 @@ struct Header {
     unsigned long long total;     // ids numbered in the current epoch (committed by the last launch of a call)
     unsigned long long nbig;      // oversized buckets of the running call (0 between calls)
     unsigned long long pad0[14];
-    unsigned long long appended;  // ids the running call has added (0 between calls)
-    unsigned long long pad1[15];
+    struct { unsigned long long n, pad[15]; } added[MAXG];   // ids the running call has added, per array group (0 between calls)
     unsigned long long or_mask;   // OR / AND over the ids the running call has added (0 / ~0 between calls)
     unsigned long long and_mask;
     unsigned long long pad2[14];
     unsigned long long overflow;  // sticky: more ids than the capacity, or no free slot
     unsigned long long pad3[15];
 };
-constexpr size_t HEADER_BYTES = 512;
+constexpr size_t HEADER_BYTES = 384 + 128 * MAXG;
 static_assert(sizeof(Header) == HEADER_BYTES, "hashed state header layout");
 
 struct Table {
     Header* hdr;
     unsigned long long* keys;   // [slots]
-    uint32_t* vals;             // [slots] local id, UNNUMBERED or PENDING0 + g
+    uint32_t* vals;             // [slots] local id, or UNNUMBERED
     uint32_t* used;             // [capacity] slot of the k-th id of the epoch
     int64_t capacity, slots;
 };
@@ -209,11 +209,31 @@ __device__ __forceinline__ bool locate(const Arrays& a, int64_t t, int* g_out, i
 // What a call works with: ids numbered before it and (from the order launches on) ids it added.
 __device__ __forceinline__ int64_t ids_before(const Table& t, int reset) { return reset ? 0 : (int64_t)t.hdr->total; }
 __device__ __forceinline__ int64_t ids_added(const Table& t, const Scratch& s, int64_t before) {
-    int64_t n = (int64_t)t.hdr->appended;
+    int64_t n = 0;
+#pragma unroll
+    for (int g = 0; g < MAXG; ++g) n += (int64_t)t.hdr->added[g].n;
     const int64_t room = t.capacity - before;
     if (n > room) n = room;
     if (n > s.ncap) n = s.ncap;
     return n < 0 ? 0 : n;
+}
+// array group of the k-th id the call added (groups are appended one after the other)
+__device__ __forceinline__ uint32_t group_of(const Table& t, int64_t k) {
+    uint32_t g = 0;
+    int64_t end = 0;
+#pragma unroll
+    for (int q = 0; q < MAXG - 1; ++q) {
+        end += (int64_t)t.hdr->added[q].n;
+        g += k >= end ? 1u : 0u;
+    }
+    return g;
+}
+__device__ __forceinline__ void clear_call_fields(Header* h) {
+#pragma unroll
+    for (int g = 0; g < MAXG; ++g) h->added[g].n = 0;
+    h->or_mask = 0;
+    h->and_mask = ~0ull;
+    h->nbig = 0;
 }
 
 __global__ __launch_bounds__(BLOCK) void init_kernel(Table t) {
@@ -224,11 +244,8 @@ __global__ __launch_bounds__(BLOCK) void init_kernel(Table t) {
     }
     if (tid == 0) {
         t.hdr->total = 0;
-        t.hdr->appended = 0;
-        t.hdr->or_mask = 0;
-        t.hdr->and_mask = ~0ull;
         t.hdr->overflow = 0;
-        t.hdr->nbig = 0;
+        clear_call_fields(t.hdr);
     }
 }
 
@@ -256,29 +273,28 @@ __global__ __launch_bounds__(BLOCK) void prep_kernel(Table t, Scratch s, int fre
     }
     if (fresh && tid == 0) {
         t.hdr->total = 0;
-        t.hdr->appended = 0;
-        t.hdr->or_mask = 0;
-        t.hdr->and_mask = ~0ull;
         t.hdr->overflow = 0;
-        t.hdr->nbig = 0;
+        clear_call_fields(t.hdr);
     }
 }
 
 // IPT ids per thread: a tile of 256 * IPT ids per block (small calls take small tiles so that the chip has
 // blocks to run; large ones take large tiles, which fold more repeats before the table is touched).
+// grp: the array group whose ids this launch adds (grouped mode: one launch per array, in array order, so that
+// an id belongs to the first array that holds it; otherwise one launch, group 0, over all arrays).  flat_base:
+// index of the launch's first element among the elements of all arrays (slot_of is indexed over all of them).
 template <int IPT>
-__global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratch s, int reset, int grouped) {
+__global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratch s, int reset, int grp, int64_t flat_base) {
     constexpr int TILE = BLOCK * IPT;
     constexpr int LDS_SLOTS = 2 * TILE;      // load <= 0.5
     __shared__ unsigned long long s_key[LDS_SLOTS];
-    __shared__ uint32_t s_aux[LDS_SLOTS];       // first the smallest array index that holds the id, then its table slot
+    __shared__ uint32_t s_aux[LDS_SLOTS];       // table slot of the id
     __shared__ int32_t s_won;
     __shared__ long long s_base;
     __shared__ unsigned long long s_or, s_and;
 #pragma unroll
     for (int q = 0; q < LDS_SLOTS / BLOCK; ++q) {
         s_key[q * BLOCK + threadIdx.x] = EMPTY;
-        s_aux[q * BLOCK + threadIdx.x] = MAXG;
     }
     if (threadIdx.x == 0) {
         s_won = 0;
@@ -288,17 +304,14 @@ __global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratc
     const int64_t t0 = (int64_t)blockIdx.x * TILE + threadIdx.x;
     // the tile's ids (every load issued before the first LDS probe)
     int64_t id[IPT];
-    int32_t grp[IPT];
+    bool live[IPT];
 #pragma unroll
     for (int q = 0; q < IPT; ++q) {
         id[q] = -1;
-        grp[q] = -1;                      // -1: no element
         int g;
         int64_t i;
-        if (locate(a, t0 + (int64_t)q * BLOCK, &g, &i)) {
-            id[q] = a.ids[g][i];
-            grp[q] = g;
-        }
+        live[q] = locate(a, t0 + (int64_t)q * BLOCK, &g, &i);
+        if (live[q]) id[q] = a.ids[g][i];
     }
     __syncthreads();
     int32_t ls[IPT];                      // LDS slot of the id; -1: negative id or no element
@@ -316,9 +329,7 @@ __global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratc
             h = (h + 1) & (LDS_SLOTS - 1);
         }
         ls[q] = (int32_t)h;
-        if (grouped) atomicMin(&s_aux[h], (uint32_t)grp[q]);
     }
-    if (grouped) __syncthreads();          // an owner needs the smallest array index of its id
     // every owner finds or claims the table slot of its id: first probes of all its ids in flight together
     const int64_t before = ids_before(t, reset);
     uint64_t h[IPT];
@@ -342,7 +353,6 @@ __global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratc
         pos[q] = 0;
         if (!owner[q]) continue;
         const unsigned long long me = (unsigned long long)id[q];
-        const uint32_t g_min = s_aux[ls[q]];
         unsigned long long k = k0[q];
         bool placed = false;
         for (int64_t probes = 0; probes < t.slots; ++probes) {
@@ -367,9 +377,6 @@ __global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratc
             continue;
         }
         s_aux[ls[q]] = (uint32_t)h[q];
-        // grouped: an id that has no local id yet belongs to the first array that holds it (a local id is
-        // smaller than every PENDING value, so ids of earlier calls keep theirs)
-        if (grouped) atomicMin(&t.vals[h[q]], PENDING0 + g_min);
         if (won[q]) {
             pos[q] = atomicAdd(&s_won, 1);
             my_or |= me;
@@ -383,7 +390,9 @@ __global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratc
     if (lost) atomicOr(&t.hdr->overflow, 1ull);
     __syncthreads();
     if (threadIdx.x == 0 && s_won > 0) {
-        s_base = (long long)atomicAdd(&t.hdr->appended, (unsigned long long)s_won);
+        long long prev = 0;                 // ids added by the launches of the groups before this one
+        for (int g = 0; g < grp; ++g) prev += (long long)t.hdr->added[g].n;
+        s_base = prev + (long long)atomicAdd(&t.hdr->added[grp].n, (unsigned long long)s_won);
         // the two masks settle after the first few blocks: an atomic only when this block still changes them
         // (they move one way only, so a stale reading costs a redundant atomic, never a missing one)
         if (s_or & ~__hip_atomic_load(&t.hdr->or_mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicOr(&t.hdr->or_mask, s_or);
@@ -400,7 +409,7 @@ __global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratc
                 t.used[before + k] = (uint32_t)h[q];
             }
         }
-        if (grp[q] >= 0) s.slot_of[t0 + (int64_t)q * BLOCK] = ls[q] < 0 ? NONE : s_aux[ls[q]];
+        if (live[q]) s.slot_of[flat_base + t0 + (int64_t)q * BLOCK] = ls[q] < 0 ? NONE : s_aux[ls[q]];
     }
 }
 
@@ -464,12 +473,6 @@ __device__ __forceinline__ uint32_t bucket_of(const Codec& c, uint64_t id, uint3
     return (g << kb) | (uint32_t)top;
 }
 
-__device__ __forceinline__ uint32_t group_of(const Table& t, uint32_t slot, int grouped) {
-    if (!grouped) return 0;
-    const uint32_t g = t.vals[slot] - PENDING0;
-    return g < (uint32_t)MAXG ? g : 0;
-}
-
 // ---- atomic route -------------------------------------------------------------------------------
 __global__ __launch_bounds__(BLOCK) void hist_kernel(Table t, Scratch s, int reset, int grouped, int glog) {
     __shared__ Codec s_codec;
@@ -479,7 +482,7 @@ __global__ __launch_bounds__(BLOCK) void hist_kernel(Table t, Scratch s, int res
     const int64_t before = ids_before(t, reset);
     const int64_t n = ids_added(t, s, before);
     for (int64_t k = (int64_t)blockIdx.x * BLOCK + threadIdx.x; k < n; k += (int64_t)gridDim.x * BLOCK) {
-        const uint32_t g = grouped ? group_of(t, t.used[before + k], 1) : 0;
+        const uint32_t g = grouped ? group_of(t, k) : 0;
         const uint32_t b = bucket_of(c, s.list_id[k], g, s.nb_log, glog);
         s.list_b[k] = b;
         atomicAdd(&s.cnt[b], 1u);
@@ -643,7 +646,7 @@ __global__ __launch_bounds__(BLOCK) void sortkey_kernel(Table t, Scratch s, int 
     if (blockIdx.x == 0 && threadIdx.x == 0) *n_out = n;      // the sort's live length
     for (int64_t k = (int64_t)blockIdx.x * BLOCK + threadIdx.x; k < n; k += (int64_t)gridDim.x * BLOCK) {
         const uint32_t slot = t.used[before + k];
-        const uint32_t b = bucket_of(c, s.list_id[k], group_of(t, slot, grouped), SORT_KEY_LOG, glog);
+        const uint32_t b = bucket_of(c, s.list_id[k], grouped ? group_of(t, k) : 0, SORT_KEY_LOG, glog);
         s.key_a[k] = ((uint64_t)b << SORT_KEY_SHIFT) | slot;
     }
 }
@@ -724,10 +727,7 @@ __global__ __launch_bounds__(BLOCK) void lookup_kernel(Arrays a, Table t, Scratc
         U_dev[0] = void_result ? INT64_MAX : before + n;
         U_dev[1] = before;
         t.hdr->total = (unsigned long long)(before + n);
-        t.hdr->appended = 0;
-        t.hdr->or_mask = 0;
-        t.hdr->and_mask = ~0ull;
-        t.hdr->nbig = 0;
+        clear_call_fields(t.hdr);
     }
     for (int64_t x = i0; x < a.start[a.G]; x += (int64_t)gridDim.x * BLOCK) {
         int g;
@@ -737,7 +737,7 @@ __global__ __launch_bounds__(BLOCK) void lookup_kernel(Arrays a, Table t, Scratc
         int64_t local = -1;
         if (h != NONE) {
             const uint32_t v = t.vals[h];
-            if (v < PENDING0) local = (int64_t)v;
+            if (v != UNNUMBERED) local = (int64_t)v;
         }
         a.out[g][i] = local;
     }
@@ -749,7 +749,7 @@ int32_t check_capacity(int64_t capacity) {
     return SGL_OK;
 }
 
-using InsertKernel = void (*)(Arrays, Table, Scratch, int, int);
+using InsertKernel = void (*)(Arrays, Table, Scratch, int, int, int64_t);
 
 int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const int64_t* const* ids, const int64_t* len_max,
             const int64_t* const* len_dev, int64_t* const* local_out, int64_t* unique_out, int64_t unique_capacity,
@@ -785,12 +785,31 @@ int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const i
     if (total > 0) {
         // tile of the insert: 1024 ids per block (larger tiles fold more repeats before the table is touched but
         // leave fewer waves per compute unit to hide the table's latency: 2048 ids per block is 10 % slower
-        // on 15.6M ids); small calls take smaller tiles so that the chip still has a few hundred blocks
-        int ipt = 4;
-        while (ipt > 1 && total / (BLOCK * ipt) < 256) ipt >>= 1;
-        const InsertKernel ins = ipt == 4 ? insert_kernel<4> : ipt == 2 ? insert_kernel<2> : insert_kernel<1>;
-        hipLaunchKernelGGL(ins, dim3((unsigned)ceil_div<int64_t>(total, BLOCK * ipt)), dim3(BLOCK), 0, st, all, t, s, reset, grouped);
-        SGL_LAUNCH_CHECK();
+        // on 15.6M ids); small launches take smaller tiles so that the chip still has a few hundred blocks
+        auto launch_insert = [&](const Arrays& arr, int64_t n, int grp, int64_t flat_base) -> int32_t {
+            int ipt = 4;
+            while (ipt > 1 && n / (BLOCK * ipt) < 256) ipt >>= 1;
+            const InsertKernel ins = ipt == 4 ? insert_kernel<4> : ipt == 2 ? insert_kernel<2> : insert_kernel<1>;
+            hipLaunchKernelGGL(ins, dim3((unsigned)ceil_div<int64_t>(n, BLOCK * ipt)), dim3(BLOCK), 0, st, arr, t, s, reset, grp, flat_base);
+            SGL_LAUNCH_CHECK();
+            return SGL_OK;
+        };
+        int32_t rc_ins = SGL_OK;
+        if (!grouped) {
+            rc_ins = launch_insert(all, total, 0, 0);
+        } else {
+            for (int g = 0; g < G && rc_ins == SGL_OK; ++g) {   // array by array: an id belongs to the first array that holds it
+                if (all.len_max[g] == 0) continue;
+                Arrays sub = all;
+                sub.G = 1;
+                sub.ids[0] = all.ids[g]; sub.out[0] = all.out[g];
+                sub.len_dev[0] = all.len_dev[g]; sub.len_max[0] = all.len_max[g];
+                sub.start[0] = 0;
+                for (int q = 1; q <= MAXG; ++q) sub.start[q] = sub.len_max[0];
+                rc_ins = launch_insert(sub, sub.len_max[0], g, all.start[g]);
+            }
+        }
+        if (rc_ins != SGL_OK) return rc_ins;
         if (!s.radix) {
             hipLaunchKernelGGL(hist_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, grouped, glog);
             SGL_LAUNCH_CHECK();
