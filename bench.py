@@ -249,6 +249,22 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     res["gather_memory_30pct_host"] = {"ms": round(ms, 4), "rows": u1, "GBps": round(u1 * (8 + 4 + 800 + 16) / ms / 1e6, 1)}
     ms = _time_launches(torch, lambda: hot.gather_multi(plan))
     res["gather_all_three_one_launch"] = {"ms": round(ms, 4), "GBps": round((u1 * (2 * 812 + 16) + e1 * 1384) / ms / 1e6, 1)}
+    # the launch is bound by the rows that cross PCIe: memory rows (400 B + 8 B last update) and node rows (400 B) of the
+    # unique nodes whose owner is remote.  Host memory is read in 128-byte lines: a 400-byte row at a 16-byte-aligned
+    # offset always spans 4 of them (512 B), its 8-byte time another one.
+    st3 = hot.be.zeros(3)
+    hot.gather(c_mem, ubuf, o_mem, out_ts=o_ts, N_dev=U[0:1], stats=st3)
+    n_cold = int(st3[1].item())
+    cold_alg, cold_lines = n_cold * (400 + 8 + 400), n_cold * (512 + 128 + 512)
+    probe = torch.empty(cold_alg, dtype=torch.uint8, device=dev)
+    src_h = mem_cold.view(torch.uint8).reshape(-1)[:cold_alg]
+    ms_cp = _time_launches(torch, lambda: probe.copy_(src_h, non_blocking=True), reps=5)
+    res["gather_all_three_one_launch"].update({
+        "cold_rows": n_cold, "cold_bytes": cold_alg, "cold_GBps": round(cold_alg / ms / 1e6, 2),
+        "cold_GBps_in_128B_lines": round(cold_lines / ms / 1e6, 2),
+        "memcpy_h2d_same_bytes_GBps": round(cold_alg / ms_cp / 1e6, 2),
+        "cold_rate_over_memcpy": round(ms_cp / ms, 3), "line_rate_over_memcpy": round(cold_lines / cold_alg * ms_cp / ms, 3)})
+    del probe
     p_h = hot.with_root_hint(p, s_in[4])
     ms = _time_launches(torch, lambda: hot.sample_khop(dg, s_in[0], ts_ptr, s_in[1], s_in[2], s_in[3], 1, p_h, finalize=False, out=kr))
     res["sample_recent_1hop"] = {"ms": round(ms, 4), "edges_per_s": round(e1 / ms * 1e3, 1)}

@@ -12,6 +12,8 @@
 //   prep    : empties the table (everything for a workspace table; for a
 //             persistent one only on reset, and then only the slots the last
 //             epoch used when those are few) and zeroes the bucket counters;
+//             for calls of up to 2^20 ids it also leaves OR and AND over the
+//             call's ids, one pair per block, for the insert to fold;
 //   insert  : a block folds its tile of ids through an LDS set, so an id that
 //             repeats inside the tile reaches the global table once; the
 //             element that put an id into the LDS set probes the table for it
@@ -20,7 +22,14 @@
 //             remembers the table slot of its id (4 bytes), so nothing is ever
 //             probed twice.  The ids a block added are appended - id and slot -
 //             to the call's list with ONE returning atomic per block; OR and
-//             AND over them are kept.  In grouped mode (an id belongs to the first
+//             AND over them are kept.  Calls of up to 2^20 ids are bound by the
+//             chain of round trips, not by the number of atomics: their probes
+//             are an atomicCAS straight away (one round trip per probe instead
+//             of two), the table is sparser (load <= 1/3), and the insert
+//             itself counts the bucket sizes (the squeezed key below is then
+//             made from the bits in which the call's ids differ, known from
+//             prep, a superset of the bits in which the new ones do).
+//             In grouped mode (an id belongs to the first
 //             array that holds it) the arrays are inserted by one launch each, in
 //             array order, so the ids an array adds are exactly those new to it;
 //   order   : the new ids have to be numbered in ascending order.  The bits in
@@ -28,21 +37,26 @@
 //             short key that keeps the order (in grouped mode the array that
 //             owns the id is the top digit), and the top bits of that key cut
 //             the ids into buckets of a few ids each:
-//             - calls of up to 2^20 ids: hist (bucket sizes by spread atomics),
-//               scan (one block), scatter (ids move to their bucket's segment);
+//             - calls of up to 2^20 ids: the insert counts the bucket sizes with one
+//               returning atomic per new id (what comes back is the id's place inside
+//               its bucket); scatter moves the ids to their bucket's segment, every
+//               block making the prefix of the at most 8192 sizes for itself in LDS
+//               (its first block leaves the first places and the list of oversized
+//               buckets in memory for the numbering launch);
 //             - larger calls, where an atomic per id costs more than a pass
 //               over the data: three 8-bit passes of the library's radix sort
 //               on the top 24 bits of the key;
 //   number  : an id's rank = first place of its bucket + ids of the bucket
-//             that are smaller (a handful); rank + ids numbered before = local
-//             id, written to the table and the local->global list.  Oversized
-//             buckets (skewed id distributions) are sorted by a block each with
-//             a bitonic network in place;
+//             that are smaller (a handful, compared from a tile of ids parked in
+//             LDS); rank + ids numbered before = local id, written to the table and
+//             the local->global list.  Oversized buckets (skewed id distributions)
+//             are sorted by a block each with a bitonic network in place;
 //   lookup  : out[i] = local id at the slot element i remembered.
 //
 // Numbering is by ascending id inside each group, so the result equals the dense
 // path and the reference's sort + unique (csrc/include/starrygl/sample.cu.hpp:
 // 1786-1852) bit for bit.
+#include <algorithm>
 #include "common.hpp"
 #include "radix.hpp"
 
@@ -55,12 +69,14 @@ constexpr unsigned long long EMPTY = ~0ull;
 constexpr uint32_t NONE = 0xFFFFFFFFu;   // slot of an element whose id is negative
 constexpr uint32_t UNNUMBERED = 0x7FFFFFFFu;  // value of a slot whose id has no local id yet
 constexpr int64_t MAX_CAPACITY = 0x7FFFFF00ll;
-constexpr int NB_MIN_LOG = 8, NB_MAX_LOG = 15;   // buckets of the atomic route: 32 consecutive counters per scan thread
+constexpr int NB_MIN_LOG = 8, NB_MAX_LOG = 13;   // buckets of the atomic route: at least one per thread of a block, at most what a block scans in LDS
 constexpr int64_t ATOMIC_ROUTE_MAX = 1ll << 20;  // most ids a call may add for the atomic route to be taken
 constexpr int SORT_KEY_LOG = 24;         // bucket bits of the radix route (three 8-bit passes)
 constexpr int SORT_KEY_SHIFT = 64 - SORT_KEY_LOG;
 constexpr int SMALL_BUCKET = 512;        // buckets up to this size are ranked by counting
-constexpr int SCAN_BLOCK = 1024;
+constexpr int IDS_PER_BUCKET = 32;      // of the atomic route, when every id of the call is new
+constexpr int64_t SPARSE_CAPACITY = 1ll << 20;   // tables up to this capacity are three times the capacity
+constexpr int NMASK = BLOCK;             // most blocks of prep that leave an OR / AND pair
 constexpr int MAX_GRID = 4096;
 
 // Every field that blocks of one launch hammer with atomics has a 128-byte line of its own: a line that
@@ -87,7 +103,8 @@ struct Table {
     int64_t capacity, slots;
 };
 
-int64_t slots_of(int64_t capacity) { return capacity + capacity / 2 + 64; }
+// (small tables are cheap to empty, and a short probe sequence is what a small call's time is made of)
+int64_t slots_of(int64_t capacity) { return (capacity <= SPARSE_CAPACITY ? 3 * capacity : capacity + capacity / 2) + 64; }
 
 size_t state_bytes(int64_t capacity) {
     const int64_t s = slots_of(capacity);
@@ -115,11 +132,13 @@ struct Scratch {
     uint32_t* slot_of;          // [total] table slot of every input element (NONE: negative id)
     unsigned long long* list_id;  // [ncap] ids added by this call, in the order of their appends
     uint32_t* list_b;           // [ncap] their buckets
+    uint32_t* list_r;           // [ncap] how many ids the bucket held when they were counted into it
     unsigned long long* part_id;  // [ncap] the same ids grouped by bucket
     uint32_t* part_slot;        // [ncap]
     uint32_t* part_b;           // [ncap]
-    uint32_t* cnt;              // [nb + 1] bucket sizes, later the scatter cursors
-    uint32_t* off;              // [nb + 1] bucket offsets
+    uint32_t* cnt;              // [nb + 1] bucket sizes
+    uint32_t* off;              // [nb + 1] first places of the buckets (only with the one-block scan)
+    unsigned long long* mask_part;  // [2 * NMASK] OR / AND over the call's ids, one pair per block of prep
     uint32_t* big;              // [ncap / SMALL_BUCKET + 2] oversized buckets (atomic route) / their first places (radix route)
     uint64_t* key_a;            // [ncap] radix route
     uint64_t* key_b;
@@ -129,6 +148,7 @@ struct Scratch {
     int64_t ncap;               // most ids one call can add
     int32_t nb_log;             // log2 of the number of buckets
     int32_t radix;              // 1: radix route
+    int32_t nmask;              // pairs in mask_part
 };
 
 bool radix_route(int64_t ncap) { return ncap > ATOMIC_ROUTE_MAX; }
@@ -136,7 +156,7 @@ bool radix_route(int64_t ncap) { return ncap > ATOMIC_ROUTE_MAX; }
 int nb_log_of(int64_t ncap) {
     if (radix_route(ncap)) return SORT_KEY_LOG;
     int l = NB_MIN_LOG;
-    while (l < NB_MAX_LOG && (32ll << l) < ncap) ++l;     // ~32 ids per bucket when every id of the call is new
+    while (l < NB_MAX_LOG && ((int64_t)IDS_PER_BUCKET << l) < ncap) ++l;
     return l;
 }
 
@@ -147,7 +167,8 @@ size_t scratch_bytes(int64_t total, int64_t ncap) {
     if (radix_route(ncap))
         b += 3 * align_up((size_t)(ncap + 1) * 8) + radix_sort_workspace_bytes(ncap) + 256;
     else
-        b += align_up((size_t)(ncap + 1) * 8) + 3 * align_up((size_t)(ncap + 1) * 4) + 2 * align_up((size_t)(nb + 1) * 4);
+        b += align_up((size_t)(ncap + 1) * 8) + 4 * align_up((size_t)(ncap + 1) * 4) + 2 * align_up((size_t)(nb + 1) * 4) +
+             align_up((size_t)2 * NMASK * 8);
     return b;
 }
 
@@ -169,10 +190,12 @@ Scratch carve_scratch(Arena& ar, int64_t total, int64_t ncap) {
     } else {
         s.part_id = ar.take<unsigned long long>(ncap + 1);
         s.list_b = ar.take<uint32_t>(ncap + 1);
+        s.list_r = ar.take<uint32_t>(ncap + 1);
         s.part_slot = ar.take<uint32_t>(ncap + 1);
         s.part_b = ar.take<uint32_t>(ncap + 1);
         s.cnt = ar.take<uint32_t>(nb + 1);
         s.off = ar.take<uint32_t>(nb + 1);
+        s.mask_part = ar.take<unsigned long long>(2 * NMASK);
     }
     return s;
 }
@@ -236,183 +259,6 @@ __device__ __forceinline__ void clear_call_fields(Header* h) {
     h->nbig = 0;
 }
 
-__global__ __launch_bounds__(BLOCK) void init_kernel(Table t) {
-    const int64_t tid = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
-    for (int64_t i = tid; i < t.slots; i += (int64_t)gridDim.x * BLOCK) {
-        t.keys[i] = EMPTY;
-        t.vals[i] = UNNUMBERED;
-    }
-    if (tid == 0) {
-        t.hdr->total = 0;
-        t.hdr->overflow = 0;
-        clear_call_fields(t.hdr);
-    }
-}
-
-__global__ __launch_bounds__(BLOCK) void prep_kernel(Table t, Scratch s, int fresh, int reset) {
-    const int64_t tid = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * BLOCK;
-    // every block reads the header before anyone writes it: only a fresh (workspace) table's header is
-    // written here, and nobody reads that one
-    const int64_t prev = fresh ? 0 : (int64_t)t.hdr->total;
-    if (fresh || (reset && prev * 4 >= t.slots)) {
-        for (int64_t i = tid; i < t.slots; i += stride) {
-            t.keys[i] = EMPTY;
-            t.vals[i] = UNNUMBERED;
-        }
-    } else if (reset) {
-        for (int64_t k = tid; k < prev; k += stride) {
-            const uint32_t h = t.used[k];
-            t.keys[h] = EMPTY;
-            t.vals[h] = UNNUMBERED;
-        }
-    }
-    if (!s.radix) {
-        const int64_t nb = 1ll << s.nb_log;
-        for (int64_t i = tid; i <= nb; i += stride) s.cnt[i] = 0;
-    }
-    if (fresh && tid == 0) {
-        t.hdr->total = 0;
-        t.hdr->overflow = 0;
-        clear_call_fields(t.hdr);
-    }
-}
-
-// IPT ids per thread: a tile of 256 * IPT ids per block (small calls take small tiles so that the chip has
-// blocks to run; large ones take large tiles, which fold more repeats before the table is touched).
-// grp: the array group whose ids this launch adds (grouped mode: one launch per array, in array order, so that
-// an id belongs to the first array that holds it; otherwise one launch, group 0, over all arrays).  flat_base:
-// index of the launch's first element among the elements of all arrays (slot_of is indexed over all of them).
-template <int IPT>
-__global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratch s, int reset, int grp, int64_t flat_base) {
-    constexpr int TILE = BLOCK * IPT;
-    constexpr int LDS_SLOTS = 2 * TILE;      // load <= 0.5
-    __shared__ unsigned long long s_key[LDS_SLOTS];
-    __shared__ uint32_t s_aux[LDS_SLOTS];       // table slot of the id
-    __shared__ int32_t s_won;
-    __shared__ long long s_base;
-    __shared__ unsigned long long s_or, s_and;
-#pragma unroll
-    for (int q = 0; q < LDS_SLOTS / BLOCK; ++q) {
-        s_key[q * BLOCK + threadIdx.x] = EMPTY;
-    }
-    if (threadIdx.x == 0) {
-        s_won = 0;
-        s_or = 0;
-        s_and = ~0ull;
-    }
-    const int64_t t0 = (int64_t)blockIdx.x * TILE + threadIdx.x;
-    // the tile's ids (every load issued before the first LDS probe)
-    int64_t id[IPT];
-    bool live[IPT];
-#pragma unroll
-    for (int q = 0; q < IPT; ++q) {
-        id[q] = -1;
-        int g;
-        int64_t i;
-        live[q] = locate(a, t0 + (int64_t)q * BLOCK, &g, &i);
-        if (live[q]) id[q] = a.ids[g][i];
-    }
-    __syncthreads();
-    int32_t ls[IPT];                      // LDS slot of the id; -1: negative id or no element
-    bool owner[IPT];                      // this element put the id into the LDS set
-#pragma unroll
-    for (int q = 0; q < IPT; ++q) {
-        ls[q] = -1;
-        owner[q] = false;
-        if (id[q] < 0) continue;
-        uint32_t h = (uint32_t)mix((uint64_t)id[q]) & (LDS_SLOTS - 1);
-        while (true) {
-            const unsigned long long prev = atomicCAS(&s_key[h], EMPTY, (unsigned long long)id[q]);
-            if (prev == EMPTY) owner[q] = true;
-            if (prev == EMPTY || prev == (unsigned long long)id[q]) break;
-            h = (h + 1) & (LDS_SLOTS - 1);
-        }
-        ls[q] = (int32_t)h;
-    }
-    // every owner finds or claims the table slot of its id: first probes of all its ids in flight together
-    const int64_t before = ids_before(t, reset);
-    uint64_t h[IPT];
-    unsigned long long k0[IPT];
-#pragma unroll
-    for (int q = 0; q < IPT; ++q) {
-        h[q] = 0;
-        k0[q] = 0;
-        if (owner[q]) {
-            h[q] = __umul64hi(mix((uint64_t)id[q]), (uint64_t)t.slots);
-            k0[q] = t.keys[h[q]];       // a slot never changes once it holds an id: a cached value is good
-        }
-    }
-    bool won[IPT];
-    int32_t pos[IPT];
-    unsigned long long my_or = 0, my_and = ~0ull;
-    bool lost = false;
-#pragma unroll
-    for (int q = 0; q < IPT; ++q) {
-        won[q] = false;
-        pos[q] = 0;
-        if (!owner[q]) continue;
-        const unsigned long long me = (unsigned long long)id[q];
-        unsigned long long k = k0[q];
-        bool placed = false;
-        for (int64_t probes = 0; probes < t.slots; ++probes) {
-            if (probes > 0) k = t.keys[h[q]];
-            if (k == EMPTY) {
-                k = atomicCAS(&t.keys[h[q]], EMPTY, me);
-                if (k == EMPTY) {
-                    won[q] = true;
-                    k = me;
-                }
-            }
-            if (k == me) {
-                placed = true;
-                break;
-            }
-            h[q] = h[q] + 1 == (uint64_t)t.slots ? 0 : h[q] + 1;
-        }
-        if (!placed) {          // the table is full
-            lost = true;
-            won[q] = false;
-            s_aux[ls[q]] = NONE;
-            continue;
-        }
-        s_aux[ls[q]] = (uint32_t)h[q];
-        if (won[q]) {
-            pos[q] = atomicAdd(&s_won, 1);
-            my_or |= me;
-            my_and &= me;
-        }
-    }
-    if (my_or != 0 || my_and != ~0ull) {
-        atomicOr(&s_or, my_or);
-        atomicAnd(&s_and, my_and);
-    }
-    if (lost) atomicOr(&t.hdr->overflow, 1ull);
-    __syncthreads();
-    if (threadIdx.x == 0 && s_won > 0) {
-        long long prev = 0;                 // ids added by the launches of the groups before this one
-        for (int g = 0; g < grp; ++g) prev += (long long)t.hdr->added[g].n;
-        s_base = prev + (long long)atomicAdd(&t.hdr->added[grp].n, (unsigned long long)s_won);
-        // the two masks settle after the first few blocks: an atomic only when this block still changes them
-        // (they move one way only, so a stale reading costs a redundant atomic, never a missing one)
-        if (s_or & ~__hip_atomic_load(&t.hdr->or_mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicOr(&t.hdr->or_mask, s_or);
-        if (~s_and & __hip_atomic_load(&t.hdr->and_mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicAnd(&t.hdr->and_mask, s_and);
-        if (before + s_base + s_won > t.capacity || s_base + s_won > s.ncap) atomicOr(&t.hdr->overflow, 1ull);
-    }
-    __syncthreads();
-#pragma unroll
-    for (int q = 0; q < IPT; ++q) {
-        if (won[q]) {
-            const int64_t k = s_base + pos[q];
-            if (k < s.ncap && before + k < t.capacity) {
-                s.list_id[k] = (unsigned long long)id[q];
-                t.used[before + k] = (uint32_t)h[q];
-            }
-        }
-        if (live[q]) s.slot_of[flat_base + t0 + (int64_t)q * BLOCK] = ls[q] < 0 ? NONE : s_aux[ls[q]];
-    }
-}
-
 // The bits in which the new ids differ, squeezed into a key that keeps their order: up to three runs
 // of such bits from the top, then one span down to the lowest of them (it may hold bits that do not
 // differ; only the top bits of the key select the bucket).
@@ -473,100 +319,374 @@ __device__ __forceinline__ uint32_t bucket_of(const Codec& c, uint64_t id, uint3
     return (g << kb) | (uint32_t)top;
 }
 
-// ---- atomic route -------------------------------------------------------------------------------
-__global__ __launch_bounds__(BLOCK) void hist_kernel(Table t, Scratch s, int reset, int grouped, int glog) {
-    __shared__ Codec s_codec;
-    if (threadIdx.x == 0) s_codec = make_codec(t.hdr->or_mask, t.hdr->and_mask);
-    __syncthreads();
-    const Codec c = s_codec;
-    const int64_t before = ids_before(t, reset);
-    const int64_t n = ids_added(t, s, before);
-    for (int64_t k = (int64_t)blockIdx.x * BLOCK + threadIdx.x; k < n; k += (int64_t)gridDim.x * BLOCK) {
-        const uint32_t g = grouped ? group_of(t, k) : 0;
-        const uint32_t b = bucket_of(c, s.list_id[k], g, s.nb_log, glog);
-        s.list_b[k] = b;
-        atomicAdd(&s.cnt[b], 1u);
+__global__ __launch_bounds__(BLOCK) void init_kernel(Table t) {
+    const int64_t tid = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    for (int64_t i = tid; i < t.slots; i += (int64_t)gridDim.x * BLOCK) {
+        t.keys[i] = EMPTY;
+        t.vals[i] = UNNUMBERED;
+    }
+    if (tid == 0) {
+        t.hdr->total = 0;
+        t.hdr->overflow = 0;
+        clear_call_fields(t.hdr);
     }
 }
 
-// One block: exclusive prefix of the bucket sizes, cursors zeroed, oversized buckets listed.  The counters
-// are read with coalesced loads, all of them in flight before the first is used, and pass through LDS
-// in chunks of CHUNK so that thread t can scan CHUNK / SCAN_BLOCK consecutive ones.
-__global__ __launch_bounds__(SCAN_BLOCK) void scan_kernel(Table t, Scratch s) {
-    constexpr int NW = SCAN_BLOCK / WAVE;
-    constexpr int RUN = 8;                          // consecutive counters per thread and chunk
-    constexpr int CHUNK = SCAN_BLOCK * RUN;
-    constexpr int NCHUNK = (1 << NB_MAX_LOG) / CHUNK;
-    __shared__ uint32_t s_c[CHUNK];
-    __shared__ uint32_t s_w[2][NW];
-    __shared__ uint32_t s_nbig;
-    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
-    const int nb = 1 << s.nb_log;
-    if (threadIdx.x == 0) s_nbig = 0;
-    uint32_t v[NCHUNK][RUN];
+// OR / AND over the values of a block's threads, left in s_or / s_and (both set up before the call)
+__device__ __forceinline__ void block_or_and(unsigned long long o, unsigned long long n, unsigned long long* s_or,
+                                             unsigned long long* s_and) {
 #pragma unroll
-    for (int c = 0; c < NCHUNK; ++c)
-#pragma unroll
-        for (int j = 0; j < RUN; ++j) {
-            const int i = c * CHUNK + j * SCAN_BLOCK + threadIdx.x;
-            v[c][j] = (c * CHUNK < nb && i < nb) ? s.cnt[i] : 0;
-        }
-    uint32_t carry = 0;
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) {
-        if (c * CHUNK >= nb) break;                 // uniform
-#pragma unroll
-        for (int j = 0; j < RUN; ++j) s_c[j * SCAN_BLOCK + threadIdx.x] = v[c][j];
-        __syncthreads();
-        uint32_t w[RUN];
-        uint32_t sum = 0;
-#pragma unroll
-        for (int j = 0; j < RUN; ++j) {
-            w[j] = s_c[threadIdx.x * RUN + j];
-            sum += w[j];
-        }
-        uint32_t inc = sum;
-        for (int d = 1; d < WAVE; d <<= 1) {
-            const uint32_t y = __shfl_up(inc, d);
-            if (lane >= d) inc += y;
-        }
-        if (lane == WAVE - 1) s_w[c & 1][wid] = inc;
-        __syncthreads();
-        uint32_t o = carry + inc - sum, chunk_total = 0;
-#pragma unroll
-        for (int q = 0; q < NW; ++q) {
-            const uint32_t x = s_w[c & 1][q];
-            if (q < wid) o += x;
-            chunk_total += x;
-        }
-        carry += chunk_total;
-        const int i0 = c * CHUNK + threadIdx.x * RUN;
-#pragma unroll
-        for (int j = 0; j < RUN; ++j) {
-            if (i0 + j < nb) {
-                s.off[i0 + j] = o;
-                s.cnt[i0 + j] = 0;
-                if (w[j] > (uint32_t)SMALL_BUCKET) s.big[atomicAdd(&s_nbig, 1u)] = (uint32_t)(i0 + j);
-                o += w[j];
+    for (int d = WAVE / 2; d > 0; d >>= 1) {
+        o |= __shfl_xor(o, d);
+        n &= __shfl_xor(n, d);
+    }
+    if (threadIdx.x % WAVE == 0) {
+        atomicOr(s_or, o);
+        atomicAnd(s_and, n);
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void prep_kernel(Arrays a, Table t, Scratch s, int fresh, int reset) {
+    __shared__ unsigned long long s_or, s_and;
+    const int64_t tid = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * BLOCK;
+    // every block reads the header before anyone writes it: only a fresh (workspace) table's header is
+    // written here, and nobody reads that one.  Only the keys are emptied: whoever claims a slot sets its value.
+    const int64_t prev = fresh ? 0 : (int64_t)t.hdr->total;
+    if (fresh || (reset && prev * 4 >= t.slots)) {
+        for (int64_t i = tid; i < t.slots; i += stride) t.keys[i] = EMPTY;
+    } else if (reset) {
+        for (int64_t k = tid; k < prev; k += stride) t.keys[t.used[k]] = EMPTY;
+    }
+    if (!s.radix) {
+        const int64_t nb = 1ll << s.nb_log;
+        for (int64_t i = tid; i <= nb; i += stride) s.cnt[i] = 0;
+        if ((int)blockIdx.x < s.nmask) {     // block-uniform
+            if (threadIdx.x == 0) {
+                s_or = 0;
+                s_and = ~0ull;
+            }
+            __syncthreads();
+            unsigned long long o = 0, n = ~0ull;
+            for (int64_t x = tid; x < a.start[a.G]; x += (int64_t)s.nmask * BLOCK) {
+                int g;
+                int64_t i;
+                if (!locate(a, x, &g, &i)) continue;
+                const int64_t id = a.ids[g][i];
+                if (id >= 0) {
+                    o |= (unsigned long long)id;
+                    n &= (unsigned long long)id;
+                }
+            }
+            block_or_and(o, n, &s_or, &s_and);
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                s.mask_part[2 * blockIdx.x] = s_or;
+                s.mask_part[2 * blockIdx.x + 1] = s_and;
             }
         }
     }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        s.off[nb] = carry;
-        t.hdr->nbig = s_nbig;
+    if (fresh && tid == 0) {
+        t.hdr->total = 0;
+        t.hdr->overflow = 0;
+        clear_call_fields(t.hdr);
     }
 }
 
-__global__ __launch_bounds__(BLOCK) void scatter_kernel(Table t, Scratch s, int reset) {
+// IPT ids per thread: a tile of 256 * IPT ids per block (small calls take small tiles so that the chip has
+// blocks to run; large ones take large tiles, which fold more repeats before the table is touched).
+// grp: the array group whose ids this launch adds (grouped mode: one launch per array, in array order, so that
+// an id belongs to the first array that holds it; otherwise one launch, group 0, over all arrays).  flat_base:
+// index of the launch's first element among the elements of all arrays (slot_of is indexed over all of them).
+// SMALL (calls of the atomic route): probes are an atomicCAS straight away, and the ids the block adds are
+// counted into their buckets here, with the key made from the masks prep left; otherwise a probe is a plain load
+// first and OR / AND over the added ids go to the header for the launches that follow.
+template <int IPT, bool SMALL>
+__global__ __launch_bounds__(BLOCK) void insert_kernel(Arrays a, Table t, Scratch s, int reset, int grp, int glog,
+                                                       int64_t flat_base) {
+    constexpr int TILE = BLOCK * IPT;
+    constexpr int LDS_SLOTS = 2 * TILE;      // load <= 0.5
+    __shared__ unsigned long long s_key[LDS_SLOTS];
+    __shared__ uint32_t s_aux[LDS_SLOTS];       // table slot of the id
+    __shared__ int32_t s_won;
+    __shared__ long long s_base;
+    __shared__ unsigned long long s_or, s_and;  // SMALL: over the call's ids; otherwise over the ids the block added
+#pragma unroll
+    for (int q = 0; q < LDS_SLOTS / BLOCK; ++q) {
+        s_key[q * BLOCK + threadIdx.x] = EMPTY;
+    }
+    if (threadIdx.x == 0) {
+        s_won = 0;
+        s_or = 0;
+        s_and = ~0ull;
+    }
+    const int64_t t0 = (int64_t)blockIdx.x * TILE + threadIdx.x;
+    // the tile's ids (every load issued before the first LDS probe)
+    int64_t id[IPT];
+    bool live[IPT];
+#pragma unroll
+    for (int q = 0; q < IPT; ++q) {
+        // the id is loaded beside the array's live length, not after it (the arrays hold len_max entries)
+        const int64_t x = t0 + (int64_t)q * BLOCK;
+        id[q] = -1;
+        live[q] = false;
+        if (x < a.start[a.G]) {
+            int g = 0;
+#pragma unroll
+            for (int w = 1; w < MAXG; ++w)
+                if (w < a.G && x >= a.start[w]) g = w;
+            const int64_t i = x - a.start[g];
+            const int64_t v = a.ids[g][i];
+            live[q] = i < live_count(a.len_dev[g], a.len_max[g]);
+            if (live[q]) id[q] = v;
+        }
+    }
+    unsigned long long part_or = 0, part_and = ~0ull;
+    if constexpr (SMALL) {
+        if ((int)threadIdx.x < s.nmask) {
+            part_or = s.mask_part[2 * threadIdx.x];
+            part_and = s.mask_part[2 * threadIdx.x + 1];
+        }
+    }
+    __syncthreads();
+    if constexpr (SMALL) block_or_and(part_or, part_and, &s_or, &s_and);
+    int32_t ls[IPT];                      // LDS slot of the id; -1: negative id or no element
+    bool owner[IPT];                      // this element put the id into the LDS set
+#pragma unroll
+    for (int q = 0; q < IPT; ++q) {
+        ls[q] = -1;
+        owner[q] = false;
+        if (id[q] < 0) continue;
+        uint32_t h = (uint32_t)mix((uint64_t)id[q]) & (LDS_SLOTS - 1);
+        while (true) {
+            const unsigned long long prev = atomicCAS(&s_key[h], EMPTY, (unsigned long long)id[q]);
+            if (prev == EMPTY) owner[q] = true;
+            if (prev == EMPTY || prev == (unsigned long long)id[q]) break;
+            h = (h + 1) & (LDS_SLOTS - 1);
+        }
+        ls[q] = (int32_t)h;
+    }
+    // every owner finds or claims the table slot of its id: first probes of all its ids in flight together
     const int64_t before = ids_before(t, reset);
+    uint64_t h[IPT];
+    unsigned long long k0[IPT];
+#pragma unroll
+    for (int q = 0; q < IPT; ++q) {
+        h[q] = 0;
+        k0[q] = 0;
+        if (owner[q]) {
+            h[q] = __umul64hi(mix((uint64_t)id[q]), (uint64_t)t.slots);
+            if constexpr (SMALL) k0[q] = atomicCAS(&t.keys[h[q]], EMPTY, (unsigned long long)id[q]);
+            else k0[q] = t.keys[h[q]];  // a slot never changes once it holds an id: a cached value is good
+        }
+    }
+    Codec codec{};
+    if constexpr (SMALL) {
+        __syncthreads();                 // the masks are folded
+        codec = make_codec(s_or, s_and);
+    }
+    bool won[IPT];
+    int32_t pos[IPT];
+    uint32_t bkt[IPT], rnk[IPT];          // SMALL: bucket of a new id and how many ids the bucket held before it
+    unsigned long long my_or = 0, my_and = ~0ull;
+    bool lost = false;
+#pragma unroll
+    for (int q = 0; q < IPT; ++q) {
+        won[q] = false;
+        pos[q] = 0;
+        bkt[q] = rnk[q] = 0;
+        if (!owner[q]) continue;
+        const unsigned long long me = (unsigned long long)id[q];
+        unsigned long long k = k0[q];
+        bool placed = false;
+        for (int64_t probes = 0; probes < t.slots; ++probes) {
+            if constexpr (SMALL) {
+                if (probes > 0) k = atomicCAS(&t.keys[h[q]], EMPTY, me);
+                if (k == EMPTY) {
+                    won[q] = true;
+                    k = me;
+                }
+            } else {
+                if (probes > 0) k = t.keys[h[q]];
+                if (k == EMPTY) {
+                    k = atomicCAS(&t.keys[h[q]], EMPTY, me);
+                    if (k == EMPTY) {
+                        won[q] = true;
+                        k = me;
+                    }
+                }
+            }
+            if (k == me) {
+                placed = true;
+                break;
+            }
+            h[q] = h[q] + 1 == (uint64_t)t.slots ? 0 : h[q] + 1;
+        }
+        if (!placed) {          // the table is full
+            lost = true;
+            won[q] = false;
+            s_aux[ls[q]] = NONE;
+            continue;
+        }
+        s_aux[ls[q]] = (uint32_t)h[q];
+        if (won[q]) {
+            pos[q] = atomicAdd(&s_won, 1);
+            t.vals[h[q]] = UNNUMBERED;
+            if constexpr (SMALL) {       // counted here, so that this round trip runs beside the block's append
+                bkt[q] = bucket_of(codec, me, (uint32_t)grp, s.nb_log, glog);
+                rnk[q] = atomicAdd(&s.cnt[bkt[q]], 1u);
+            }
+            my_or |= me;
+            my_and &= me;
+        }
+    }
+    if constexpr (!SMALL) {
+        if (my_or != 0 || my_and != ~0ull) {
+            atomicOr(&s_or, my_or);
+            atomicAnd(&s_and, my_and);
+        }
+    }
+    if (lost) atomicOr(&t.hdr->overflow, 1ull);
+    __syncthreads();
+    if (threadIdx.x == 0 && s_won > 0) {
+        long long prev = 0;                 // ids added by the launches of the groups before this one
+        for (int g = 0; g < grp; ++g) prev += (long long)t.hdr->added[g].n;
+        s_base = prev + (long long)atomicAdd(&t.hdr->added[grp].n, (unsigned long long)s_won);
+        if (before + s_base + s_won > t.capacity || s_base + s_won > s.ncap) atomicOr(&t.hdr->overflow, 1ull);
+    }
+    if constexpr (!SMALL) {
+        // lanes of two other waves, so that the three round trips to the header run side by side.  The two masks
+        // settle after the first few blocks: an atomic only when this block still changes them (they move one
+        // way only, so a stale reading costs a redundant atomic, never a missing one)
+        if (threadIdx.x == WAVE && s_won > 0 &&
+            (s_or & ~__hip_atomic_load(&t.hdr->or_mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)))
+            atomicOr(&t.hdr->or_mask, s_or);
+        if (threadIdx.x == 2 * WAVE && s_won > 0 &&
+            (~s_and & __hip_atomic_load(&t.hdr->and_mask, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)))
+            atomicAnd(&t.hdr->and_mask, s_and);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < IPT; ++q) {
+        if (won[q]) {
+            const int64_t k = s_base + pos[q];
+            if (k < s.ncap && before + k < t.capacity) {
+                s.list_id[k] = (unsigned long long)id[q];
+                t.used[before + k] = (uint32_t)h[q];
+                if constexpr (SMALL) {
+                    s.list_b[k] = bkt[q];
+                    s.list_r[k] = rnk[q];
+                }
+            }
+        }
+        if (live[q]) s.slot_of[flat_base + t0 + (int64_t)q * BLOCK] = ls[q] < 0 ? NONE : s_aux[ls[q]];
+    }
+}
+
+// ---- atomic route -------------------------------------------------------------------------------
+// Exclusive prefix of the nb <= 2^NB_MAX_LOG bucket sizes (and their total at [nb]) into LDS, by every block for
+// itself: thread t loads its nb / BLOCK consecutive sizes (16 bytes at a time) and adds them up, the block scans
+// the sums.  Entry i sits at i + i / 32, so that the threads' runs do not all start in the same bank.
+constexpr int NB_MAX = 1 << NB_MAX_LOG;
+constexpr int PRE_WORDS = NB_MAX + NB_MAX / 32 + 2;
+__device__ __forceinline__ int pre_at(int i) { return i + (i >> 5); }
+
+__device__ void block_prefix(const uint32_t* __restrict__ cnt, int nb, uint32_t* s_pre, uint32_t* s_wave) {
+    constexpr int NW = BLOCK / WAVE;
+    constexpr int PER_MAX = NB_MAX / BLOCK;
+    const int per = nb / BLOCK;                // nb is a power of two >= BLOCK
+    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    uint32_t v[PER_MAX];
+#pragma unroll
+    for (int j = 0; j < PER_MAX; ++j) v[j] = 0;
+    if (per >= 4) {
+        const uint4* src = reinterpret_cast<const uint4*>(cnt + (size_t)threadIdx.x * per);   // (the counters are 256-byte aligned)
+#pragma unroll
+        for (int j = 0; j < PER_MAX / 4; ++j) {
+            if (4 * j < per) {
+                const uint4 x = src[j];
+                v[4 * j] = x.x; v[4 * j + 1] = x.y; v[4 * j + 2] = x.z; v[4 * j + 3] = x.w;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            if (j < per) v[j] = cnt[threadIdx.x * per + j];
+    }
+    uint32_t sum = 0;
+#pragma unroll
+    for (int j = 0; j < PER_MAX; ++j) sum += v[j];
+    uint32_t inc = sum;
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const uint32_t y = __shfl_up(inc, d);
+        if (lane >= d) inc += y;
+    }
+    if (lane == WAVE - 1) s_wave[wid] = inc;
+    __syncthreads();
+    uint32_t o = inc - sum, total = 0;
+#pragma unroll
+    for (int q = 0; q < NW; ++q) {
+        const uint32_t x = s_wave[q];
+        if (q < wid) o += x;
+        total += x;
+    }
+#pragma unroll
+    for (int j = 0; j < PER_MAX; ++j) {
+        if (j < per) {
+            s_pre[pre_at(threadIdx.x * per + j)] = o;
+            o += v[j];
+        }
+    }
+    if (threadIdx.x == 0) s_pre[pre_at(nb)] = total;
+    __syncthreads();
+}
+
+// An id's place: first place of its bucket + the count the insert got back when it counted the id into the bucket.
+// The list entries are loaded before the number of live ones is known (the arrays hold ncap entries).
+__global__ __launch_bounds__(BLOCK) void scatter_kernel(Table t, Scratch s, int reset) {
+    __shared__ uint32_t s_pre[PRE_WORDS];
+    __shared__ uint32_t s_wave[BLOCK / WAVE];
+    constexpr int PER = 2;
+    const int64_t k0 = (int64_t)blockIdx.x * (PER * BLOCK) + threadIdx.x;
+    uint32_t b[PER], r[PER];
+    unsigned long long id[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int64_t k = k0 + j * BLOCK;
+        b[j] = r[j] = 0;
+        id[j] = 0;
+        if (k < s.ncap) {
+            b[j] = s.list_b[k];
+            r[j] = s.list_r[k];
+            id[j] = s.list_id[k];
+        }
+    }
+    const int nb = 1 << s.nb_log;
+    const int64_t before = ids_before(t, reset);       // (read before the barriers of the prefix, not after)
     const int64_t n = ids_added(t, s, before);
-    for (int64_t k = (int64_t)blockIdx.x * BLOCK + threadIdx.x; k < n; k += (int64_t)gridDim.x * BLOCK) {
-        const uint32_t b = s.list_b[k];
-        const uint32_t p = s.off[b] + atomicAdd(&s.cnt[b], 1u);
-        s.part_id[p] = s.list_id[k];
+    block_prefix(s.cnt, nb, s_pre, s_wave);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int64_t k = k0 + j * BLOCK;
+        if (k >= n) continue;
+        const int64_t p = (int64_t)s_pre[pre_at((int)(b[j] & (uint32_t)(nb - 1)))] + r[j];
+        if (p >= n) continue;            // only after an overflow (the result is void then)
+        s.part_id[p] = id[j];
         s.part_slot[p] = t.used[before + k];
-        s.part_b[p] = b;
+        s.part_b[p] = b[j];
+    }
+    if (blockIdx.x == 0) {               // for the numbering launch: the first places, and which buckets are oversized
+        __shared__ uint32_t s_nbig;
+        if (threadIdx.x == 0) s_nbig = 0;
+        __syncthreads();
+        for (int i = threadIdx.x; i <= nb; i += BLOCK) {
+            const uint32_t f = s_pre[pre_at(i)];
+            s.off[i] = f;
+            if (i < nb && s_pre[pre_at(i + 1)] - f > (uint32_t)SMALL_BUCKET) s.big[atomicAdd(&s_nbig, 1u)] = (uint32_t)i;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) t.hdr->nbig = s_nbig;
     }
 }
 
@@ -605,31 +725,76 @@ __device__ void block_sort(IdT* ids, PayloadT* payload, int64_t n) {
     }
 }
 
+// A block takes NUMBER_TILE consecutive places and parks their ids in LDS: an id is ranked against the ids of
+// its bucket from there (a chain of LDS reads instead of one of trips to the L2); only the part of a bucket that
+// lies outside the tile is read from memory.  Oversized buckets (skewed id distributions), listed by the scatter
+// launch, are taken in turn by the blocks and sorted in place.
+constexpr int NUMBER_TILE = 2 * BLOCK;
 __global__ __launch_bounds__(BLOCK) void number_kernel(Table t, Scratch s, int reset, int64_t* __restrict__ unique_out,
                                                        int64_t unique_capacity) {
+    __shared__ unsigned long long s_id[NUMBER_TILE];
+    constexpr int PER = NUMBER_TILE / BLOCK;
+    const int64_t p0 = (int64_t)blockIdx.x * NUMBER_TILE;
+    const int nb = 1 << s.nb_log;
+    uint32_t slot[PER];
+    int64_t lo[PER], hi[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {       // loaded before the number of live places is known (the arrays hold ncap entries)
+        const int64_t p = p0 + j * BLOCK + threadIdx.x;
+        slot[j] = 0;
+        lo[j] = hi[j] = 0;
+        if (p < s.ncap) {
+            s_id[j * BLOCK + threadIdx.x] = s.part_id[p];
+            slot[j] = s.part_slot[p];
+            const uint32_t bucket = s.part_b[p] & (uint32_t)(nb - 1);
+            lo[j] = s.off[bucket];
+            hi[j] = s.off[bucket + 1];
+        }
+    }
     const int64_t before = ids_before(t, reset);
     const int64_t n = ids_added(t, s, before);
-    for (int64_t p = (int64_t)blockIdx.x * BLOCK + threadIdx.x; p < n; p += (int64_t)gridDim.x * BLOCK) {
-        const uint32_t b = s.part_b[p];
-        const uint32_t lo = s.off[b], hi = s.off[b + 1];
-        if (hi - lo > (uint32_t)SMALL_BUCKET) continue;       // sorted below
-        const unsigned long long id = s.part_id[p];
-        uint32_t r = lo;
-        for (uint32_t q = lo; q < hi; ++q) r += s.part_id[q] < id ? 1u : 0u;
+    const int64_t nbig = (int64_t)t.hdr->nbig;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int64_t p = p0 + j * BLOCK + threadIdx.x;
+        if (p >= n) continue;
+        if (lo[j] > n) lo[j] = n;         // (beyond n only after an overflow)
+        if (hi[j] > n) hi[j] = n;
+        if (hi[j] - lo[j] > SMALL_BUCKET) continue;       // sorted below
+        const unsigned long long id = s_id[j * BLOCK + threadIdx.x];
+        int64_t r = lo[j];
+        if (lo[j] >= p0 && hi[j] <= p0 + NUMBER_TILE) {    // the whole bucket is in the tile (all but the buckets at its ends)
+            const int a = (int)(lo[j] - p0), e = (int)(hi[j] - p0);
+            int q = a;
+            for (; q + 4 <= e; q += 4) {
+                const unsigned long long o0 = s_id[q], o1 = s_id[q + 1], o2 = s_id[q + 2], o3 = s_id[q + 3];
+                r += (o0 < id ? 1 : 0) + (o1 < id ? 1 : 0) + (o2 < id ? 1 : 0) + (o3 < id ? 1 : 0);
+            }
+            for (; q < e; ++q) r += s_id[q] < id ? 1 : 0;
+        } else {
+            for (int64_t q = lo[j]; q < hi[j]; ++q) {
+                const int64_t rel = q - p0;
+                const unsigned long long other = (rel >= 0 && rel < NUMBER_TILE) ? s_id[rel] : s.part_id[q];
+                r += other < id ? 1 : 0;
+            }
+        }
         const int64_t local = before + r;
         if (local < unique_capacity) unique_out[local] = (int64_t)id;
-        t.vals[s.part_slot[p]] = (uint32_t)local;
+        t.vals[slot[j]] = (uint32_t)local;
     }
-    const int64_t nbig = (int64_t)t.hdr->nbig;
     for (int64_t q = blockIdx.x; q < nbig; q += gridDim.x) {
-        const uint32_t b = s.big[q];
-        const int64_t lo = s.off[b], len = (int64_t)s.off[b + 1] - lo;
+        const uint32_t bucket = s.big[q];
+        int64_t blo = s.off[bucket], bhi = s.off[bucket + 1];
+        if (blo > n) blo = n;
+        if (bhi > n) bhi = n;
+        const int64_t len = bhi - blo;
         __syncthreads();
-        block_sort(s.part_id + lo, s.part_slot + lo, len);
+        block_sort(s.part_id + blo, s.part_slot + blo, len);
         for (int64_t j = threadIdx.x; j < len; j += BLOCK) {
-            const int64_t local = before + lo + j;
-            if (local < unique_capacity) unique_out[local] = (int64_t)s.part_id[lo + j];
-            t.vals[s.part_slot[lo + j]] = (uint32_t)local;
+            const int64_t local = before + blo + j;
+            if (local < unique_capacity) unique_out[local] = (int64_t)s.part_id[blo + j];
+            t.vals[s.part_slot[blo + j]] = (uint32_t)local;
         }
     }
 }
@@ -749,7 +914,7 @@ int32_t check_capacity(int64_t capacity) {
     return SGL_OK;
 }
 
-using InsertKernel = void (*)(Arrays, Table, Scratch, int, int, int64_t);
+using InsertKernel = void (*)(Arrays, Table, Scratch, int, int, int, int64_t);
 
 int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const int64_t* const* ids, const int64_t* len_max,
             const int64_t* const* len_dev, int64_t* const* local_out, int64_t* unique_out, int64_t unique_capacity,
@@ -768,7 +933,7 @@ int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const i
     const int64_t total = all.start[MAXG];
     if (total > MAX_CAPACITY) return fail(SGL_ENOTSUP, "unique_compact: too many ids");
     const int64_t ncap = total < t.capacity ? total : t.capacity;
-    const Scratch s = carve_scratch(ar, total, ncap);
+    Scratch s = carve_scratch(ar, total, ncap);
     int64_t* n_sort = ar.take<int64_t>(1);
     if (!ar.ok()) return fail(SGL_ENOMEM, "unique_compact: workspace too small");
     const int grouped = (mode == SGL_UNIQUE_GROUPED && G > 1) ? 1 : 0;
@@ -779,8 +944,11 @@ int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const i
         int64_t b = ceil_div<int64_t>(work > 0 ? work : 1, per_block);
         return dim3((unsigned)(b > MAX_GRID ? MAX_GRID : b));
     };
-    const int64_t clear_work = (fresh || reset) ? t.slots : (s.radix ? 1 : (1ll << s.nb_log));
-    hipLaunchKernelGGL(prep_kernel, grid(clear_work, 4 * BLOCK), dim3(BLOCK), 0, st, t, s, fresh ? 1 : 0, reset);
+    int64_t prep_work = (fresh || reset) ? t.slots : 1;
+    if (!s.radix) prep_work = std::max<int64_t>(prep_work, std::max<int64_t>(1ll << s.nb_log, total));
+    const dim3 prep_grid = grid(prep_work, 4 * BLOCK);
+    s.nmask = s.radix ? 0 : (int32_t)std::min<unsigned>(prep_grid.x, (unsigned)NMASK);
+    hipLaunchKernelGGL(prep_kernel, prep_grid, dim3(BLOCK), 0, st, all, t, s, fresh ? 1 : 0, reset);
     SGL_LAUNCH_CHECK();
     if (total > 0) {
         // tile of the insert: 1024 ids per block (larger tiles fold more repeats before the table is touched but
@@ -789,8 +957,9 @@ int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const i
         auto launch_insert = [&](const Arrays& arr, int64_t n, int grp, int64_t flat_base) -> int32_t {
             int ipt = 4;
             while (ipt > 1 && n / (BLOCK * ipt) < 256) ipt >>= 1;
-            const InsertKernel ins = ipt == 4 ? insert_kernel<4> : ipt == 2 ? insert_kernel<2> : insert_kernel<1>;
-            hipLaunchKernelGGL(ins, dim3((unsigned)ceil_div<int64_t>(n, BLOCK * ipt)), dim3(BLOCK), 0, st, arr, t, s, reset, grp, flat_base);
+            const InsertKernel ins = s.radix ? (ipt == 4 ? insert_kernel<4, false> : ipt == 2 ? insert_kernel<2, false> : insert_kernel<1, false>)
+                                             : (ipt == 4 ? insert_kernel<4, true> : ipt == 2 ? insert_kernel<2, true> : insert_kernel<1, true>);
+            hipLaunchKernelGGL(ins, dim3((unsigned)ceil_div<int64_t>(n, BLOCK * ipt)), dim3(BLOCK), 0, st, arr, t, s, reset, grp, glog, flat_base);
             SGL_LAUNCH_CHECK();
             return SGL_OK;
         };
@@ -811,13 +980,10 @@ int32_t run(Table t, bool fresh, int32_t reset, int32_t mode, int32_t G, const i
         }
         if (rc_ins != SGL_OK) return rc_ins;
         if (!s.radix) {
-            hipLaunchKernelGGL(hist_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, grouped, glog);
+            hipLaunchKernelGGL(scatter_kernel, dim3((unsigned)ceil_div<int64_t>(std::max<int64_t>(ncap, 1), 2 * BLOCK)), dim3(BLOCK), 0, st, t, s, reset);
             SGL_LAUNCH_CHECK();
-            hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, t, s);
-            SGL_LAUNCH_CHECK();
-            hipLaunchKernelGGL(scatter_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset);
-            SGL_LAUNCH_CHECK();
-            hipLaunchKernelGGL(number_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, unique_out, unique_capacity);
+            hipLaunchKernelGGL(number_kernel, dim3((unsigned)ceil_div<int64_t>(std::max<int64_t>(ncap, 1), NUMBER_TILE)), dim3(BLOCK), 0, st, t, s, reset,
+                               unique_out, unique_capacity);
             SGL_LAUNCH_CHECK();
         } else {
             hipLaunchKernelGGL(sortkey_kernel, grid(ncap, BLOCK), dim3(BLOCK), 0, st, t, s, reset, grouped, glog, n_sort);
