@@ -140,10 +140,16 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     mem = torch.randn((n, 100), device=dev, generator=gen)
     mem_ts = torch.randint(0, 1 << 40, (n,), device=dev, generator=gen)
     nfeat = torch.randn((n, 100), device=dev, generator=gen)
-    mem_hot, mem_cold = tiered(mem)
-    ts_hot, ts_cold = tiered(mem_ts)
+    mem_hot, mem_cold_packed = tiered(mem)
+    ts_hot, ts_cold_packed = tiered(mem_ts)
     nf_hot, nf_cold = tiered(nfeat)
+    # the host tier of the memory keeps a row and its time in one 512-byte record (views of one pinned buffer);
+    # the packed tables (one for the rows, one for the times) stay for the comparison below
+    mem_cold, ts_cold, _rec = hot.interleaved_cold(n, 100)
+    mem_cold.copy_(mem_cold_packed)
+    ts_cold.copy_(ts_cold_packed)
     c_mem = hot.cache(400, mem_hot, rows=n, cold=mem_cold, hot_slot=slot, ts_hot=ts_hot, ts_cold=ts_cold)
+    c_mem_packed = hot.cache(400, mem_hot, rows=n, cold=mem_cold_packed, hot_slot=slot, ts_hot=ts_hot, ts_cold=ts_cold_packed)
     c_nf = hot.cache(400, nf_hot, rows=n, cold=nf_cold, hot_slot=slot)
     del mem, nfeat
     efeat = torch.empty((m, 172), device=dev)
@@ -231,7 +237,7 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     wall, (e_tot, u_tot) = timed(len(pipes))
     P0 = pipes[0]
     kr, ubuf, U, E, plan, s_in = P0.kr, P0.ubuf, P0.U, P0.E, P0.plan, P0.s_in
-    o_mem, o_ts, o_ef, o_te = P0.o_mem, P0.o_ts, P0.o_ef, P0.o_te
+    o_mem, o_ts, o_ef, o_te, o_nf = P0.o_mem, P0.o_ts, P0.o_ef, P0.o_te, P0.o_nf
     with torch.cuda.stream(streams[0]):
         P0.s_all.copy_(packed[0]); P0.body()
     torch.cuda.synchronize()
@@ -249,22 +255,47 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     res["gather_memory_30pct_host"] = {"ms": round(ms, 4), "rows": u1, "GBps": round(u1 * (8 + 4 + 800 + 16) / ms / 1e6, 1)}
     ms = _time_launches(torch, lambda: hot.gather_multi(plan))
     res["gather_all_three_one_launch"] = {"ms": round(ms, 4), "GBps": round((u1 * (2 * 812 + 16) + e1 * 1384) / ms / 1e6, 1)}
+    plan_packed = hot.gather_plan([(c_mem_packed, ubuf, o_mem, o_ts, U[0:1]), (c_nf, ubuf, o_nf, None, U[0:1]),
+                                   (c_ef, kr.hops[0].neighbors_eid, o_ef, None, E)])
+    ms_packed = _time_launches(torch, lambda: hot.gather_multi(plan_packed))
     # the launch is bound by the rows that cross PCIe: memory rows (400 B + 8 B last update) and node rows (400 B) of the
     # unique nodes whose owner is remote.  Host memory is read in 128-byte lines: a 400-byte row at a 16-byte-aligned
-    # offset always spans 4 of them (512 B), its 8-byte time another one.
+    # offset always spans 4 of them (512 B); a time in a table of its own costs another one, in the row's record none.
     st3 = hot.be.zeros(3)
     hot.gather(c_mem, ubuf, o_mem, out_ts=o_ts, N_dev=U[0:1], stats=st3)
     n_cold = int(st3[1].item())
-    cold_alg, cold_lines = n_cold * (400 + 8 + 400), n_cold * (512 + 128 + 512)
+    cold_alg, cold_lines, cold_lines_packed = n_cold * (400 + 8 + 400), n_cold * (512 + 512), n_cold * (512 + 128 + 512)
     probe = torch.empty(cold_alg, dtype=torch.uint8, device=dev)
-    src_h = mem_cold.view(torch.uint8).reshape(-1)[:cold_alg]
+    src_h = mem_cold_packed.view(torch.uint8).reshape(-1)[:cold_alg]
     ms_cp = _time_launches(torch, lambda: probe.copy_(src_h, non_blocking=True), reps=5)
     res["gather_all_three_one_launch"].update({
         "cold_rows": n_cold, "cold_bytes": cold_alg, "cold_GBps": round(cold_alg / ms / 1e6, 2),
         "cold_GBps_in_128B_lines": round(cold_lines / ms / 1e6, 2),
         "memcpy_h2d_same_bytes_GBps": round(cold_alg / ms_cp / 1e6, 2),
-        "cold_rate_over_memcpy": round(ms_cp / ms, 3), "line_rate_over_memcpy": round(cold_lines / cold_alg * ms_cp / ms, 3)})
+        "cold_rate_over_memcpy": round(ms_cp / ms, 3), "line_rate_over_memcpy": round(cold_lines / cold_alg * ms_cp / ms, 3),
+        "ceiling_of_cold_rate_over_memcpy": round(cold_alg / cold_lines, 3),
+        "times_in_a_table_of_their_own": {"ms": round(ms_packed, 4), "cold_GBps": round(cold_alg / ms_packed / 1e6, 2),
+                                          "cold_rate_over_memcpy": round(ms_cp / ms_packed, 3),
+                                          "line_rate_over_memcpy": round(cold_lines_packed / cold_alg * ms_cp / ms_packed, 3)}})
     del probe
+    # what a row read over PCIe costs by its size: all-cold gathers of 8 MB of random rows from a pinned table
+    # (rows aligned to their size; 400-byte rows packed and in 512-byte records).  Isolated 64- and 128-byte
+    # reads cost about the same; from 256 contiguous bytes on the rate is that of a plain copy.
+    by_size = {}
+    pin = torch.empty(256 << 20, dtype=torch.uint8, pin_memory=True)
+    pin.view(torch.int64)[::512] = 1                                  # touch every page
+    none_hot = torch.full(((256 << 20) // 64,), -1, dtype=torch.int32, device=dev)
+    o_probe = torch.empty(8 << 20, dtype=torch.uint8, device=dev)
+    for label, rb, stride in (("64", 64, 64), ("128", 128, 128), ("256", 256, 256), ("512", 512, 512), ("4096", 4096, 4096),
+                              ("400_packed", 400, 400), ("400_in_512_records", 400, 512)):
+        nrows = (256 << 20) // stride
+        tab = pin[:nrows * stride].view(nrows, stride)[:, :rb]
+        c_probe = hot.cache(rb, None, rows=nrows, cold=tab, hot_slot=none_hot[:nrows])
+        ids_p = torch.randint(0, nrows, ((8 << 20) // rb,), device=dev, generator=gen)
+        ms_p = _time_launches(torch, lambda: hot.gather(c_probe, ids_p, o_probe), reps=5)
+        by_size[label] = round(ids_p.numel() * rb / ms_p / 1e6, 2)
+    res["host_read_GBps_by_row_bytes"] = by_size
+    del pin, o_probe, none_hot
     p_h = hot.with_root_hint(p, s_in[4])
     ms = _time_launches(torch, lambda: hot.sample_khop(dg, s_in[0], ts_ptr, s_in[1], s_in[2], s_in[3], 1, p_h, finalize=False, out=kr))
     res["sample_recent_1hop"] = {"ms": round(ms, 4), "edges_per_s": round(e1 / ms * 1e3, 1)}

@@ -410,7 +410,11 @@ int32_t sgl_unique_compact_hashed(void* state, int64_t capacity, int32_t reset,
  *   loc  = g2l ? g2l[key] : key              (-1 / out of range = not resident)
  *   slot = hot_slot ? hot_slot[loc] : loc    (>= 0: row `slot` of `hot`,
  *                                             < 0 : row `loc` of `cold`)
- * A non-resident id yields an all-zero row, out_ts = 0 and bumps stats[2]. */
+ * A non-resident id yields an all-zero row, out_ts = 0 and bumps stats[2].
+ * The two strides let the cold tier keep a row and its time in one record
+ * (cold = base, ts_cold = base + row_bytes, both strides = the record size, best
+ * a multiple of 128): reads over PCIe are paid for in whole 128-byte lines, and
+ * an 8-byte time in a table of its own costs as much as a third of a 400-byte row. */
 typedef struct sgl_cache {
     int64_t        rows;      /* logical (local) rows                          */
     int64_t        row_bytes; /* multiple of 4                                 */
@@ -423,6 +427,10 @@ typedef struct sgl_cache {
     const void*    cold;      /* device-visible pinned host [rows, row_bytes]  */
     const int64_t* ts_hot;    /* optional last-update time per hot row         */
     const int64_t* ts_cold;   /* optional last-update time per logical row     */
+    int64_t        cold_stride;    /* bytes from one cold row to the next; 0 = row_bytes (a
+                                    * multiple of 4, >= row_bytes)                       */
+    int64_t        ts_cold_stride; /* bytes from one ts_cold entry to the next; 0 = 8 (a
+                                    * multiple of 8)                                     */
 } sgl_cache;
 
 /* out[i, :] = row(ids[i]); out_ts[i] = its last-update time when out_ts and the

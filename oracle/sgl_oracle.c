@@ -772,6 +772,12 @@ int32_t sglo_unique_compact_hashed(void* state, int64_t capacity, int32_t reset,
 
 /* ------------------------------------------------------------ cache gather */
 
+/* cold rows and their times may sit at a stride of their own (0 = packed) */
+static int64_t cold_stride(const sgl_cache* c) { return c->cold_stride ? c->cold_stride : c->row_bytes; }
+static int64_t* cold_ts_at(const sgl_cache* c, const int64_t* base, int64_t loc) {
+    return (int64_t*)((char*)base + loc * (c->ts_cold_stride ? c->ts_cold_stride : 8));
+}
+
 static int64_t cache_loc(const sgl_cache* c, int64_t id) {
     int64_t key = id & c->id_mask;
     if (id < 0) return -1;
@@ -811,8 +817,8 @@ int32_t sglo_gather(const sgl_cache* c, const int64_t* ids, int64_t N_max,
             if (out_ts) out_ts[i] = c->ts_hot ? c->ts_hot[slot] : 0;
             hit++;
         } else {
-            memcpy(dst, (const char*)c->cold + loc * c->row_bytes, (size_t)c->row_bytes);
-            if (out_ts) out_ts[i] = c->ts_cold ? c->ts_cold[loc] : 0;
+            memcpy(dst, (const char*)c->cold + loc * cold_stride(c), (size_t)c->row_bytes);
+            if (out_ts) out_ts[i] = c->ts_cold ? *cold_ts_at(c, c->ts_cold, loc) : 0;
             cold++;
         }
     }
@@ -837,8 +843,8 @@ int32_t sglo_scatter_update(const sgl_cache* c, void* hot_rw, void* cold_rw,
             memcpy((char*)hot_rw + slot * c->row_bytes, srcp, (size_t)c->row_bytes);
             if (ts && ts_hot_rw) ts_hot_rw[slot] = ts[i];
         } else {
-            memcpy((char*)cold_rw + loc * c->row_bytes, srcp, (size_t)c->row_bytes);
-            if (ts && ts_cold_rw) ts_cold_rw[loc] = ts[i];
+            memcpy((char*)cold_rw + loc * cold_stride(c), srcp, (size_t)c->row_bytes);
+            if (ts && ts_cold_rw) *cold_ts_at(c, ts_cold_rw, loc) = ts[i];
         }
     }
     return SGL_OK;

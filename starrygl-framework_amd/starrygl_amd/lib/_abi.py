@@ -44,7 +44,7 @@ class Cache(C.Structure):
     _fields_ = [("rows", i64), ("row_bytes", i64), ("id_mask", i64),
                 ("g2l", vp), ("g2l_len", i64), ("hot_slot", vp),
                 ("hot", vp), ("hot_rows", i64), ("cold", vp),
-                ("ts_hot", vp), ("ts_cold", vp)]
+                ("ts_hot", vp), ("ts_cold", vp), ("cold_stride", i64), ("ts_cold_stride", i64)]
 
 
 class GatherSeg(C.Structure):

@@ -12,6 +12,22 @@ from . import _abi
 from ._abi import (TCSR, Cache, GatherSeg, HopOut, SampleParams, SeedQuery, WindowParams, check, i64, vp)
 
 
+def _itemsize(a):
+    return a.element_size() if hasattr(a, "element_size") else a.itemsize
+
+
+def _byte_strides(a):
+    """strides in bytes of a torch tensor or a numpy array"""
+    if hasattr(a, "element_size"):
+        return tuple(int(x) * a.element_size() for x in a.stride())
+    return tuple(int(x) for x in a.strides)
+
+
+def _address(a):
+    """address of the first element (the array may be a strided view)"""
+    return a.data_ptr() if hasattr(a, "data_ptr") else a.ctypes.data
+
+
 class TorchBackend:
     """Device memory and stream plumbing through PyTorch-ROCm."""
 
@@ -470,15 +486,51 @@ class HotPath:
     # ------------------------------------------------------------- gather
     def cache(self, row_bytes, hot, rows=None, cold=None, hot_slot=None, g2l=None,
               id_mask=-1, ts_hot=None, ts_cold=None):
+        """`cold` may be a row-strided view ([rows, width] with unit stride inside a row) and `ts_cold`
+        a strided 1-D view: their strides travel in the struct, so a cold tier that keeps a row and its
+        time in one record (see `interleaved_cold`) is read in place."""
         be = self.be
         hot_rows = 0 if hot is None else int(hot.shape[0])
         if rows is None:
             rows = int(cold.shape[0]) if cold is not None else hot_rows
+        cold_stride = ts_cold_stride = 0
+        cold_ptr, ts_cold_ptr = None, None
+        if cold is not None:
+            st = _byte_strides(cold)
+            if len(st) == 2 and cold.shape[0] > 1 and st[0] != cold.shape[1] * st[1]:
+                if st[1] != _itemsize(cold):
+                    raise ValueError("cache: the cold table must have unit stride inside a row")
+                cold_stride = int(st[0])
+            cold_ptr = _address(cold)
+        if ts_cold is not None:
+            st = _byte_strides(ts_cold)
+            if len(st) == 1 and ts_cold.shape[0] > 1 and st[0] != _itemsize(ts_cold):
+                ts_cold_stride = int(st[0])
+            ts_cold_ptr = _address(ts_cold)
         c = Cache(int(rows), int(row_bytes), int(id_mask), be.ptr(g2l),
                   0 if g2l is None else int(g2l.shape[0]), be.ptr(hot_slot), be.ptr(hot),
-                  hot_rows, be.ptr(cold), be.ptr(ts_hot), be.ptr(ts_cold))
+                  hot_rows, cold_ptr, be.ptr(ts_hot), ts_cold_ptr, cold_stride, ts_cold_stride)
         c._keep = (hot, cold, hot_slot, g2l, ts_hot, ts_cold)  # keep the arrays alive
         return c
+
+    def interleaved_cold(self, rows, width, dtype=None, record_bytes=None):
+        """Pinned host memory for a cold tier whose records hold a row and its last-update time side by
+        side: -> (data [rows, width] view, ts [rows] int64 view, record buffer).  Reads over PCIe are paid
+        for in whole 128-byte lines, so a time kept in a table of its own costs a line per row; in a
+        record of a multiple of 128 bytes it rides in the row's last line."""
+        torch = self.be.torch
+        dtype = dtype or torch.float32
+        item = torch.empty((), dtype=dtype).element_size()
+        row_bytes = width * item
+        ts_off = (row_bytes + 7) // 8 * 8
+        if record_bytes is None:
+            record_bytes = (ts_off + 8 + 127) // 128 * 128
+        if record_bytes % 8 or record_bytes % item or record_bytes < ts_off + 8:
+            raise ValueError("interleaved_cold: record size %d does not fit row + time" % record_bytes)
+        buf = torch.zeros((rows, record_bytes), dtype=torch.uint8, pin_memory=self.be.device.type == "cuda")
+        data = buf.view(dtype)[:, :width]
+        ts = buf.view(torch.int64)[:, ts_off // 8]
+        return data, ts, buf
 
     def gather(self, cache, ids, out, out_ts=None, stats=None, N_dev=None):
         self._chk("i64", ids=ids, out_ts=out_ts, stats=stats, N_dev=N_dev)
@@ -504,8 +556,9 @@ class HotPath:
     def scatter_update(self, cache, hot_rw, cold_rw, ts_hot_rw, ts_cold_rw, ids, values, ts=None):
         self._chk("i64", ids=ids, ts=ts)
         be = self.be
-        self._ck(self.lib.scatter_update(C.byref(cache), be.ptr(hot_rw), be.ptr(cold_rw),
-                                         be.ptr(ts_hot_rw), be.ptr(ts_cold_rw), be.ptr(ids),
+        addr = lambda a: None if a is None else _address(a)     # (the cold tier may be strided views of a record buffer)
+        self._ck(self.lib.scatter_update(C.byref(cache), be.ptr(hot_rw), addr(cold_rw),
+                                         be.ptr(ts_hot_rw), addr(ts_cold_rw), be.ptr(ids),
                                          int(ids.shape[0]), be.ptr(values), be.ptr(ts),
                                          be.stream()))
 

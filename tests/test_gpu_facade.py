@@ -245,6 +245,10 @@ def test_dist_node_state(mode, tiered):
     ns.to("cuda:0")
     d, tt = ns[q]
     assert torch.equal(d.cpu(), ref_data[q_loc]) and torch.equal(tt.cpu(), ref_ts[q_loc])
+    ns.to("cpu")             # back into records of pinned memory (row and time side by side)
+    d, tt = ns[q]
+    assert ns.data.is_pinned() and torch.equal(d.cpu(), ref_data[q_loc]) and torch.equal(tt.cpu(), ref_ts[q_loc])
+    assert torch.equal(ns.data, ref_data) and torch.equal(ns.ts, ref_ts)
     ns.reset()
     assert not ns[q][0].any()
 

@@ -135,6 +135,61 @@ def test_scatter_update_roundtrip(oracle, hot):
     assert np.array_equal(np_of(out)[keep], vals[keep])
 
 
+@pytest.mark.parametrize("dim", [100, 3, 172])
+def test_interleaved_cold_records(oracle, hot, dim):
+    """cold tier whose records hold a row and its last-update time side by side (cold_stride / ts_cold_stride of
+    sgl_cache): gather with times, scatter_update and a multi-segment gather read and write the records in place;
+    byte-exact against numpy on the same values and against the oracle on a numpy copy of the record buffer."""
+    rows, N = 6000, 20_000
+    full, h, c, slot = _tables(rows, dim, np.float32, 0.2, 40 + dim)
+    rng = np.random.default_rng(dim)
+    ts_full = rng.integers(1, 10**9, rows).astype(np.int64)
+    data, ts, rec = hot.interleaved_cold(rows, dim)
+    assert rec.is_pinned() and rec.shape[1] % 128 == 0 and data.shape == (rows, dim) and ts.shape == (rows,)
+    data.copy_(torch.from_numpy(c))
+    ts.copy_(torch.from_numpy(ts_full))
+    hot_ids = np.nonzero(slot >= 0)[0]
+    ts_hot_np = np.zeros(h.shape[0], np.int64)
+    ts_hot_np[slot[hot_ids]] = ts_full[hot_ids]
+    t_hot, t_slot, t_ts_hot = torch.from_numpy(h).to(hot.be.device), to_dev(hot, slot, "i32"), to_dev(hot, ts_hot_np)
+    cache = hot.cache(dim * 4, t_hot, rows=rows, cold=data, hot_slot=t_slot, ts_hot=t_ts_hot, ts_cold=ts)
+    assert cache.cold_stride == rec.shape[1] and cache.ts_cold_stride == rec.shape[1]
+    ids = rng.integers(-2, rows, N).astype(np.int64)
+    out = torch.empty((N, dim), dtype=torch.float32, device=hot.be.device)
+    out_ts = hot.be.empty(N)
+    hot.gather(cache, to_dev(hot, ids), out, out_ts=out_ts)
+    ok = ids >= 0
+    assert np.array_equal(np_of(out)[ok], full[ids[ok]]) and not np_of(out)[~ok].any()
+    assert np.array_equal(np_of(out_ts)[ok], ts_full[ids[ok]]) and not np_of(out_ts)[~ok].any()
+    # the oracle on a numpy copy of the same records
+    o_rec = rec.numpy().copy()
+    o_data = o_rec.view(np.float32)[:, :dim]
+    o_ts = o_rec.view(np.int64)[:, (dim * 4 + 7) // 8]
+    oh, oth = h.copy(), ts_hot_np.copy()
+    oc = oracle.cache(dim * 4, oh, rows=rows, cold=o_data, hot_slot=slot, ts_hot=oth, ts_cold=o_ts)
+    o_out, o_out_ts = np.empty((N, dim), np.float32), np.empty(N, np.int64)
+    oracle.gather(oc, ids, o_out, out_ts=o_out_ts)
+    assert np.array_equal(np_of(out), o_out) and np.array_equal(np_of(out_ts), o_out_ts)
+    # rows and times written back in place
+    upd = rng.permutation(rows)[:2000].astype(np.int64)
+    vals = rng.standard_normal((2000, dim)).astype(np.float32)
+    new_ts = rng.integers(10**9, 2 * 10**9, 2000).astype(np.int64)
+    hot.scatter_update(cache, t_hot, data, t_ts_hot, ts, to_dev(hot, upd), to_dev(hot, vals, "f32"), to_dev(hot, new_ts))
+    torch.cuda.synchronize()
+    oracle.scatter_update(oc, oh, o_data, oth, o_ts, upd, vals, new_ts)
+    assert np.array_equal(rec.numpy(), o_rec) and np.array_equal(np_of(t_hot), oh) and np.array_equal(np_of(t_ts_hot), oth)
+    if dim % 4 == 0:        # a strided segment beside a packed one in one launch
+        out2 = torch.empty((N, dim), dtype=torch.float32, device=hot.be.device)
+        out_ts2 = hot.be.empty(N)
+        other = torch.from_numpy(full).to(hot.be.device)
+        out3 = torch.empty((N, dim), dtype=torch.float32, device=hot.be.device)
+        ids_d = to_dev(hot, np.where(ids < 0, 0, ids))
+        hot.gather_multi(hot.gather_plan([(cache, ids_d, out2, out_ts2, None), (hot.cache(dim * 4, other), ids_d, out3, None, None)]))
+        full[upd], ts_full[upd] = vals, new_ts
+        idc = np.where(ids < 0, 0, ids)
+        assert np.array_equal(np_of(out2), full[idc]) and np.array_equal(np_of(out_ts2), ts_full[idc])
+
+
 def test_gather_multi_equals_single_gathers(oracle, hot):
     """three segments (tiered 400 B rows with timestamps and a device-side count, all-HBM 688 B
     rows, all-HBM 256 B rows) in one launch == three sgl_gather calls, byte for byte."""
