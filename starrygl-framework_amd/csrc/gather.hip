@@ -43,6 +43,15 @@ struct GatherArgs {
 __host__ __device__ __forceinline__ int64_t cold_stride(const sgl_cache& c) { return c.cold_stride ? c.cold_stride : c.row_bytes; }
 __host__ __device__ __forceinline__ int64_t ts_cold_stride(const sgl_cache& c) { return c.ts_cold_stride ? c.ts_cold_stride : 8; }
 
+// lc / cpr for a chunk index inside a block's tile (lc < 2^22: a tile holds at most 1024 rows of at most 1024
+// chunks, or one row of at most 65536): one multiply and a fix-up in place of an integer division per chunk.
+__device__ __forceinline__ int32_t row_of_chunk(int32_t lc, int32_t cpr, float inv_cpr) {
+    int32_t r = (int32_t)(((float)lc + 0.5f) * inv_cpr);
+    r -= (r * cpr > lc) ? 1 : 0;
+    r += ((r + 1) * cpr <= lc) ? 1 : 0;
+    return r;
+}
+
 // id -> (source row address, last-update time); nullptr when not resident.
 // tier: 0 hot, 1 cold, 2 absent.
 __device__ __forceinline__ const char* resolve(const sgl_cache& c, int64_t id, int64_t* ts_out,
@@ -80,6 +89,7 @@ __global__ __launch_bounds__(BLOCK) void gather_kernel(GatherArgs a) {
     const int64_t N = live_count(a.N_dev, a.N_max);
     if (threadIdx.x < 3) s_tier[threadIdx.x] = 0;
     const int32_t cpr = a.cpr;
+    const float inv_cpr = 1.0f / (float)cpr;
     const int64_t first_row = (int64_t)blockIdx.x * a.rpb;
     if (a.stats != nullptr) __syncthreads();  // s_tier is zero before the first atomicAdd
     for (int64_t row0 = first_row; row0 < N; row0 += (int64_t)gridDim.x * a.rpb) {
@@ -102,7 +112,7 @@ __global__ __launch_bounds__(BLOCK) void gather_kernel(GatherArgs a) {
                 const int32_t lc = base + u * BLOCK + threadIdx.x;
                 V v = {};
                 if (lc < total) {
-                    const int32_t r = lc / cpr;
+                    const int32_t r = row_of_chunk(lc, cpr, inv_cpr);
                     const int32_t part = lc - r * cpr;
                     const V* src = reinterpret_cast<const V*>(s_src[r]);
                     if (src != nullptr) v = NT ? __builtin_nontemporal_load(src + part) : src[part];
@@ -155,6 +165,7 @@ __global__ __launch_bounds__(BLOCK) void gather_multi_kernel(MultiArgs m) {
         const MultiSeg& a = m.seg[t];
         const int64_t N = live_count(a.N_dev, a.N_max);
         const int32_t cpr = a.cpr;
+        const float inv_cpr = 1.0f / (float)cpr;
         for (int64_t row0 = (int64_t)blockIdx.x * a.rpb; row0 < N; row0 += (int64_t)gridDim.x * a.rpb) {
             const int32_t rows = (int32_t)((N - row0) < a.rpb ? (N - row0) : a.rpb);
             __syncthreads();  // s_src of the previous tile has been consumed
@@ -174,7 +185,7 @@ __global__ __launch_bounds__(BLOCK) void gather_multi_kernel(MultiArgs m) {
                     const int32_t lc = base + u * BLOCK + threadIdx.x;
                     u32x4 v = {};
                     if (lc < total) {
-                        const int32_t r = lc / cpr;
+                        const int32_t r = row_of_chunk(lc, cpr, inv_cpr);
                         const int32_t part = lc - r * cpr;
                         const u32x4* src = reinterpret_cast<const u32x4*>(s_src[r]);
                         if (src != nullptr) v = src[part];
@@ -232,10 +243,11 @@ __global__ __launch_bounds__(BLOCK) void scatter_kernel(ScatterArgs a) {
         }
         __syncthreads();
         const int32_t cpr = a.cpr;
+        const float inv_cpr = 1.0f / (float)cpr;
         const int32_t total = rows * cpr;
         const V* __restrict__ src = reinterpret_cast<const V*>(a.values + row0 * a.c.row_bytes);
         for (int32_t lc = threadIdx.x; lc < total; lc += BLOCK) {
-            const int32_t r = lc / cpr;
+            const int32_t r = row_of_chunk(lc, cpr, inv_cpr);
             const int32_t part = lc - r * cpr;
             V* d = reinterpret_cast<V*>(s_dst[r]);
             if (d != nullptr) d[part] = src[lc];

@@ -386,6 +386,72 @@ __device__ __forceinline__ int64_t bounded(uint64_t bits, int64_t range) {
     return (int64_t)__umul64hi(bits, (uint64_t)range);
 }
 
+// x of lane j of every G-lane group of the wave, handed to the group's lanes (j is wave-uniform): lane reads
+// into scalar registers and a select per group instead of a trip through the LDS crossbar.
+template <int G>
+__device__ __forceinline__ int32_t group_bcast(int32_t x, int j, int wlane) {
+    int32_t r = __builtin_amdgcn_readlane(x, j);
+#pragma unroll
+    for (int g = 1; g < WAVE / G; ++g) {
+        const int32_t y = __builtin_amdgcn_readlane(x, g * G + j);
+        r = wlane >= g * G ? y : r;
+    }
+    return r;
+}
+
+// Floyd's subset of k of [0, len) for every drawing group of the wave (draw is uniform inside a group; lane
+// lig < k holds draw tj from [0, len - k + lig]): step j keeps its draw unless an earlier step holds the same
+// value, then it takes len - k + j.  -> the lane's pick and its rank among the k picks (all distinct).
+// Two draws of a group collide only in windows of a few thousand edges or fewer: the ranks are counted on the raw
+// draws first, and the sequential construction runs only in waves where some group saw two equal draws.
+// Windows of 2^31 edges and more take the 64-bit variant.
+template <int G>
+__device__ __forceinline__ void floyd_subset(bool draw, int lig, int wlane, int gshift, int32_t k, int64_t len, int64_t tj,
+                                             int64_t* pick, int32_t* rank) {
+    const bool mine_on = draw && lig < k;
+    if (__all(!draw || len <= (int64_t)INT32_MAX)) {          // wave-uniform
+        int32_t v = mine_on ? (int32_t)tj : -1 - lig;            // (idle lanes hold distinct negatives)
+        int32_t r = 0;
+        bool dup = false;
+        for (int32_t j = 0; j < k; ++j) {
+            const int32_t o = group_bcast<G>(v, j, wlane);
+            r += o < v ? 1 : 0;
+            dup |= o == v && j != lig;
+        }
+        if (__any(mine_on && dup)) {
+            int32_t m = -1;
+            for (int32_t j = 0; j < k; ++j) {
+                const int32_t cand = group_bcast<G>(v, j, wlane);
+                const bool hit = group_ballot<G>(draw && lig < j && m == cand, gshift) != 0;
+                if (lig == j) m = hit ? (int32_t)(len - k + j) : cand;
+            }
+            v = mine_on ? m : -1 - lig;
+            r = 0;
+            for (int32_t j = 0; j < k; ++j) r += group_bcast<G>(v, j, wlane) < v ? 1 : 0;
+        }
+        if (draw) {
+            *pick = (int64_t)v;
+            *rank = r;
+        }
+        return;
+    }
+    int64_t mine = -1;
+    for (int32_t j = 0; j < k; ++j) {
+        const int64_t cand = shfl_i64(tj, (wlane - lig) + j);
+        const bool hit = group_ballot<G>(draw && lig < j && mine == cand, gshift) != 0;
+        if (lig == j) mine = hit ? (len - k + j) : cand;
+    }
+    int32_t r = 0;
+    for (int32_t j = 0; j < k; ++j) {
+        const int64_t other = shfl_i64(mine, (wlane - lig) + j);
+        r += (other < mine) ? 1 : 0;
+    }
+    if (draw) {
+        *pick = mine;
+        *rank = r;
+    }
+}
+
 template <int G, bool UNIFORM>
 __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     constexpr int SPB = BLOCK / G;
@@ -594,23 +660,9 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
                 if (a.replace) {
                     if (draw) sel = tj;  // draw order is kept
                 } else {
-                    // Floyd: step j picks t_j from [0, len-k+j]; a repeat is replaced by len-k+j
-                    int64_t mine = -1;
-                    for (int32_t j = 0; j < k; ++j) {
-                        const int64_t cand = shfl_i64(tj, (wlane - lig) + j);
-                        const bool dup = group_ballot<G>(draw && lig < j && mine == cand, gshift) != 0;
-                        if (lig == j) mine = dup ? (len - k + j) : cand;
-                    }
-                    // rank among the k picks (all distinct) = output position
-                    int32_t r = 0;
-                    for (int32_t j = 0; j < k; ++j) {
-                        const int64_t other = shfl_i64(mine, (wlane - lig) + j);
-                        r += (other < mine) ? 1 : 0;
-                    }
-                    if (draw) {
-                        sel = mine;
-                        rank = r;
-                    }
+                    // Floyd: step j picks t_j from [0, len-k+j]; a repeat is replaced by len-k+j; rank among
+                    // the k picks (all distinct) = output position
+                    floyd_subset<G>(draw, lig, wlane, gshift, k, len, tj, &sel, &rank);
                 }
             }
             if (active && lig < c) {
@@ -869,21 +921,7 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
             if (a.replace) {
                 if (draw) sel = tj;
             } else {
-                int64_t mine = -1;
-                for (int32_t j = 0; j < k; ++j) {
-                    const int64_t cand = shfl_i64(tj, gbase + j);
-                    const bool dup = group_ballot<FG>(draw && lig < j && mine == cand, gshift) != 0;
-                    if (lig == j) mine = dup ? (len - k + j) : cand;
-                }
-                int32_t r = 0;
-                for (int32_t j = 0; j < k; ++j) {
-                    const int64_t other = shfl_i64(mine, gbase + j);
-                    r += (other < mine) ? 1 : 0;
-                }
-                if (draw) {
-                    sel = mine;
-                    rank = r;
-                }
+                floyd_subset<FG>(draw, lig, wlane, gshift, k, len, tj, &sel, &rank);
             }
             int64_t placed = sel;
             for (int32_t j = 0; j < k; ++j) {
