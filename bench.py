@@ -402,6 +402,17 @@ def workload_large_partition(hot, torch, np, synth, _abi, n=100_000_000, m=1_000
         ms_m = float(np.mean(ms_u))
         res[tag] = {"ms": round(ms_m, 4), "edges_per_batch": e_u / NB, "edges_per_s": round(e_u / NB / ms_m * 1e3, 1),
                     "over_recent": round(ms_m / ms, 2)}
+    # what the picks alone cost: as many 32-byte records as a uniform batch samples, gathered from uniformly
+    # random positions of the record array into a contiguous output by the library's gather (one scattered
+    # sector read and 32 bytes written per pick; the sampler adds the draws, the windows and three more outputs)
+    n_pick = int(e_u / NB)
+    pick_ids = torch.randint(0, g.m, (n_pick,), device=dev, generator=torch.Generator(device=dev).manual_seed(3))
+    pick_out = torch.empty((n_pick, 4), dtype=torch.int64, device=dev)
+    c_rec = hot.cache(32, g.rec.view(-1, 4))
+    ms_p = _time_launches(torch, lambda: hot.gather(c_rec, pick_ids, pick_out), reps=5, warm=1)
+    res["scattered_record_gather_same_picks"] = {"ms": round(ms_p, 4), "records": n_pick, "records_per_s": round(n_pick / ms_p * 1e3, 1),
+                                                 "over_recent": round(ms_p / ms, 2)}
+    del pick_ids, pick_out, c_rec
     del ku
     g.rec = None
     g.view.rec = None

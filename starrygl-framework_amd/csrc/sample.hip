@@ -530,15 +530,14 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     }
     int par = 0;
     for (int64_t it = first; it < first + run && it < S; it += SPB, par ^= 1) {
-        if (it != first) {
-            slot = it + gib;
-            active = slot < S;
-            start = len = t = 0;
-            if (active) {
-                start = a.w_start[slot];
-                len = a.w_len[slot];
-                t = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
-            }
+        // the next iteration's slot is loaded now, so that its latency runs beside this iteration's picks and copies
+        const int64_t nslot = it + SPB + gib;
+        const bool nactive = it + SPB < first + run && nslot < S;
+        int64_t nstart = 0, nlen = 0, nt = 0;
+        if (nactive) {
+            nstart = a.w_start[nslot];
+            nlen = a.w_len[nslot];
+            nt = a.derive ? a.slot_ts_out[nslot] : a.slot_ts[nslot];
         }
         const int32_t c = (int32_t)(len < k ? len : k);
         // exclusive prefix of c over the iteration's slots: scan inside the wave (one
@@ -675,6 +674,11 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
                 if (a.hint_out != nullptr) a.hint_out[off + rank] = ed.hint;
             }
         }
+        slot = nslot;
+        active = nactive;
+        start = nstart;
+        len = nlen;
+        t = nt;
     }
 }
 
