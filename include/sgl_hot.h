@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define SGL_ABI_VERSION 5
+#define SGL_ABI_VERSION 6
 
 /* ------------------------------------------------------------------ status */
 #define SGL_OK        0

@@ -5,7 +5,7 @@ header declares.  The product library exports them as ``sgl_*``.
 """
 import ctypes as C
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
