@@ -463,9 +463,15 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
     const int gshift = wlane / G * G;
     const int32_t k = a.k;
-    // first iteration's slot data: loaded before the live count arrives when the grid is
+    // The uniform strategy with a group per slot gives each of the block's waves a stretch of the run of its own
+    // (below): its waves spend their time on draws and scattered picks and gain from running apart (857k slots of
+    // 20 picks: 647 -> 590 us).  The copies of the most-recent strategy lose 8 % that way (a block's waves then write
+    // four distant pieces of the output at a time) and keep walking the run with the whole block, one iteration's
+    // slots at a time, as does the uniform kernel with a wavefront per slot (its subset construction needs block barriers).
+    constexpr bool WAVE_RUNS = UNIFORM && G != WAVE;
+    // (whole-block walk) first iteration's slot data: loaded before the live count arrives when the grid is
     // not capped (see count_kernel), and before the prefix sum, so the loads overlap both
-    const bool fixed = a.align == SPB && (int64_t)gridDim.x * SPB >= a.S_max;
+    const bool fixed = !WAVE_RUNS && a.align == SPB && (int64_t)gridDim.x * SPB >= a.S_max;
     int64_t slot = (int64_t)blockIdx.x * SPB + gib;
     int64_t start = 0, len = 0, t = 0;
     if (fixed && slot < a.S_max) {
@@ -477,7 +483,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     int64_t first, run;
     block_run(S, a.align, &first, &run);
     bool active = first < S && first + gib < S;
-    if (!fixed) {
+    if (!fixed && !WAVE_RUNS) {
         slot = first + gib;
         if (active) {
             start = a.w_start[slot];
@@ -486,6 +492,33 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
         }
     }
     if (!active) start = len = t = 0;   // speculative loads of slots beyond the live count
+    // (a stretch per wave) the wave's stretch, its first slots and the edges of the stretch: loaded before the
+    // block's offset is worked out, so that the latencies run side by side
+    int64_t wfirst = 0, wend = 0;
+    if constexpr (WAVE_RUNS) {
+        constexpr int SPW = WAVE / G;
+        int64_t rw = ceil_div<int64_t>(run, (int64_t)NWAVE);
+        rw = ceil_div<int64_t>(rw, (int64_t)SPW) * SPW;
+        const int64_t run_end = first + run < S ? first + run : S;
+        wfirst = first + (int64_t)wid * rw;
+        if (wfirst > run_end) wfirst = run_end;
+        wend = wfirst + rw < run_end ? wfirst + rw : run_end;
+        slot = wfirst + wlane / G;
+        active = slot < wend;
+        start = len = t = 0;
+        if (active) {
+            start = a.w_start[slot];
+            len = a.w_len[slot];
+            t = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
+        }
+        int32_t wsum = 0;
+        for (int64_t j = wfirst + wlane; j < wend; j += WAVE) {
+            const int64_t l = a.w_len[j];
+            wsum += (int32_t)(l < k ? l : k);
+        }
+        for (int d = WAVE / 2; d > 0; d >>= 1) wsum += __shfl(wsum, wlane ^ d);
+        if (wlane == 0) s_wtot[0][wid] = wsum;
+    }
     // exclusive prefix of this block: read it (scan_kernel ran) or add up the sums of
     // the blocks before it
     int64_t run_off = 0;
@@ -528,6 +561,162 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
             a.root_end_ptr[S] = E;
         }
     }
+    // one slot of the hop: its two offsets, then its edges (copied, or picked and copied)
+    auto emit_slot = [&](int64_t slot, bool active, int64_t start, int64_t len, int64_t t, int32_t c, int64_t off) {
+            if (active && lig == 0) {
+                a.root_start_ptr[slot] = off;
+                a.root_end_ptr[slot] = off + c;
+            }
+            if constexpr (!UNIFORM) {
+                if (active) {
+                    // up to ROUNDS * G edges per pass, every load issued before the first store
+                    constexpr int ROUNDS = 4;
+                    for (int32_t j0 = lig; j0 < c; j0 += ROUNDS * G) {
+                        int64_t ets[ROUNDS], dst[ROUNDS], id[ROUNDS];
+    #pragma unroll
+                        for (int r = 0; r < ROUNDS; ++r) {
+                            const int32_t j = j0 + r * G;
+                            if (j < c) {
+                                const int64_t e = start + j;
+                                ets[r] = a.ts[e];
+                                dst[r] = a.col[e];
+                                id[r] = a.eid[e];
+                                if (a.hint_out != nullptr) a.hint_out[off + j] = a.hint[e];
+                            }
+                        }
+    #pragma unroll
+                        for (int r = 0; r < ROUNDS; ++r) {
+                            const int32_t j = j0 + r * G;
+                            if (j < c) {
+                                a.nbr[off + j] = dst[r];
+                                if (a.mark != nullptr) mark_id(a, dst[r]);
+                                a.nbr_ts[off + j] = ets[r];
+                                a.nbr_eid[off + j] = id[r];
+                                a.nbr_dt[off + j] = ets[r] - t;
+                            }
+                        }
+                    }
+                }
+            } else if (G == WAVE && k > G) {
+                // ---- uniform with a fanout beyond one wavefront (a wave per slot, picks in dynamic LDS) ----
+                // Block-uniform control flow (the loops run to k for every wave, idle waves skip the work),
+                // so that block barriers order the LDS accesses of the sequential subset construction.
+                extern __shared__ int64_t s_wide[];
+                int64_t* pk = s_wide + (size_t)wid * k;
+                const bool draw = active && len > k;
+                auto emit = [&](int64_t sel, int64_t place) {
+                    const Edge ed = load_picked_edge(a, start + sel);
+                    a.nbr[off + place] = ed.col;
+                    if (a.mark != nullptr) mark_id(a, ed.col);
+                    a.nbr_ts[off + place] = a.keep_root_time ? t : ed.ts;
+                    a.nbr_eid[off + place] = ed.eid;
+                    a.nbr_dt[off + place] = ed.ts - t;
+                    if (a.hint_out != nullptr) a.hint_out[off + place] = ed.hint;
+                };
+                if (active && !draw)                      // the whole window, in storage order
+                    for (int32_t j = lig; j < c; j += G) emit(j, j);
+                if (draw)
+                    for (int32_t j = lig; j < k; j += G) {
+                        const uint64_t bits = draw_bits(a.seed, a.hop, slot, j);
+                        pk[j] = a.replace ? bounded(bits, len) : bounded(bits, len - k + j + 1);
+                    }
+                __syncthreads();
+                if (a.replace) {                          // kernel argument: uniform; draw order is kept
+                    if (draw)
+                        for (int32_t j = lig; j < k; j += G) emit(pk[j], j);
+                } else {
+                    // Floyd: step j keeps its draw unless an earlier step holds the same value, then it takes len-k+j
+                    for (int32_t j = 1; j < k; ++j) {
+                        bool dup = false;
+                        if (draw) {
+                            const int64_t cand = pk[j];
+                            for (int32_t i = lig; i < j; i += G) dup |= pk[i] == cand;
+                        }
+                        dup = __any(dup);
+                        __syncthreads();
+                        if (draw && dup && lig == 0) pk[j] = len - k + j;
+                        __syncthreads();
+                    }
+                    // ascending: the place of a pick is the number of smaller picks (all distinct)
+                    if (draw)
+                        for (int32_t j = lig; j < k; j += G) {
+                            const int64_t mine = pk[j];
+                            int32_t r = 0;
+                            for (int32_t i = 0; i < k; ++i) r += pk[i] < mine ? 1 : 0;
+                            emit(mine, r);
+                        }
+                }
+                __syncthreads();                          // the picks are reused by the next iteration
+            } else {
+                // ---- uniform: k <= G ----------------------------------------------------
+                const bool draw = active && len > k;  // uniform inside the group
+                int64_t sel = lig;                    // offset inside the window; copy path: identity
+                int32_t rank = lig;
+                const bool any_draw = __any(draw);
+                if (any_draw) {                       // wave-uniform branch
+                    int64_t tj = 0;
+                    if (draw && lig < k) {
+                        const uint64_t bits = draw_bits(a.seed, a.hop, slot, lig);
+                        tj = a.replace ? bounded(bits, len) : bounded(bits, len - k + lig + 1);
+                    }
+                    if (a.replace) {
+                        if (draw) sel = tj;  // draw order is kept
+                    } else {
+                        // Floyd: step j picks t_j from [0, len-k+j]; a repeat is replaced by len-k+j; rank among
+                        // the k picks (all distinct) = output position
+                        floyd_subset<G>(draw, lig, wlane, gshift, k, len, tj, &sel, &rank);
+                    }
+                }
+                if (active && lig < c) {
+                    const Edge ed = load_picked_edge(a, start + sel);
+                    a.nbr[off + rank] = ed.col;
+                    if (a.mark != nullptr) mark_id(a, ed.col);
+                    a.nbr_ts[off + rank] = a.keep_root_time ? t : ed.ts;
+                    a.nbr_eid[off + rank] = ed.eid;
+                    a.nbr_dt[off + rank] = ed.ts - t;
+                    if (a.hint_out != nullptr) a.hint_out[off + rank] = ed.hint;
+                }
+            }
+    };
+    // A stretch of the run per wave: a wave adds up the edges of its stretch, one barrier hands every wave the edges
+    // of the waves before it, and from there on the waves run without barriers (a slot's offset is a prefix inside
+    // its wave), each loading its next slots while it copies the current ones.
+    if constexpr (WAVE_RUNS) {
+        constexpr int SPW = WAVE / G;
+        const int gw = wlane / G;
+        __syncthreads();                 // the waves' edge totals are in s_wtot[0]
+        int64_t wave_off = run_off;
+#pragma unroll
+        for (int q = 0; q < NWAVE; ++q)
+            if (q < wid) wave_off += s_wtot[0][q];
+        for (int64_t it = wfirst; it < wend; it += SPW) {
+            // the next iteration's slot is loaded now, so that its latency runs beside this iteration's picks and copies
+            const int64_t nslot = it + SPW + gw;
+            const bool nactive = nslot < wend;
+            int64_t nstart = 0, nlen = 0, nt = 0;
+            if (nactive) {
+                nstart = a.w_start[nslot];
+                nlen = a.w_len[nslot];
+                nt = a.derive ? a.slot_ts_out[nslot] : a.slot_ts[nslot];
+            }
+            const int32_t c = (int32_t)(len < k ? len : k);
+            int32_t inc = (lig == 0) ? c : 0;
+            for (int d = 1; d < WAVE; d <<= 1) {
+                const int32_t x = __shfl_up(inc, d);
+                if (wlane >= d) inc += x;
+            }
+            const int32_t excl = __shfl(inc - ((lig == 0) ? c : 0), wlane - lig);
+            const int32_t iter_total = __shfl(inc, WAVE - 1);
+            emit_slot(slot, active, start, len, t, c, wave_off + excl);
+            wave_off += iter_total;
+            slot = nslot;
+            active = nactive;
+            start = nstart;
+            len = nlen;
+            t = nt;
+        }
+        return;
+    }
     int par = 0;
     for (int64_t it = first; it < first + run && it < S; it += SPB, par ^= 1) {
         // the next iteration's slot is loaded now, so that its latency runs beside this iteration's picks and copies
@@ -560,120 +749,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
         }
         const int64_t off = run_off + wave_off + excl;
         run_off += iter_total;
-        if (active && lig == 0) {
-            a.root_start_ptr[slot] = off;
-            a.root_end_ptr[slot] = off + c;
-        }
-        if constexpr (!UNIFORM) {
-            if (active) {
-                // up to ROUNDS * G edges per pass, every load issued before the first store
-                constexpr int ROUNDS = 4;
-                for (int32_t j0 = lig; j0 < c; j0 += ROUNDS * G) {
-                    int64_t ets[ROUNDS], dst[ROUNDS], id[ROUNDS];
-#pragma unroll
-                    for (int r = 0; r < ROUNDS; ++r) {
-                        const int32_t j = j0 + r * G;
-                        if (j < c) {
-                            const int64_t e = start + j;
-                            ets[r] = a.ts[e];
-                            dst[r] = a.col[e];
-                            id[r] = a.eid[e];
-                            if (a.hint_out != nullptr) a.hint_out[off + j] = a.hint[e];
-                        }
-                    }
-#pragma unroll
-                    for (int r = 0; r < ROUNDS; ++r) {
-                        const int32_t j = j0 + r * G;
-                        if (j < c) {
-                            a.nbr[off + j] = dst[r];
-                            if (a.mark != nullptr) mark_id(a, dst[r]);
-                            a.nbr_ts[off + j] = ets[r];
-                            a.nbr_eid[off + j] = id[r];
-                            a.nbr_dt[off + j] = ets[r] - t;
-                        }
-                    }
-                }
-            }
-        } else if (G == WAVE && k > G) {
-            // ---- uniform with a fanout beyond one wavefront (a wave per slot, picks in dynamic LDS) ----
-            // Block-uniform control flow (the loops run to k for every wave, idle waves skip the work),
-            // so that block barriers order the LDS accesses of the sequential subset construction.
-            extern __shared__ int64_t s_wide[];
-            int64_t* pk = s_wide + (size_t)wid * k;
-            const bool draw = active && len > k;
-            auto emit = [&](int64_t sel, int64_t place) {
-                const Edge ed = load_picked_edge(a, start + sel);
-                a.nbr[off + place] = ed.col;
-                if (a.mark != nullptr) mark_id(a, ed.col);
-                a.nbr_ts[off + place] = a.keep_root_time ? t : ed.ts;
-                a.nbr_eid[off + place] = ed.eid;
-                a.nbr_dt[off + place] = ed.ts - t;
-                if (a.hint_out != nullptr) a.hint_out[off + place] = ed.hint;
-            };
-            if (active && !draw)                      // the whole window, in storage order
-                for (int32_t j = lig; j < c; j += G) emit(j, j);
-            if (draw)
-                for (int32_t j = lig; j < k; j += G) {
-                    const uint64_t bits = draw_bits(a.seed, a.hop, slot, j);
-                    pk[j] = a.replace ? bounded(bits, len) : bounded(bits, len - k + j + 1);
-                }
-            __syncthreads();
-            if (a.replace) {                          // kernel argument: uniform; draw order is kept
-                if (draw)
-                    for (int32_t j = lig; j < k; j += G) emit(pk[j], j);
-            } else {
-                // Floyd: step j keeps its draw unless an earlier step holds the same value, then it takes len-k+j
-                for (int32_t j = 1; j < k; ++j) {
-                    bool dup = false;
-                    if (draw) {
-                        const int64_t cand = pk[j];
-                        for (int32_t i = lig; i < j; i += G) dup |= pk[i] == cand;
-                    }
-                    dup = __any(dup);
-                    __syncthreads();
-                    if (draw && dup && lig == 0) pk[j] = len - k + j;
-                    __syncthreads();
-                }
-                // ascending: the place of a pick is the number of smaller picks (all distinct)
-                if (draw)
-                    for (int32_t j = lig; j < k; j += G) {
-                        const int64_t mine = pk[j];
-                        int32_t r = 0;
-                        for (int32_t i = 0; i < k; ++i) r += pk[i] < mine ? 1 : 0;
-                        emit(mine, r);
-                    }
-            }
-            __syncthreads();                          // the picks are reused by the next iteration
-        } else {
-            // ---- uniform: k <= G ----------------------------------------------------
-            const bool draw = active && len > k;  // uniform inside the group
-            int64_t sel = lig;                    // offset inside the window; copy path: identity
-            int32_t rank = lig;
-            const bool any_draw = __any(draw);
-            if (any_draw) {                       // wave-uniform branch
-                int64_t tj = 0;
-                if (draw && lig < k) {
-                    const uint64_t bits = draw_bits(a.seed, a.hop, slot, lig);
-                    tj = a.replace ? bounded(bits, len) : bounded(bits, len - k + lig + 1);
-                }
-                if (a.replace) {
-                    if (draw) sel = tj;  // draw order is kept
-                } else {
-                    // Floyd: step j picks t_j from [0, len-k+j]; a repeat is replaced by len-k+j; rank among
-                    // the k picks (all distinct) = output position
-                    floyd_subset<G>(draw, lig, wlane, gshift, k, len, tj, &sel, &rank);
-                }
-            }
-            if (active && lig < c) {
-                const Edge ed = load_picked_edge(a, start + sel);
-                a.nbr[off + rank] = ed.col;
-                if (a.mark != nullptr) mark_id(a, ed.col);
-                a.nbr_ts[off + rank] = a.keep_root_time ? t : ed.ts;
-                a.nbr_eid[off + rank] = ed.eid;
-                a.nbr_dt[off + rank] = ed.ts - t;
-                if (a.hint_out != nullptr) a.hint_out[off + rank] = ed.hint;
-            }
-        }
+        emit_slot(slot, active, start, len, t, c, off);
         slot = nslot;
         active = nactive;
         start = nstart;
