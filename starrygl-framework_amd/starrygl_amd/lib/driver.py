@@ -7,6 +7,7 @@ the package uses; anything else that offers the same five methods can drive a
 library with the same ABI on host memory.
 """
 import ctypes as C
+import os
 
 from . import _abi
 from ._abi import (TCSR, Cache, GatherSeg, HopOut, SampleParams, SeedQuery, WindowParams, check, i64, vp)
@@ -163,6 +164,7 @@ class HotPath:
                                    f"bytes, the binding {C.sizeof(mirror)}")
         self._ws = {}
         self.recoveries = 0     # calls re-issued because a block had given up its bounded wait
+        self.check_hints = os.environ.get("SGL_CHECK_HINTS", "0") not in ("", "0")   # see verify_root_hint
 
     # ------------------------------------------------------------ helpers
     def _workspace(self, nbytes):
@@ -240,6 +242,28 @@ class HotPath:
         self._ck(self.lib.window_end(C.byref(g.view), self.be.ptr(node), self.be.ptr(t), int(node.shape[0]),
                                      self.be.ptr(out), self.be.stream()))
         return out
+
+    def verify_root_hint(self, g, roots, ts_ptr, root_ts, p):
+        """Debug check (SGL_CHECK_HINTS=1 in the environment makes the sampling calls run it, at the price of a
+        window search per positive slot and one host synchronisation): every root hint that is not -1 must
+        be what `window_end` finds for its slot on this graph.  The kernels clamp a hint to the root's row, so
+        a stale or foreign hint cannot cause a stray access, but it silently changes that slot's sample."""
+        hint = getattr(p, "_keep", (None, None))[1] if getattr(p, "_root_hint_len", None) is not None else None
+        if hint is None or not hasattr(self.be, "torch"):
+            return
+        torch = self.be.torch
+        S_pos = int(root_ts.shape[0])
+        if S_pos == 0:
+            return
+        slots = torch.arange(S_pos, device=root_ts.device)
+        node = roots[torch.searchsorted(ts_ptr, slots, right=True) - 1]
+        want = self.window_end(g, node.contiguous(), root_ts)
+        h = hint[:S_pos]
+        bad = (h >= 0) & (h != want)
+        if bool(bad.any()):
+            i = int(torch.nonzero(bad)[0])
+            raise ValueError(f"root_hint[{i}] = {int(h[i])}, but the window of slot {i} (node {int(node[i])}, "
+                             f"time {int(root_ts[i])}) ends at {int(want[i])} on this graph")
 
     def with_root_hint(self, p, root_hint):
         """Copy of the sampling parameters `p` that hands the k-hop sampler the window ends of the
@@ -365,6 +389,8 @@ class HotPath:
         R, S_pos, N_neg = int(roots.shape[0]), int(root_ts.shape[0]), int(neg_roots.shape[0])
         S0 = S_pos + N_neg
         _check_root_hint(p, S_pos)
+        if self.check_hints:
+            self.verify_root_hint(g, roots, ts_ptr, root_ts, p)
         res = out if out is not None else self.khop_buffers(S0, layers, p.fanout)
         if res.S0 < S0 or len(res.hops) != layers or res.fanout < p.fanout:
             raise MemoryError("khop buffers are smaller than this call needs")
@@ -395,6 +421,8 @@ class HotPath:
         fan = max(p.fanout for p in params)
         for p, res in zip(params, outs):
             _check_root_hint(p, S_pos)
+            if self.check_hints:
+                self.verify_root_hint(g, roots, ts_ptr, root_ts, p)
             if res.S0 < S0 or len(res.hops) != layers or res.fanout < p.fanout:
                 raise MemoryError("khop buffers are smaller than this call needs")
         head = outs[0]

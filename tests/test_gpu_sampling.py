@@ -375,6 +375,14 @@ def test_root_hints_give_the_same_samples(oracle, hot, sample_type):
     wild = to_dev(hot, rng.integers(-5, 2 * g.m, S_pos).astype(np.int64))
     res = hot.sample_khop(dg, *dev, 1, hot.with_root_hint(hot.params(sample_type, 17), wild))
     assert 0 <= res.hops[0].E <= (S_pos + n_neg) * 17
+    # ... and the driver's debug check (SGL_CHECK_HINTS=1) refuses them, while it passes hints that are right or -1
+    hot.check_hints = True
+    try:
+        with pytest.raises(ValueError, match="root_hint"):
+            hot.sample_khop(dg, *dev, 1, hot.with_root_hint(hot.params(sample_type, 17), wild))
+        hot.sample_khop(dg, *dev, 1, hot.with_root_hint(hot.params(sample_type, 17), hint))
+    finally:
+        hot.check_hints = False
 
 
 def test_window_end_edge_cases(oracle, hot):
