@@ -452,7 +452,7 @@ __device__ __forceinline__ void floyd_subset(bool draw, int lig, int wlane, int 
     }
 }
 
-template <int G, bool UNIFORM>
+template <int G>
 __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     constexpr int SPB = BLOCK / G;
     __shared__ int64_t s_red[NWAVE];
@@ -463,12 +463,11 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
     const int gshift = wlane / G * G;
     const int32_t k = a.k;
-    // The uniform strategy with a group per slot gives each of the block's waves a stretch of the run of its own
-    // (below): its waves spend their time on draws and scattered picks and gain from running apart (857k slots of
-    // 20 picks: 647 -> 590 us).  The copies of the most-recent strategy lose 8 % that way (a block's waves then write
-    // four distant pieces of the output at a time) and keep walking the run with the whole block, one iteration's
-    // slots at a time, as does the uniform kernel with a wavefront per slot (its subset construction needs block barriers).
-    constexpr bool WAVE_RUNS = UNIFORM && G != WAVE;
+    // With a group of lanes per slot each of the block's waves gets a stretch of the run of its own (below): the waves
+    // spend their time on draws and scattered picks and gain from running apart (857k slots of 20 picks: 647 -> 590 us).
+    // With a wavefront per slot the whole block walks the run, one iteration's slots at a time (the subset
+    // construction in LDS needs block barriers).
+    constexpr bool WAVE_RUNS = G != WAVE;
     // (whole-block walk) first iteration's slot data: loaded before the live count arrives when the grid is
     // not capped (see count_kernel), and before the prefix sum, so the loads overlap both
     const bool fixed = !WAVE_RUNS && a.align == SPB && (int64_t)gridDim.x * SPB >= a.S_max;
@@ -567,37 +566,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
                 a.root_start_ptr[slot] = off;
                 a.root_end_ptr[slot] = off + c;
             }
-            if constexpr (!UNIFORM) {
-                if (active) {
-                    // up to ROUNDS * G edges per pass, every load issued before the first store
-                    constexpr int ROUNDS = 4;
-                    for (int32_t j0 = lig; j0 < c; j0 += ROUNDS * G) {
-                        int64_t ets[ROUNDS], dst[ROUNDS], id[ROUNDS];
-    #pragma unroll
-                        for (int r = 0; r < ROUNDS; ++r) {
-                            const int32_t j = j0 + r * G;
-                            if (j < c) {
-                                const int64_t e = start + j;
-                                ets[r] = a.ts[e];
-                                dst[r] = a.col[e];
-                                id[r] = a.eid[e];
-                                if (a.hint_out != nullptr) a.hint_out[off + j] = a.hint[e];
-                            }
-                        }
-    #pragma unroll
-                        for (int r = 0; r < ROUNDS; ++r) {
-                            const int32_t j = j0 + r * G;
-                            if (j < c) {
-                                a.nbr[off + j] = dst[r];
-                                if (a.mark != nullptr) mark_id(a, dst[r]);
-                                a.nbr_ts[off + j] = ets[r];
-                                a.nbr_eid[off + j] = id[r];
-                                a.nbr_dt[off + j] = ets[r] - t;
-                            }
-                        }
-                    }
-                }
-            } else if (G == WAVE && k > G) {
+            if (G == WAVE && k > G) {
                 // ---- uniform with a fanout beyond one wavefront (a wave per slot, picks in dynamic LDS) ----
                 // Block-uniform control flow (the loops run to k for every wave, idle waves skip the work),
                 // so that block barriers order the LDS accesses of the sequential subset construction.
@@ -758,10 +727,164 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     }
 }
 
-// Lanes per slot.  Uniform needs fanout <= G (one lane per draw).  Recent copies any
-// fanout with any G; with many slots 8 lanes per slot keep twice as many slots in
-// flight per compute unit, which is what bounds a launch once the slots exceed one
-// wave-residency round (8192 waves): 53k slots run ~25 % faster than with 16 lanes.
+
+// Most-recent copy with a lane per EDGE instead of a group of lanes per slot.  A block takes its run in chunks of
+// FLAT_SLOTS slots: their counts are scanned into LDS (with the slots' window starts and times), then the chunk's
+// edges are walked flat - edge x of the chunk belongs to the slot whose offsets enclose x (a 9-step search in LDS),
+// comes from start + (x - offset) and goes to run offset + x.  Every lane has an edge whatever the slots hold
+// (slots of deeper hops hold two edges on average on a power-law graph: a group of 8 lanes per slot left six idle),
+// and the stores of a block-iteration are one contiguous piece per output array.
+constexpr int FLAT_SLOTS = 2 * BLOCK;
+__global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
+    __shared__ int64_t s_red[NWAVE];
+    __shared__ int32_t s_redb[NWAVE];
+    __shared__ int32_t s_w[NWAVE];
+    __shared__ int32_t s_off[FLAT_SLOTS + 1];
+    __shared__ int64_t s_start[FLAT_SLOTS], s_t[FLAT_SLOTS];
+    const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    const int32_t k = a.k;
+    const int64_t S = live_count(a.S_dev, a.S_max);
+    int64_t first, run;
+    block_run(S, a.align, &first, &run);
+    const int64_t run_end = first + run < S ? first + run : S;
+    // the first chunk's slots (two consecutive ones per thread): loaded beside the block's offset
+    constexpr int SPT = FLAT_SLOTS / BLOCK;      // consecutive slots per thread
+    int64_t st[SPT], ln[SPT], tt[SPT];
+    auto load_slots = [&](int64_t chunk0) {
+#pragma unroll
+        for (int q = 0; q < SPT; ++q) {
+            const int64_t slot = chunk0 + SPT * threadIdx.x + q;
+            st[q] = ln[q] = tt[q] = 0;
+            if (slot < run_end) {
+                st[q] = a.w_start[slot];
+                ln[q] = a.w_len[slot];
+                tt[q] = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
+            }
+        }
+    };
+    load_slots(first);
+    int64_t run_off = 0;
+    if (a.scanned) {
+        constexpr int CH = MAX_BLOCKS / SCAN_BLOCK;
+        const int c0 = (int)blockIdx.x / CH * CH;
+        run_off = a.chunk_off[blockIdx.x / CH];
+#pragma unroll
+        for (int q = 0; q < CH - 1; ++q)
+            if (c0 + q < (int)blockIdx.x) run_off += a.block_sum[c0 + q];
+    } else {
+        int64_t part = 0;
+        int32_t partb = 0;
+        const bool last = blockIdx.x == gridDim.x - 1;
+        for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += BLOCK) {
+            part += a.block_sum[b];
+            if (last) partb += a.block_bad[b];
+        }
+        for (int d = WAVE / 2; d > 0; d >>= 1) {
+            part += shfl_i64(part, wlane ^ d);
+            partb += __shfl(partb, wlane ^ d);
+        }
+        if (wlane == 0) {
+            s_red[wid] = part;
+            s_redb[wid] = partb;
+        }
+        __syncthreads();
+        int32_t bad_total = 0;
+#pragma unroll
+        for (int q = 0; q < NWAVE; ++q) {
+            run_off += s_red[q];
+            bad_total += s_redb[q];
+        }
+        if (last && threadIdx.x == 0) {
+            const int64_t E = run_off + a.block_sum[blockIdx.x];
+            a.counts[0] = S;
+            a.counts[1] = E;
+            a.counts[2] = bad_total + a.block_bad[blockIdx.x];
+            a.root_start_ptr[S] = E;
+            a.root_end_ptr[S] = E;
+        }
+    }
+    for (int64_t chunk0 = first; chunk0 < run_end; chunk0 += FLAT_SLOTS) {      // block-uniform
+        if (chunk0 != first) load_slots(chunk0);
+        // exclusive prefix of the chunk's counts
+        int32_t c[SPT], sum = 0;
+#pragma unroll
+        for (int q = 0; q < SPT; ++q) {
+            c[q] = (int32_t)(ln[q] < k ? ln[q] : k);
+            sum += c[q];
+        }
+        int32_t inc = sum;
+        for (int d = 1; d < WAVE; d <<= 1) {
+            const int32_t y = __shfl_up(inc, d);
+            if (wlane >= d) inc += y;
+        }
+        if (wlane == WAVE - 1) s_w[wid] = inc;
+        __syncthreads();                 // (also: the previous chunk's edges are done with the LDS arrays)
+        int32_t excl = inc - sum, total = 0;
+#pragma unroll
+        for (int q = 0; q < NWAVE; ++q) {
+            const int32_t y = s_w[q];
+            if (q < wid) excl += y;
+            total += y;
+        }
+        if (threadIdx.x == 0) s_off[FLAT_SLOTS] = total;
+#pragma unroll
+        for (int q = 0; q < SPT; ++q) {
+            const int j = SPT * threadIdx.x + q;
+            s_off[j] = excl;
+            s_start[j] = st[q];
+            s_t[j] = tt[q];
+            const int64_t slot = chunk0 + j;
+            if (slot < run_end) {
+                a.root_start_ptr[slot] = run_off + excl;
+                a.root_end_ptr[slot] = run_off + excl + c[q];
+            }
+            excl += c[q];
+        }
+        __syncthreads();
+        // the chunk's edges, flat: up to ROUNDS per lane, every load issued before the first store
+        constexpr int ROUNDS = 4;
+        for (int32_t x0 = threadIdx.x; x0 < total; x0 += ROUNDS * BLOCK) {
+            int64_t ets[ROUNDS], dst[ROUNDS], id[ROUNDS], hnt[ROUNDS], tslot[ROUNDS];
+#pragma unroll
+            for (int r = 0; r < ROUNDS; ++r) {
+                const int32_t x = x0 + r * BLOCK;
+                ets[r] = dst[r] = id[r] = hnt[r] = tslot[r] = 0;
+                if (x < total) {
+                    // the slot of edge x: the last one whose offset is <= x (empty slots share the offset of the
+                    // slot after them, so the last one is the one that holds x)
+                    int lo = 0;
+#pragma unroll
+                    for (int step = FLAT_SLOTS / 2; step > 0; step >>= 1)
+                        lo += s_off[lo + step] <= x ? step : 0;
+                    const int64_t e = s_start[lo] + (x - s_off[lo]);
+                    tslot[r] = s_t[lo];
+                    ets[r] = a.ts[e];
+                    dst[r] = a.col[e];
+                    id[r] = a.eid[e];
+                    if (a.hint_out != nullptr) hnt[r] = a.hint[e];
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < ROUNDS; ++r) {
+                const int32_t x = x0 + r * BLOCK;
+                if (x < total) {
+                    const int64_t o = run_off + x;
+                    a.nbr[o] = dst[r];
+                    if (a.mark != nullptr) mark_id(a, dst[r]);
+                    a.nbr_ts[o] = ets[r];
+                    a.nbr_eid[o] = id[r];
+                    a.nbr_dt[o] = ets[r] - tslot[r];
+                    if (a.hint_out != nullptr) a.hint_out[o] = hnt[r];
+                }
+            }
+        }
+        run_off += total;
+    }
+}
+
+// Lanes per slot of the uniform strategy's draws (fanout <= G: one lane per draw).  The most-recent strategy
+// copies with a lane per edge (fill_flat_kernel); the figure returned for it only steers the group of its
+// window search (pick_search_group) and the alignment of the blocks' runs.
 int pick_group(const sgl_sample_params* p, int64_t S_max) {
     if (p->type == SGL_SAMPLE_UNIFORM) {
         if (p->fanout <= 16) return 16;
@@ -844,12 +967,12 @@ HopKernel count_fn(int G) {
 HopKernel fill_fn(int G, bool uniform) {
     if (uniform) {
         switch (G) {
-            case 16: return fill_kernel<16, true>;
-            case 32: return fill_kernel<32, true>;
-            default: return fill_kernel<64, true>;
+            case 16: return fill_kernel<16>;
+            case 32: return fill_kernel<32>;
+            default: return fill_kernel<64>;
         }
     }
-    return G == 8 ? fill_kernel<8, false> : fill_kernel<16, false>;
+    return fill_flat_kernel;
 }
 
 // Gc lanes per slot search, Gf lanes per slot copy or draw

@@ -153,6 +153,9 @@ struct Scratch {
 
 bool radix_route(int64_t ncap) { return ncap > ATOMIC_ROUTE_MAX; }
 
+// entries of Scratch::big: a call that adds at most ncap ids has fewer than ncap / SMALL_BUCKET oversized buckets
+__host__ __device__ constexpr int64_t big_capacity(int64_t ncap) { return ncap / SMALL_BUCKET + 2; }
+
 int nb_log_of(int64_t ncap) {
     if (radix_route(ncap)) return SORT_KEY_LOG;
     int l = NB_MIN_LOG;
@@ -163,7 +166,7 @@ int nb_log_of(int64_t ncap) {
 size_t scratch_bytes(int64_t total, int64_t ncap) {
     const int64_t nb = 1ll << nb_log_of(ncap);
     size_t b = align_up((size_t)(total + 1) * 4) + align_up((size_t)(ncap + 1) * 8) +
-               align_up((size_t)(ncap / SMALL_BUCKET + 2) * 4) + 1024;
+               align_up((size_t)big_capacity(ncap) * 4) + 1024;
     if (radix_route(ncap))
         b += 3 * align_up((size_t)(ncap + 1) * 8) + radix_sort_workspace_bytes(ncap) + 256;
     else
@@ -180,7 +183,7 @@ Scratch carve_scratch(Arena& ar, int64_t total, int64_t ncap) {
     const int64_t nb = 1ll << s.nb_log;
     s.slot_of = ar.take<uint32_t>(total + 1);
     s.list_id = ar.take<unsigned long long>(ncap + 1);
-    s.big = ar.take<uint32_t>(ncap / SMALL_BUCKET + 2);
+    s.big = ar.take<uint32_t>(big_capacity(ncap));
     if (s.radix) {
         s.key_a = ar.take<uint64_t>(ncap + 1);
         s.key_b = ar.take<uint64_t>(ncap + 1);
@@ -683,10 +686,13 @@ __global__ __launch_bounds__(BLOCK) void scatter_kernel(Table t, Scratch s, int 
         for (int i = threadIdx.x; i <= nb; i += BLOCK) {
             const uint32_t f = s_pre[pre_at(i)];
             s.off[i] = f;
-            if (i < nb && s_pre[pre_at(i + 1)] - f > (uint32_t)SMALL_BUCKET) s.big[atomicAdd(&s_nbig, 1u)] = (uint32_t)i;
+            if (i < nb && s_pre[pre_at(i + 1)] - f > (uint32_t)SMALL_BUCKET) {
+                const uint32_t q = atomicAdd(&s_nbig, 1u);
+                if ((int64_t)q < big_capacity(s.ncap)) s.big[q] = (uint32_t)i;    // (more only after an overflow)
+            }
         }
         __syncthreads();
-        if (threadIdx.x == 0) t.hdr->nbig = s_nbig;
+        if (threadIdx.x == 0) t.hdr->nbig = (int64_t)s_nbig < big_capacity(s.ncap) ? s_nbig : (uint32_t)big_capacity(s.ncap);
     }
 }
 
