@@ -403,31 +403,46 @@ __device__ __forceinline__ int32_t group_bcast(int32_t x, int j, int wlane) {
 // lig < k holds draw tj from [0, len - k + lig]): step j keeps its draw unless an earlier step holds the same
 // value, then it takes len - k + j.  -> the lane's pick and its rank among the k picks (all distinct).
 // Two draws of a group collide only in windows of a few thousand edges or fewer: the ranks are counted on the raw
-// draws first, and the sequential construction runs only in waves where some group saw two equal draws.
-// Windows of 2^31 edges and more take the 64-bit variant.
+// draws first, and the sequential construction runs only in waves where some group saw two equal draws.  Counting
+// goes through LDS: every lane parks its draw, then reads its group's draws four at a time (lanes of a group read
+// the same words: a broadcast) - a fifth of the instructions of handing the draws round lane by lane, and this
+// part is what the uniform kernels spend their issue slots on.  The groups never leave their wavefront, whose LDS
+// accesses are served in program order.  Windows close to 2^31 edges and more take the 64-bit variant.
 template <int G>
 __device__ __forceinline__ void floyd_subset(bool draw, int lig, int wlane, int gshift, int32_t k, int64_t len, int64_t tj,
                                              int64_t* pick, int32_t* rank) {
+    __shared__ __attribute__((aligned(16))) int32_t s_draw[BLOCK];
     const bool mine_on = draw && lig < k;
-    if (__all(!draw || len <= (int64_t)INT32_MAX)) {          // wave-uniform
-        int32_t v = mine_on ? (int32_t)tj : -1 - lig;            // (idle lanes hold distinct negatives)
-        int32_t r = 0;
-        bool dup = false;
-        for (int32_t j = 0; j < k; ++j) {
-            const int32_t o = group_bcast<G>(v, j, wlane);
-            r += o < v ? 1 : 0;
-            dup |= o == v && j != lig;
-        }
-        if (__any(mine_on && dup)) {
+    if (__all(!draw || len < (int64_t)INT32_MAX - WAVE)) {          // wave-uniform
+        const int gbase = (int)threadIdx.x - lig;                     // (a multiple of G >= 16: 16-byte aligned words)
+        int32_t v = mine_on ? (int32_t)tj : INT32_MAX - lig;          // (idle lanes hold distinct values above every draw)
+        // rank of v among the group's values = how many are smaller; eq = how many are equal (itself included)
+        auto count = [&](int32_t* smaller, int32_t* equal) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            s_draw[threadIdx.x] = v;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            int32_t r = 0, e = 0;
+            for (int32_t j = 0; j < k; j += 4) {                      // (k <= G, G a multiple of 4: inside the group's words)
+                const int4 o = *reinterpret_cast<const int4*>(&s_draw[gbase + j]);
+                r += (o.x < v ? 1 : 0) + (o.y < v ? 1 : 0) + (o.z < v ? 1 : 0) + (o.w < v ? 1 : 0);
+                e += (o.x == v ? 1 : 0) + (o.y == v ? 1 : 0) + (o.z == v ? 1 : 0) + (o.w == v ? 1 : 0);
+            }
+            *smaller = r;
+            *equal = e;
+        };
+        int32_t r, e;
+        count(&r, &e);
+        if (__any(mine_on && e > 1)) {
             int32_t m = -1;
             for (int32_t j = 0; j < k; ++j) {
                 const int32_t cand = group_bcast<G>(v, j, wlane);
                 const bool hit = group_ballot<G>(draw && lig < j && m == cand, gshift) != 0;
                 if (lig == j) m = hit ? (int32_t)(len - k + j) : cand;
             }
-            v = mine_on ? m : -1 - lig;
-            r = 0;
-            for (int32_t j = 0; j < k; ++j) r += group_bcast<G>(v, j, wlane) < v ? 1 : 0;
+            v = mine_on ? m : INT32_MAX - lig;
+            count(&r, &e);
         }
         if (draw) {
             *pick = (int64_t)v;
@@ -658,31 +673,87 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
 #pragma unroll
         for (int q = 0; q < NWAVE; ++q)
             if (q < wid) wave_off += s_wtot[0][q];
-        for (int64_t it = wfirst; it < wend; it += SPW) {
-            // the next iteration's slot is loaded now, so that its latency runs beside this iteration's picks and copies
-            const int64_t nslot = it + SPW + gw;
-            const bool nactive = nslot < wend;
-            int64_t nstart = 0, nlen = 0, nt = 0;
-            if (nactive) {
-                nstart = a.w_start[nslot];
-                nlen = a.w_len[nslot];
-                nt = a.derive ? a.slot_ts_out[nslot] : a.slot_ts[nslot];
+        // Two iterations' slots per trip: the draws of both are made, then the picked edges of both are loaded,
+        // then both are stored - twice the loads in flight per wave, and the prefix work is shared.
+        auto load_slot_of = [&](int64_t sl, bool on, int64_t* st_, int64_t* ln_, int64_t* t_) {
+            *st_ = *ln_ = *t_ = 0;
+            if (on) {
+                *st_ = a.w_start[sl];
+                *ln_ = a.w_len[sl];
+                *t_ = a.derive ? a.slot_ts_out[sl] : a.slot_ts[sl];
             }
-            const int32_t c = (int32_t)(len < k ? len : k);
-            int32_t inc = (lig == 0) ? c : 0;
+        };
+        // the pick of this lane for its slot: position inside the window and output place
+        auto choose = [&](int64_t sl, bool on, int64_t ln_, int64_t* sel, int32_t* rank) {
+            const bool draw = on && ln_ > k;
+            *sel = lig;
+            *rank = lig;
+            if (__any(draw)) {                    // wave-uniform
+                int64_t tj = 0;
+                if (draw && lig < k) {
+                    const uint64_t bits = draw_bits(a.seed, a.hop, sl, lig);
+                    tj = a.replace ? bounded(bits, ln_) : bounded(bits, ln_ - k + lig + 1);
+                }
+                if (a.replace) {
+                    if (draw) *sel = tj;
+                } else {
+                    floyd_subset<G>(draw, lig, wlane, gshift, k, ln_, tj, sel, rank);
+                }
+            }
+        };
+        auto store = [&](bool on, int64_t t_, int64_t o, const Edge& ed) {
+            if (!on) return;
+            a.nbr[o] = ed.col;
+            if (a.mark != nullptr) mark_id(a, ed.col);
+            a.nbr_ts[o] = a.keep_root_time ? t_ : ed.ts;
+            a.nbr_eid[o] = ed.eid;
+            a.nbr_dt[o] = ed.ts - t_;
+            if (a.hint_out != nullptr) a.hint_out[o] = ed.hint;
+        };
+        int64_t slot_b = slot + SPW, start_b, len_b, t_b;
+        bool active_b = slot_b < wend;
+        load_slot_of(slot_b, active_b, &start_b, &len_b, &t_b);
+        for (int64_t it = wfirst; it < wend; it += 2 * SPW) {
+            // the next trip's slots are loaded now, so that their latency runs beside this trip's draws and picks
+            const int64_t nslot = it + 2 * SPW + gw, nslot_b = nslot + SPW;
+            const bool nactive = nslot < wend, nactive_b = nslot_b < wend;
+            int64_t nstart, nlen, nt, nstart_b, nlen_b, nt_b;
+            load_slot_of(nslot, nactive, &nstart, &nlen, &nt);
+            load_slot_of(nslot_b, nactive_b, &nstart_b, &nlen_b, &nt_b);
+            const int32_t c = (int32_t)(len < k ? len : k), c_b = (int32_t)(len_b < k ? len_b : k);
+            // exclusive prefix over the trip's slots: the first iteration's groups, then the second's
+            int32_t inc = (lig == 0) ? c : 0, inc_b = (lig == 0) ? c_b : 0;
             for (int d = 1; d < WAVE; d <<= 1) {
-                const int32_t x = __shfl_up(inc, d);
-                if (wlane >= d) inc += x;
+                const int32_t x = __shfl_up(inc, d), y = __shfl_up(inc_b, d);
+                if (wlane >= d) {
+                    inc += x;
+                    inc_b += y;
+                }
             }
-            const int32_t excl = __shfl(inc - ((lig == 0) ? c : 0), wlane - lig);
-            const int32_t iter_total = __shfl(inc, WAVE - 1);
-            emit_slot(slot, active, start, len, t, c, wave_off + excl);
-            wave_off += iter_total;
-            slot = nslot;
-            active = nactive;
-            start = nstart;
-            len = nlen;
-            t = nt;
+            const int32_t total_a = __shfl(inc, WAVE - 1), total_b = __shfl(inc_b, WAVE - 1);
+            const int64_t off = wave_off + __shfl(inc - ((lig == 0) ? c : 0), wlane - lig);
+            const int64_t off_b = wave_off + total_a + __shfl(inc_b - ((lig == 0) ? c_b : 0), wlane - lig);
+            int64_t sel, sel_b;
+            int32_t rank, rank_b;
+            choose(slot, active, len, &sel, &rank);
+            choose(slot_b, active_b, len_b, &sel_b, &rank_b);
+            const bool on = active && lig < c, on_b = active_b && lig < c_b;
+            Edge ed{}, ed_b{};
+            if (on) ed = load_picked_edge(a, start + sel);
+            if (on_b) ed_b = load_picked_edge(a, start_b + sel_b);
+            if (active && lig == 0) {
+                a.root_start_ptr[slot] = off;
+                a.root_end_ptr[slot] = off + c;
+            }
+            if (active_b && lig == 0) {
+                a.root_start_ptr[slot_b] = off_b;
+                a.root_end_ptr[slot_b] = off_b + c_b;
+            }
+            store(on, t, off + rank, ed);
+            store(on_b, t_b, off_b + rank_b, ed_b);
+            wave_off += total_a + total_b;
+            slot = nslot; active = nactive; start = nstart; len = nlen; t = nt;
+            slot_b = nslot_b; active_b = nactive_b; start_b = nstart_b; len_b = nlen_b; t_b = nt_b;
         }
         return;
     }

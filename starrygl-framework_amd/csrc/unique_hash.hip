@@ -126,7 +126,7 @@ Table carve(void* state, int64_t capacity) {
     return t;
 }
 
-// Per-call scratch.  Atomic route: list_b, part_*, cnt, off.  Radix route: key_a/b (bucket << 40 | table
+// Per-call scratch.  Atomic route: list_b, list_r, part_*, cnt, off, mask_part.  Radix route: key_a/b (bucket << 40 | table
 // slot) with the ids as the sort's values (id_a/b), and the sort's own workspace.
 struct Scratch {
     uint32_t* slot_of;          // [total] table slot of every input element (NONE: negative id)
@@ -137,7 +137,7 @@ struct Scratch {
     uint32_t* part_slot;        // [ncap]
     uint32_t* part_b;           // [ncap]
     uint32_t* cnt;              // [nb + 1] bucket sizes
-    uint32_t* off;              // [nb + 1] first places of the buckets (only with the one-block scan)
+    uint32_t* off;              // [nb + 1] first places of the buckets, left by the first block of the scatter launch
     unsigned long long* mask_part;  // [2 * NMASK] OR / AND over the call's ids, one pair per block of prep
     uint32_t* big;              // [ncap / SMALL_BUCKET + 2] oversized buckets (atomic route) / their first places (radix route)
     uint64_t* key_a;            // [ncap] radix route
