@@ -472,6 +472,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE readings can be scaled")
     ap.add_argument("--no-fused-mark", action="store_true",
                     help="unique runs its own marking pass instead of the sampler recording the ids it emits")
+    ap.add_argument("--no-edge-records", action="store_true",
+                    help="do not build the interleaved edge records (the uniform strategy then reads the separate arrays)")
     ap.add_argument("--no-hop-hint", action="store_true",
                     help="sample without the graph's next-hop index (every slot of hops >= 1 searches its window)")
     ap.add_argument("--loader-root-hints", action="store_true",
@@ -520,6 +522,12 @@ def main():
         hot.build_hop_hint(dg)
         torch.cuda.synchronize()
         log(f"[setup] next-hop index of {m} edges built in {(time.perf_counter() - t_h) * 1e3:.1f} ms")
+    if not args.no_edge_records:  # the 32-byte edge records: a pick of the uniform strategy costs one memory sector, not one per array
+        torch.cuda.synchronize()
+        t_h = time.perf_counter()
+        hot.build_records(dg)
+        torch.cuda.synchronize()
+        log(f"[setup] edge records of {m} edges built in {(time.perf_counter() - t_h) * 1e3:.1f} ms")
     gen = torch.Generator(device=dev).manual_seed(20242)
     node_feat = torch.randn((n, 100), device=dev, generator=gen)
     edge_feat = None
@@ -1142,7 +1150,7 @@ def main():
                                "negatives (12000 roots): 2-hop recent 10x10 + unique + node/edge gather + 2-hop uniform 10x10",
                    "nodes": n, "edges": m, "roots_per_batch": S0, "fanout": [k, k],
                    "node_feat": "100xfp32", "edge_feat": "172xfp32" if has_edge_feat else None,
-                   "next_hop_index": not args.no_hop_hint, "root_hints_in_batch": use_root_hint},
+                   "next_hop_index": not args.no_hop_hint, "edge_records": not args.no_edge_records, "root_hints_in_batch": use_root_hint},
         "edges_per_step": {"recent": float(np.mean(e_rec)), "uniform": float(np.mean(e_uni))},
         "mean_rows_per_step": {"gather_node_feat": float(np.mean(cl[:, 4])), "gather_edge_feat_hop1": float(np.mean(cl[:, 0])),
                                "gather_edge_feat_hop2": float(np.mean(cl[:, 1]))},
