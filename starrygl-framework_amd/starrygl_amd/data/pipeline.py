@@ -100,7 +100,8 @@ class MiniBatch:
 class MiniBatchPipeline:
     def __init__(self, graph, num_pos_slots, num_neg, layers, fanout, sample_type="recent", node_tables=None,
                  edge_tables=None, time_encoder=None, allowed_offset=-1, equal_root_time=False,
-                 keep_root_time=False, seed=0, use_graph=True, stream=None, root_hints=False):
+                 keep_root_time=False, seed=0, use_graph=True, stream=None, root_hints=False, remap="dense",
+                 remap_capacity=None):
         """graph: the native graph object (`pyGraph.g`, i.e. `CUDAGraph`).
         num_pos_slots / num_neg: positive root timestamps and negatives per batch
         (fixed, they size every buffer).  node_tables / edge_tables: name ->
@@ -110,6 +111,10 @@ class MiniBatchPipeline:
         root_hints: every run() also takes `root_hint`, the window ends of the positive slots
         (`graph.window_end(roots, root_ts)`, which a loader looks up once for all the events it will
         train on; -1 = search): those roots are then sampled without a search.
+        remap: "dense" numbers the batch's ids through a table over the graph's n nodes (the sampler marks the ids
+        it emits there, unique skips its first pass); "hashed" through the LDS-staged hash set, whose state is sized
+        by `remap_capacity` distinct ids per batch (default: the batch's worst case) and not by n - for graphs whose
+        id space has no room for a table per pipeline.  Same local ids either way.
         stream: run every batch on this stream instead of the caller's current one (see
         MiniBatchPipelinePool); inputs handed to run() must then be complete on the host side
         or long-lived, and results are read through MiniBatch.finalize(), which waits for it."""
@@ -141,9 +146,15 @@ class MiniBatchPipeline:
         self.local = [be.empty(c) for c in caps]
         self.ucap = min(sum(caps), graph._n)
         self.ubuf, self.U = be.empty(max(self.ucap, 1)), self.live[3 * self.layers:]
-        self.state = hp.remap_state(graph._n)
-        # the sampler records the ids it emits as pending in the remap state: unique skips its first pass
-        self.p = hp.marking(self.p, self.state)
+        if remap not in ("dense", "hashed"):
+            raise ValueError("remap must be 'dense' or 'hashed'")
+        self.hashed = remap == "hashed"
+        if self.hashed:
+            self.state = hp.remap_hashed_state(int(remap_capacity) if remap_capacity else max(self.ucap, 1))
+        else:
+            self.state = hp.remap_state(graph._n)
+            # the sampler records the ids it emits as pending in the remap state: unique skips its first pass
+            self.p = hp.marking(self.p, self.state)
         self.S0_dev = torch.tensor([self.S0], dtype=torch.int64, device=self.dev)
         f32 = torch.float32
         self.node_out, self.node_ts_out, self.edge_out = {}, {}, {}
@@ -161,8 +172,10 @@ class MiniBatchPipeline:
         self._views = {}
         # the unique stage's scratch belongs to this pipeline: its pointer is baked into the pipeline's HIP
         # graph, and graphs of different pipelines replay side by side on different streams
-        self.uws = be.empty(max(int(hp.lib.unique_workspace_bytes(graph._n, 1 + self.layers,
-                                                                  (_abi.i64 * (1 + self.layers))(*caps))), 256), "u8")
+        lens_c = (_abi.i64 * (1 + self.layers))(*caps)
+        need = (hp.lib.unique_hashed_workspace_bytes(self.state.universe, 1 + self.layers, lens_c) if self.hashed
+                else hp.lib.unique_workspace_bytes(graph._n, 1 + self.layers, lens_c))
+        self.uws = be.empty(max(int(need), 256), "u8")
         self.use_graph, self._graph = use_graph, None
         self._plans, self._slow = None, []
         self.stream = stream
@@ -186,6 +199,9 @@ class MiniBatchPipeline:
         cur = torch.cuda.current_stream(self.dev)
         with torch.cuda.stream(self.stream if self.stream is not None else cur):
             hp._reinit_marked(self.p)
+            if self.hashed:          # a hashed state whose capacity an epoch outgrew stays void until it is initialised again
+                be = hp.be
+                hp._ck(hp.lib.remap_hashed_init(be.ptr(self.state.buf), be.nbytes(self.state.buf), self.state.universe, be.stream()))
             self._chain(multi_launch=True)
             torch.cuda.current_stream(self.dev).synchronize()
         hp.recoveries += 1
@@ -196,9 +212,9 @@ class MiniBatchPipeline:
                        hp.multi_launch(self.p) if multi_launch else self.p, finalize=False, out=kr)
         arrays = [kr.slot_node0] + [h.neighbors for h in kr.hops]
         lens = [self.S0_dev] + [h.counts[1:2] for h in kr.hops]
-        hp.unique_compact(arrays, _abi.UNIQUE_SORTED | (_abi.UNIQUE_MULTI_LAUNCH if multi_launch else 0), self.state, True,
+        hp.unique_compact(arrays, _abi.UNIQUE_SORTED | (_abi.UNIQUE_MULTI_LAUNCH if multi_launch and not self.hashed else 0), self.state, True,
                           lens_dev=lens, out_arrays=self.local, finalize=False, unique_out=self.ubuf, U_out=self.U,
-                          premarked=True, workspace=self.uws)
+                          premarked=not self.hashed, workspace=self.uws)
         if self._plans is None:      # every gather of the batch in as few launches as possible
             segs = [(c, self.ubuf, self.node_out[name], self.node_ts_out.get(name), self.U[0:1])
                     for name, c in self.node_tables.items()]
