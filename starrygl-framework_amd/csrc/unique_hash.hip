@@ -666,6 +666,10 @@ __global__ __launch_bounds__(BLOCK) void scatter_kernel(Table t, Scratch s, int 
         }
     }
     const int nb = 1 << s.nb_log;
+    // After an overflow (more ids than the capacity, or a full table) the counts the insert got back no longer
+    // number the listed ids 0..n-1 bucket by bucket (ids without a place in the list were counted too), so places
+    // would stay unwritten: the result is void anyway, and neither this launch nor the numbering one touches it.
+    if (t.hdr->overflow != 0) return;                  // the same for every thread of the launch
     const int64_t before = ids_before(t, reset);       // (read before the barriers of the prefix, not after)
     const int64_t n = ids_added(t, s, before);
     block_prefix(s.cnt, nb, s_pre, s_wave);
@@ -674,7 +678,7 @@ __global__ __launch_bounds__(BLOCK) void scatter_kernel(Table t, Scratch s, int 
         const int64_t k = k0 + j * BLOCK;
         if (k >= n) continue;
         const int64_t p = (int64_t)s_pre[pre_at((int)(b[j] & (uint32_t)(nb - 1)))] + r[j];
-        if (p >= n) continue;            // only after an overflow (the result is void then)
+        if (p >= n) continue;            // (cannot happen without an overflow)
         s.part_id[p] = id[j];
         s.part_slot[p] = t.used[before + k];
         s.part_b[p] = b[j];
@@ -742,6 +746,7 @@ __global__ __launch_bounds__(BLOCK) void number_kernel(Table t, Scratch s, int r
     constexpr int PER = NUMBER_TILE / BLOCK;
     const int64_t p0 = (int64_t)blockIdx.x * NUMBER_TILE;
     const int nb = 1 << s.nb_log;
+    if (t.hdr->overflow != 0) return;                  // the scatter launch left nothing to number (see there)
     uint32_t slot[PER];
     int64_t lo[PER], hi[PER];
 #pragma unroll
@@ -787,7 +792,7 @@ __global__ __launch_bounds__(BLOCK) void number_kernel(Table t, Scratch s, int r
         }
         const int64_t local = before + r;
         if (local < unique_capacity) unique_out[local] = (int64_t)id;
-        t.vals[slot[j]] = (uint32_t)local;
+        if ((int64_t)slot[j] < t.slots) t.vals[slot[j]] = (uint32_t)local;
     }
     for (int64_t q = blockIdx.x; q < nbig; q += gridDim.x) {
         const uint32_t bucket = s.big[q];

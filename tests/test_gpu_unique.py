@@ -216,6 +216,28 @@ def test_hashed_state_reports_an_outgrown_capacity(hot):
     assert th == 900 and np.array_equal(np_of(lh[0]), np.arange(900))
 
 
+@pytest.mark.parametrize("n_ids,capacity", [(5_000, 50), (30_000, 1_000), (2_000_000, 1_500_000)])
+def test_hashed_state_overflow_leaves_scratch_contents_alone(hot, n_ids, capacity):
+    """An epoch that outgrows its state (far more distinct ids than the capacity, also more than the table has
+    slots; both routes) on a workspace full of 0xFF bytes: whatever the call's scratch held before, nothing of it is
+    used as an index - the call completes, reports a void result, and a state of sufficient capacity then numbers
+    the same ids correctly with the same workspace."""
+    import torch
+    ids = to_dev(hot, np.random.default_rng(3).permutation(n_ids).astype(np.int64) * 3)
+    lens = (_abi.i64 * 1)(n_ids)
+    big = hot.remap_hashed_state(n_ids)
+    need = max(int(hot.lib.unique_hashed_workspace_bytes(capacity, 1, lens)), int(hot.lib.unique_hashed_workspace_bytes(n_ids, 1, lens)))
+    ws = torch.full((need,), 0xFF, dtype=torch.uint8, device=ids.device)
+    small = hot.remap_hashed_state(capacity)
+    out, uniq, U = hot.unique_compact([ids], _abi.UNIQUE_SORTED, small, True, finalize=False, workspace=ws)
+    torch.cuda.synchronize()
+    assert int(U[0]) == np.iinfo(np.int64).max
+    ws.fill_(0xFF)
+    lh, uh, (th, _) = hot.unique_compact([ids], _abi.UNIQUE_SORTED, big, True, workspace=ws)
+    assert th == n_ids and np.array_equal(np_of(uh), np.arange(n_ids) * 3)
+    assert np.array_equal(np_of(uh)[np_of(lh[0])], np_of(ids))
+
+
 @pytest.mark.parametrize("n", [30_000, 1_300_000])
 def test_hash_unique_is_captured_and_replayed_in_a_hip_graph(oracle, hot, n):
     """The hash-set path is a fixed launch sequence without host synchronisation: captured once, replayed
