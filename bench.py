@@ -483,6 +483,10 @@ def main():
     ap.add_argument("--pipelines", type=int, default=3,
                     help="independent copies of the step (own buffers, graph and stream) that take the batches of the "
                          "timed region in turn, as a loader with that many batches in flight does; 1 = one batch at a time")
+    ap.add_argument("--hold-ms", type=float, default=0.0,
+                    help="keep the pipelines' streams waiting behind that many ms of filler work while the host enqueues "
+                         "the timed steps, and clock the steps from the moment the wait ends: under a profiler the host "
+                         "enqueues more slowly than the GPU works, and only then does a trace show the GPU-bound schedule")
     ap.add_argument("--separate-samplers", action="store_true",
                     help="one library call per sampler (the uniform one on a second graph branch) instead of one call for both")
     ap.add_argument("--serial", action="store_true", help="capture the step as one serial chain of kernels")
@@ -759,9 +763,13 @@ def main():
              and edge_cache is not None)
     main_stream = torch.cuda.current_stream()
 
-    def timed_region(run_batch, accs):
+    filler = torch.empty(1 << 29, dtype=torch.float32, device=dev) if args.hold_ms > 0 else None   # 2 GiB
+
+    def timed_region(run_batch, accs, streams=()):
         """W untimed steps, then exactly K steps on the wall clock with no host synchronisation inside
-        -> (seconds, host seconds spent enqueueing, the accumulated device-side counts)."""
+        -> (seconds, host seconds spent enqueueing, the accumulated device-side counts).
+        --hold-ms: `streams` first wait for filler work on the main stream, the K steps are enqueued behind that
+        wait, and the clock starts when the wait ends (the host must have finished enqueueing by then)."""
         for i in range(W):
             run_batch(i, i % NB)
         torch.cuda.set_stream(main_stream)
@@ -769,10 +777,22 @@ def main():
         for a_ in accs:
             a_.zero_()
         torch.cuda.synchronize()
+        gate = None
+        if filler is not None and streams:
+            for _ in range(max(1, int(args.hold_ms / 0.8))):     # ~0.8 ms per pass over 2 GiB, read and written
+                filler.mul_(1.0)
+            gate = torch.cuda.Event()
+            gate.record(main_stream)
+            for st_ in streams:
+                st_.wait_event(gate)
         t_start = time.perf_counter()
         for i in range(K):
             run_batch(i, (W + i) % NB)
         submit = time.perf_counter() - t_start      # the host's share: K batch copies + K graph launches enqueued
+        if gate is not None:
+            assert not gate.query(), "--hold-ms: the filler work ended before the host had enqueued the steps"
+            gate.synchronize()
+            t_start = time.perf_counter()
         torch.cuda.synchronize()
         wall_ = time.perf_counter() - t_start
         torch.cuda.set_stream(main_stream)
@@ -787,7 +807,10 @@ def main():
         # ---- the headline: K steps dealt in turn to the pipelines
         pipes = [make_pipeline(st_, use_root_hint) for st_ in pipe_streams]
         mode += f", {args.pipelines} batches in flight (one pipeline of buffers, graph and stream each)"
-        wall, host_submit, tot = timed_region(lambda i, b: pipes[i % len(pipes)].run(b), [P.acc for P in pipes])
+        if args.hold_ms > 0:
+            mode += ", timed steps enqueued behind a stream wait (--hold-ms) and clocked from its end"
+        wall, host_submit, tot = timed_region(lambda i, b: pipes[i % len(pipes)].run(b), [P.acc for P in pipes],
+                                              pipe_streams)
         del pipes
         # ---- the same K steps with the other choice about root hints (reported beside the headline)
         pipes = [make_pipeline(st_, not use_root_hint) for st_ in pipe_streams]
