@@ -2,11 +2,13 @@
 //
 // out[i, j] = cos(fl32(fl32(w[j] * float(dt[i])) + b[j])): the product and the
 // sum are rounded separately (no FMA contraction), which is what a K=1
-// `nn.Linear` followed by `torch.cos` computes.  A block owns RPB rows: their
-// converted dt values are parked in LDS, then all threads emit the block's
-// RPB x dim outputs as flat, coalesced 16-byte stores (4-byte stores when dim
-// is not a multiple of 4); the cosine is computed by cos_f32 below.  One pass over the output: the [N, dim] tensor is
-// written once instead of written, re-read and re-written by a GEMM + cos pair.
+// `nn.Linear` followed by `torch.cos` computes.  One pass over the output: the
+// [N, dim] tensor is written once, in 16-byte stores (4-byte stores when dim is
+// not a multiple of 4), instead of written, re-read and re-written by a GEMM +
+// cos pair; the cosine is computed by cos_core / cos_f32 below.  The kernel is
+// bound by the cosine's fp64 arithmetic, with the stores hidden behind it as long
+// as a wave does not load from global memory between two stores
+// (time_encode_cols_kernel); time_encode_kernel is the general form (any dim).
 //
 // Replaces TimeEncoder.forward (starrygl/nn/model/time_encoder.py:29-31).
 #include "common.hpp"
@@ -40,8 +42,9 @@ struct TEArgs {
 // operations, all straight-line.  The library cosf takes ~2.5x as long (its
 // large-argument path is a Payne-Hanek reduction).  Arguments beyond 2^45 (not
 // reachable from int64 timestamps times w <= 1 in practice) take the library routine.
-__device__ __forceinline__ float cos_f32(float af) {
-    if (!(__builtin_fabsf(af) < 3.5e13f)) return cosf(af);   // also NaN / inf
+constexpr float COS_CORE_LIMIT = 3.5e13f;
+// |af| < COS_CORE_LIMIT
+__device__ __forceinline__ float cos_core(float af) {
     const double x = (double)af;
     // n = nearest integer to x/pi without a rounding instruction: adding 1.5 * 2^52 leaves n in the low
     // mantissa bits of the sum (|x/pi| < 2^44 here), whose lowest bit is the parity of n
@@ -64,8 +67,80 @@ __device__ __forceinline__ float cos_f32(float af) {
     return __uint_as_float(__float_as_uint(c) ^ (odd << 31));
 }
 
+__device__ __forceinline__ float cos_f32(float af) {
+    if (!(__builtin_fabsf(af) < COS_CORE_LIMIT)) return cosf(af);   // also NaN / inf
+    return cos_core(af);
+}
+
 __device__ __forceinline__ float enc(float w, float x, float b) {
     return cos_f32(__fadd_rn(__fmul_rn(w, x), b));
+}
+
+// four columns of one row; the test for the library fallback is made once for the four
+__device__ __forceinline__ f32x4 enc4(const f32x4 w, float x, const f32x4 b) {
+    const float a0 = __fadd_rn(__fmul_rn(w.x, x), b.x), a1 = __fadd_rn(__fmul_rn(w.y, x), b.y);
+    const float a2 = __fadd_rn(__fmul_rn(w.z, x), b.z), a3 = __fadd_rn(__fmul_rn(w.w, x), b.w);
+    const float m = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(a0), __builtin_fabsf(a1)),
+                                    __builtin_fmaxf(__builtin_fabsf(a2), __builtin_fabsf(a3)));
+    const bool nan = a0 != a0 || a1 != a1 || a2 != a2 || a3 != a3;    // (fmax drops a NaN operand)
+    f32x4 y;
+    if (m < COS_CORE_LIMIT && !nan) {
+        y.x = cos_core(a0); y.y = cos_core(a1); y.z = cos_core(a2); y.w = cos_core(a3);
+    } else {
+        y.x = cos_f32(a0); y.y = cos_f32(a1); y.z = cos_f32(a2); y.w = cos_f32(a3);
+    }
+    return y;
+}
+
+// dim % 4 == 0 and dim / 4 <= BLOCK: a thread owns one 4-column chunk for its whole life and keeps the
+// chunk's w and b in registers; the block's threads form RPI = BLOCK / (dim / 4) rows of such chunks and
+// walk a tile of `un` * RPI rows, RPI rows (one contiguous piece of the output) per trip.  The tile's dt
+// values are converted once and parked in LDS together with w and b (dynamic LDS: un * RPI + 2 * dim
+// floats), so after the one barrier of a tile a wave issues no global load: loads and stores return
+// through one in-order counter, and a wave that loads w, b or dt between two stores waits for the first
+// store's completion as well, with the arithmetic units idling behind the latency of the stores.  What a
+// block pays before its first result (launch, the loads, the barrier) is paid once per tile: tiles of
+// 8 * RPI rows and more take 0.8 of the time of tiles of 4 * RPI rows (1.32M x 100); the host shrinks the
+// tile when the call is too small to give every CU several blocks.
+constexpr int COLS_UN_MAX = 16;
+constexpr int COLS_MIN_BLOCKS = 512;
+__global__ __launch_bounds__(BLOCK) void time_encode_cols_kernel(TEArgs a, int32_t un) {
+    extern __shared__ __align__(16) float s_dyn[];
+    const int32_t cpr = a.dim / 4;
+    const int32_t rpi = BLOCK / cpr;
+    const int32_t tile = rpi * un;
+    float* __restrict__ s_w = s_dyn;
+    float* __restrict__ s_b = s_dyn + a.dim;
+    float* __restrict__ s_x = s_dyn + 2 * a.dim;
+    const int32_t rl = threadIdx.x / cpr;
+    const int32_t j = (threadIdx.x - rl * cpr) * 4;
+    const bool active = rl < rpi;
+    for (int32_t i = threadIdx.x; i < a.dim; i += BLOCK) {
+        s_w[i] = a.w[i];
+        s_b[i] = a.b[i];
+    }
+    f32x4 w = {0.f, 0.f, 0.f, 0.f}, b = {0.f, 0.f, 0.f, 0.f};
+    const int64_t N = live_count(a.N_dev, a.N_max);
+    bool first = true;
+    for (int64_t row0 = (int64_t)blockIdx.x * tile; row0 < N; row0 += (int64_t)gridDim.x * tile) {
+        const int32_t rows = (int32_t)((N - row0) < tile ? (N - row0) : tile);
+        __syncthreads();
+        for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
+            s_x[r] = a.dt_dtype == SGL_DT_I64 ? (float)static_cast<const int64_t*>(a.dt)[row0 + r]
+                                               : static_cast<const float*>(a.dt)[row0 + r];
+        }
+        __syncthreads();
+        if (first && active) {
+            w = *reinterpret_cast<const f32x4*>(s_w + j);
+            b = *reinterpret_cast<const f32x4*>(s_b + j);
+        }
+        first = false;
+        float* __restrict__ dst = a.out + (row0 + rl) * a.dim + j;
+        const int64_t step = (int64_t)rpi * a.dim;
+        for (int32_t r = rl; r < rows; r += rpi, dst += step) {
+            if (active) *reinterpret_cast<f32x4*>(dst) = enc4(w, s_x[r], b);
+        }
+    }
 }
 
 template <int VEC>
@@ -132,7 +207,16 @@ extern "C" int32_t sgl_time_encode(const void* dt, int32_t dt_dtype, int64_t N_m
     if (N_dev != nullptr && blocks > 8192) blocks = 8192;   // live count usually far below capacity
     if (blocks > 0x3FFFFFll) blocks = 0x3FFFFFll;
     hipStream_t st = as_stream(stream);
-    if (vec4)
+    if (vec4 && cpr <= BLOCK) {
+        const int64_t rpi = BLOCK / cpr;
+        int64_t un = N_max / (rpi * COLS_MIN_BLOCKS);
+        un = un < 1 ? 1 : (un > COLS_UN_MAX ? COLS_UN_MAX : un);
+        blocks = ceil_div<int64_t>(N_max, rpi * un);
+        if (N_dev != nullptr && blocks > 8192) blocks = 8192;
+        if (blocks > 0x3FFFFFll) blocks = 0x3FFFFFll;
+        const size_t lds = (size_t)(rpi * un + 2 * dim) * sizeof(float);     // <= 16 KB + 8 KB
+        hipLaunchKernelGGL(time_encode_cols_kernel, dim3((unsigned)blocks), dim3(BLOCK), lds, st, a, (int32_t)un);
+    } else if (vec4)
         hipLaunchKernelGGL(time_encode_kernel<4>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
     else
         hipLaunchKernelGGL(time_encode_kernel<1>, dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);

@@ -45,6 +45,41 @@ def test_time_encode_f32_input_and_device_count(oracle, hot):
     assert np.abs(got[:777] - want[:777]).max() <= TOL and not got[777:].any()
 
 
+@pytest.mark.parametrize("dim,rows,live", [
+    (100, 50_000, None),        # 10 rows of 25 chunks per trip, tiles of several trips
+    (100, 400_000, None),       # the largest tile
+    (4, 1_200_000, None),       # one chunk per row: 256 rows per trip
+    (1024, 5_000, None),        # 256 chunks per row: one row per trip
+    (1028, 300, None),          # 257 chunks per row: more than a block has threads
+    (172, 30_011, None),        # 43 chunks per row: 41 threads of a block idle
+    (512, 300_000, 290_001),    # more tiles than the capped grid has blocks, live count on the device
+])
+def test_time_encode_tiles(oracle, hot, dim, rows, live):
+    """every tile shape of the kernels (a thread owns one 4-column chunk and walks the rows of a tile; the tile's
+    size follows the call's size) against the oracle, bit for bit where the oracle is correctly rounded too."""
+    rng = np.random.default_rng(dim + rows)
+    dt = rng.integers(-2**40, 2**40, rows).astype(np.int64)
+    dt[:5] = [0, 1, -1, 2**40, -(2**40)]
+    w, b = _w(dim), rng.standard_normal(dim).astype(np.float32)
+    n = rows if live is None else live
+    out = hot.be.zeros((rows, dim), "f32")
+    hot.time_encode(to_dev(hot, dt), to_dev(hot, w, "f32"), to_dev(hot, b, "f32"), out=out,
+                    N_dev=None if live is None else to_dev(hot, np.array([live], dtype=np.int64)))
+    got = np_of(out)
+    step = 50_000_000 // dim            # the oracle works in float64: bounded pieces
+    worst, same, total = 0.0, 0, 0
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        want = oracle.time_encode(dt[lo:hi], w, b)
+        err = np.abs(got[lo:hi].astype(np.float64) - want)
+        worst = max(worst, float(err.max()))
+        same += int((got[lo:hi] == want).sum())
+        total += want.size
+    assert worst <= 1.2e-7, worst
+    assert same / total > 0.99
+    assert not got[n:].any()
+
+
 def test_time_encode_is_within_one_ulp_everywhere(oracle, hot):
     """denser check of the in-kernel cosine: <= 1 ulp (1.2e-7 absolute, |y| <= 1) against the
     correctly rounded oracle over small, mid-range and huge arguments, including the
