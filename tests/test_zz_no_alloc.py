@@ -19,9 +19,11 @@ def _hop_pair(hot, dg, node, t, p, S_dev=None):
     S = int(node.shape[0])
     want = hot.sample_hop(dg, node, t, p, S_dev=S_dev, finalize=False)
     got = HopResult(hot.be, S, S * p.fanout)
-    before = torch.cuda.memory_allocated()
+    # the binding allocates nothing either: the allocator's count of allocations made so far stays put
+    # (bytes in use would also move when Python's collector frees another test's tensors during the call)
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
     hot.sample_hop_static(dg, node, t, p, got, S_dev=S_dev)
-    assert torch.cuda.memory_allocated() == before      # the binding allocated nothing either
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
     torch.cuda.synchronize()
     cw, cg = np_of(want.counts), np_of(got.counts)
     assert np.array_equal(cw, cg), (cw, cg)
