@@ -27,6 +27,12 @@ for _p in (ROOT, os.path.join(ROOT, "starrygl-framework_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
+def graph_capture(graph, stream=None):
+    """torch.cuda.graph with Python's cycle collector held off during the capture (see the library's helper)."""
+    from starrygl_amd.lib.driver import graph_capture as capture
+    return capture(graph, stream)
+
+
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes moved per algorithmic byte by the step's gather launch (node rows + hop-1 + hop-2 edge rows),
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (summary and commands:
@@ -207,7 +213,7 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
         with torch.cuda.stream(stream):
             P.s_all.copy_(packed[0]); body(); stream.synchronize()
             P.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(P.graph, stream=stream):
+            with graph_capture(P.graph, stream=stream):
                 body()
 
         def run(b):
@@ -690,7 +696,7 @@ def main():
             step()
             P.stream.synchronize()
             P.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(P.graph, stream=P.stream):
+            with graph_capture(P.graph, stream=P.stream):
                 step()
 
         def run(b):          # (set_stream, not the context manager: the host's share of a step is what bounds
@@ -723,7 +729,7 @@ def main():
         torch.cuda.synchronize()
         g_step = torch.cuda.CUDAGraph()
         if args.serial or not args.separate_samplers:
-            with torch.cuda.graph(g_step):
+            with graph_capture(g_step):
                 body()
         else:
             # independent stages become parallel branches of the graph: the uniform sampler
@@ -736,7 +742,7 @@ def main():
             # independent branch first delays the chain and costs ~10 % of the step; two graphs on
             # two streams, or the edge gather on a branch beside unique, were slower as well.)
             br = torch.cuda.Stream()
-            with torch.cuda.graph(g_step):
+            with graph_capture(g_step):
                 cur = torch.cuda.current_stream()
                 st_recent()
                 ev0 = torch.cuda.Event()
@@ -751,7 +757,7 @@ def main():
         graphs = []
         for f in stages_fn:
             gs = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gs):
+            with graph_capture(gs):
                 f()
             graphs.append(gs)
         mode = ("hipgraph, both samplers in one launch" if not args.separate_samplers else
@@ -910,7 +916,7 @@ def main():
             call()
             cap_s.synchronize()
             g_alt = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g_alt, stream=cap_s):
+            with graph_capture(g_alt, stream=cap_s):
                 call()
             ms = _time_launches(torch, g_alt.replay, reps=20)
         torch.cuda.current_stream().wait_stream(cap_s)
@@ -1094,7 +1100,7 @@ def main():
                 calls()
                 cap.synchronize()
                 gcalls = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(gcalls, stream=cap):
+                with graph_capture(gcalls, stream=cap):
                     calls()
                 ms = _time_launches(torch, gcalls.replay, reps=3, warm=1) / REPS
             torch.cuda.current_stream().wait_stream(cap)

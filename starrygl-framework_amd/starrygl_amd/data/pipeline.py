@@ -18,7 +18,7 @@ import torch
 
 from ..graph.graph import Block
 from ..lib import _abi, hot_path
-from ..lib.driver import POISON, check_sample_bad, check_unique_total
+from ..lib.driver import POISON, check_sample_bad, check_unique_total, graph_capture
 
 
 class MiniBatch:
@@ -271,7 +271,7 @@ class MiniBatchPipeline:
             torch.cuda.current_stream(self.dev).wait_stream(side)
             torch.cuda.current_stream(self.dev).synchronize()
             g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
+            with graph_capture(g):
                 self._chain()
             self._graph = g
             g.replay()

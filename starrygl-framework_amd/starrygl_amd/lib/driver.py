@@ -6,7 +6,9 @@ where arrays live: `TorchBackend` (device tensors, current HIP stream) is what
 the package uses; anything else that offers the same five methods can drive a
 library with the same ABI on host memory.
 """
+import contextlib
 import ctypes as C
+import gc
 import os
 
 from . import _abi
@@ -696,6 +698,25 @@ class HotPath:
         self._ck(self.lib.time_encode(be.ptr(dt), dt_dtype, N, be.ptr(N_dev), be.ptr(w),
                                       be.ptr(b), dim, be.ptr(out), be.stream()))
         return out
+
+
+@contextlib.contextmanager
+def graph_capture(graph, stream=None):
+    """`torch.cuda.graph(graph, stream=stream)` with Python's cycle collector held off.  A collection that runs
+    while a stream is capturing may free a dead object that owns another CUDAGraph (a dropped pipeline, say);
+    that graph's destructor calls the runtime, the runtime refuses calls of that kind from a capturing thread,
+    and an error thrown from a destructor ends the process in std::terminate.  Dead cycles are collected before
+    the capture starts instead (torch itself no longer does that by default)."""
+    import torch
+    gc.collect()
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph, stream=stream):
+            yield
+    finally:
+        if was_enabled:
+            gc.enable()
 
 
 class RemapState:

@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 
 from starrygl_amd.lib import _abi
+from starrygl_amd.lib.driver import graph_capture
 from util import np_of, to_dev
 
 pytestmark = pytest.mark.gpu
@@ -261,7 +262,7 @@ def test_hash_unique_is_captured_and_replayed_in_a_hip_graph(oracle, hot, n):
         call(state)                      # warm-up outside the capture
     stream.synchronize()
     g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g, stream=stream):
+    with graph_capture(g, stream=stream):
         call(state)
     for rep, m in enumerate((n, 17, 12_345, 0, n)):
         a = _encode(rng, 4, n // 3, n).astype(np.int64)
