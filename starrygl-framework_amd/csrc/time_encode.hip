@@ -37,9 +37,9 @@ struct TEArgs {
 // magnitude the path produces (|a| up to 2^40 and beyond): the argument is reduced
 // in double precision by multiples of pi (two-constant Cody-Waite, exact through
 // FMA) to r in [-pi/2, pi/2]; then cos(r) = 1 - 2 sin^2(r/2) with one odd
-// polynomial for sin on [-pi/4, pi/4] - no quadrant-dependent coefficients, so no
-// selects - and the sign (-1)^n is applied to the sign bit of the result.  About 16 fp64
-// operations, all straight-line.  The library cosf takes ~2.5x as long (its
+// polynomial for sqrt(2) sin on [-pi/4, pi/4] - no quadrant-dependent coefficients, so no
+// selects - and the sign (-1)^n is applied to the sign bit of the result.  14 fp64
+// operations and two conversions, all straight-line.  The library cosf takes ~2.5x as long (its
 // large-argument path is a Payne-Hanek reduction).  Arguments beyond 2^45 (not
 // reachable from int64 timestamps times w <= 1 in practice) take the library routine.
 constexpr float COS_CORE_LIMIT = 3.5e13f;
@@ -54,15 +54,16 @@ __device__ __forceinline__ float cos_core(float af) {
     const double n = t - SHIFT;
     double r = __builtin_fma(-n, 3.14159265358979311600e+00, x);        // pi, high part
     r = __builtin_fma(-n, 1.22464679914735317723e-16, r);               // pi, low part
-    const double h = 0.5 * r, h2 = h * h;
-    // sin(h) = h + h*h2*S(h2) on [-pi/4, pi/4]
-    double p = -2.505210838544171878e-08;                               // -1/11!
-    p = __builtin_fma(p, h2, 2.755731922398589065e-06);                 //  1/9!
-    p = __builtin_fma(p, h2, -1.984126984126984127e-04);                // -1/7!
-    p = __builtin_fma(p, h2, 8.333333333333333333e-03);                 //  1/5!
-    p = __builtin_fma(p, h2, -1.666666666666666667e-01);                // -1/3!
-    const double sn = __builtin_fma(p, h * h2, h);
-    const float c = (float)__builtin_fma(-2.0 * sn, sn, 1.0);           // cos(r)
+    // cos r = 1 - 2 sin^2(r/2) = 1 - q^2 with q = sqrt(2) sin(r/2), odd in u = r/sqrt(2) on [-1.12, 1.12]:
+    // q = u + u*u2*Q(u2), Q the cubic through (q/u - 1)/u2 at the four Chebyshev points of [0, 1.235]
+    // (|cos r - result| < 4e-11 before the rounding to fp32, as with the series up to u^11)
+    const double u = 0.70710678118654752440 * r, u2 = u * u;
+    double p = 1.7031108097175238e-07;
+    p = __builtin_fma(p, u2, -2.4800106945370714e-05);
+    p = __builtin_fma(p, u2, 2.083332968131731e-03);
+    p = __builtin_fma(p, u2, -8.33333333192484e-02);
+    const double q = __builtin_fma(p, u * u2, u);
+    const float c = (float)__builtin_fma(-q, q, 1.0);                   // cos(r)
     // (-1)^n: flip the sign bit of the rounded result
     return __uint_as_float(__float_as_uint(c) ^ (odd << 31));
 }
@@ -82,9 +83,9 @@ __device__ __forceinline__ f32x4 enc4(const f32x4 w, float x, const f32x4 b) {
     const float a2 = __fadd_rn(__fmul_rn(w.z, x), b.z), a3 = __fadd_rn(__fmul_rn(w.w, x), b.w);
     const float m = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(a0), __builtin_fabsf(a1)),
                                     __builtin_fmaxf(__builtin_fabsf(a2), __builtin_fabsf(a3)));
-    const bool nan = a0 != a0 || a1 != a1 || a2 != a2 || a3 != a3;    // (fmax drops a NaN operand)
+    // (the maximum drops a NaN operand; cos_core turns a NaN into a NaN, so one may take either route)
     f32x4 y;
-    if (m < COS_CORE_LIMIT && !nan) {
+    if (m < COS_CORE_LIMIT) {
         y.x = cos_core(a0); y.y = cos_core(a1); y.z = cos_core(a2); y.w = cos_core(a3);
     } else {
         y.x = cos_f32(a0); y.y = cos_f32(a1); y.z = cos_f32(a2); y.w = cos_f32(a3);
