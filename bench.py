@@ -918,7 +918,7 @@ def main():
             g_alt = torch.cuda.CUDAGraph()
             with graph_capture(g_alt, stream=cap_s):
                 call()
-            ms = _time_launches(torch, g_alt.replay, reps=20)
+            ms = _time_launches(torch, g_alt.replay, reps=200, warm=20)
         torch.cuda.current_stream().wait_stream(cap_s)
         stages[tag] = {"ms": round(ms, 4), "ids_per_s": round(n_ids / ms * 1e3, 1), "unique": int(u_alt[0].item()),
                        "GBps": round((16 * n_ids + 8 * int(u_alt[0].item())) / ms / 1e6, 1)}
