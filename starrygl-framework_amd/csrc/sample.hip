@@ -1474,7 +1474,7 @@ __device__ __forceinline__ void fused2_body(const Fused2Args& f, const int64_t b
 template <bool UNIFORM>
 __global__ __launch_bounds__(BLOCK) void fused2_kernel(Fused2Args f) {
     extern __shared__ int64_t s_dyn[];
-    fused2_body<UNIFORM, 10>(f, blockIdx.x, gridDim.x, s_dyn);
+    fused2_body<UNIFORM, 8>(f, blockIdx.x, gridDim.x, s_dyn);
 }
 
 // Two calls over the same roots in one launch, a most-recent one (even blocks) and a uniform one (odd
