@@ -486,7 +486,7 @@ def main():
                     help="headline steps take the window ends of their positive roots from a lookup done before the timed "
                          "region (a loader that knows its event stream can do that); by default every root is searched "
                          "inside the step and the variant with hints is only reported beside it")
-    ap.add_argument("--pipelines", type=int, default=3,
+    ap.add_argument("--pipelines", type=int, default=4,
                     help="independent copies of the step (own buffers, graph and stream) that take the batches of the "
                          "timed region in turn, as a loader with that many batches in flight does; 1 = one batch at a time")
     ap.add_argument("--hold-ms", type=float, default=0.0,
@@ -1183,7 +1183,7 @@ def main():
         "value": round(value, 1), "unit": "sampled edges/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 4), "host_submit_ms_per_step": round(host_submit / K * 1e3, 4), "one_batch_in_flight": one_in_flight, "other_root_hint_choice": hinted_variant, "step_ms_spread": step_spread,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int64", "data": "synthetic", "launch_mode": mode,
+        "dtype": "int64", "data": "synthetic", "launch_mode": mode, "batches_in_flight": args.pipelines if piped else 1,
         "config": {"workload": "configs[1]: 1M nodes / 20M edges Zipf(1.1) out-degree, batches of 4000 events + 4000 "
                                "negatives (12000 roots): 2-hop recent 10x10 + unique + node/edge gather + 2-hop uniform 10x10",
                    "nodes": n, "edges": m, "roots_per_batch": S0, "fanout": [k, k],
