@@ -1,4 +1,4 @@
-"""GPU: a seeded sweep of random shapes through every stage (T-CSR build, k-hop sampling of both
+"""GPU: seeded sweeps of random shapes through every stage (T-CSR build, k-hop sampling of both
 kinds and both in one call, unique in both modes over the dense table and the hash set, seed extraction,
 slicing, pair unique) against the CPU oracle, bit-exact.  The parametrised tests pin chosen edge cases;
 this one walks the combinations nobody chose."""
@@ -114,3 +114,165 @@ def test_random_shapes_match_the_oracle(oracle, hot, first):
             _one_case(seed, oracle, hot)
         except AssertionError as exc:
             raise AssertionError(f"seed {seed}: {exc}") from exc
+
+
+# ---- two-tier gather and multi-segment gather against numpy
+
+def _random_table(rng, hot):
+    import torch
+    dev = hot.be.device
+    rows = int(rng.choice([1, 2, 33, 1000, 20_000]))
+    dim = int(rng.choice([1, 2, 3, 4, 6, 16, 100, 172, 64, 500]))
+    frac = float(rng.choice([0.0, 0.1, 0.5, 1.0]))
+    full = rng.standard_normal((rows, dim)).astype(np.float32)
+    ts_full = rng.integers(0, 10**9, rows).astype(np.int64)
+    hot_rows = int(rows * frac)
+    hot_ids = rng.permutation(rows)[:hot_rows]
+    slot = np.full(rows, -1, np.int32)
+    slot[hot_ids] = np.arange(hot_rows, dtype=np.int32)
+    cold, tsc = full.copy(), ts_full.copy()
+    cold[hot_ids] = 0          # a hot row must never be served from the cold tier
+    tsc[hot_ids] = 0
+    G = rows * 3 + 5
+    g2l = None
+    if rng.random() < 0.4:     # global id -> local row through a dense map
+        g2l = np.full(G + 1, -1, np.int64)
+        g2l[rng.permutation(G)[:rows]] = np.arange(rows)
+    t_hot = torch.from_numpy(full[hot_ids].copy()).to(dev) if hot_rows else None
+    if rng.random() < 0.4:     # row and time side by side in one pinned record
+        t_cold, t_tsc, _ = hot.interleaved_cold(rows, dim)
+        t_cold.copy_(torch.from_numpy(cold))
+        t_tsc.copy_(torch.from_numpy(tsc))
+    else:
+        t_cold, t_tsc = torch.from_numpy(cold).pin_memory(), torch.from_numpy(tsc).pin_memory()
+    kw = {}
+    if frac < 1.0 or rng.random() < 0.5:
+        kw.update(cold=t_cold, hot_slot=to_dev(hot, slot, "i32"), ts_cold=t_tsc)
+        if t_hot is not None:
+            kw.update(ts_hot=to_dev(hot, ts_full[hot_ids].copy()))
+    else:                      # one HBM table in row order, no index
+        t_hot = torch.from_numpy(full).to(dev)
+        kw.update(ts_hot=to_dev(hot, ts_full))
+    if g2l is not None:
+        kw.update(g2l=to_dev(hot, g2l))
+    return dict(rows=rows, dim=dim, full=full, ts=ts_full, g2l=g2l, G=G, cache=hot.cache(dim * 4, t_hot, rows=rows, **kw))
+
+
+def _one_gather_case(seed, hot):
+    import torch
+    rng = np.random.default_rng(seed)
+    dev = hot.be.device
+    tabs = [_random_table(rng, hot) for _ in range(int(rng.integers(1, 4)))]
+    segs, wants = [], []
+    for T in tabs:
+        n = int(rng.choice([0, 1, 7, 300, 5000, 40_000]))
+        hi = T["G"] + 1 if T["g2l"] is not None else T["rows"]
+        ids = rng.integers(0, hi, n).astype(np.int64)
+        if n > 3:
+            ids[rng.integers(0, n, max(1, n // 50))] = -7
+            ids[rng.integers(0, n, max(1, n // 50))] = hi + 11
+        ok = (ids >= 0) & (ids < hi)
+        loc = np.where(ok, T["g2l"][np.clip(ids, 0, hi - 1)] if T["g2l"] is not None else ids, -1)
+        good = loc >= 0
+        w_rows = np.where(good[:, None], T["full"][np.clip(loc, 0, T["rows"] - 1)], 0).astype(np.float32)
+        w_ts = np.where(good, T["ts"][np.clip(loc, 0, T["rows"] - 1)], 0)
+        live = None if rng.random() < 0.5 or n == 0 else int(rng.integers(0, n + 1))
+        out = torch.zeros((max(n, 1), T["dim"]), dtype=torch.float32, device=dev)[:n]
+        out_ts = hot.be.zeros(max(n, 1))[:n] if rng.random() < 0.5 else None
+        n_dev = None if live is None else to_dev(hot, np.array([live], dtype=np.int64))
+        segs.append((T["cache"], to_dev(hot, ids), out, out_ts, n_dev))
+        wants.append((w_rows, w_ts, n if live is None else live))
+    live_segs = [s for s in segs if s[2].shape[0]]
+    if rng.random() < 0.5 and live_segs and all(T["dim"] % 4 == 0 for T in tabs):
+        hot.gather_multi(hot.gather_plan(live_segs))
+    else:
+        for c, ids, out, ots, nd in live_segs:
+            hot.gather(c, ids, out, out_ts=ots, N_dev=nd)
+    for (c, ids, out, ots, nd), (w_rows, w_ts, m) in zip(segs, wants):
+        g = np_of(out)
+        assert np.array_equal(g[:m].view(np.uint32), w_rows[:m].view(np.uint32)) and not g[m:].any(), f"seed {seed}: rows"
+        if ots is not None:
+            gt = np_of(ots)
+            assert np.array_equal(gt[:m], w_ts[:m]) and not gt[m:].any(), f"seed {seed}: times"
+
+
+@pytest.mark.parametrize("first", [0, 150])
+def test_random_gathers_match_numpy(hot, first):
+    """random tables (tiers, index, interleaved cold records, row widths), id lists with absent ids and
+    device-side live counts, one launch per table or one for all"""
+    for seed in range(first, first + 150):
+        _one_gather_case(9000 + seed, hot)
+
+
+# ---- sequences of calls on a hashed remap state, up to and past its capacity
+
+@pytest.mark.parametrize("first", [0, 200])
+def test_random_sequences_on_a_hashed_state(oracle, hot, first):
+    """every call of a sequence equals the oracle's; when a sequence outgrows the state, both sides say so"""
+    for seq in range(first, first + 200):
+        rng = np.random.default_rng(7000 + seq)
+        cap = int(rng.choice([1, 7, 300, 5000, 70_000, 400_000]))
+        mode = int(rng.choice([_abi.UNIQUE_SORTED, _abi.UNIQUE_GROUPED]))
+        kind = str(rng.choice(["dense", "wide", "encoded", "squares", "neg"]))
+
+        def draw(n):
+            if kind == "dense": return rng.integers(0, max(2, cap // 2), n)
+            if kind == "wide": return rng.integers(0, 2**62, n)
+            if kind == "encoded": return (rng.integers(0, 8, n) << 48) | rng.integers(0, max(2, cap), n)
+            if kind == "squares": return rng.integers(0, 50_000, n) ** 2 + (1 << 40)
+            x = rng.integers(0, max(2, cap), n)
+            x[rng.random(n) < 0.2] = -rng.integers(1, 100)
+            return x
+
+        so, sh = oracle.remap_hashed_state(cap), hot.remap_hashed_state(cap)
+        for c in range(int(rng.integers(1, 7))):
+            G = int(rng.integers(1, 4))
+            arrs = [draw(int(rng.choice([0, 1, 5, 300, 4000, 60_000, 9000]))).astype(np.int64) for _ in range(G)]
+            reset = bool(rng.random() < 0.4) or c == 0
+            try:
+                lo, uo, (to_, bo) = oracle.unique_compact([a.copy() for a in arrs], mode, so, reset)
+            except RuntimeError:
+                lo = None
+            try:
+                lh, uh, (th, bh) = hot.unique_compact([to_dev(hot, a) for a in arrs], mode, sh, reset)
+            except RuntimeError:
+                lh = None
+            assert (lo is None) == (lh is None), f"sequence {seq} call {c}: only one side reports the outgrown state"
+            if lo is None:
+                break          # both states are void
+            assert (th, bh) == (to_, bo), f"sequence {seq} call {c}"
+            assert np.array_equal(np_of(uh)[bh:th], uo[bo:to_]), f"sequence {seq} call {c}: unique list"
+            for g in range(G):
+                assert np.array_equal(np_of(lh[g]), lo[g]), f"sequence {seq} call {c} array {g}"
+
+
+# ---- time encoding over random widths, sizes and live counts
+
+def test_random_time_encodings(oracle, hot):
+    for it in range(250):
+        rng = np.random.default_rng(5000 + it)
+        dim = int(rng.choice([1, 3, 4, 8, 12, 100, 128, 172, 256, 1020, 1024, 1028, int(rng.integers(1, 1100))]))
+        N = int(rng.choice([0, 1, 9, 10, 11, 255, 257, 4096, 5121, 40000, int(rng.integers(0, 60000))]))
+        N = min(N, 20_000_000 // dim)
+        span = int(rng.choice([50, 10**7, 2**40, 2**62]))
+        dt = rng.integers(-span, span, N).astype(np.int64)
+        w = (1.0 / 10 ** np.linspace(0, 9, dim, dtype=np.float32)).astype(np.float32)
+        if rng.random() < 0.3:
+            w = rng.standard_normal(dim).astype(np.float32)
+        b = rng.standard_normal(dim).astype(np.float32)
+        live = None if rng.random() < 0.5 or N == 0 else int(rng.integers(0, N + 1))
+        out = hot.be.zeros((max(N, 1), dim), "f32")[:N]
+        n_dev = None if live is None else to_dev(hot, np.array([live], dtype=np.int64))
+        if rng.random() < 0.3:
+            x = dt.astype(np.float32)
+            want = oracle.time_encode(x, w, b, dt_dtype=_abi.DT_F32)
+            hot.time_encode(to_dev(hot, x, "f32"), to_dev(hot, w, "f32"), to_dev(hot, b, "f32"), dt_dtype=_abi.DT_F32,
+                            out=out, N_dev=n_dev)
+        else:
+            want = oracle.time_encode(dt, w, b)
+            hot.time_encode(to_dev(hot, dt), to_dev(hot, w, "f32"), to_dev(hot, b, "f32"), out=out, N_dev=n_dev)
+        got = np_of(out)
+        n = N if live is None else live
+        if n:
+            assert np.abs(got[:n].astype(np.float64) - want[:n]).max() <= 1.2e-7, f"case {it}: dim {dim} N {N}"
+        assert not got[n:].any(), f"case {it}: rows beyond the live count were written"
