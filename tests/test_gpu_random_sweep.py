@@ -155,7 +155,8 @@ def _random_table(rng, hot):
         kw.update(ts_hot=to_dev(hot, ts_full))
     if g2l is not None:
         kw.update(g2l=to_dev(hot, g2l))
-    return dict(rows=rows, dim=dim, full=full, ts=ts_full, g2l=g2l, G=G, cache=hot.cache(dim * 4, t_hot, rows=rows, **kw))
+    return dict(rows=rows, dim=dim, full=full, ts=ts_full, g2l=g2l, G=G, cache=hot.cache(dim * 4, t_hot, rows=rows, **kw),
+                t_hot=t_hot, t_cold=kw.get("cold"), t_ts_hot=kw.get("ts_hot"), t_ts_cold=kw.get("ts_cold"))
 
 
 def _one_gather_case(seed, hot):
@@ -194,6 +195,47 @@ def _one_gather_case(seed, hot):
         if ots is not None:
             gt = np_of(ots)
             assert np.array_equal(gt[:m], w_ts[:m]) and not gt[m:].any(), f"seed {seed}: times"
+
+
+def _one_update_case(seed, hot):
+    """scatter_update of distinct rows (some ids absent) into both tiers, read back through the gather"""
+    import torch
+    rng = np.random.default_rng(seed)
+    T = _random_table(rng, hot)
+    if T["t_ts_hot"] is None and T["t_hot"] is not None:
+        return
+    rows, dim = T["rows"], T["dim"]
+    hi = T["G"] + 1 if T["g2l"] is not None else rows
+    n = int(rng.integers(0, min(rows, 3000) + 1))
+    loc = rng.permutation(rows)[:n].astype(np.int64)                   # distinct local rows
+    ids = np.nonzero(np.isin(T["g2l"], loc))[0].astype(np.int64) if T["g2l"] is not None else loc.copy()
+    if T["g2l"] is not None:
+        loc = T["g2l"][ids]
+    ids_w = ids.copy()
+    if n > 5:
+        ids_w[::17] = -3                                               # skipped
+    vals = rng.standard_normal((n, dim)).astype(np.float32)
+    new_ts = rng.integers(1, 10**9, n).astype(np.int64)
+    hot.scatter_update(T["cache"], T["t_hot"], T["t_cold"], T["t_ts_hot"], T["t_ts_cold"], to_dev(hot, ids_w),
+                       to_dev(hot, vals, "f32"), to_dev(hot, new_ts))
+    want, want_ts = T["full"].copy(), T["ts"].copy()
+    keep = ids_w >= 0
+    want[loc[keep]] = vals[keep]
+    want_ts[loc[keep]] = new_ts[keep]
+    probe = rng.integers(0, hi, 4000).astype(np.int64)
+    ploc = T["g2l"][probe] if T["g2l"] is not None else probe
+    good = ploc >= 0
+    out = torch.zeros((4000, dim), dtype=torch.float32, device=hot.be.device)
+    out_ts = hot.be.zeros(4000)
+    hot.gather(T["cache"], to_dev(hot, probe), out, out_ts=out_ts)
+    w_rows = np.where(good[:, None], want[np.clip(ploc, 0, rows - 1)], 0).astype(np.float32)
+    assert np.array_equal(np_of(out).view(np.uint32), w_rows.view(np.uint32)), f"seed {seed}: rows after the update"
+    assert np.array_equal(np_of(out_ts), np.where(good, want_ts[np.clip(ploc, 0, rows - 1)], 0)), f"seed {seed}: times"
+
+
+def test_random_updates_read_back(hot):
+    for seed in range(120):
+        _one_update_case(12000 + seed, hot)
 
 
 @pytest.mark.parametrize("first", [0, 150])
@@ -240,6 +282,32 @@ def test_random_sequences_on_a_hashed_state(oracle, hot, first):
             assert (lo is None) == (lh is None), f"sequence {seq} call {c}: only one side reports the outgrown state"
             if lo is None:
                 break          # both states are void
+            assert (th, bh) == (to_, bo), f"sequence {seq} call {c}"
+            assert np.array_equal(np_of(uh)[bh:th], uo[bo:to_]), f"sequence {seq} call {c}: unique list"
+            for g in range(G):
+                assert np.array_equal(np_of(lh[g]), lo[g]), f"sequence {seq} call {c} array {g}"
+
+
+def test_random_sequences_on_a_dense_state(oracle, hot):
+    """'r' / 'f' sequences on the dense remap state, ids outside the universe among them"""
+    for seq in range(150):
+        rng = np.random.default_rng(8000 + seq)
+        universe = int(rng.choice([1, 9, 700, 50_000, 3_000_000]))
+        mode = int(rng.choice([_abi.UNIQUE_SORTED, _abi.UNIQUE_GROUPED]))
+        so, sh = oracle.remap_state(universe), hot.remap_state(universe)
+        for c in range(int(rng.integers(1, 6))):
+            G = int(rng.integers(1, 4))
+            arrs = []
+            for _ in range(G):
+                n = int(rng.choice([0, 1, 5, 300, 4000, 60_000]))
+                a = rng.integers(0, universe, n).astype(np.int64)
+                if n > 4:
+                    a[1] = -4
+                    a[3] = universe + 2
+                arrs.append(a)
+            reset = bool(rng.random() < 0.4) or c == 0
+            lo, uo, (to_, bo) = oracle.unique_compact([a.copy() for a in arrs], mode, so, reset)
+            lh, uh, (th, bh) = hot.unique_compact([to_dev(hot, a) for a in arrs], mode, sh, reset)
             assert (th, bh) == (to_, bo), f"sequence {seq} call {c}"
             assert np.array_equal(np_of(uh)[bh:th], uo[bo:to_]), f"sequence {seq} call {c}: unique list"
             for g in range(G):
