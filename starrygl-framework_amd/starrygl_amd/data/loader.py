@@ -16,12 +16,13 @@ from .pipeline import MiniBatchPipelinePool
 
 class EventBatchLoader:
     def __init__(self, graph, src, dst, ts, batch_size, num_neg, layers, fanout, sample_type="recent",
-                 node_tables=None, edge_tables=None, time_encoder=None, prefetch=3, negative_sampler=None,
+                 node_tables=None, edge_tables=None, time_encoder=None, prefetch=4, negative_sampler=None,
                  drop_last=True, **pipeline_kwargs):
         """graph: `pyGraph.g` / `CUDAGraph`.  src/dst/ts: the events in training order (int64, any device).
         num_neg: negatives per batch (their times repeat the batch's event times).  negative_sampler: an
         object with `sample(num_samples, num_groups)` (NegSamplingSet); default: uniform over all nodes.
-        prefetch: batches in flight (pipelines of the pool).  Remaining keywords go to MiniBatchPipeline.
+        prefetch: batches in flight (pipelines of the pool; a process has four hardware queues, and
+        pipelines that share one take turns).  Remaining keywords go to MiniBatchPipeline.
         Only full batches are produced (every buffer of a pipeline is planned for one batch shape)."""
         if not drop_last:
             raise ValueError("EventBatchLoader produces full batches only (drop_last=True)")

@@ -159,7 +159,7 @@ def test_pipeline_with_root_hints(oracle, hot, sample_type):
         plain.run(to_dev(hot, b[0]), to_dev(hot, b[2]), to_dev(hot, b[3]), to_dev(hot, b[4]), root_hint=hint)
 
 
-@pytest.mark.parametrize("prefetch", [1, 3])
+@pytest.mark.parametrize("prefetch", [1, 3, 4])
 def test_event_batch_loader(oracle, hot, prefetch):
     """The loader walks the event stream batch by batch with `prefetch` batches in flight and the window ends
     of all event endpoints looked up once; every yielded batch equals the oracle's result for its own events
