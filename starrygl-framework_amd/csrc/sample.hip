@@ -1134,10 +1134,6 @@ __device__ __forceinline__ int64_t lane_lower_bound(const int64_t* __restrict__ 
     return lo;
 }
 
-// `b` of `nb`: the block's index among the blocks of this call (set by the kernels below)
-// PRE: hop-2 slots of a most-recent call whose edges are loaded while the block waits for the
-// totals of the blocks before it (6 registers per slot).  s_pick: k * BLOCK entries of dynamic LDS
-// (uniform only): the draws of a hop-2 slot are made by the slot's lane; its k picks live there, pick-major.
 // What a lane carries from the counting half of the single-launch sampler (fused2_count: windows and
 // counts of its root and of its hop-2 slot, the block's totals published) to the writing half
 // (fused2_write: offsets from the totals of the blocks before, then the outputs).
@@ -1291,6 +1287,10 @@ __device__ __forceinline__ void fused2_count(const Fused2Args& f, const int64_t 
     s.in_range = in_range; s.e_on = e_on;
 }
 
+// `b` of `nb`: the block's index among the blocks of this call (set by the kernels below)
+// PRE: hop-2 slots of a most-recent call whose edges are loaded while the block waits for the
+// totals of the blocks before it (6 registers per slot).  s_pick: k * BLOCK entries of dynamic LDS
+// (uniform only): the draws of a hop-2 slot are made by the slot's lane; its k picks live there, pick-major.
 template <bool UNIFORM, int PRE>
 __device__ __forceinline__ void fused2_write(const Fused2Args& f, const int64_t b, const int64_t nb, int64_t* s_pick,
                                              const F2Lane& s) {
