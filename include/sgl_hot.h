@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define SGL_ABI_VERSION 6
+#define SGL_ABI_VERSION 7
 
 /* ------------------------------------------------------------------ status */
 #define SGL_OK        0
@@ -316,6 +316,47 @@ int32_t sgl_sample_khop_multi(const sgl_tcsr* g,
                               const sgl_hop_out* outs,
                               void* workspace, size_t workspace_bytes, void* stream);
 
+/* B mini-batches sampled by ONE k-hop launch sequence, per-batch results
+ * addressable on the device.  The reference keeps several windows in flight at
+ * once - AsyncGraphBlob submits one query per window (graph.py:274-293),
+ * AsyncTemporalSampler::submit_query queues them (sample.cu.hpp:1990-2020),
+ * the loader prefetches (`prefetch_factor`, test/test.py:212-221) - but runs
+ * them one after the other; a 12 000-root query is bound by launch floors and
+ * by its chain of dependent loads, B of them in one call are bound by
+ * throughput.
+ *   slot_node/slot_ts [S_max]  the hop-0 slots of all batches, batch after
+ *                              batch (per batch: its positive root timestamps,
+ *                              then its negatives, as sgl_sample_khop lays
+ *                              them out);
+ *   batch_ptr  device int64[B+1], ascending: batch b owns the slots
+ *              [batch_ptr[b], batch_ptr[b+1]); batch_ptr[B] <= S_max is the
+ *              live slot count (trailing batches may be empty);
+ *   slot_hint  optional device int64[S_max]: where slot s's window ends
+ *              (sgl_window_end), -1 = search; used when equal_root_time == 0;
+ *   p[q], outs[q * layers + l]  Q queries over the same slots, as
+ *              sgl_sample_khop_multi (mark_state must be NULL: the batches
+ *              have id spaces of their own, see sgl_unique_compact_batched).
+ * The result equals ONE sgl_sample_khop call whose root slots are slot_node /
+ * slot_ts (the generator of the uniform strategy is keyed by the slot's index
+ * in the whole call); for the most-recent strategy that is the concatenation
+ * of the batches' own results.
+ *   seg  device int64[Q][layers+1][B+1]: seg[q][0][b] = batch_ptr[b];
+ *        seg[q][l+1][b] = outs[q*layers+l].root_start_ptr[seg[q][l][b]], i.e.
+ *        batch b owns the edges [seg[q][l+1][b], seg[q][l+1][b+1]) of hop l
+ *        (which are the slots of hop l+1).
+ * Always the launch-per-hop route (nothing waits for another block). */
+size_t  sgl_sample_khop_batched_workspace_bytes(int64_t S_max, int32_t layers,
+                                                int32_t fanout, int32_t Q);
+int32_t sgl_sample_khop_batched(const sgl_tcsr* g, int32_t B,
+                                const int64_t* batch_ptr, int64_t S_max,
+                                const int64_t* slot_node, const int64_t* slot_ts,
+                                const int64_t* slot_hint,
+                                int32_t layers, int32_t Q,
+                                const sgl_sample_params* p,
+                                const sgl_hop_out* outs, int64_t* seg,
+                                void* workspace, size_t workspace_bytes,
+                                void* stream);
+
 /* ------------------------------------------------------ unique / compaction */
 #define SGL_UNIQUE_SORTED  0 /* all arrays form one group: == np.unique(return_inverse) */
 #define SGL_UNIQUE_GROUPED 1 /* per array: ids new to the epoch, ascending, appended    */
@@ -399,6 +440,36 @@ int32_t sgl_unique_compact_hashed(void* state, int64_t capacity, int32_t reset,
                                   int64_t* U_dev,
                                   void* workspace, size_t workspace_bytes,
                                   void* stream);
+
+/* Unique + compaction of B mini-batches, each with a local-id space of its
+ * own, in one launch sequence (the loader's batches are independent: every one
+ * starts a new epoch, Remapper with op 'r', sample.cu.hpp:1825-1852; np.unique
+ * per batch in prepare_sample.py:205-213).  The state spans B copies of the
+ * universe [0, universe) (B <= SGL_BATCH_MAX); every call starts a new epoch.
+ *   ids[g] / local_out[g]  G arrays of len_max[g] entries holding all batches;
+ *   seg[g]     device int64[B+1]: elements [seg[g][b], seg[g][b+1]) of array g
+ *              belong to batch b (seg[g][B] = live length <= len_max[g]) -
+ *              what sgl_sample_khop_batched writes per hop;
+ *   unique_out batch b's distinct ids, ascending, at [U_off[b], U_off[b+1]);
+ *   U_off      device int64[B+1], U_off[B] = number of rows of unique_out;
+ *   local_out  position of the id in its batch's list (-1 for ids outside
+ *              [0, universe)).
+ * Per batch this is sgl_unique_compact(..., reset = 1, SGL_UNIQUE_SORTED) over
+ * the batch's slices. */
+#define SGL_BATCH_MAX 64
+size_t  sgl_remap_batched_state_bytes(int64_t universe, int32_t B);
+int32_t sgl_remap_batched_init(void* state, size_t state_bytes, int64_t universe,
+                               int32_t B, void* stream);
+size_t  sgl_unique_batched_workspace_bytes(int64_t universe, int32_t B);
+int32_t sgl_unique_compact_batched(void* state, int64_t universe, int32_t B,
+                                   int32_t G, const int64_t* const* ids,
+                                   const int64_t* len_max,
+                                   const int64_t* const* seg,
+                                   int64_t* const* local_out,
+                                   int64_t* unique_out, int64_t unique_capacity,
+                                   int64_t* U_off,
+                                   void* workspace, size_t workspace_bytes,
+                                   void* stream);
 
 /* ------------------------------------------------------------ cache gather */
 /* Two-tier row store (replaces IDMapper.to_local + DistNodeState.__getitem__,

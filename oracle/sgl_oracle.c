@@ -567,6 +567,58 @@ int32_t sglo_sample_khop_multi(const sgl_tcsr* g, int64_t R, const int64_t* root
     return SGL_OK;
 }
 
+/* B mini-batches in one call.  The reference queues one query per window and runs them one after the other
+ * (AsyncGraphBlob, graph.py:274-293; submit_query, sample.cu.hpp:1990-2020); by definition the batched call
+ * is the k-hop driver (sample.cu.hpp:1532-1716) over the concatenated root slots, plus the table that says
+ * where each batch's edges begin in every hop.  slot_hint is an accelerator of the kernels: the oracle
+ * searches, and refuses a hint that is not the window end it finds itself. */
+size_t sglo_sample_khop_batched_workspace_bytes(int64_t S_max, int32_t layers, int32_t fanout, int32_t Q) {
+    (void)S_max; (void)layers; (void)fanout; (void)Q;
+    return 0;
+}
+
+int32_t sglo_sample_khop_batched(const sgl_tcsr* g, int32_t B, const int64_t* batch_ptr, int64_t S_max,
+                                 const int64_t* slot_node, const int64_t* slot_ts, const int64_t* slot_hint,
+                                 int32_t layers, int32_t Q, const sgl_sample_params* p, const sgl_hop_out* outs,
+                                 int64_t* seg, void* ws, size_t ws_bytes, void* stream) {
+    if (!g || B < 1 || !batch_ptr || S_max < 0 || layers < 1 || Q < 1 || !p || !outs || !seg)
+        return fail(SGL_EINVAL, "sample_khop_batched: bad argument");
+    const int64_t S = batch_ptr[B];
+    if (S < 0 || S > S_max) return fail(SGL_EINVAL, "sample_khop_batched: batch_ptr[B] outside [0, S_max]");
+    for (int32_t b = 0; b < B; ++b)
+        if (batch_ptr[b] < 0 || batch_ptr[b] > batch_ptr[b + 1])
+            return fail(SGL_EINVAL, "sample_khop_batched: batch_ptr does not ascend");
+    for (int32_t q = 0; q < Q; ++q) {
+        if (p[q].mark_state) return fail(SGL_EINVAL, "sample_khop_batched: mark_state is not supported");
+        if (slot_hint && !p[q].equal_root_time)
+            for (int64_t s = 0; s < S; ++s) {
+                int64_t v = slot_node[s], h = slot_hint[s];
+                if (h < 0 || v < 0 || v >= g->n) continue;
+                if (h != lower_bound_ts(g->ts, g->row_ptr[v], g->row_ptr[v + 1], slot_ts[s]))
+                    return fail(SGL_EINVAL, "sample_khop_batched: a slot_hint entry is not the window end");
+            }
+        const sgl_hop_out* oq = outs + (size_t)q * layers;
+        const int64_t* sn = slot_node; const int64_t* st = slot_ts;
+        int64_t Sl = S;
+        for (int32_t l = 0; l < layers; ++l) {
+            sgl_sample_params pl = p[q]; pl.hop = l;
+            int32_t rc = sglo_sample_hop(g, sn, st, Sl, NULL, &pl, &oq[l], ws, ws_bytes, stream);
+            if (rc != SGL_OK) return rc;
+            sn = oq[l].neighbors; st = oq[l].neighbors_ts; Sl = oq[l].counts[1];
+        }
+        int64_t* sq = seg + (size_t)q * (layers + 1) * (B + 1);
+        for (int32_t b = 0; b <= B; ++b) {
+            int64_t x = batch_ptr[b];
+            sq[b] = x;
+            for (int32_t l = 0; l < layers; ++l) {
+                x = oq[l].root_start_ptr[x];
+                sq[(size_t)(l + 1) * (B + 1) + b] = x;
+            }
+        }
+    }
+    return SGL_OK;
+}
+
 /* ----------------------------------------------------- unique / compaction */
 
 /* state layout: int64 header[3] = {epoch, id_count, universe}; then
@@ -768,6 +820,75 @@ int32_t sglo_unique_compact_hashed(void* state, int64_t capacity, int32_t reset,
     if (rc == SGL_OK && U_dev[0] == INT64_MAX) h[2] = 1;
     if (rc == SGL_OK && h[2]) U_dev[0] = INT64_MAX;      /* sticky */
     return rc;
+}
+
+/* B independent unique problems: per batch np.unique(return_inverse) over the batch's slices of the arrays
+ * (_get_unique_pairs, prepare_sample.py:205-213; Remapper::insert with a fresh epoch per batch,
+ * sample.cu.hpp:1825-1852).  State: int64 header {universe, B}. */
+size_t sglo_remap_batched_state_bytes(int64_t universe, int32_t B) {
+    if (universe <= 0 || B < 1 || B > SGL_BATCH_MAX) return 0;
+    return 2 * sizeof(int64_t);
+}
+
+int32_t sglo_remap_batched_init(void* state, size_t bytes, int64_t universe, int32_t B, void* stream) {
+    (void)stream;
+    if (!state || universe <= 0 || B < 1 || B > SGL_BATCH_MAX || bytes < 2 * sizeof(int64_t))
+        return fail(SGL_EINVAL, "remap_batched_init: bad argument");
+    ((int64_t*)state)[0] = universe; ((int64_t*)state)[1] = B;
+    return SGL_OK;
+}
+
+size_t sglo_unique_batched_workspace_bytes(int64_t universe, int32_t B) { (void)universe; (void)B; return 0; }
+
+int32_t sglo_unique_compact_batched(void* state, int64_t universe, int32_t B, int32_t G,
+                                    const int64_t* const* ids, const int64_t* len_max,
+                                    const int64_t* const* seg, int64_t* const* local_out,
+                                    int64_t* unique_out, int64_t unique_capacity, int64_t* U_off,
+                                    void* ws, size_t ws_bytes, void* stream) {
+    (void)ws; (void)ws_bytes; (void)stream;
+    if (!state || G < 1 || !ids || !len_max || !seg || !local_out || !U_off)
+        return fail(SGL_EINVAL, "unique_compact_batched: null");
+    const int64_t* h = (const int64_t*)state;
+    if (h[0] != universe || h[1] != B) return fail(SGL_EINVAL, "unique_compact_batched: universe / B differ from remap_batched_init");
+    int64_t total = 0;
+    for (int32_t g = 0; g < G; ++g) {
+        if (seg[g][B] < 0 || seg[g][B] > len_max[g]) return fail(SGL_EINVAL, "unique_compact_batched: bad live length");
+        for (int32_t b = 0; b < B; ++b)
+            if (seg[g][b] < 0 || seg[g][b] > seg[g][b + 1]) return fail(SGL_EINVAL, "unique_compact_batched: seg does not ascend");
+        total += seg[g][B];
+    }
+    int64_t* tmp = (int64_t*)malloc((size_t)(total + 1) * sizeof(int64_t));
+    if (!tmp) return fail(SGL_ENOMEM, "malloc");
+    int64_t count = 0;
+    for (int32_t b = 0; b < B; ++b) {
+        U_off[b] = count;
+        int64_t nt = 0;
+        for (int32_t g = 0; g < G; ++g)
+            for (int64_t i = seg[g][b]; i < seg[g][b + 1]; ++i) {
+                int64_t id = ids[g][i];
+                if (id >= 0 && id < universe) tmp[nt++] = id;
+            }
+        qsort(tmp, (size_t)nt, sizeof(int64_t), i64_cmp);
+        int64_t nu = 0;
+        for (int64_t i = 0; i < nt; ++i)
+            if (i == 0 || tmp[i] != tmp[i - 1]) tmp[nu++] = tmp[i];
+        if (count + nu > unique_capacity) { free(tmp); return fail(SGL_ENOMEM, "unique_out too small"); }
+        for (int64_t i = 0; i < nu; ++i) unique_out[count + i] = tmp[i];
+        for (int32_t g = 0; g < G; ++g)
+            for (int64_t i = seg[g][b]; i < seg[g][b + 1]; ++i) {
+                int64_t id = ids[g][i], loc = -1;
+                if (id >= 0 && id < universe) {
+                    int64_t lo = 0, hi = nu;
+                    while (lo < hi) { int64_t mid = (lo + hi) >> 1; if (tmp[mid] < id) lo = mid + 1; else hi = mid; }
+                    loc = lo;
+                }
+                local_out[g][i] = loc;
+            }
+        count += nu;
+    }
+    U_off[B] = count;
+    free(tmp);
+    return SGL_OK;
 }
 
 /* ------------------------------------------------------------ cache gather */

@@ -52,6 +52,8 @@ struct HopArgs {
     const int64_t* rec;  // interleaved edge records of the graph (sgl_tcsr.rec), or nullptr
     const int64_t* slot_hint;  // per explicit slot: where its window ends (the index entry of the edge the slot
                                // came from), or nullptr: search
+    int32_t hint_optional;     // 1: slot_hint comes from a caller (the root slots of a batched call) and an entry
+                               // of -1 means "search"; 0: every entry is an index entry of the graph
     int64_t* hint_out;   // per emitted edge: its index entry, for the next hop's slots; or nullptr
     const int64_t* root_hint;  // derived slots only: per positive slot, where its window ends according to the
                                // caller (sgl_sample_params.root_hint; -1: search), or nullptr
@@ -260,13 +262,14 @@ __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
         }
         const int64_t t_hi = t + (a.equal_root_time ? 1 : 0);
         int64_t hi;
-        if (a.slot_hint != nullptr) {     // kernel argument: uniform across the wave
+        if (a.slot_hint != nullptr && !a.hint_optional) {     // kernel arguments: uniform across the wave
             // the slot is (destination, time) of an edge whose index entry says where the window ends;
             // an entry of -1 belongs to a destination outside [0,n), which is a bad slot anyway
             const int64_t h = active ? a.slot_hint[slot] : 0;
             hi = clamp_to_row(h, rs, re);     // an index that does not belong to this graph cannot lead outside the row
         } else {
             // positive roots whose window end the caller knows are not searched
+            if (a.slot_hint != nullptr && active) rh = a.slot_hint[slot];     // (explicit root slots of a batched call)
             const bool told = active && rh >= 0;
             hi = group_lower_bound<G>(a.ts, rs, re, t_hi, lig, gshift, active && !told);
             if (told) hi = clamp_to_row(rh, rs, re);
@@ -1558,7 +1561,8 @@ struct RootSpec {  // hop-0 slot source of the k-hop driver
 
 int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot_ts, const RootSpec* derive,
                 int64_t S_max, const int64_t* S_dev, const sgl_sample_params* p, const sgl_hop_out* out, void* ws,
-                size_t ws_bytes, hipStream_t st, const int64_t* slot_hint = nullptr, int64_t* hint_out = nullptr) {
+                size_t ws_bytes, hipStream_t st, const int64_t* slot_hint = nullptr, int64_t* hint_out = nullptr,
+                bool hint_optional = false) {
     if (!derive && S_max > 0 && (!slot_node || !slot_ts)) return fail(SGL_EINVAL, "sample: slot array is NULL");
     if (ws_bytes < hop_workspace_bytes(S_max) || !ws)
         return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, hop_workspace_bytes(S_max));
@@ -1566,7 +1570,7 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
     HopArgs a{};
     a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint; a.rec = g->rec;
     a.slot_node = slot_node; a.slot_ts = slot_ts; a.S_max = S_max; a.S_dev = S_dev;
-    a.slot_hint = slot_hint; a.hint_out = hint_out;
+    a.slot_hint = slot_hint; a.hint_out = hint_out; a.hint_optional = hint_optional ? 1 : 0;
     a.root_hint = (derive && !p->equal_root_time) ? p->root_hint : nullptr;
     a.derive = derive ? 1 : 0;
     if (derive) {
@@ -1853,5 +1857,110 @@ extern "C" int32_t sgl_sample_khop_multi(const sgl_tcsr* g, int64_t R, const int
                                            static_cast<char*>(ws) + (size_t)q * per, per, stream);
         if (rc != SGL_OK) return rc;
     }
+    return SGL_OK;
+}
+
+// ---- sgl_sample_khop_batched: the root slots of B mini-batches sampled as one k-hop call --------------
+namespace {
+constexpr int SEG_MAX_CHAINS = 16;      // queries x layers one launch of batch_seg_kernel follows
+struct SegArgs {
+    int32_t B, layers, Q;
+    int64_t S_max;
+    const int64_t* batch_ptr;
+    const int64_t* rsp[SEG_MAX_CHAINS];      // [q * layers + l]: root_start_ptr of hop l of query q
+    int64_t cap[SEG_MAX_CHAINS];             // its capacity_slots
+    int64_t* seg;                            // [Q][layers + 1][B + 1]
+};
+// seg[q][0][b] = first root slot of batch b; seg[q][l+1][b] = root_start_ptr_l[seg[q][l][b]]: where batch b's
+// edges of hop l begin (hop l's terminating entry root_start_ptr[S_l] = E_l closes the last batch).
+__global__ void batch_seg_kernel(SegArgs a) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b > a.B) return;
+    const int64_t S = live_count(a.batch_ptr + a.B, a.S_max);
+    int64_t x0 = a.batch_ptr[b];
+    x0 = x0 < 0 ? 0 : (x0 > S ? S : x0);
+    for (int q = 0; q < a.Q; ++q) {
+        int64_t* out = a.seg + (size_t)q * (a.layers + 1) * (a.B + 1);
+        int64_t x = x0;
+        out[b] = x;
+        for (int l = 0; l < a.layers; ++l) {
+            const int64_t cap = a.cap[q * a.layers + l];        // (an index is kept inside the array whatever it holds)
+            x = a.rsp[q * a.layers + l][x < 0 ? 0 : (x > cap ? cap : x)];
+            out[(size_t)(l + 1) * (a.B + 1) + b] = x;
+        }
+    }
+}
+}  // namespace
+
+extern "C" size_t sgl_sample_khop_batched_workspace_bytes(int64_t S_max, int32_t layers, int32_t fanout, int32_t Q) {
+    return (size_t)(Q > 0 ? Q : 1) * sgl_sample_khop_workspace_bytes(S_max, layers, fanout);
+}
+
+extern "C" int32_t sgl_sample_khop_batched(const sgl_tcsr* g, int32_t B, const int64_t* batch_ptr, int64_t S_max,
+                                           const int64_t* slot_node, const int64_t* slot_ts, const int64_t* slot_hint,
+                                           int32_t layers, int32_t Q, const sgl_sample_params* p,
+                                           const sgl_hop_out* outs, int64_t* seg, void* ws, size_t ws_bytes,
+                                           void* stream) {
+    int32_t rc;
+    if ((rc = check_graph(g)) != SGL_OK) return rc;
+    if (B < 1 || !batch_ptr || S_max < 0 || layers < 1 || Q < 1 || !p || !outs || !seg)
+        return fail(SGL_EINVAL, "sample_khop_batched: bad B, S_max, layers, Q or NULL argument");
+    if (S_max > 0 && (!slot_node || !slot_ts)) return fail(SGL_EINVAL, "sample_khop_batched: slot array is NULL");
+    if ((int64_t)Q * layers > SEG_MAX_CHAINS)
+        return fail(SGL_ENOTSUP, "sample_khop_batched: Q * layers > %d", SEG_MAX_CHAINS);
+    int32_t fan = 0;
+    for (int32_t q = 0; q < Q; ++q) {
+        if ((rc = check_params(&p[q])) != SGL_OK) return rc;
+        if (p[q].mark_state) return fail(SGL_EINVAL, "sample_khop_batched: mark_state is not supported (the batches have id spaces of their own)");
+        fan = p[q].fanout > fan ? p[q].fanout : fan;
+        for (int32_t l = 0; l < layers; ++l) {
+            const int64_t s = worst_slots(S_max, l, p[q].fanout);
+            if (s == INT64_MAX) return fail(SGL_ENOTSUP, "sample_khop_batched: worst-case slot count overflows");
+            if ((rc = check_out(&outs[(size_t)q * layers + l], s, p[q].fanout)) != SGL_OK) return rc;
+        }
+    }
+    const size_t per = sgl_sample_khop_workspace_bytes(S_max, layers, fan);
+    if (!ws || ws_bytes < (size_t)Q * per)
+        return fail(SGL_ENOMEM, "sample_khop_batched: workspace %zu < %zu bytes", ws_bytes, (size_t)Q * per);
+    hipStream_t st = as_stream(stream);
+    for (int32_t q = 0; q < Q; ++q) {
+        const sgl_sample_params* pq = &p[q];
+        const sgl_hop_out* oq = outs + (size_t)q * layers;
+        char* wq = static_cast<char*>(ws) + (size_t)q * per;
+        int64_t worst = S_max;
+        for (int32_t l = 0; l < layers; ++l) worst = worst_slots(S_max, l, pq->fanout) > worst ? worst_slots(S_max, l, pq->fanout) : worst;
+        const size_t hop_ws = hop_workspace_bytes(worst);
+        // as sgl_sample_khop: with the graph's next-hop index the slots of hops >= 1 are not searched
+        const bool carry = layers > 1 && g->hop_hint != nullptr && !pq->equal_root_time &&
+                           !(pq->type == SGL_SAMPLE_UNIFORM && pq->keep_root_time) && per >= hop_ws + hint_carry_bytes(worst);
+        int64_t* carry_buf[2] = {nullptr, nullptr};
+        if (carry) {
+            carry_buf[0] = reinterpret_cast<int64_t*>(wq + hop_ws);
+            carry_buf[1] = reinterpret_cast<int64_t*>(wq + hop_ws + align_up((size_t)(worst + 1) * 8));
+        }
+        const int64_t* sn = slot_node;
+        const int64_t* stt = slot_ts;
+        const int64_t* S_dev = batch_ptr + B;
+        for (int32_t l = 0; l < layers; ++l) {
+            sgl_sample_params pl = *pq;
+            pl.hop = l;
+            const int64_t s_max = worst_slots(S_max, l, pq->fanout);
+            const int64_t* hint_in = l == 0 ? (pq->equal_root_time ? nullptr : slot_hint) : (carry ? carry_buf[(l - 1) & 1] : nullptr);
+            rc = run_hop(g, sn, stt, nullptr, s_max, S_dev, &pl, &oq[l], wq, carry ? hop_ws : per, st, hint_in,
+                         (carry && l + 1 < layers) ? carry_buf[l & 1] : nullptr, l == 0);
+            if (rc != SGL_OK) return rc;
+            sn = oq[l].neighbors;
+            stt = oq[l].neighbors_ts;
+            S_dev = oq[l].counts + 1;
+        }
+    }
+    SegArgs sa{};
+    sa.B = B; sa.layers = layers; sa.Q = Q; sa.S_max = S_max; sa.batch_ptr = batch_ptr; sa.seg = seg;
+    for (int32_t i = 0; i < Q * layers; ++i) {
+        sa.rsp[i] = outs[i].root_start_ptr;
+        sa.cap[i] = outs[i].capacity_slots;
+    }
+    hipLaunchKernelGGL(batch_seg_kernel, dim3((unsigned)ceil_div<int>(B + 1, 256)), dim3(256), 0, st, sa);
+    SGL_LAUNCH_CHECK();
     return SGL_OK;
 }

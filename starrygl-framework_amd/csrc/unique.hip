@@ -452,6 +452,180 @@ __global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a, int fo
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Batched call: B mini-batches, each with a local-id space of its own, numbered by ONE launch sequence.
+// Batch b's ids live at [b * stride, b * stride + universe) of a state over B * stride ids (stride: the
+// universe rounded up to whole tiles of flag words, so that a tile belongs to one batch); array g's
+// elements [seg[g][b], seg[g][b+1]) belong to batch b.  Ascending numbering over the big universe is
+// batch-major and ascending inside a batch: batch b's local id = global rank - U_off[b], where U_off[b]
+// is the offset of the first tile of batch b.  Every call starts a new epoch, so marking needs no table
+// read.
+constexpr int BATCH_MAX = SGL_BATCH_MAX;
+constexpr int64_t BATCH_STRIDE_ALIGN = (int64_t)TILE * 64;   // ids per tile of a bitmap state (a byte-flag tile holds TILE * 8)
+
+struct Batched {
+    int32_t B;
+    int64_t stride, universe;
+    const int64_t* seg[MAXG];
+};
+
+inline int64_t batch_stride(int64_t universe) { return ceil_div<int64_t>(universe, BATCH_STRIDE_ALIGN) * BATCH_STRIDE_ALIGN; }
+
+State carve_batched(void* state, int64_t universe, int32_t B) {
+    State s;
+    char* p = static_cast<char*>(state);
+    s.universe = (int64_t)B * batch_stride(universe);
+    s.bytes = remap_byte_flags(s.universe) ? 1 : 0;
+    s.words = ceil_div<int64_t>(s.universe, s.bytes ? 8 : 64);
+    s.hdr = reinterpret_cast<Header*>(p);
+    s.table = reinterpret_cast<uint64_t*>(p + HEADER_BYTES);
+    s.bitmap = s.table + s.universe;
+    s.planes = 1;
+    s.desc = s.bitmap + s.words;
+    return s;
+}
+
+// batch of element i of an array whose batch offsets are seg[0..B] (in LDS): the last b with seg[b] <= i
+__device__ __forceinline__ int batch_of(const int64_t* seg, int B, int64_t i) {
+    int lo = 0, hi = B;     // seg[lo] <= i < seg[hi] for a live element
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (seg[mid] <= i) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+__device__ __forceinline__ void stage_segs(const Batched& bt, int G, int64_t (*s_seg)[BATCH_MAX + 1]) {
+    for (int x = threadIdx.x; x < G * (bt.B + 1); x += blockDim.x) {
+        const int g = x / (bt.B + 1), b = x - g * (bt.B + 1);
+        s_seg[g][b] = bt.seg[g][b];
+    }
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(BLOCK) void mark_batched_kernel(State s, Arrays a, Batched bt) {
+    __shared__ int64_t s_seg[MAXG][BATCH_MAX + 1];
+    stage_segs(bt, a.G, s_seg);
+    int64_t len[MAXG], max_len = 0;
+#pragma unroll
+    for (int g = 0; g < MAXG; ++g) {
+        len[g] = 0;
+        if (g < a.G) {
+            const int64_t l = s_seg[g][bt.B];
+            len[g] = l < 0 ? 0 : (l > a.len_max[g] ? a.len_max[g] : l);
+        }
+        max_len = len[g] > max_len ? len[g] : max_len;
+    }
+    for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < max_len; i += (int64_t)gridDim.x * BLOCK) {
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) {
+            if (g < a.G && i < len[g]) {
+                const int64_t id = a.ids[g][i];
+                if (id >= 0 && id < bt.universe)
+                    remap_set_pending(s.bitmap, s.bytes, id + (int64_t)batch_of(s_seg[g], bt.B, i) * bt.stride);
+            }
+        }
+    }
+}
+
+// Numbers the set flags (tile_sum holds the exclusive tile offsets, the total at [nt]); the first tile of
+// every batch records where the batch's list begins.
+__global__ __launch_bounds__(BLOCK) void assign_batched_kernel(State s, const int64_t* tile_sum, int64_t nt, Batched bt,
+                                                               int64_t* unique_out, int64_t unique_capacity,
+                                                               int64_t* U_off, int64_t* U_dev, uint32_t* stamp_ws) {
+    __shared__ int32_t s_wave[BLOCK / WAVE];
+    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
+    uint64_t word = (w < s.words) ? s.bitmap[w] : 0ull;
+    const int32_t c = __popcll(word);
+    int32_t inc = c;
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const int32_t x = __shfl_up(inc, d);
+        if (lane >= d) inc += x;
+    }
+    if (lane == WAVE - 1) s_wave[wid] = inc;
+    __syncthreads();
+    int32_t wave_off = 0;
+    for (int q = 0; q < wid; ++q) wave_off += s_wave[q];
+    const int64_t tile_off = tile_sum[blockIdx.x];
+    const int ipw = s.bytes ? 8 : 64;                       // ids per flag word
+    const int64_t tile_id0 = (int64_t)blockIdx.x * TILE * ipw;
+    const int64_t b = tile_id0 / bt.stride;                 // the tile's batch (a stride is a whole number of tiles)
+    if (threadIdx.x == 0) {
+        if (tile_id0 == b * bt.stride) U_off[b] = tile_off;
+        if (blockIdx.x == nt - 1) {
+            const int64_t total = tile_sum[nt];
+            U_off[bt.B] = total;
+            U_dev[0] = total;
+            stamp_ws[0] = eff_stamp(s, 1);
+        }
+    }
+    if (c == 0) return;
+    int64_t local = tile_off + wave_off + (inc - c);
+    const uint64_t stamp = (uint64_t)eff_stamp(s, 1) << 32;
+    const int64_t id0 = w * ipw;
+    const int shift = s.bytes ? 3 : 0;
+    const int64_t base = b * bt.stride;
+    while (word) {
+        const int bit = __ffsll((unsigned long long)word) - 1;
+        word &= word - 1;
+        const int64_t id = id0 + (bit >> shift);
+        s.table[id] = stamp | (uint64_t)(uint32_t)local;
+        if (local < unique_capacity) unique_out[local] = id - base;
+        ++local;
+    }
+    s.bitmap[w] = 0;
+}
+
+// Rewrites every array through the table, batch by batch (local id = global rank - start of the batch's list),
+// and commits the epoch.
+__global__ __launch_bounds__(BLOCK) void lookup_batched_kernel(State s, Arrays a, Batched bt, const int64_t* U_off,
+                                                               const uint32_t* stamp_ws, int64_t* U_dev) {
+    __shared__ int64_t s_seg[MAXG][BATCH_MAX + 1];
+    __shared__ int64_t s_uoff[BATCH_MAX + 1];
+    for (int x = threadIdx.x; x <= bt.B; x += BLOCK) s_uoff[x] = U_off[x];
+    stage_segs(bt, a.G, s_seg);
+    const uint32_t stamp = stamp_ws[0];
+    if (blockIdx.x == 0 && threadIdx.x == 0) commit(s, 1, 1, 1, U_dev);
+    int64_t len[MAXG], max_len = 0;
+#pragma unroll
+    for (int g = 0; g < MAXG; ++g) {
+        len[g] = 0;
+        if (g < a.G) {
+            const int64_t l = s_seg[g][bt.B];
+            len[g] = l < 0 ? 0 : (l > a.len_max[g] ? a.len_max[g] : l);
+        }
+        max_len = len[g] > max_len ? len[g] : max_len;
+    }
+    for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < max_len; i += (int64_t)gridDim.x * BLOCK) {
+        int64_t id[MAXG];
+        int bb[MAXG];
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g) {
+            id[g] = -1;
+            bb[g] = 0;
+            if (g < a.G && i < len[g]) {
+                id[g] = a.ids[g][i];       // ids may alias out
+                bb[g] = batch_of(s_seg[g], bt.B, i);
+            }
+        }
+        uint64_t e[MAXG];
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g)
+            e[g] = (id[g] >= 0 && id[g] < bt.universe) ? s.table[id[g] + (int64_t)bb[g] * bt.stride] : 0ull;
+#pragma unroll
+        for (int g = 0; g < MAXG; ++g)
+            if (g < a.G && i < len[g])
+                a.out[g][i] = ((uint32_t)(e[g] >> 32) == stamp) ? (int64_t)(e[g] & 0xFFFFFFFFull) - s_uoff[bb[g]] : -1;
+    }
+}
+
+size_t batched_workspace_bytes(int64_t universe, int32_t B) {
+    const int64_t big = (int64_t)B * batch_stride(universe);
+    const int64_t words = ceil_div<int64_t>(big, remap_byte_flags(big) ? 8 : 64);
+    return align_up((size_t)(ceil_div<int64_t>(words, TILE) + 2) * 8) + align_up(16) + align_up(16) + 512;
+}
+
 size_t dense_workspace_bytes(int64_t universe) {
     const int64_t words = ceil_div<int64_t>(universe, remap_byte_flags(universe) ? 8 : 64);
     return align_up((size_t)(MAXG * ceil_div<int64_t>(words, TILE) + 2) * 8) + 512;
@@ -620,5 +794,93 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
                            stamp_ws, U_dev);
         SGL_LAUNCH_CHECK();
     }
+    return SGL_OK;
+}
+
+// ---- batched: B mini-batches with local-id spaces of their own in one launch sequence ------------------
+extern "C" size_t sgl_remap_batched_state_bytes(int64_t universe, int32_t B) {
+    if (universe <= 0 || B < 1 || B > BATCH_MAX) return 0;
+    const int64_t big = (int64_t)B * batch_stride(universe);
+    const int64_t words = ceil_div<int64_t>(big, remap_byte_flags(big) ? 8 : 64);
+    return HEADER_BYTES + (size_t)big * 8 + (size_t)words * 8 + (size_t)ceil_div<int64_t>(words, TILE) * 8 + 8;
+}
+
+extern "C" int32_t sgl_remap_batched_init(void* state, size_t state_bytes, int64_t universe, int32_t B, void* stream) {
+    if (!state || universe <= 0) return fail(SGL_EINVAL, "remap_batched_init: state is NULL or universe <= 0");
+    if (B < 1 || B > BATCH_MAX) return fail(SGL_ENOTSUP, "remap_batched_init: B must be 1..%d", BATCH_MAX);
+    if ((int64_t)B * batch_stride(universe) > 0xFFFFFFFFll) return fail(SGL_ENOTSUP, "remap_batched_init: B * universe > 2^32");
+    if (state_bytes < sgl_remap_batched_state_bytes(universe, B))
+        return fail(SGL_ENOMEM, "remap_batched_init: state %zu < %zu bytes", state_bytes, sgl_remap_batched_state_bytes(universe, B));
+    if (reinterpret_cast<uintptr_t>(state) % 8) return fail(SGL_EINVAL, "remap_batched_init: state must be 8-byte aligned");
+    State s = carve_batched(state, universe, B);
+    int64_t blocks = ceil_div<int64_t>(s.universe, 256);
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(init_state_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), s);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}
+
+extern "C" size_t sgl_unique_batched_workspace_bytes(int64_t universe, int32_t B) {
+    if (universe <= 0 || B < 1 || B > BATCH_MAX) return 512;
+    return batched_workspace_bytes(universe, B);
+}
+
+extern "C" int32_t sgl_unique_compact_batched(void* state, int64_t universe, int32_t B, int32_t G,
+                                              const int64_t* const* ids, const int64_t* len_max,
+                                              const int64_t* const* seg, int64_t* const* local_out,
+                                              int64_t* unique_out, int64_t unique_capacity, int64_t* U_off,
+                                              void* ws, size_t ws_bytes, void* stream) {
+    if (!state || G < 1 || !ids || !len_max || !seg || !local_out || !U_off)
+        return fail(SGL_EINVAL, "unique_compact_batched: NULL argument or G < 1");
+    if (universe <= 0 || B < 1 || B > BATCH_MAX || (int64_t)B * batch_stride(universe) > 0xFFFFFFFFll)
+        return fail(SGL_EINVAL, "unique_compact_batched: bad universe or B (1..%d)", BATCH_MAX);
+    if (G > MAXG) return fail(SGL_ENOTSUP, "unique_compact_batched: more than %d arrays", MAXG);
+    if (unique_capacity < 0 || (unique_capacity > 0 && !unique_out))
+        return fail(SGL_EINVAL, "unique_compact_batched: unique_out is NULL");
+    if (!ws || ws_bytes < batched_workspace_bytes(universe, B))
+        return fail(SGL_ENOMEM, "unique_compact_batched: workspace %zu < %zu bytes", ws_bytes, batched_workspace_bytes(universe, B));
+    Arrays all;
+    all.G = G;
+    all.start[0] = 0;
+    Batched bt;
+    bt.B = B; bt.universe = universe; bt.stride = batch_stride(universe);
+    int64_t longest = 0;
+    for (int g = 0; g < MAXG; ++g) {
+        const bool live = g < G;
+        if (live && (len_max[g] < 0 || !seg[g] || (len_max[g] > 0 && (!ids[g] || !local_out[g]))))
+            return fail(SGL_EINVAL, "unique_compact_batched: array %d: negative length or NULL pointer", g);
+        all.ids[g] = live ? ids[g] : nullptr;
+        all.out[g] = live ? local_out[g] : nullptr;
+        all.len_dev[g] = nullptr;
+        all.len_max[g] = live ? len_max[g] : 0;
+        all.start[g + 1] = all.start[g] + all.len_max[g];
+        bt.seg[g] = live ? seg[g] : nullptr;
+        longest = all.len_max[g] > longest ? all.len_max[g] : longest;
+    }
+    if (ceil_div<int64_t>(all.start[MAXG], BLOCK) > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "unique_compact_batched: too many ids");
+    hipStream_t st = as_stream(stream);
+    State s = carve_batched(state, universe, B);
+    Arena ar(ws, ws_bytes);
+    const int64_t nt = ceil_div<int64_t>(s.words, TILE);
+    int64_t* tile_sum = ar.take<int64_t>(nt + 2);
+    uint32_t* stamp_ws = ar.take<uint32_t>(4);
+    int64_t* U_dev = ar.take<int64_t>(2);
+    if (!ar.ok()) return fail(SGL_ENOMEM, "unique_compact_batched: workspace too small");
+    int64_t mb = ceil_div<int64_t>(longest > 0 ? longest : 1, BLOCK);
+    if (mb > MAX_GRID) mb = MAX_GRID;
+    if (longest > 0) {
+        hipLaunchKernelGGL(mark_batched_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, all, bt);
+        SGL_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
+    SGL_LAUNCH_CHECK();
+    hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, tile_sum, nt);
+    SGL_LAUNCH_CHECK();
+    hipLaunchKernelGGL(assign_batched_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, bt, unique_out,
+                       unique_capacity, U_off, U_dev, stamp_ws);
+    SGL_LAUNCH_CHECK();
+    // (always launched: thread 0 of block 0 commits the epoch)
+    hipLaunchKernelGGL(lookup_batched_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, all, bt, U_off, stamp_ws, U_dev);
+    SGL_LAUNCH_CHECK();
     return SGL_OK;
 }

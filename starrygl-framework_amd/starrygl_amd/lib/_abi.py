@@ -5,12 +5,13 @@ header declares.  The product library exports them as ``sgl_*``.
 """
 import ctypes as C
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
 UNIFORM_MAX_FANOUT = 1024
 STATIC_HOP_MAX_SLOTS = 65536
+BATCH_MAX = 64
 UNIQUE_SORTED, UNIQUE_GROUPED, UNIQUE_PREMARKED, UNIQUE_MULTI_LAUNCH = 0, 1, 0x100, 0x200
 SAMPLE_MULTI_LAUNCH = 1
 DT_I64, DT_F32 = 0, 1
@@ -90,6 +91,8 @@ PROTOTYPES = {
     "sample_khop_multi_workspace_bytes": (sz, [i64, i32, i32, i32]),
     "sample_khop_multi": (i32, [P(TCSR), i64, vp, vp, i64, vp, i64, vp, vp, i32, i32,
                                 P(SampleParams), vp, vp, P(HopOut), vp, sz, vp]),
+    "sample_khop_batched_workspace_bytes": (sz, [i64, i32, i32, i32]),
+    "sample_khop_batched": (i32, [P(TCSR), i32, vp, i64, vp, vp, vp, i32, i32, P(SampleParams), P(HopOut), vp, vp, sz, vp]),
     "remap_state_bytes": (sz, [i64]),
     "remap_init": (i32, [vp, sz, i64, vp]),
     "unique_workspace_bytes": (sz, [i64, i32, P(i64)]),
@@ -100,6 +103,10 @@ PROTOTYPES = {
     "unique_hashed_workspace_bytes": (sz, [i64, i32, P(i64)]),
     "unique_compact_hashed": (i32, [vp, i64, i32, i32, i32, P(vp), P(i64), P(vp), P(vp),
                                     vp, i64, vp, vp, sz, vp]),
+    "remap_batched_state_bytes": (sz, [i64, i32]),
+    "remap_batched_init": (i32, [vp, sz, i64, i32, vp]),
+    "unique_batched_workspace_bytes": (sz, [i64, i32]),
+    "unique_compact_batched": (i32, [vp, i64, i32, i32, P(vp), P(i64), P(vp), P(vp), vp, i64, vp, vp, sz, vp]),
     "gather": (i32, [P(Cache), vp, i64, vp, vp, vp, vp, vp]),
     "gather_multi": (i32, [i32, P(GatherSeg), vp]),
     "scatter_update": (i32, [P(Cache), vp, vp, vp, vp, vp, i64, vp, vp, vp]),

@@ -441,6 +441,96 @@ class HotPath:
             res.slot_node0, res.slot_ts0, res.S0_live = head.slot_node0, head.slot_ts0, S0
         return outs
 
+    # ---------------------------------------------- several batches per call
+    def khop_batched_buffers(self, S_max, B, layers, fanout, Q=1, counts=None):
+        """Worst-case output buffers of `sample_khop_batched` for Q queries over up to S_max root slots in
+        B batches; reusable across calls.  `counts` (int64[Q * 3 * layers], zeroed) may be the caller's."""
+        be = self.be
+        if counts is None:
+            counts = be.zeros(Q * 3 * max(layers, 1))
+        queries = []
+        for q in range(Q):
+            outs, cap = [], S_max
+            cq = counts[q * 3 * layers: (q + 1) * 3 * layers]
+            for l in range(layers):
+                outs.append(HopResult(be, cap, cap * fanout, cq[3 * l: 3 * l + 3]))
+                cap *= fanout
+            r = KHopResult(self, None, None, outs, cq)
+            r.S0, r.fanout = S_max, fanout
+            queries.append(r)
+        res = KHopBatched(self, queries, B, S_max, layers, fanout, counts)
+        res.seg = be.zeros((Q, layers + 1, B + 1))
+        res.structs = (HopOut * max(Q * layers, 1))(*[o.struct for r in queries for o in r.hops])
+        res.ws_bytes = int(self.lib.sample_khop_batched_workspace_bytes(S_max, layers, fanout, Q))
+        res.ws = be.empty(max(res.ws_bytes, 256), "u8")
+        return res
+
+    def sample_khop_batched(self, g, slot_node, slot_ts, batch_ptr, layers, params, out=None, slot_hint=None,
+                            finalize=False):
+        """The root slots of B mini-batches (slot_node/slot_ts, batch b owning [batch_ptr[b], batch_ptr[b+1]);
+        batch_ptr: device int64[B+1]) sampled by one k-hop call per entry of `params`; -> KHopBatched whose
+        `seg[q, l+1]` says where each batch's edges of hop l begin.  slot_hint: window ends of the slots
+        (`window_end`; -1 = search)."""
+        self._chk("i64", slot_node=slot_node, slot_ts=slot_ts, batch_ptr=batch_ptr, slot_hint=slot_hint)
+        be, Q = self.be, len(params)
+        S_max, B = int(slot_node.shape[0]), int(batch_ptr.shape[0]) - 1
+        if int(slot_ts.shape[0]) != S_max or (slot_hint is not None and int(slot_hint.shape[0]) < S_max):
+            raise ValueError("sample_khop_batched: slot_node, slot_ts and slot_hint differ in length")
+        fan = max(p.fanout for p in params)
+        res = out if out is not None else self.khop_batched_buffers(S_max, B, layers, fan, Q)
+        if res.S_max < S_max or res.B != B or res.layers != layers or res.fanout < fan or len(res.queries) != Q:
+            raise MemoryError("khop batched buffers do not fit this call")
+        pa = (_abi.SampleParams * Q)(*params)
+        self._ck(self.lib.sample_khop_batched(C.byref(g.view), B, be.ptr(batch_ptr), S_max, be.ptr(slot_node),
+                                              be.ptr(slot_ts), be.ptr(slot_hint), layers, Q, pa, res.structs,
+                                              be.ptr(res.seg), be.ptr(res.ws), be.nbytes(res.ws), be.stream()))
+        res.slot_node, res.slot_ts, res.batch_ptr = slot_node, slot_ts, batch_ptr
+        res.final = False
+        for r in res.queries:
+            r.slot_node0, r.slot_ts0, r.final = slot_node, slot_ts, False
+        return res.finalize() if finalize else res
+
+    def remap_batched_state(self, universe, B):
+        """Remap state for `unique_compact_batched`: B copies of the id universe [0, universe)."""
+        nbytes = int(self.lib.remap_batched_state_bytes(universe, B))
+        if nbytes == 0:
+            raise ValueError(f"remap_batched_state: universe must be positive and B in 1..{_abi.BATCH_MAX}")
+        st = self.be.empty(max(nbytes, 8), "u8")
+        self._ck(self.lib.remap_batched_init(self.be.ptr(st), nbytes, universe, B, self.be.stream()))
+        rs = RemapState(st, universe)
+        rs.B = int(B)
+        return rs
+
+    def unique_compact_batched(self, arrays, segs, state, out_arrays=None, unique_out=None, U_off=None,
+                               workspace=None, finalize=True):
+        """Per batch np.unique(return_inverse) over the batch's slices of `arrays` (segs[g]: device int64[B+1]
+        offsets of array g, segs[g][B] = its live length).  -> (local arrays, unique_out, U_off) where batch
+        b's distinct ids are unique_out[U_off[b]: U_off[b+1]]; finalize reads U_off on the host and narrows."""
+        self._chk("i64", **{f"arrays[{i}]": a for i, a in enumerate(arrays)})
+        self._chk("i64", **{f"segs[{i}]": a for i, a in enumerate(segs)})
+        be, G, B = self.be, len(arrays), state.B
+        if len(segs) != G or any(int(sg.shape[0]) != B + 1 for sg in segs):
+            raise ValueError("unique_compact_batched: one segment table of B + 1 entries per array")
+        len_max = (i64 * max(G, 1))(*[int(a.shape[0]) for a in arrays])
+        ids = (vp * max(G, 1))(*[be.ptr(a) for a in arrays])
+        sg = (vp * max(G, 1))(*[be.ptr(a) for a in segs])
+        if out_arrays is None:
+            out_arrays = [be.empty(int(a.shape[0])) for a in arrays]
+        outs = (vp * max(G, 1))(*[be.ptr(a) for a in out_arrays])
+        if unique_out is None:
+            unique_out = be.empty(max(min(sum(len_max[:G]), B * state.universe), 1))
+        if U_off is None:
+            U_off = be.zeros(B + 1)
+        need = int(self.lib.unique_batched_workspace_bytes(state.universe, B))
+        ws, wsb = (workspace, be.nbytes(workspace)) if workspace is not None else self._workspace(need)
+        self._ck(self.lib.unique_compact_batched(be.ptr(state.buf), state.universe, B, G, ids, len_max, sg, outs,
+                                                 be.ptr(unique_out), int(unique_out.shape[0]), be.ptr(U_off),
+                                                 be.ptr(ws), wsb, be.stream()))
+        if not finalize:
+            return out_arrays, unique_out, U_off
+        off = be.tolist(U_off)
+        return out_arrays, unique_out[: off[B]], off
+
     # ------------------------------------------------------------- unique
     def remap_state(self, universe):
         nbytes = self.lib.remap_state_bytes(universe)
@@ -754,3 +844,32 @@ class KHopResult:
                 self.slot_node0, self.slot_ts0 = self.slot_node0[:S0], self.slot_ts0[:S0]
             self.final = True
         return self
+
+
+class KHopBatched:
+    """Result of `HotPath.sample_khop_batched`: `queries[q]` is a KHopResult over all batches' slots;
+    `seg[q, l]` (device, B + 1 entries) delimits the batches in the slots of hop l (= the edges of hop l - 1)."""
+
+    def __init__(self, hp, queries, B, S_max, layers, fanout, counts):
+        self.hp, self.queries, self.B, self.S_max, self.layers, self.fanout = hp, queries, B, S_max, layers, fanout
+        self.counts, self.final, self.seg_host = counts, False, None
+
+    def finalize(self):
+        """One synchronising read of the segment table and the counts; narrows every query's arrays."""
+        if not self.final:
+            be = self.hp.be
+            self.seg_host = be.tolist(self.seg)
+            c = be.tolist(self.counts)
+            L = self.layers
+            S = self.seg_host[0][0][self.B]
+            for q, r in enumerate(self.queries):
+                r.S0_live = S
+                r.finalize(c[q * 3 * L: (q + 1) * 3 * L])
+            self.final = True
+        return self
+
+    def batch(self, q, b):
+        """Batch b of query q: [(slot range), (edge range of hop 0), ...] as python ints (after finalize)."""
+        self.finalize()
+        sg = self.seg_host[q]
+        return [(sg[l][b], sg[l][b + 1]) for l in range(self.layers + 1)]
