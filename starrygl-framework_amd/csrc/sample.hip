@@ -84,7 +84,7 @@ struct HopArgs {
     int64_t mark_universe;
     int32_t mark_bytes;  // 1: a flag byte per id, 0: a bit per id
     // workspace
-    int64_t* w_start;    // [S_max] first candidate position (recent: first copied edge)
+    int64_t* w_start;    // [S_max] first candidate position (the window's first edge, whatever the strategy)
     int64_t* w_len;      // [S_max] window length
     int64_t* block_sum;  // [gridDim] edges counted by each block
     int32_t* block_bad;  // [gridDim] out-of-range slots seen by each block
@@ -280,7 +280,7 @@ __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
         const int64_t len = hi - lo;
         const int32_t c = (int32_t)(len < a.k ? len : a.k);
         if (lig == 0 && slot < S) {
-            a.w_start[slot] = (a.type == SGL_SAMPLE_RECENT) ? hi - c : lo;
+            a.w_start[slot] = lo;
             a.w_len[slot] = active ? len : 0;
             if (a.derive) {
                 a.slot_node_out[slot] = v;
@@ -470,8 +470,11 @@ __device__ __forceinline__ void floyd_subset(bool draw, int lig, int wlane, int 
     }
 }
 
+// Uniform picks with a wavefront per slot, for fanouts beyond 32 (G = WAVE is the only instantiation; smaller
+// fanouts take fill_uniform_flat_kernel): the block walks its run one iteration's slots at a time.
 template <int G>
 __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
+    static_assert(G == WAVE, "a wavefront per slot");
     constexpr int SPB = BLOCK / G;
     __shared__ int64_t s_red[NWAVE];
     __shared__ int32_t s_redb[NWAVE];
@@ -481,14 +484,9 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
     const int gshift = wlane / G * G;
     const int32_t k = a.k;
-    // With a group of lanes per slot each of the block's waves gets a stretch of the run of its own (below): the waves
-    // spend their time on draws and scattered picks and gain from running apart (857k slots of 20 picks: 647 -> 590 us).
-    // With a wavefront per slot the whole block walks the run, one iteration's slots at a time (the subset
-    // construction in LDS needs block barriers).
-    constexpr bool WAVE_RUNS = G != WAVE;
-    // (whole-block walk) first iteration's slot data: loaded before the live count arrives when the grid is
+    // first iteration's slot data: loaded before the live count arrives when the grid is
     // not capped (see count_kernel), and before the prefix sum, so the loads overlap both
-    const bool fixed = !WAVE_RUNS && a.align == SPB && (int64_t)gridDim.x * SPB >= a.S_max;
+    const bool fixed = a.align == SPB && (int64_t)gridDim.x * SPB >= a.S_max;
     int64_t slot = (int64_t)blockIdx.x * SPB + gib;
     int64_t start = 0, len = 0, t = 0;
     if (fixed && slot < a.S_max) {
@@ -500,7 +498,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
     int64_t first, run;
     block_run(S, a.align, &first, &run);
     bool active = first < S && first + gib < S;
-    if (!fixed && !WAVE_RUNS) {
+    if (!fixed) {
         slot = first + gib;
         if (active) {
             start = a.w_start[slot];
@@ -509,33 +507,6 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
         }
     }
     if (!active) start = len = t = 0;   // speculative loads of slots beyond the live count
-    // (a stretch per wave) the wave's stretch, its first slots and the edges of the stretch: loaded before the
-    // block's offset is worked out, so that the latencies run side by side
-    int64_t wfirst = 0, wend = 0;
-    if constexpr (WAVE_RUNS) {
-        constexpr int SPW = WAVE / G;
-        int64_t rw = ceil_div<int64_t>(run, (int64_t)NWAVE);
-        rw = ceil_div<int64_t>(rw, (int64_t)SPW) * SPW;
-        const int64_t run_end = first + run < S ? first + run : S;
-        wfirst = first + (int64_t)wid * rw;
-        if (wfirst > run_end) wfirst = run_end;
-        wend = wfirst + rw < run_end ? wfirst + rw : run_end;
-        slot = wfirst + wlane / G;
-        active = slot < wend;
-        start = len = t = 0;
-        if (active) {
-            start = a.w_start[slot];
-            len = a.w_len[slot];
-            t = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
-        }
-        int32_t wsum = 0;
-        for (int64_t j = wfirst + wlane; j < wend; j += WAVE) {
-            const int64_t l = a.w_len[j];
-            wsum += (int32_t)(l < k ? l : k);
-        }
-        for (int d = WAVE / 2; d > 0; d >>= 1) wsum += __shfl(wsum, wlane ^ d);
-        if (wlane == 0) s_wtot[0][wid] = wsum;
-    }
     // exclusive prefix of this block: read it (scan_kernel ran) or add up the sums of
     // the blocks before it
     int64_t run_off = 0;
@@ -665,101 +636,6 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
                 }
             }
     };
-    // A stretch of the run per wave: a wave adds up the edges of its stretch, one barrier hands every wave the edges
-    // of the waves before it, and from there on the waves run without barriers (a slot's offset is a prefix inside
-    // its wave), each loading its next slots while it copies the current ones.
-    if constexpr (WAVE_RUNS) {
-        constexpr int SPW = WAVE / G;
-        const int gw = wlane / G;
-        __syncthreads();                 // the waves' edge totals are in s_wtot[0]
-        int64_t wave_off = run_off;
-#pragma unroll
-        for (int q = 0; q < NWAVE; ++q)
-            if (q < wid) wave_off += s_wtot[0][q];
-        // Two iterations' slots per trip: the draws of both are made, then the picked edges of both are loaded,
-        // then both are stored - twice the loads in flight per wave, and the prefix work is shared.
-        auto load_slot_of = [&](int64_t sl, bool on, int64_t* st_, int64_t* ln_, int64_t* t_) {
-            *st_ = *ln_ = *t_ = 0;
-            if (on) {
-                *st_ = a.w_start[sl];
-                *ln_ = a.w_len[sl];
-                *t_ = a.derive ? a.slot_ts_out[sl] : a.slot_ts[sl];
-            }
-        };
-        // the pick of this lane for its slot: position inside the window and output place
-        auto choose = [&](int64_t sl, bool on, int64_t ln_, int64_t* sel, int32_t* rank) {
-            const bool draw = on && ln_ > k;
-            *sel = lig;
-            *rank = lig;
-            if (__any(draw)) {                    // wave-uniform
-                int64_t tj = 0;
-                if (draw && lig < k) {
-                    const uint64_t bits = draw_bits(a.seed, a.hop, sl, lig);
-                    tj = a.replace ? bounded(bits, ln_) : bounded(bits, ln_ - k + lig + 1);
-                }
-                if (a.replace) {
-                    if (draw) *sel = tj;
-                } else {
-                    floyd_subset<G>(draw, lig, wlane, gshift, k, ln_, tj, sel, rank);
-                }
-            }
-        };
-        auto store = [&](bool on, int64_t t_, int64_t o, const Edge& ed) {
-            if (!on) return;
-            a.nbr[o] = ed.col;
-            if (a.mark != nullptr) mark_id(a, ed.col);
-            a.nbr_ts[o] = a.keep_root_time ? t_ : ed.ts;
-            a.nbr_eid[o] = ed.eid;
-            a.nbr_dt[o] = ed.ts - t_;
-            if (a.hint_out != nullptr) a.hint_out[o] = ed.hint;
-        };
-        int64_t slot_b = slot + SPW, start_b, len_b, t_b;
-        bool active_b = slot_b < wend;
-        load_slot_of(slot_b, active_b, &start_b, &len_b, &t_b);
-        for (int64_t it = wfirst; it < wend; it += 2 * SPW) {
-            // the next trip's slots are loaded now, so that their latency runs beside this trip's draws and picks
-            const int64_t nslot = it + 2 * SPW + gw, nslot_b = nslot + SPW;
-            const bool nactive = nslot < wend, nactive_b = nslot_b < wend;
-            int64_t nstart, nlen, nt, nstart_b, nlen_b, nt_b;
-            load_slot_of(nslot, nactive, &nstart, &nlen, &nt);
-            load_slot_of(nslot_b, nactive_b, &nstart_b, &nlen_b, &nt_b);
-            const int32_t c = (int32_t)(len < k ? len : k), c_b = (int32_t)(len_b < k ? len_b : k);
-            // exclusive prefix over the trip's slots: the first iteration's groups, then the second's
-            int32_t inc = (lig == 0) ? c : 0, inc_b = (lig == 0) ? c_b : 0;
-            for (int d = 1; d < WAVE; d <<= 1) {
-                const int32_t x = __shfl_up(inc, d), y = __shfl_up(inc_b, d);
-                if (wlane >= d) {
-                    inc += x;
-                    inc_b += y;
-                }
-            }
-            const int32_t total_a = __shfl(inc, WAVE - 1), total_b = __shfl(inc_b, WAVE - 1);
-            const int64_t off = wave_off + __shfl(inc - ((lig == 0) ? c : 0), wlane - lig);
-            const int64_t off_b = wave_off + total_a + __shfl(inc_b - ((lig == 0) ? c_b : 0), wlane - lig);
-            int64_t sel, sel_b;
-            int32_t rank, rank_b;
-            choose(slot, active, len, &sel, &rank);
-            choose(slot_b, active_b, len_b, &sel_b, &rank_b);
-            const bool on = active && lig < c, on_b = active_b && lig < c_b;
-            Edge ed{}, ed_b{};
-            if (on) ed = load_picked_edge(a, start + sel);
-            if (on_b) ed_b = load_picked_edge(a, start_b + sel_b);
-            if (active && lig == 0) {
-                a.root_start_ptr[slot] = off;
-                a.root_end_ptr[slot] = off + c;
-            }
-            if (active_b && lig == 0) {
-                a.root_start_ptr[slot_b] = off_b;
-                a.root_end_ptr[slot_b] = off_b + c_b;
-            }
-            store(on, t, off + rank, ed);
-            store(on_b, t_b, off_b + rank_b, ed_b);
-            wave_off += total_a + total_b;
-            slot = nslot; active = nactive; start = nstart; len = nlen; t = nt;
-            slot_b = nslot_b; active_b = nactive_b; start_b = nstart_b; len_b = nlen_b; t_b = nt_b;
-        }
-        return;
-    }
     int par = 0;
     for (int64_t it = first; it < first + run && it < S; it += SPB, par ^= 1) {
         // the next iteration's slot is loaded now, so that its latency runs beside this iteration's picks and copies
@@ -817,6 +693,10 @@ __global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
     __shared__ int64_t s_start[FLAT_SLOTS], s_t[FLAT_SLOTS];
     const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
     const int32_t k = a.k;
+    // Runs of up to 16 edges come from the graph's interleaved records when it has them: a run then lies in one
+    // stretch of memory instead of one per array (slots of a deeper hop hold a few edges: three 64-byte sectors for
+    // 16 useful bytes each become one or two); longer runs read fewer bytes from the arrays.
+    const bool use_rec = a.rec != nullptr && k <= 16;
     const int64_t S = live_count(a.S_dev, a.S_max);
     int64_t first, run;
     block_run(S, a.align, &first, &run);
@@ -830,8 +710,8 @@ __global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
             const int64_t slot = chunk0 + SPT * threadIdx.x + q;
             st[q] = ln[q] = tt[q] = 0;
             if (slot < run_end) {
-                st[q] = a.w_start[slot];
                 ln[q] = a.w_len[slot];
+                st[q] = a.w_start[slot] + (ln[q] > k ? ln[q] - k : 0);       // the last min(len, k) edges of the window
                 tt[q] = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
             }
         }
@@ -932,10 +812,15 @@ __global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
                         lo += s_off[lo + step] <= x ? step : 0;
                     const int64_t e = s_start[lo] + (x - s_off[lo]);
                     tslot[r] = s_t[lo];
-                    ets[r] = a.ts[e];
-                    dst[r] = a.col[e];
-                    id[r] = a.eid[e];
-                    if (a.hint_out != nullptr) hnt[r] = a.hint[e];
+                    if (use_rec) {       // kernel argument: uniform across the launch
+                        const Edge ed = load_picked_edge(a, e);
+                        ets[r] = ed.ts; dst[r] = ed.col; id[r] = ed.eid; hnt[r] = ed.hint;
+                    } else {
+                        ets[r] = a.ts[e];
+                        dst[r] = a.col[e];
+                        id[r] = a.eid[e];
+                        if (a.hint_out != nullptr) hnt[r] = a.hint[e];
+                    }
                 }
             }
 #pragma unroll
@@ -949,6 +834,268 @@ __global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
                     a.nbr_eid[o] = id[r];
                     a.nbr_dt[o] = ets[r] - tslot[r];
                     if (a.hint_out != nullptr) a.hint_out[o] = hnt[r];
+                }
+            }
+        }
+        run_off += total;
+    }
+}
+
+// Uniform picks with a lane per PICK.  As fill_flat_kernel a block takes its run in chunks of SLOTS slots and walks
+// the chunk's output edges flat; what differs is where an edge comes from.  A slot whose window holds at most k edges
+// copies it whole.  For the others ("drawing" slots, listed compactly in LDS) the block first makes the k raw draws
+// of every such slot, one (slot, draw) pair per lane - the generator is most of the cost, and with a group of lanes
+// per slot the lanes of slots that do not draw (most slots of a deeper hop hold a handful of edges) idle through it
+// - then a group of KP lanes turns a slot's draws into its ascending picks in place: rank = number of smaller draws;
+// only when two draws of the slot are equal does one lane replay Floyd's construction (step j keeps its draw
+// unless an earlier step holds that value, then it takes len - k + j).  Picks are kept as 32-bit offsets into the
+// window; a window of 2^32 edges or more (no row of a graph this library can hold today) is picked lane by lane.
+// The k picks of one slot whose window has 2^32 edges or more, by one lane, into `row` (global memory: the slot's
+// own k entries of an output array, which the copy that follows overwrites): Floyd's construction and an insertion
+// sort, or the draws in their order when drawing with replacement.
+__device__ __forceinline__ void huge_window_picks(const HopArgs& a, int64_t slot, int64_t len, int64_t* row) {
+    const int32_t k = a.k;
+    for (int32_t j = 0; j < k; ++j) {
+        const uint64_t bits = draw_bits(a.seed, a.hop, slot, j);
+        int64_t pj = a.replace ? bounded(bits, len) : bounded(bits, len - k + j + 1);
+        if (!a.replace) {
+            bool dup = false;
+            for (int32_t i = 0; i < j; ++i) dup |= row[i] == pj;
+            if (dup) pj = len - k + j;
+        }
+        row[j] = pj;
+    }
+    if (a.replace) return;
+    for (int32_t x = 1; x < k; ++x) {
+        const int64_t v = row[x];
+        int32_t y = x - 1;
+        while (y >= 0 && row[y] > v) {
+            row[y + 1] = row[y];
+            --y;
+        }
+        row[y + 1] = v;
+    }
+}
+
+template <int KP, int SLOTS>
+__global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
+    static_assert(SLOTS % BLOCK == 0 && BLOCK % KP == 0 && KP % 4 == 0 && KP < WAVE, "chunk layout");
+    constexpr int SPT = SLOTS / BLOCK;
+    __shared__ int64_t s_red[NWAVE];
+    __shared__ int32_t s_redb[NWAVE];
+    __shared__ int32_t s_w[NWAVE];
+    __shared__ int32_t s_off[SLOTS + 1];
+    __shared__ int64_t s_start[SLOTS], s_t[SLOTS], s_len[SLOTS];
+    __shared__ int32_t s_dl[SLOTS];          // chunk-local index of the q-th drawing slot
+    __shared__ int32_t s_didx[SLOTS];        // slot -> its place in s_dl, -1: copies its window, -2: window >= 2^32 edges
+    __shared__ __attribute__((aligned(16))) uint32_t s_pick[SLOTS * KP];
+    const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    const int32_t k = a.k;
+    const int64_t S = live_count(a.S_dev, a.S_max);
+    int64_t first, run;
+    block_run(S, a.align, &first, &run);
+    const int64_t run_end = first + run < S ? first + run : S;
+    int64_t st[SPT], ln[SPT], tt[SPT];
+    auto load_slots = [&](int64_t chunk0) {
+#pragma unroll
+        for (int q = 0; q < SPT; ++q) {
+            const int64_t slot = chunk0 + SPT * threadIdx.x + q;
+            st[q] = ln[q] = tt[q] = 0;
+            if (slot < run_end) {
+                st[q] = a.w_start[slot];
+                ln[q] = a.w_len[slot];
+                tt[q] = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
+            }
+        }
+    };
+    load_slots(first);
+    int64_t run_off = 0;
+    if (a.scanned) {
+        constexpr int CH = MAX_BLOCKS / SCAN_BLOCK;
+        const int c0 = (int)blockIdx.x / CH * CH;
+        run_off = a.chunk_off[blockIdx.x / CH];
+#pragma unroll
+        for (int q = 0; q < CH - 1; ++q)
+            if (c0 + q < (int)blockIdx.x) run_off += a.block_sum[c0 + q];
+    } else {
+        int64_t part = 0;
+        int32_t partb = 0;
+        const bool last = blockIdx.x == gridDim.x - 1;
+        for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += BLOCK) {
+            part += a.block_sum[b];
+            if (last) partb += a.block_bad[b];
+        }
+        for (int d = WAVE / 2; d > 0; d >>= 1) {
+            part += shfl_i64(part, wlane ^ d);
+            partb += __shfl(partb, wlane ^ d);
+        }
+        if (wlane == 0) {
+            s_red[wid] = part;
+            s_redb[wid] = partb;
+        }
+        __syncthreads();
+        int32_t bad_total = 0;
+#pragma unroll
+        for (int q = 0; q < NWAVE; ++q) {
+            run_off += s_red[q];
+            bad_total += s_redb[q];
+        }
+        if (last && threadIdx.x == 0) {
+            const int64_t E = run_off + a.block_sum[blockIdx.x];
+            a.counts[0] = S;
+            a.counts[1] = E;
+            a.counts[2] = bad_total + a.block_bad[blockIdx.x];
+            a.root_start_ptr[S] = E;
+            a.root_end_ptr[S] = E;
+        }
+    }
+    constexpr int DSH = 20;                      // packed scan: edges in the low 20 bits (<= SLOTS * 64), drawing slots above
+    for (int64_t chunk0 = first; chunk0 < run_end; chunk0 += SLOTS) {      // block-uniform
+        if (chunk0 != first) load_slots(chunk0);
+        int32_t c[SPT], sum = 0;
+        bool dr[SPT];
+#pragma unroll
+        for (int q = 0; q < SPT; ++q) {
+            c[q] = (int32_t)(ln[q] < k ? ln[q] : k);
+            dr[q] = ln[q] > k;
+            sum += c[q] + (dr[q] ? (1 << DSH) : 0);
+        }
+        int32_t inc = sum;
+        for (int d = 1; d < WAVE; d <<= 1) {
+            const int32_t y = __shfl_up(inc, d);
+            if (wlane >= d) inc += y;
+        }
+        if (wlane == WAVE - 1) s_w[wid] = inc;
+        __syncthreads();                 // (also: the previous chunk's edges are done with the LDS arrays)
+        int32_t excl = inc - sum, all = 0;
+#pragma unroll
+        for (int q = 0; q < NWAVE; ++q) {
+            const int32_t y = s_w[q];
+            if (q < wid) excl += y;
+            all += y;
+        }
+        const int32_t total = all & ((1 << DSH) - 1), nd = all >> DSH;
+        if (threadIdx.x == 0) s_off[SLOTS] = total;
+#pragma unroll
+        for (int q = 0; q < SPT; ++q) {
+            const int j = SPT * threadIdx.x + q;
+            const int32_t eoff = excl & ((1 << DSH) - 1), dpos = excl >> DSH;
+            s_off[j] = eoff;
+            s_start[j] = st[q];
+            s_t[j] = tt[q];
+            s_len[j] = ln[q];
+            const bool huge = dr[q] && (ln[q] >> 32) != 0;
+            s_didx[j] = dr[q] ? (huge ? -2 : dpos) : -1;
+            if (dr[q]) s_dl[dpos] = huge ? -1 : j;
+            const int64_t slot = chunk0 + j;
+            if (slot < run_end) {
+                a.root_start_ptr[slot] = run_off + eoff;
+                a.root_end_ptr[slot] = run_off + eoff + c[q];
+            }
+            excl += c[q] + (dr[q] ? (1 << DSH) : 0);
+        }
+        __syncthreads();
+        if (nd > 0) {                    // block-uniform
+            // the raw draws, one (drawing slot, draw) pair per lane
+            for (int32_t x = threadIdx.x; x < nd * k; x += BLOCK) {
+                const int32_t di = x / k, d = x - di * k;
+                const int j = s_dl[di];
+                if (j >= 0) {
+                    const int64_t len = s_len[j];
+                    const uint64_t bits = draw_bits(a.seed, a.hop, chunk0 + j, d);
+                    s_pick[di * KP + d] = (uint32_t)(a.replace ? bounded(bits, len) : bounded(bits, len - k + d + 1));
+                }
+            }
+            // (windows of 2^32 edges or more: 64-bit picks, parked in the slot's own stretch of the output)
+            for (int j = threadIdx.x; j < SLOTS; j += BLOCK)
+                if (s_didx[j] == -2) huge_window_picks(a, chunk0 + j, s_len[j], &a.nbr_dt[run_off + s_off[j]]);
+            __syncthreads();
+            if (!a.replace) {
+                // ascending picks in place, a group of KP lanes per drawing slot (all inside one wavefront, whose LDS
+                // accesses are served in program order: the group reads its row, then writes it)
+                const int lig = threadIdx.x % KP;
+                for (int32_t di0 = 0; di0 < nd; di0 += BLOCK / KP) {           // block-uniform trip count
+                    const int32_t di = di0 + (int)threadIdx.x / KP;
+                    const bool on = di < nd && s_dl[di < nd ? di : 0] >= 0;
+                    const uint32_t mine = (on && lig < k) ? s_pick[di * KP + lig] : 0xFFFFFFFFu;
+                    int32_t r = 0, e = 0;
+                    if (on) {
+                        for (int32_t q = 0; q < k; q += 4) {
+                            const uint4 o = *reinterpret_cast<const uint4*>(&s_pick[di * KP + q]);
+                            r += (o.x < mine ? 1 : 0) + ((q + 1 < k && o.y < mine) ? 1 : 0) + ((q + 2 < k && o.z < mine) ? 1 : 0) +
+                                 ((q + 3 < k && o.w < mine) ? 1 : 0);
+                            e += (o.x == mine ? 1 : 0) + ((q + 1 < k && o.y == mine) ? 1 : 0) + ((q + 2 < k && o.z == mine) ? 1 : 0) +
+                                 ((q + 3 < k && o.w == mine) ? 1 : 0);
+                        }
+                    }
+                    const bool clash = on && lig < k && e > 1;
+                    const uint64_t cm = __ballot(clash);
+                    const int gsh = wlane / KP * KP;
+                    const bool gclash = ((cm >> gsh) & ((1ull << KP) - 1ull)) != 0;
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    if (on && !gclash && lig < k) s_pick[di * KP + r] = mine;
+                    if (on && gclash && lig == 0) {
+                        // two equal draws: Floyd's construction step by step, then an insertion sort, by one lane
+                        const int64_t len = s_len[s_dl[di]];
+                        uint32_t* row = &s_pick[di * KP];
+                        for (int32_t j = 1; j < k; ++j) {
+                            const uint32_t cand = row[j];
+                            bool dup = false;
+                            for (int32_t i = 0; i < j; ++i) dup |= row[i] == cand;
+                            if (dup) row[j] = (uint32_t)(len - k + j);
+                        }
+                        for (int32_t x = 1; x < k; ++x) {
+                            const uint32_t v = row[x];
+                            int32_t y = x - 1;
+                            while (y >= 0 && row[y] > v) {
+                                row[y + 1] = row[y];
+                                --y;
+                            }
+                            row[y + 1] = v;
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        // the chunk's edges, flat: up to ROUNDS per lane, every load issued before the first store
+        constexpr int ROUNDS = 4;
+        for (int32_t x0 = threadIdx.x; x0 < total; x0 += ROUNDS * BLOCK) {
+            Edge ed[ROUNDS];
+            int64_t tslot[ROUNDS];
+#pragma unroll
+            for (int r = 0; r < ROUNDS; ++r) {
+                const int32_t x = x0 + r * BLOCK;
+                ed[r] = Edge{0, 0, 0, -1};
+                tslot[r] = 0;
+                if (x < total) {
+                    int lo = 0;
+#pragma unroll
+                    for (int step = SLOTS / 2; step > 0; step >>= 1)
+                        lo += s_off[lo + step] <= x ? step : 0;
+                    const int32_t j = x - s_off[lo], di = s_didx[lo];
+                    int64_t sel = j;
+                    if (di >= 0) {
+                        sel = (int64_t)s_pick[di * KP + j];
+                    } else if (di == -2) {
+                        sel = a.nbr_dt[run_off + x];      // parked there by huge_window_picks (this lane overwrites it below)
+                    }
+                    tslot[r] = s_t[lo];
+                    ed[r] = load_picked_edge(a, s_start[lo] + sel);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < ROUNDS; ++r) {
+                const int32_t x = x0 + r * BLOCK;
+                if (x < total) {
+                    const int64_t o = run_off + x;
+                    a.nbr[o] = ed[r].col;
+                    if (a.mark != nullptr) mark_id(a, ed[r].col);
+                    a.nbr_ts[o] = a.keep_root_time ? tslot[r] : ed[r].ts;
+                    a.nbr_eid[o] = ed[r].eid;
+                    a.nbr_dt[o] = ed[r].ts - tslot[r];
+                    if (a.hint_out != nullptr) a.hint_out[o] = ed[r].hint;
                 }
             }
         }
@@ -975,7 +1122,7 @@ int pick_group(const sgl_sample_params* p, int64_t S_max) {
 // search) keeps 8x the slots in flight and issues ~2.5x fewer loads than 8 lanes do
 // (857k slots over rows of up to 1M edges: 187 us against 330 us).
 int pick_search_group(int Gf, int64_t S_max) {
-    if (S_max >= 262144) return 1;
+    if (S_max >= 131072) return 1;
     if (S_max >= 32768 && Gf > 8) return 8;   // as the recent strategy: one wave-residency round for the search
     return Gf;
 }
@@ -1041,30 +1188,47 @@ HopKernel count_fn(int G) {
 HopKernel fill_fn(int G, bool uniform) {
     if (uniform) {
         switch (G) {
-            case 16: return fill_kernel<16>;
-            case 32: return fill_kernel<32>;
-            default: return fill_kernel<64>;
+            case 16: return fill_uniform_flat_kernel<16, 256>;
+            case 32: return fill_uniform_flat_kernel<32, 256>;
+            default: return fill_kernel<64>;      // fanouts beyond 32: a wavefront per slot
         }
     }
     return fill_flat_kernel;
 }
 
-// Gc lanes per slot search, Gf lanes per slot copy or draw
-int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf) {
-    a.align = BLOCK / (Gc < Gf ? Gc : Gf);
-    int64_t blocks = ceil_div<int64_t>(a.S_max > 0 ? a.S_max : 1, a.align);
-    if (blocks > MAX_BLOCKS) blocks = MAX_BLOCKS;
+// Gc lanes per slot search, Gf lanes per slot copy or draw.  do_count / do_fill: the two halves of a hop; a second
+// query over the same slots with the same window rule and fanout runs only the fill, on the first query's
+// window arrays and block sums (same grid and run alignment: hop_grid).
+struct HopGrid {
+    int32_t align;
+    int64_t blocks;
+};
+HopGrid hop_grid(int64_t S_max, int Gc, int Gf) {
+    HopGrid hg;
+    hg.align = BLOCK / (Gc < Gf ? Gc : Gf);
+    hg.blocks = ceil_div<int64_t>(S_max > 0 ? S_max : 1, hg.align);
+    if (hg.blocks > MAX_BLOCKS) hg.blocks = MAX_BLOCKS;
+    return hg;
+}
+
+int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf, bool do_count = true, bool do_fill = true) {
+    const HopGrid hg = hop_grid(a.S_max, Gc, Gf);
+    a.align = hg.align;
+    const int64_t blocks = hg.blocks;
     // a block counts the edges of its run of slots in 32 bits (count_kernel's partial sums, scan_kernel's staging)
     const int64_t run = ceil_div<int64_t>(ceil_div<int64_t>(a.S_max > 0 ? a.S_max : 1, blocks), a.align) * a.align;
     if (a.k > 0 && run > (int64_t)INT32_MAX / a.k)
         return fail(SGL_ENOTSUP, "sample: %lld slots x fanout %d exceed what a block counts in 32 bits", (long long)a.S_max, a.k);
     a.scanned = blocks > FUSED_PREFIX_MAX ? 1 : 0;
-    hipLaunchKernelGGL(count_fn(Gc), dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
-    SGL_LAUNCH_CHECK();
-    if (a.scanned) {
-        hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, a, (int)blocks);
+    if (do_count) {
+        hipLaunchKernelGGL(count_fn(Gc), dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
         SGL_LAUNCH_CHECK();
+        if (a.scanned) {
+            hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, a, (int)blocks);
+            SGL_LAUNCH_CHECK();
+        }
     }
+    if (!do_fill) return SGL_OK;
     // a uniform fanout beyond one wavefront keeps a slot's picks in LDS (one wave per slot)
     const size_t wide_lds = (a.type == SGL_SAMPLE_UNIFORM && a.k > WAVE) ? (size_t)NWAVE * a.k * sizeof(int64_t) : 0;
     hipLaunchKernelGGL(fill_fn(Gf, a.type == SGL_SAMPLE_UNIFORM), dim3((unsigned)blocks), dim3(BLOCK), wide_lds, st, a);
@@ -1562,7 +1726,7 @@ struct RootSpec {  // hop-0 slot source of the k-hop driver
 int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot_ts, const RootSpec* derive,
                 int64_t S_max, const int64_t* S_dev, const sgl_sample_params* p, const sgl_hop_out* out, void* ws,
                 size_t ws_bytes, hipStream_t st, const int64_t* slot_hint = nullptr, int64_t* hint_out = nullptr,
-                bool hint_optional = false) {
+                bool hint_optional = false, bool do_count = true) {
     if (!derive && S_max > 0 && (!slot_node || !slot_ts)) return fail(SGL_EINVAL, "sample: slot array is NULL");
     if (ws_bytes < hop_workspace_bytes(S_max) || !ws)
         return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, hop_workspace_bytes(S_max));
@@ -1594,7 +1758,7 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
     a.nbr = out->neighbors; a.nbr_ts = out->neighbors_ts; a.nbr_eid = out->neighbors_eid;
     a.nbr_dt = out->neighbors_dt; a.counts = out->counts;
     const int Gf = pick_group(p, S_max);
-    return launch_hop(a, st, pick_search_group(Gf, S_max), Gf);
+    return launch_hop(a, st, pick_search_group(Gf, S_max), Gf, do_count, true);
 }
 
 
@@ -1871,6 +2035,17 @@ struct SegArgs {
     int64_t cap[SEG_MAX_CHAINS];             // its capacity_slots
     int64_t* seg;                            // [Q][layers + 1][B + 1]
 };
+// What scan_kernel publishes for a hop, for a second query that shares the hop's counting pass
+__global__ void share_counts_kernel(const int64_t* src_counts, int64_t* counts, int64_t* rsp, int64_t* rep, int64_t cap) {
+    const int64_t S = src_counts[0], E = src_counts[1];
+    counts[0] = S;
+    counts[1] = E;
+    counts[2] = src_counts[2];
+    if (S >= 0 && S <= cap) {
+        rsp[S] = E;
+        rep[S] = E;
+    }
+}
 // seg[q][0][b] = first root slot of batch b; seg[q][l+1][b] = root_start_ptr_l[seg[q][l][b]]: where batch b's
 // edges of hop l begin (hop l's terminating entry root_start_ptr[S_l] = E_l closes the last batch).
 __global__ void batch_seg_kernel(SegArgs a) {
@@ -1923,35 +2098,57 @@ extern "C" int32_t sgl_sample_khop_batched(const sgl_tcsr* g, int32_t B, const i
     if (!ws || ws_bytes < (size_t)Q * per)
         return fail(SGL_ENOMEM, "sample_khop_batched: workspace %zu < %zu bytes", ws_bytes, (size_t)Q * per);
     hipStream_t st = as_stream(stream);
+    // Hop-major order: a query that asks for the same windows and fanout as query 0 runs only the fill of hop 0,
+    // on query 0's window arrays and block sums (its root slots are the same; they are searched once).
+    const int64_t* sn[SEG_MAX_CHAINS];
+    const int64_t* stt[SEG_MAX_CHAINS];
+    const int64_t* S_dev[SEG_MAX_CHAINS];
     for (int32_t q = 0; q < Q; ++q) {
-        const sgl_sample_params* pq = &p[q];
-        const sgl_hop_out* oq = outs + (size_t)q * layers;
-        char* wq = static_cast<char*>(ws) + (size_t)q * per;
-        int64_t worst = S_max;
-        for (int32_t l = 0; l < layers; ++l) worst = worst_slots(S_max, l, pq->fanout) > worst ? worst_slots(S_max, l, pq->fanout) : worst;
-        const size_t hop_ws = hop_workspace_bytes(worst);
-        // as sgl_sample_khop: with the graph's next-hop index the slots of hops >= 1 are not searched
-        const bool carry = layers > 1 && g->hop_hint != nullptr && !pq->equal_root_time &&
-                           !(pq->type == SGL_SAMPLE_UNIFORM && pq->keep_root_time) && per >= hop_ws + hint_carry_bytes(worst);
-        int64_t* carry_buf[2] = {nullptr, nullptr};
-        if (carry) {
-            carry_buf[0] = reinterpret_cast<int64_t*>(wq + hop_ws);
-            carry_buf[1] = reinterpret_cast<int64_t*>(wq + hop_ws + align_up((size_t)(worst + 1) * 8));
-        }
-        const int64_t* sn = slot_node;
-        const int64_t* stt = slot_ts;
-        const int64_t* S_dev = batch_ptr + B;
-        for (int32_t l = 0; l < layers; ++l) {
+        sn[q] = slot_node;
+        stt[q] = slot_ts;
+        S_dev[q] = batch_ptr + B;
+    }
+    const int Gf0 = pick_group(&p[0], S_max);
+    const HopGrid grid0 = hop_grid(S_max, pick_search_group(Gf0, S_max), Gf0);
+    for (int32_t l = 0; l < layers; ++l) {
+        for (int32_t q = 0; q < Q; ++q) {
+            const sgl_sample_params* pq = &p[q];
+            const sgl_hop_out* oq = outs + (size_t)q * layers;
+            char* wq = static_cast<char*>(ws) + (size_t)q * per;
+            int64_t worst = S_max;
+            for (int32_t j = 0; j < layers; ++j) worst = worst_slots(S_max, j, pq->fanout) > worst ? worst_slots(S_max, j, pq->fanout) : worst;
+            const size_t hop_ws = hop_workspace_bytes(worst);
+            // as sgl_sample_khop: with the graph's next-hop index the slots of hops >= 1 are not searched
+            const bool carry = layers > 1 && g->hop_hint != nullptr && !pq->equal_root_time &&
+                               !(pq->type == SGL_SAMPLE_UNIFORM && pq->keep_root_time) && per >= hop_ws + hint_carry_bytes(worst);
+            int64_t* carry_buf[2] = {nullptr, nullptr};
+            if (carry) {
+                carry_buf[0] = reinterpret_cast<int64_t*>(wq + hop_ws);
+                carry_buf[1] = reinterpret_cast<int64_t*>(wq + hop_ws + align_up((size_t)(worst + 1) * 8));
+            }
             sgl_sample_params pl = *pq;
             pl.hop = l;
             const int64_t s_max = worst_slots(S_max, l, pq->fanout);
             const int64_t* hint_in = l == 0 ? (pq->equal_root_time ? nullptr : slot_hint) : (carry ? carry_buf[(l - 1) & 1] : nullptr);
-            rc = run_hop(g, sn, stt, nullptr, s_max, S_dev, &pl, &oq[l], wq, carry ? hop_ws : per, st, hint_in,
-                         (carry && l + 1 < layers) ? carry_buf[l & 1] : nullptr, l == 0);
+            bool share = false;
+            if (l == 0 && q > 0) {
+                const int Gfq = pick_group(pq, S_max);
+                const HopGrid gq = hop_grid(S_max, pick_search_group(Gfq, S_max), Gfq);
+                share = pq->fanout == p[0].fanout && pq->allowed_offset == p[0].allowed_offset &&
+                        (pq->equal_root_time != 0) == (p[0].equal_root_time != 0) && gq.align == grid0.align &&
+                        gq.blocks == grid0.blocks;      // (a hop's scratch is carved by its own slot count: same places)
+            }
+            rc = run_hop(g, sn[q], stt[q], nullptr, s_max, S_dev[q], &pl, &oq[l], share ? static_cast<char*>(ws) : wq,
+                         carry ? hop_ws : per, st, hint_in, (carry && l + 1 < layers) ? carry_buf[l & 1] : nullptr, l == 0, !share);
             if (rc != SGL_OK) return rc;
-            sn = oq[l].neighbors;
-            stt = oq[l].neighbors_ts;
-            S_dev = oq[l].counts + 1;
+            if (share && grid0.blocks > FUSED_PREFIX_MAX) {   // the scan launch of query 0 published that query's counts only
+                hipLaunchKernelGGL(share_counts_kernel, dim3(1), dim3(1), 0, st, outs[0].counts, oq[0].counts,
+                                   oq[0].root_start_ptr, oq[0].root_end_ptr, oq[0].capacity_slots);
+                SGL_LAUNCH_CHECK();
+            }
+            sn[q] = oq[l].neighbors;
+            stt[q] = oq[l].neighbors_ts;
+            S_dev[q] = oq[l].counts + 1;
         }
     }
     SegArgs sa{};

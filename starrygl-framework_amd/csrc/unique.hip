@@ -457,9 +457,9 @@ __global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a, int fo
 // Batch b's ids live at [b * stride, b * stride + universe) of a state over B * stride ids (stride: the
 // universe rounded up to whole tiles of flag words, so that a tile belongs to one batch); array g's
 // elements [seg[g][b], seg[g][b+1]) belong to batch b.  Ascending numbering over the big universe is
-// batch-major and ascending inside a batch: batch b's local id = global rank - U_off[b], where U_off[b]
-// is the offset of the first tile of batch b.  Every call starts a new epoch, so marking needs no table
-// read.
+// batch-major and ascending inside a batch: batch b's local id = global rank - rank of the batch's first
+// tile.  Every call numbers afresh and looks up only ids it has numbered itself, so the table needs
+// neither epoch stamps nor clearing: 4 bytes per id, written by assign, read by lookup.
 constexpr int BATCH_MAX = SGL_BATCH_MAX;
 constexpr int64_t BATCH_STRIDE_ALIGN = (int64_t)TILE * 64;   // ids per tile of a bitmap state (a byte-flag tile holds TILE * 8)
 
@@ -469,20 +469,29 @@ struct Batched {
     const int64_t* seg[MAXG];
 };
 
+struct BState {
+    uint32_t* table;    // [B * stride] local id inside the batch
+    uint64_t* flags;    // pending flags: a byte per id (8 per word) or a bit per id
+    int64_t universe, words;
+    int32_t bytes;
+};
+
 inline int64_t batch_stride(int64_t universe) { return ceil_div<int64_t>(universe, BATCH_STRIDE_ALIGN) * BATCH_STRIDE_ALIGN; }
 
-State carve_batched(void* state, int64_t universe, int32_t B) {
-    State s;
+BState carve_batched(void* state, int64_t universe, int32_t B) {
+    BState s;
     char* p = static_cast<char*>(state);
     s.universe = (int64_t)B * batch_stride(universe);
     s.bytes = remap_byte_flags(s.universe) ? 1 : 0;
     s.words = ceil_div<int64_t>(s.universe, s.bytes ? 8 : 64);
-    s.hdr = reinterpret_cast<Header*>(p);
-    s.table = reinterpret_cast<uint64_t*>(p + HEADER_BYTES);
-    s.bitmap = s.table + s.universe;
-    s.planes = 1;
-    s.desc = s.bitmap + s.words;
+    s.flags = reinterpret_cast<uint64_t*>(p + HEADER_BYTES);
+    s.table = reinterpret_cast<uint32_t*>(s.flags + s.words);
     return s;
+}
+
+__global__ void init_batched_kernel(BState s) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < s.words; i += stride) s.flags[i] = 0;
 }
 
 // batch of element i of an array whose batch offsets are seg[0..B] (in LDS): the last b with seg[b] <= i
@@ -503,90 +512,12 @@ __device__ __forceinline__ void stage_segs(const Batched& bt, int G, int64_t (*s
     __syncthreads();
 }
 
-__global__ __launch_bounds__(BLOCK) void mark_batched_kernel(State s, Arrays a, Batched bt) {
+// LOOKUP == false: sets the flag of every id (a new numbering per call: no table read);
+// LOOKUP == true : rewrites every array through the table.
+template <bool LOOKUP>
+__global__ __launch_bounds__(BLOCK) void walk_batched_kernel(BState s, Arrays a, Batched bt) {
     __shared__ int64_t s_seg[MAXG][BATCH_MAX + 1];
     stage_segs(bt, a.G, s_seg);
-    int64_t len[MAXG], max_len = 0;
-#pragma unroll
-    for (int g = 0; g < MAXG; ++g) {
-        len[g] = 0;
-        if (g < a.G) {
-            const int64_t l = s_seg[g][bt.B];
-            len[g] = l < 0 ? 0 : (l > a.len_max[g] ? a.len_max[g] : l);
-        }
-        max_len = len[g] > max_len ? len[g] : max_len;
-    }
-    for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < max_len; i += (int64_t)gridDim.x * BLOCK) {
-#pragma unroll
-        for (int g = 0; g < MAXG; ++g) {
-            if (g < a.G && i < len[g]) {
-                const int64_t id = a.ids[g][i];
-                if (id >= 0 && id < bt.universe)
-                    remap_set_pending(s.bitmap, s.bytes, id + (int64_t)batch_of(s_seg[g], bt.B, i) * bt.stride);
-            }
-        }
-    }
-}
-
-// Numbers the set flags (tile_sum holds the exclusive tile offsets, the total at [nt]); the first tile of
-// every batch records where the batch's list begins.
-__global__ __launch_bounds__(BLOCK) void assign_batched_kernel(State s, const int64_t* tile_sum, int64_t nt, Batched bt,
-                                                               int64_t* unique_out, int64_t unique_capacity,
-                                                               int64_t* U_off, int64_t* U_dev, uint32_t* stamp_ws) {
-    __shared__ int32_t s_wave[BLOCK / WAVE];
-    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
-    const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
-    uint64_t word = (w < s.words) ? s.bitmap[w] : 0ull;
-    const int32_t c = __popcll(word);
-    int32_t inc = c;
-    for (int d = 1; d < WAVE; d <<= 1) {
-        const int32_t x = __shfl_up(inc, d);
-        if (lane >= d) inc += x;
-    }
-    if (lane == WAVE - 1) s_wave[wid] = inc;
-    __syncthreads();
-    int32_t wave_off = 0;
-    for (int q = 0; q < wid; ++q) wave_off += s_wave[q];
-    const int64_t tile_off = tile_sum[blockIdx.x];
-    const int ipw = s.bytes ? 8 : 64;                       // ids per flag word
-    const int64_t tile_id0 = (int64_t)blockIdx.x * TILE * ipw;
-    const int64_t b = tile_id0 / bt.stride;                 // the tile's batch (a stride is a whole number of tiles)
-    if (threadIdx.x == 0) {
-        if (tile_id0 == b * bt.stride) U_off[b] = tile_off;
-        if (blockIdx.x == nt - 1) {
-            const int64_t total = tile_sum[nt];
-            U_off[bt.B] = total;
-            U_dev[0] = total;
-            stamp_ws[0] = eff_stamp(s, 1);
-        }
-    }
-    if (c == 0) return;
-    int64_t local = tile_off + wave_off + (inc - c);
-    const uint64_t stamp = (uint64_t)eff_stamp(s, 1) << 32;
-    const int64_t id0 = w * ipw;
-    const int shift = s.bytes ? 3 : 0;
-    const int64_t base = b * bt.stride;
-    while (word) {
-        const int bit = __ffsll((unsigned long long)word) - 1;
-        word &= word - 1;
-        const int64_t id = id0 + (bit >> shift);
-        s.table[id] = stamp | (uint64_t)(uint32_t)local;
-        if (local < unique_capacity) unique_out[local] = id - base;
-        ++local;
-    }
-    s.bitmap[w] = 0;
-}
-
-// Rewrites every array through the table, batch by batch (local id = global rank - start of the batch's list),
-// and commits the epoch.
-__global__ __launch_bounds__(BLOCK) void lookup_batched_kernel(State s, Arrays a, Batched bt, const int64_t* U_off,
-                                                               const uint32_t* stamp_ws, int64_t* U_dev) {
-    __shared__ int64_t s_seg[MAXG][BATCH_MAX + 1];
-    __shared__ int64_t s_uoff[BATCH_MAX + 1];
-    for (int x = threadIdx.x; x <= bt.B; x += BLOCK) s_uoff[x] = U_off[x];
-    stage_segs(bt, a.G, s_seg);
-    const uint32_t stamp = stamp_ws[0];
-    if (blockIdx.x == 0 && threadIdx.x == 0) commit(s, 1, 1, 1, U_dev);
     int64_t len[MAXG], max_len = 0;
 #pragma unroll
     for (int g = 0; g < MAXG; ++g) {
@@ -599,31 +530,93 @@ __global__ __launch_bounds__(BLOCK) void lookup_batched_kernel(State s, Arrays a
     }
     for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < max_len; i += (int64_t)gridDim.x * BLOCK) {
         int64_t id[MAXG];
-        int bb[MAXG];
+        int64_t at[MAXG];
 #pragma unroll
         for (int g = 0; g < MAXG; ++g) {
             id[g] = -1;
-            bb[g] = 0;
+            at[g] = 0;
             if (g < a.G && i < len[g]) {
                 id[g] = a.ids[g][i];       // ids may alias out
-                bb[g] = batch_of(s_seg[g], bt.B, i);
+                at[g] = id[g] + (int64_t)batch_of(s_seg[g], bt.B, i) * bt.stride;
             }
         }
-        uint64_t e[MAXG];
+        if constexpr (LOOKUP) {
+            uint32_t e[MAXG];
 #pragma unroll
-        for (int g = 0; g < MAXG; ++g)
-            e[g] = (id[g] >= 0 && id[g] < bt.universe) ? s.table[id[g] + (int64_t)bb[g] * bt.stride] : 0ull;
+            for (int g = 0; g < MAXG; ++g) e[g] = (id[g] >= 0 && id[g] < bt.universe) ? s.table[at[g]] : 0u;
 #pragma unroll
-        for (int g = 0; g < MAXG; ++g)
-            if (g < a.G && i < len[g])
-                a.out[g][i] = ((uint32_t)(e[g] >> 32) == stamp) ? (int64_t)(e[g] & 0xFFFFFFFFull) - s_uoff[bb[g]] : -1;
+            for (int g = 0; g < MAXG; ++g)
+                if (g < a.G && i < len[g]) a.out[g][i] = (id[g] >= 0 && id[g] < bt.universe) ? (int64_t)e[g] : -1;
+        } else {
+#pragma unroll
+            for (int g = 0; g < MAXG; ++g)
+                if (id[g] >= 0 && id[g] < bt.universe) remap_set_pending(s.flags, s.bytes, at[g]);
+        }
     }
+}
+
+__global__ __launch_bounds__(BLOCK) void reduce_batched_kernel(BState s, int64_t* tile_sum) {
+    __shared__ int32_t s_w[BLOCK / WAVE];
+    const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
+    int32_t c = (w < s.words) ? __popcll(s.flags[w]) : 0;
+    for (int d = WAVE / 2; d > 0; d >>= 1) c += __shfl_down(c, d);
+    if (threadIdx.x % WAVE == 0) s_w[threadIdx.x / WAVE] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int64_t sum = 0;
+        for (int q = 0; q < BLOCK / WAVE; ++q) sum += s_w[q];
+        tile_sum[blockIdx.x] = sum;
+    }
+}
+
+// Numbers the set flags (tile_sum holds the exclusive tile offsets, the total at [nt]): an id's local id is its
+// rank inside its batch, i.e. the global rank minus the offset of the batch's first tile; the first tile of
+// every batch records where the batch's list begins.
+__global__ __launch_bounds__(BLOCK) void assign_batched_kernel(BState s, const int64_t* tile_sum, int64_t nt, Batched bt,
+                                                               int64_t* unique_out, int64_t unique_capacity, int64_t* U_off) {
+    __shared__ int32_t s_wave[BLOCK / WAVE];
+    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
+    uint64_t word = (w < s.words) ? s.flags[w] : 0ull;
+    const int32_t c = __popcll(word);
+    int32_t inc = c;
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const int32_t x = __shfl_up(inc, d);
+        if (lane >= d) inc += x;
+    }
+    if (lane == WAVE - 1) s_wave[wid] = inc;
+    __syncthreads();
+    int32_t wave_off = 0;
+    for (int q = 0; q < wid; ++q) wave_off += s_wave[q];
+    const int64_t tile_off = tile_sum[blockIdx.x];
+    const int ipw = s.bytes ? 8 : 64;                       // ids per flag word
+    const int64_t tiles_per_batch = bt.stride / ((int64_t)TILE * ipw);
+    const int64_t b = (int64_t)blockIdx.x / tiles_per_batch;        // the tile's batch (a stride is a whole number of tiles)
+    const int64_t batch_off = tile_sum[b * tiles_per_batch];
+    if (threadIdx.x == 0) {
+        if ((int64_t)blockIdx.x == b * tiles_per_batch) U_off[b] = tile_off;
+        if (blockIdx.x == nt - 1) U_off[bt.B] = tile_sum[nt];
+    }
+    if (c == 0) return;
+    int64_t rank = tile_off + wave_off + (inc - c);
+    const int64_t id0 = w * ipw;
+    const int shift = s.bytes ? 3 : 0;
+    const int64_t base = b * bt.stride;
+    while (word) {
+        const int bit = __ffsll((unsigned long long)word) - 1;
+        word &= word - 1;
+        const int64_t id = id0 + (bit >> shift);
+        s.table[id] = (uint32_t)(rank - batch_off);
+        if (rank < unique_capacity) unique_out[rank] = id - base;
+        ++rank;
+    }
+    s.flags[w] = 0;
 }
 
 size_t batched_workspace_bytes(int64_t universe, int32_t B) {
     const int64_t big = (int64_t)B * batch_stride(universe);
     const int64_t words = ceil_div<int64_t>(big, remap_byte_flags(big) ? 8 : 64);
-    return align_up((size_t)(ceil_div<int64_t>(words, TILE) + 2) * 8) + align_up(16) + align_up(16) + 512;
+    return align_up((size_t)(ceil_div<int64_t>(words, TILE) + 2) * 8) + 512;
 }
 
 size_t dense_workspace_bytes(int64_t universe) {
@@ -802,7 +795,7 @@ extern "C" size_t sgl_remap_batched_state_bytes(int64_t universe, int32_t B) {
     if (universe <= 0 || B < 1 || B > BATCH_MAX) return 0;
     const int64_t big = (int64_t)B * batch_stride(universe);
     const int64_t words = ceil_div<int64_t>(big, remap_byte_flags(big) ? 8 : 64);
-    return HEADER_BYTES + (size_t)big * 8 + (size_t)words * 8 + (size_t)ceil_div<int64_t>(words, TILE) * 8 + 8;
+    return HEADER_BYTES + (size_t)words * 8 + (size_t)big * 4 + 8;
 }
 
 extern "C" int32_t sgl_remap_batched_init(void* state, size_t state_bytes, int64_t universe, int32_t B, void* stream) {
@@ -812,10 +805,10 @@ extern "C" int32_t sgl_remap_batched_init(void* state, size_t state_bytes, int64
     if (state_bytes < sgl_remap_batched_state_bytes(universe, B))
         return fail(SGL_ENOMEM, "remap_batched_init: state %zu < %zu bytes", state_bytes, sgl_remap_batched_state_bytes(universe, B));
     if (reinterpret_cast<uintptr_t>(state) % 8) return fail(SGL_EINVAL, "remap_batched_init: state must be 8-byte aligned");
-    State s = carve_batched(state, universe, B);
-    int64_t blocks = ceil_div<int64_t>(s.universe, 256);
+    BState s = carve_batched(state, universe, B);
+    int64_t blocks = ceil_div<int64_t>(s.words, 256);
     if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL(init_state_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), s);
+    hipLaunchKernelGGL(init_batched_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), s);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }
@@ -859,28 +852,27 @@ extern "C" int32_t sgl_unique_compact_batched(void* state, int64_t universe, int
     }
     if (ceil_div<int64_t>(all.start[MAXG], BLOCK) > 0x7FFFFFFFll) return fail(SGL_ENOTSUP, "unique_compact_batched: too many ids");
     hipStream_t st = as_stream(stream);
-    State s = carve_batched(state, universe, B);
+    BState s = carve_batched(state, universe, B);
     Arena ar(ws, ws_bytes);
     const int64_t nt = ceil_div<int64_t>(s.words, TILE);
     int64_t* tile_sum = ar.take<int64_t>(nt + 2);
-    uint32_t* stamp_ws = ar.take<uint32_t>(4);
-    int64_t* U_dev = ar.take<int64_t>(2);
     if (!ar.ok()) return fail(SGL_ENOMEM, "unique_compact_batched: workspace too small");
     int64_t mb = ceil_div<int64_t>(longest > 0 ? longest : 1, BLOCK);
     if (mb > MAX_GRID) mb = MAX_GRID;
     if (longest > 0) {
-        hipLaunchKernelGGL(mark_batched_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, all, bt);
+        hipLaunchKernelGGL(walk_batched_kernel<false>, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, all, bt);
         SGL_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
+    hipLaunchKernelGGL(reduce_batched_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
     SGL_LAUNCH_CHECK();
     hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, tile_sum, nt);
     SGL_LAUNCH_CHECK();
     hipLaunchKernelGGL(assign_batched_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, bt, unique_out,
-                       unique_capacity, U_off, U_dev, stamp_ws);
+                       unique_capacity, U_off);
     SGL_LAUNCH_CHECK();
-    // (always launched: thread 0 of block 0 commits the epoch)
-    hipLaunchKernelGGL(lookup_batched_kernel, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, all, bt, U_off, stamp_ws, U_dev);
-    SGL_LAUNCH_CHECK();
+    if (longest > 0) {
+        hipLaunchKernelGGL(walk_batched_kernel<true>, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, all, bt);
+        SGL_LAUNCH_CHECK();
+    }
     return SGL_OK;
 }
