@@ -491,6 +491,10 @@ def main():
                          "sgl_unique_compact_batched -> one gather launch over all their rows), as a loader that samples "
                          "that many batches ahead does; every batch keeps its own local-id space and its own segment of "
                          "every output.  1 = one set of library calls per mini-batch (the per-batch pipelines)")
+    ap.add_argument("--fork-uniform", action="store_true",
+                    help="batched step: the uniform query as a library call of its own on a second branch of the step's HIP "
+                         "graph, beside unique and the gather (by default both queries are one library call on one stream; "
+                         "measured within the run-to-run spread of each other)")
     ap.add_argument("--group-pipelines", type=int, default=2,
                     help="independent copies of the batched step (own buffers, HIP graph and stream each) that take the "
                          "groups of batches in turn")
@@ -558,7 +562,7 @@ def main():
 
     # batches: B consecutive events of the global time order, from the later half
     order = np.argsort(ts, kind="stable")
-    NB = min(args.steps + args.warmup, 64)
+    NB = 64
     rng = np.random.default_rng(7)
     starts = np.sort(rng.integers(m // 2, m - B, NB))
     bt = [synth.link_batch(src[order[s: s + B]], dst[order[s: s + B]], ts[order[s: s + B]], 0, B, n, B, rng)
@@ -735,7 +739,7 @@ def main():
         P = type("GroupPipeline", (), {})()
         Q = 2 if with_uniform else 1
         P.B, P.stream = B, stream
-        P.kb = hot.khop_batched_buffers(B * S0, B, 2, k, Q)
+        P.kb = hot.khop_batched_buffers(B * S0, B, 2, k, 1 if (with_uniform and args.fork_uniform) else Q)
         P.in_node, P.in_ts, P.in_hint = hot.be.empty(B * S0), hot.be.empty(B * S0), hot.be.empty(B * S0)
         P.ptr_full = D(np.arange(B + 1, dtype=np.int64) * S0)
         P.ptr = P.ptr_full.clone()
@@ -758,8 +762,17 @@ def main():
         P.acc = torch.zeros(14, dtype=torch.int64, device=dev)
         P.live = torch.zeros(14, dtype=torch.int64, device=dev)
 
+        fork = with_uniform and args.fork_uniform
+        if fork:        # the uniform query gets buffers, a workspace and a stream of its own
+            P.kb_u = hot.khop_batched_buffers(B * S0, B, 2, k, 1)
+            P.side = torch.cuda.Stream()
+
         def sample():
-            hot.sample_khop_batched(gdg, P.in_node, P.in_ts, P.ptr, 2, P.params, out=P.kb,
+            hot.sample_khop_batched(gdg, P.in_node, P.in_ts, P.ptr, 2, P.params[:1] if fork else P.params, out=P.kb,
+                                    slot_hint=P.in_hint if hinted else None)
+
+        def sample_uniform():
+            hot.sample_khop_batched(gdg, P.in_node, P.in_ts, P.ptr, 2, P.params[1:], out=P.kb_u,
                                     slot_hint=P.in_hint if hinted else None)
 
         def unique():
@@ -771,14 +784,32 @@ def main():
             hot.gather_multi(P.plan)
 
         def account():          # the same 14 places as `live` of the per-batch step
-            P.live[0: 6 * Q].copy_(P.kb.counts)
+            if fork:
+                P.live[0:6].copy_(P.kb.counts)
+                P.live[6:12].copy_(P.kb_u.counts)
+            else:
+                P.live[0: 6 * Q].copy_(P.kb.counts)
             P.live[12:13].copy_(P.uoff[B: B + 1])
             P.acc.add_(P.live)
 
         P.stage_fns = {"sample": sample, "unique": unique, "gathers": gathers}
+        if fork:
+            P.stage_fns["sample_uniform"] = sample_uniform
 
         def step():
-            sample(); unique(); gathers(); account()
+            if not fork:
+                sample(); unique(); gathers(); account()
+                return
+            # most-recent query -> unique -> gather on the step's stream; the uniform query, which only reads the batch,
+            # beside them on a second branch (its kernels are bound by the latency of scattered picks, the gather by bandwidth)
+            cur = torch.cuda.current_stream()
+            P.side.wait_stream(cur)
+            sample()
+            with torch.cuda.stream(P.side):
+                sample_uniform()
+            unique(); gathers()
+            cur.wait_stream(P.side)
+            account()
 
         def load(b0, live=B):
             """the slots of batches b0 .. b0 + live - 1 (mod NB) into the input buffers"""
@@ -795,20 +826,29 @@ def main():
             P.graph = torch.cuda.CUDAGraph()
             with graph_capture(P.graph, stream=stream):
                 step()
-        P.ptr_tail = {}
+        # a last, shorter group: the trailing batches are empty (batch_ptr is read on the device)
+        P.ptr_tail = {live: D(np.minimum(np.arange(B + 1), live).astype(np.int64) * S0) for live in {args.steps % B} - {0}}
 
         def run(b0, live=B):
             torch.cuda.set_stream(stream)
             load(b0, live)
-            if live != B:      # a last, shorter group: the trailing batches are empty (batch_ptr is read on the device)
-                if live not in P.ptr_tail:
-                    P.ptr_tail[live] = D(np.minimum(np.arange(B + 1), live).astype(np.int64) * S0)
+            if live != B:
                 P.ptr.copy_(P.ptr_tail[live], non_blocking=True)
             P.graph.replay()
             if live != B:
                 P.ptr.copy_(P.ptr_full, non_blocking=True)
         P.run = run
         return P
+
+    def pass_counts(accs, what):
+        """The accumulated counts of a pass (E0, E1 recent, E0, E1 uniform, unique ids).  counts[2] of every hop - slots
+        outside [0,n), or INT64_MAX when a block of a single-launch kernel gave up its bounded wait - must have stayed 0:
+        a pass whose sampler gave up is not a measurement."""
+        full = sum(accs).cpu().numpy()
+        bad = full[[2, 5, 8, 11]]
+        if np.any(bad != 0):
+            raise RuntimeError(f"{what}: error counts of the pass are {bad.tolist()} (a block gave up its bounded wait, or a root lies outside the graph)")
+        return full[ACC].astype(np.float64)
 
     def timed_groups(pipes, streams=()):
         """W untimed steps (whole groups), then exactly K steps in groups of B dealt to `pipes` in turn
@@ -836,7 +876,7 @@ def main():
         torch.cuda.synchronize()
         wall_ = time.perf_counter() - t_start
         torch.cuda.set_stream(main_stream)
-        return wall_, submit, sum(P.acc for P in pipes).cpu().numpy()[ACC].astype(np.float64)
+        return wall_, submit, pass_counts([P.acc for P in pipes], "batched pass")
 
     batch_rows = list(packed.unbind(0))
     K, W = args.steps, args.warmup
@@ -934,7 +974,7 @@ def main():
         torch.cuda.synchronize()
         wall_ = time.perf_counter() - t_start
         torch.cuda.set_stream(main_stream)
-        return wall_, submit, sum(accs).cpu().numpy()[ACC].astype(np.float64)
+        return wall_, submit, pass_counts(accs, "per-batch pass")
 
     def plain_batch(i, b):
         stage_inputs(b)
@@ -985,7 +1025,7 @@ def main():
         pipes = [make_pipeline(st_, use_root_hint) for st_ in pipe_streams[: args.pipelines]]
         wall_p, sub_p, tot_p = timed_region(lambda i, b: pipes[i % len(pipes)].run(b), [P_.acc for P_ in pipes])
         del pipes
-        assert np.array_equal(tot_p[SAME], tot[SAME]), "batched and per-batch passes disagree"
+        assert np.array_equal(tot_p[SAME], tot[SAME]), f"batched and per-batch passes disagree: {tot} {tot_p}"
         per_batch_calls = {"ms_per_step": round(wall_p / K * 1e3, 4), "value": round(float(tot_p[:4].sum()) / wall_p, 1),
                            "host_submit_ms_per_step": round(sub_p / K * 1e3, 4), "batches_in_flight": args.pipelines,
                            "note": "the same K steps with one set of library calls per mini-batch (sgl_sample_khop_multi as one "

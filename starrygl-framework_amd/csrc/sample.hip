@@ -316,6 +316,79 @@ __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
     }
 }
 
+// First index in [lo, hi) with ts[idx] >= key, by one lane.  (Wider searches - 8-ary per lane,
+// several probes per lane in the group search - were measured slower here: the searches are
+// bound by the number of scattered loads, not by the number of rounds.)
+__device__ __forceinline__ int64_t lane_lower_bound(const int64_t* __restrict__ ts, int64_t lo, int64_t hi, int64_t key) {
+    while (lo < hi) {
+        const int64_t mid = lo + ((hi - lo) >> 1);
+        if (ts[mid] < key) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
+// The counting pass with one lane per slot and a plain binary search per lane, for hops of so many slots that the
+// number of loads and of wavefronts in flight, not the length of one slot's chain, bound the launch.  (Several
+// slots per lane with their searches stepping together were measured slower: 116 and 122 us against 114 us per
+// 192 000-root two-hop call at two and four slots per lane.)
+__global__ __launch_bounds__(BLOCK) void count_lane_kernel(HopArgs a) {
+    __shared__ int32_t s_cnt[NWAVE];
+    __shared__ int32_t s_bad[NWAVE];
+    const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    const int64_t S = live_count(a.S_dev, a.S_max);
+    int64_t first, run;
+    block_run(S, a.align, &first, &run);
+    const int64_t end = first + run < S ? first + run : S;
+    const int64_t eq = a.equal_root_time ? 1 : 0;
+    int32_t sum = 0, nbad = 0;
+    for (int64_t slot = first + threadIdx.x; slot < end; slot += BLOCK) {
+        int64_t v, t;
+        load_slot(a, slot, &v, &t);
+        const int64_t rh = a.slot_hint != nullptr ? a.slot_hint[slot] : root_hint_of(a, slot);
+        if (v < 0 || v >= a.n) {
+            ++nbad;
+            a.w_start[slot] = 0;
+            a.w_len[slot] = 0;
+        } else {
+            const int64_t rs = a.row_ptr[v], re = a.row_ptr[v + 1];
+            // where the window ends: told by an index entry of the graph (every slot of a deeper hop), by the
+            // caller (an entry >= 0), or searched
+            const bool told = rh >= 0 || (a.slot_hint != nullptr && !a.hint_optional);
+            const int64_t hi = told ? clamp_to_row(rh, rs, re) : lane_lower_bound(a.ts, rs, re, t + eq);
+            const int64_t lo = a.allowed_offset >= 0 ? lane_lower_bound(a.ts, rs, hi, t - a.allowed_offset) : rs;
+            const int64_t len = hi - lo;
+            a.w_start[slot] = lo;
+            a.w_len[slot] = len;
+            sum += (int32_t)(len < a.k ? len : a.k);
+        }
+        if (a.derive) {
+            a.slot_node_out[slot] = v;
+            a.slot_ts_out[slot] = t;
+            if (a.mark != nullptr) mark_id(a, v);
+        }
+    }
+    for (int d = WAVE / 2; d > 0; d >>= 1) {
+        sum += __shfl(sum, wlane ^ d);
+        nbad += __shfl(nbad, wlane ^ d);
+    }
+    if (wlane == 0) {
+        s_cnt[wid] = sum;
+        s_bad[wid] = nbad;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int64_t tot = 0;
+        int32_t totb = 0;
+#pragma unroll
+        for (int i = 0; i < NWAVE; ++i) {
+            tot += s_cnt[i];
+            totb += s_bad[i];
+        }
+        a.block_sum[blockIdx.x] = tot;
+        a.block_bad[blockIdx.x] = totb;
+    }
+}
+
 // Prefix of the block sums at a granularity of CHUNK blocks, by one block (only
 // for grids beyond FUSED_PREFIX_MAX): chunk_off[c] = sum of block_sum[0 .. c*CHUNK).
 // Loads are coalesced and staged in LDS, thread t then owns the CHUNK consecutive
@@ -877,7 +950,7 @@ __device__ __forceinline__ void huge_window_picks(const HopArgs& a, int64_t slot
     }
 }
 
-template <int KP, int SLOTS>
+template <int KP, int SLOTS, int ROUNDS>
 __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
     static_assert(SLOTS % BLOCK == 0 && BLOCK % KP == 0 && KP % 4 == 0 && KP < WAVE, "chunk layout");
     constexpr int SPT = SLOTS / BLOCK;
@@ -1059,8 +1132,8 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
             }
             __syncthreads();
         }
-        // the chunk's edges, flat: up to ROUNDS per lane, every load issued before the first store
-        constexpr int ROUNDS = 4;
+        // the chunk's edges, flat: up to ROUNDS per lane, every load issued before the first store (a chunk of
+        // a deeper hop holds about as many edges as the block has lanes: more rounds only cost registers)
         for (int32_t x0 = threadIdx.x; x0 < total; x0 += ROUNDS * BLOCK) {
             Edge ed[ROUNDS];
             int64_t tslot[ROUNDS];
@@ -1175,7 +1248,7 @@ using HopKernel = void (*)(HopArgs);
 
 HopKernel count_fn(int G) {
     switch (G) {
-        case 1: return count_kernel<1>;
+        case 1: return count_lane_kernel;
         case 2: return count_kernel<2>;
         case 4: return count_kernel<4>;
         case 8: return count_kernel<8>;
@@ -1188,8 +1261,8 @@ HopKernel count_fn(int G) {
 HopKernel fill_fn(int G, bool uniform) {
     if (uniform) {
         switch (G) {
-            case 16: return fill_uniform_flat_kernel<16, 256>;
-            case 32: return fill_uniform_flat_kernel<32, 256>;
+            case 16: return fill_uniform_flat_kernel<16, 256, 2>;
+            case 32: return fill_uniform_flat_kernel<32, 256, 2>;
             default: return fill_kernel<64>;      // fanouts beyond 32: a wavefront per slot
         }
     }
@@ -1288,17 +1361,6 @@ __global__ void fused_clear_kernel(unsigned long long* desc, int n, int64_t* cou
         if (counts0_b != nullptr) counts0_b[2] = 0;
         if (counts1_b != nullptr) counts1_b[2] = 0;
     }
-}
-
-// First index in [lo, hi) with ts[idx] >= key, by one lane.  (Wider searches - 8-ary per lane,
-// several probes per lane in the group search - were measured slower here: the searches are
-// bound by the number of scattered loads, not by the number of rounds.)
-__device__ __forceinline__ int64_t lane_lower_bound(const int64_t* __restrict__ ts, int64_t lo, int64_t hi, int64_t key) {
-    while (lo < hi) {
-        const int64_t mid = lo + ((hi - lo) >> 1);
-        if (ts[mid] < key) lo = mid + 1; else hi = mid;
-    }
-    return lo;
 }
 
 // What a lane carries from the counting half of the single-launch sampler (fused2_count: windows and

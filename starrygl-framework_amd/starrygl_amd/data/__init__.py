@@ -1,2 +1,3 @@
 from .loader import EventBatchLoader  # noqa: F401
-from .pipeline import MiniBatch, MiniBatchPipeline, MiniBatchPipelinePool  # noqa: F401
+from .pipeline import (GroupedMiniBatch, MiniBatch, MiniBatchGroup, MiniBatchGroupPipeline,  # noqa: F401
+                       MiniBatchGroupPool, MiniBatchPipeline, MiniBatchPipelinePool)

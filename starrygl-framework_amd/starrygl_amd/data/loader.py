@@ -11,18 +11,22 @@ construction, and every batch then carries its values, so the sampler searches f
 """
 import torch
 
-from .pipeline import MiniBatchPipelinePool
+from .pipeline import MiniBatchGroupPool, MiniBatchPipelinePool
 
 
 class EventBatchLoader:
     def __init__(self, graph, src, dst, ts, batch_size, num_neg, layers, fanout, sample_type="recent",
                  node_tables=None, edge_tables=None, time_encoder=None, prefetch=4, negative_sampler=None,
-                 drop_last=True, **pipeline_kwargs):
+                 drop_last=True, sample_ahead=1, **pipeline_kwargs):
         """graph: `pyGraph.g` / `CUDAGraph`.  src/dst/ts: the events in training order (int64, any device).
         num_neg: negatives per batch (their times repeat the batch's event times).  negative_sampler: an
         object with `sample(num_samples, num_groups)` (NegSamplingSet); default: uniform over all nodes.
         prefetch: batches in flight (pipelines of the pool; a process has four hardware queues, and
-        pipelines that share one take turns).  Remaining keywords go to MiniBatchPipeline.
+        pipelines that share one take turns).  sample_ahead: mini-batches per pass of the library calls; above 1
+        the loader runs groups of that many consecutive batches through MiniBatchGroupPipeline objects (the
+        batched sampler and unique: a batch of a group costs a fraction of a batch sampled alone), `prefetch`
+        then counts groups in flight (two are enough), and a yielded batch stays valid until all batches of its
+        group and of the `prefetch - 2` following groups have been yielded.  Remaining keywords go to the pipelines.
         Only full batches are produced (every buffer of a pipeline is planned for one batch shape)."""
         if not drop_last:
             raise ValueError("EventBatchLoader produces full batches only (drop_last=True)")
@@ -43,9 +47,15 @@ class EventBatchLoader:
         t_rows = self.ts[: nb * B].view(nb, B)
         self._neg_ts = t_rows.repeat(1, (n_neg + B - 1) // B)[:, :n_neg].contiguous() if n_neg else t_rows[:, :0]
         self._neg_block, self._neg_at = None, 0
-        self.pool = MiniBatchPipelinePool(max(1, int(prefetch)), graph, 2 * self.B, self.num_neg, layers, fanout,
-                                          sample_type, node_tables=node_tables, edge_tables=edge_tables,
-                                          time_encoder=time_encoder, root_hints=True, **pipeline_kwargs)
+        self.sample_ahead = max(1, int(sample_ahead))
+        if self.sample_ahead > 1:
+            self.pool = MiniBatchGroupPool(max(1, int(prefetch)), graph, self.sample_ahead, 2 * self.B, self.num_neg, layers,
+                                           fanout, sample_type, node_tables=node_tables, edge_tables=edge_tables,
+                                           time_encoder=time_encoder, root_hints=True, **pipeline_kwargs)
+        else:
+            self.pool = MiniBatchPipelinePool(max(1, int(prefetch)), graph, 2 * self.B, self.num_neg, layers, fanout,
+                                              sample_type, node_tables=node_tables, edge_tables=edge_tables,
+                                              time_encoder=time_encoder, root_hints=True, **pipeline_kwargs)
 
     def __len__(self):
         return int(self.src.numel()) // self.B
@@ -68,9 +78,31 @@ class EventBatchLoader:
     def _submit(self, i):
         return self.pool.run(self._roots[i], self._root_ts[i], self._negatives(), self._neg_ts[i], root_hint=self._hint[i])
 
+    def _submit_group(self, i0, live):
+        neg = torch.stack([self._negatives() for _ in range(live)]) if self.num_neg else self._neg_ts[i0: i0 + live]
+        return self.pool.run(self._roots[i0: i0 + live], self._root_ts[i0: i0 + live], neg, self._neg_ts[i0: i0 + live],
+                             root_hint=self._hint[i0: i0 + live])
+
+    def _iter_groups(self):
+        depth, total, A = len(self.pool.pipes), len(self), self.sample_ahead
+        ahead = max(1, depth - 1)
+        queue, nxt = [], 0
+        while nxt < total and len(queue) < ahead:
+            live = min(A, total - nxt)
+            queue.append(self._submit_group(nxt, live)); nxt += live
+        while queue:
+            for mb in queue.pop(0).finalize():
+                yield mb
+            if nxt < total:
+                live = min(A, total - nxt)
+                queue.append(self._submit_group(nxt, live)); nxt += live
+
     def __iter__(self):
         """Yields the finalized MiniBatch of every full batch, in order.  A MiniBatch is valid until
         `prefetch` further batches have been submitted, i.e. until the next one is yielded."""
+        if self.sample_ahead > 1:
+            yield from self._iter_groups()
+            return
         depth, total = len(self.pool.pipes), len(self)
         # a yielded batch's pipeline is reused by the submission that follows `depth - 1` yields later, so one
         # pipeline is always kept free for the batch the consumer is looking at

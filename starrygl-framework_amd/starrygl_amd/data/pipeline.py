@@ -309,3 +309,230 @@ class MiniBatchPipelinePool:
         p = self.pipes[self._next]
         self._next = (self._next + 1) % len(self.pipes)
         return p.run(roots, root_ts, neg_roots, neg_ts, root_hint)
+
+
+class GroupedMiniBatch:
+    """One mini-batch of a `MiniBatchGroupPipeline` pass: views of the group's buffers (same attributes as a
+    finalized MiniBatch).  `root_start_ptr` / `root_end_ptr` of a hop count from the batch's first edge."""
+
+    final = True
+
+    def __init__(self, pipe, b, seg, uoff):
+        p, self._p, self.index = pipe, pipe, b
+        L = p.layers
+        self.S = [seg[l][b + 1] - seg[l][b] for l in range(L)]
+        self.E = [seg[l + 1][b + 1] - seg[l + 1][b] for l in range(L)]
+        self.num_unique = uoff[b + 1] - uoff[b]
+        s0, s1 = seg[0][b], seg[0][b + 1]
+        self.slot_node, self.slot_ts, self.slot_local = p.in_node[s0:s1], p.in_ts[s0:s1], p.local[0][s0:s1]
+        self.nid_mapper = p.ubuf[uoff[b]: uoff[b + 1]]
+        self.hops = []
+        kr = p.kb.queries[0]
+        for l, h in enumerate(kr.hops):
+            a0, a1, e0, e1 = seg[l][b], seg[l][b + 1], seg[l + 1][b], seg[l + 1][b + 1]
+            self.hops.append(dict(root_start_ptr=h.root_start_ptr[a0: a1 + 1] - e0, root_end_ptr=h.root_end_ptr[a0: a1] - e0,
+                                  neighbors=h.neighbors[e0:e1], neighbors_local=p.local[1 + l][e0:e1],
+                                  neighbors_ts=h.neighbors_ts[e0:e1], neighbors_eid=h.neighbors_eid[e0:e1],
+                                  neighbors_dt=h.neighbors_dt[e0:e1]))
+        self.node_data = {k: v[uoff[b]: uoff[b + 1]] for k, v in p.node_out.items()}
+        self.node_ts = {k: v[uoff[b]: uoff[b + 1]] for k, v in p.node_ts_out.items()}
+        self.edge_data = [{k: v[l][seg[l + 1][b]: seg[l + 1][b + 1]] for k, v in p.edge_out.items()} for l in range(L)]
+        self.time_feat = ([t[seg[l + 1][b]: seg[l + 1][b + 1]] for l, t in enumerate(p.te_out)] if p.te_out else None)
+
+    def finalize(self):
+        return self
+
+    def blocks(self, self_loop=True):
+        """Message-flow blocks, outermost hop first, local node ids (as MiniBatch.blocks)."""
+        hp = self._p.hp
+        last_nodes, last_ts = self.slot_local, self.slot_ts
+        out = []
+        for l, h in enumerate(self.hops):
+            S, E, n_prev = self.S[l], self.E[l], int(last_nodes.numel())
+            dst_off = n_prev - S if self_loop else 0
+            num_dst = n_prev if self_loop else S
+            src_off = num_dst if self_loop else 0
+            counts = torch.tensor([S, E, 0], dtype=torch.int64, device=last_nodes.device)
+            indptr, indices, _ = hp.block_build(h["root_start_ptr"].contiguous(), counts, S, E, dst_off, src_off)
+            b = Block(indptr, indices, src_off + E, num_dst)
+            if self_loop:
+                b.srcdata["nid"] = torch.cat([last_nodes, h["neighbors_local"]])
+                b.srcdata["ts"] = torch.cat([last_ts, h["neighbors_ts"]])
+            else:
+                b.srcdata["nid"], b.srcdata["ts"] = h["neighbors_local"], h["neighbors_ts"]
+            b.edata["eid"], b.edata["dt"] = h["neighbors_eid"], h["neighbors_dt"]
+            for k, v in self.edge_data[l].items():
+                b.edata[k] = v
+            if self.time_feat is not None:
+                b.edata["time_feat"] = self.time_feat[l]
+            last_nodes, last_ts = b.srcdata["nid"], b.srcdata["ts"]
+            out.append(b)
+        out.reverse()
+        return out
+
+
+class MiniBatchGroup:
+    """Result of one `MiniBatchGroupPipeline.run`: `finalize()` reads the segment table, the unique offsets and
+    the counts once (one synchronisation for the whole group) and returns the per-batch views in order."""
+
+    def __init__(self, pipe, live):
+        self._p, self.live, self.batches = pipe, live, None
+
+    def finalize(self):
+        if self.batches is None:
+            p = self._p
+            if p._done is not None:
+                p._done.synchronize()
+            # (the k-hop buffers are reused by the next pass: read the tables, leave the buffers at full size)
+            counts = p.kb.counts.tolist()
+            for l in range(p.layers):
+                check_sample_bad(counts[3 * l + 2])
+            seg, uoff = p.kb.seg[0].tolist(), p.uoff.tolist()
+            self.batches = [GroupedMiniBatch(p, b, seg, uoff) for b in range(self.live)]
+        return self.batches
+
+
+class MiniBatchGroupPipeline:
+    """B mini-batches per pass of the library calls: `sgl_sample_khop_batched` over the concatenated root slots,
+    `sgl_unique_compact_batched` (a local-id space per batch), one gather launch per 8 row lists over all batches'
+    rows, one time-encoding launch per hop.  What a loader that samples B batches ahead runs instead of B
+    MiniBatchPipeline passes: the reference keeps several windows queued (AsyncGraphBlob, graph.py:274-293;
+    prefetch_factor, test/test.py:212-221) but samples them one by one.  A 12 000-root batch alone is bound by
+    launch floors and chains of dependent loads; 16 of them per pass are bound by throughput (the most-recent
+    2-hop sampler: 6 us per batch instead of 25).  Same constructor arguments as MiniBatchPipeline after
+    `batches`; the remap is always the dense one."""
+
+    def __init__(self, graph, batches, num_pos_slots, num_neg, layers, fanout, sample_type="recent", node_tables=None,
+                 edge_tables=None, time_encoder=None, allowed_offset=-1, equal_root_time=False, keep_root_time=False,
+                 seed=0, use_graph=True, stream=None, root_hints=False):
+        self.g = graph
+        self.hp = hp = graph._hp
+        self.dev = hp.be.device
+        self.B, self.layers, self.fanout = int(batches), int(layers), int(fanout)
+        self.S_pos, self.N_neg = int(num_pos_slots), int(num_neg)
+        self.S0 = self.S_pos + self.N_neg
+        B, S0 = self.B, self.S0
+        self.p = hp.params(sample_type, fanout, allowed_offset, equal_root_time, keep_root_time, seed=seed)
+        self.node_tables, self.edge_tables = dict(node_tables or {}), dict(edge_tables or {})
+        if time_encoder is not None and not isinstance(time_encoder, tuple):
+            time_encoder = (time_encoder.w.weight.detach().reshape(-1).contiguous(),
+                            time_encoder.w.bias.detach().contiguous())
+        self.te = time_encoder
+        be = hp.be
+        self.in_node, self.in_ts = be.empty(B * S0), be.empty(B * S0)
+        self.in_hint = torch.full((B * S0,), -1, dtype=torch.int64, device=self.dev) if root_hints else None
+        self.ptr_host = [b * S0 for b in range(B + 1)]
+        self.ptr = torch.tensor(self.ptr_host, dtype=torch.int64, device=self.dev)
+        self._ptr_by_live = {B: self.ptr.clone()}
+        self.kb = hp.khop_batched_buffers(B * S0, B, self.layers, self.fanout, 1)
+        caps = [B * S0] + [B * S0 * self.fanout ** (l + 1) for l in range(self.layers)]
+        self.local = [be.empty(c) for c in caps]
+        self.ucap = min(sum(caps), B * graph._n)
+        self.ubuf, self.uoff = be.empty(max(self.ucap, 1)), be.zeros(B + 1)
+        self.state = hp.remap_batched_state(graph._n, B)
+        self.uws = be.empty(max(int(hp.lib.unique_batched_workspace_bytes(graph._n, B)), 256), "u8")
+        self.node_out, self.node_ts_out, self.edge_out = {}, {}, {}
+        for name, c in self.node_tables.items():
+            self.node_out[name] = torch.empty((self.ucap, c.row_bytes), dtype=torch.uint8, device=self.dev)
+            if c.ts_hot or c.ts_cold:
+                self.node_ts_out[name] = be.empty(self.ucap)
+        for name, c in self.edge_tables.items():
+            self.edge_out[name] = [torch.empty((caps[l + 1], c.row_bytes), dtype=torch.uint8, device=self.dev)
+                                   for l in range(self.layers)]
+        self.te_out = None
+        if self.te is not None:
+            dim = int(self.te[0].numel())
+            self.te_out = [torch.empty((caps[l + 1], dim), dtype=torch.float32, device=self.dev) for l in range(self.layers)]
+        self._views = {}
+        self.use_graph, self._graph = use_graph, None
+        self._plans, self._slow = None, []
+        self.stream = stream
+        self._done = torch.cuda.Event() if stream is not None else None
+
+    view = MiniBatchPipeline.view
+
+    def _chain(self):
+        hp, kr = self.hp, self.kb.queries[0]
+        hp.sample_khop_batched(self.g._g, self.in_node, self.in_ts, self.ptr, self.layers, [self.p], out=self.kb,
+                               slot_hint=self.in_hint)
+        arrays = [self.in_node] + [h.neighbors for h in kr.hops]
+        hp.unique_compact_batched(arrays, [self.kb.seg[0, l] for l in range(self.layers + 1)], self.state,
+                                  out_arrays=self.local, unique_out=self.ubuf, U_off=self.uoff, workspace=self.uws,
+                                  finalize=False)
+        if self._plans is None:
+            n_u = self.uoff[self.B: self.B + 1]
+            segs = [(c, self.ubuf, self.node_out[name], self.node_ts_out.get(name), n_u)
+                    for name, c in self.node_tables.items()]
+            segs += [(c, h.neighbors_eid, self.edge_out[name][l], None, h.counts[1:2])
+                     for l, h in enumerate(kr.hops) for name, c in self.edge_tables.items()]
+            fast = [s for s in segs if s[0].row_bytes % 16 == 0]
+            self._slow = [s for s in segs if s[0].row_bytes % 16 != 0]
+            self._plans = [hp.gather_plan(fast[i: i + 8]) for i in range(0, len(fast), 8)]
+        for plan in self._plans:
+            hp.gather_multi(plan)
+        for c, ids, out, out_ts, n_dev in self._slow:
+            hp.gather(c, ids, out, out_ts=out_ts, N_dev=n_dev)
+        if self.te is not None:
+            for l, h in enumerate(kr.hops):
+                hp.time_encode(h.neighbors_dt, self.te[0], self.te[1], out=self.te_out[l], N_dev=h.counts[1:2])
+
+    def run(self, roots, root_ts, neg_roots=None, neg_ts=None, root_hint=None):
+        """Enqueue one group (asynchronous).  roots / root_ts: [live, S_pos]; neg_roots / neg_ts: [live, N_neg];
+        root_hint: [live, S_pos] window ends for a pipeline built with root_hints=True.  live <= B batches (a
+        stream's last group may be short: the remaining batches of the pass are empty)."""
+        live = int(roots.shape[0]) if roots.dim() == 2 else -1
+        if live < 1 or live > self.B or tuple(roots.shape) != (live, self.S_pos) or tuple(root_ts.shape) != (live, self.S_pos):
+            raise ValueError(f"this pipeline was planned for up to {self.B} batches of {self.S_pos} positive slots")
+        if (self.in_hint is None) != (root_hint is None) or (root_hint is not None and tuple(root_hint.shape) != (live, self.S_pos)):
+            raise ValueError("root_hint goes with a pipeline built with root_hints=True, one entry per positive slot")
+        if self.N_neg and (neg_roots is None or tuple(neg_roots.shape) != (live, self.N_neg) or tuple(neg_ts.shape) != (live, self.N_neg)):
+            raise ValueError(f"this pipeline was planned for {self.N_neg} negatives per batch")
+        if self.stream is not None:
+            with torch.cuda.stream(self.stream):
+                out = self._run(live, roots, root_ts, neg_roots, neg_ts, root_hint)
+                self._done.record(self.stream)
+            return out
+        return self._run(live, roots, root_ts, neg_roots, neg_ts, root_hint)
+
+    def _run(self, live, roots, root_ts, neg_roots, neg_ts, root_hint):
+        B, S0, Sp = self.B, self.S0, self.S_pos
+        rows = lambda t: t.view(B, S0)[:live]
+        dsts, srcs = [rows(self.in_node)[:, :Sp], rows(self.in_ts)[:, :Sp]], [roots, root_ts]
+        if root_hint is not None:
+            dsts.append(rows(self.in_hint)[:, :Sp]); srcs.append(root_hint)
+        if self.N_neg:
+            dsts += [rows(self.in_node)[:, Sp:], rows(self.in_ts)[:, Sp:]]; srcs += [neg_roots, neg_ts]
+        for d, t in zip(dsts, srcs):
+            d.copy_(t, non_blocking=True)
+        if live not in self._ptr_by_live:
+            self._ptr_by_live[live] = torch.tensor([min(b, live) * S0 for b in range(B + 1)], dtype=torch.int64, device=self.dev)
+        self.ptr.copy_(self._ptr_by_live[live], non_blocking=True)
+        if not self.use_graph:
+            self._chain()
+        elif self._graph is None:
+            self._chain()
+            torch.cuda.current_stream(self.dev).synchronize()
+            g = torch.cuda.CUDAGraph()
+            with graph_capture(g):
+                self._chain()
+            self._graph = g
+            g.replay()
+        else:
+            self._graph.replay()
+        return MiniBatchGroup(self, live)
+
+
+class MiniBatchGroupPool:
+    """`n` MiniBatchGroupPipeline objects on streams of their own, taking the groups in turn (as MiniBatchPipelinePool)."""
+
+    def __init__(self, n, graph, *args, **kwargs):
+        if n < 1:
+            raise ValueError("a pool needs at least one pipeline")
+        dev = graph._hp.be.device
+        self.pipes = [MiniBatchGroupPipeline(graph, *args, stream=st, **kwargs) for st in bound_streams(n, dev)]
+        self._next = 0
+
+    def run(self, *args, **kwargs):
+        p = self.pipes[self._next]
+        self._next = (self._next + 1) % len(self.pipes)
+        return p.run(*args, **kwargs)

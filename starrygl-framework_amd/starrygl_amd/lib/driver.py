@@ -855,7 +855,8 @@ class KHopBatched:
         self.counts, self.final, self.seg_host = counts, False, None
 
     def finalize(self):
-        """One synchronising read of the segment table and the counts; narrows every query's arrays."""
+        """One synchronising read of the segment table and the counts; narrows every query's arrays (for good:
+        buffers that a later call is to reuse are read through `seg` and `counts` instead, without finalizing)."""
         if not self.final:
             be = self.hp.be
             self.seg_host = be.tolist(self.seg)

@@ -199,3 +199,97 @@ def test_event_batch_loader(oracle, hot, prefetch):
             assert np.array_equal(np_of(mb.hops[l]["neighbors_eid"]), h.neighbors_eid)
         seen += 1
     assert seen == len(loader)
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+@pytest.mark.parametrize("sample_type", ["recent", "uniform"])
+def test_group_pipeline_matches_oracle(oracle, hot, use_graph, sample_type):
+    """B mini-batches per pass: every batch of a group against the oracle - the batched sampler over the group's
+    slots (the uniform strategy is keyed by the slot's place in the call), np.unique per batch, rows, time encoding,
+    blocks - for full groups, a short last group and consecutive passes on the same buffers."""
+    from starrygl_amd.data import MiniBatchGroupPipeline
+    from starrygl_amd.lib.libstarrygl_comm import from_edge_index
+    n, m, EV, NEG, B = 4000, 80_000, 120, 70, 5
+    src, dst, ts, eid = synth.graph_stream(n, m, 1.15, 500_000, 21)
+    hg = host_graph(oracle, n, src, dst, ts, eid)
+    g = from_edge_index(n, 1, *(torch.from_numpy(x) for x in (src, dst, ts, eid)))
+    rng = np.random.default_rng(2)
+    mem = rng.standard_normal((n, 100)).astype(np.float32)
+    mem_ts = rng.integers(0, 10**6, n).astype(np.int64)
+    efeat = rng.standard_normal((m, 172)).astype(np.float32)
+    c_mem = hot.cache(400, to_dev(hot, mem, "f32"), ts_hot=to_dev(hot, mem_ts))
+    c_ef = hot.cache(688, to_dev(hot, efeat, "f32"))
+    w = (1.0 / 10 ** np.linspace(0, 9, 100, dtype=np.float32)).astype(np.float32)
+    bias = rng.standard_normal(100).astype(np.float32)
+    pipe = MiniBatchGroupPipeline(g, B, 2 * EV, NEG, 2, 5, sample_type, node_tables={"mem": c_mem}, edge_tables={"f": c_ef},
+                                  time_encoder=(to_dev(hot, w, "f32"), to_dev(hot, bias, "f32")), seed=9, use_graph=use_graph)
+    pipe.view("mem", torch.float32).view("f", torch.float32)
+    for live in (B, B, 2, B):
+        bts = [synth.link_batch(src, dst, ts, lo, lo + EV, n, NEG, rng) for lo in rng.integers(1000, m - EV, live)]
+        stack = lambda i: to_dev(hot, np.stack([b[i] for b in bts]))
+        group = pipe.run(stack(0), stack(2), stack(3), stack(4)).finalize()
+        assert len(group) == live
+        node = np.concatenate([np.concatenate([b[0], b[3]]) for b in bts])
+        t = np.concatenate([np.concatenate([b[2], b[4]]) for b in bts])
+        ptr = np.arange(live + 1, dtype=np.int64) * (2 * EV + NEG)
+        want = oracle.sample_khop_batched(hg, node, t, ptr, 2, [oracle.params(sample_type, 5, seed=9)], finalize=True)
+        seg, wq = np.asarray(want.seg_host[0]), want.queries[0]
+        for b, mb in enumerate(group):
+            assert mb.S[0] == 2 * EV + NEG and mb.E == [int(seg[l + 1][b + 1] - seg[l + 1][b]) for l in range(2)]
+            ids = [node[seg[0][b]: seg[0][b + 1]]] + [wq.hops[l].neighbors[seg[l + 1][b]: seg[l + 1][b + 1]] for l in range(2)]
+            uniq, inv = np.unique(np.concatenate(ids), return_inverse=True)
+            assert np.array_equal(np_of(mb.nid_mapper), uniq) and mb.num_unique == uniq.size, (live, b)
+            assert np.array_equal(np_of(mb.slot_local), inv[: ids[0].size])
+            assert np.array_equal(np_of(mb.node_data["mem"]), mem[uniq]) and np.array_equal(np_of(mb.node_ts["mem"]), mem_ts[uniq])
+            off = ids[0].size
+            for l in range(2):
+                lo, hi = seg[l + 1][b], seg[l + 1][b + 1]
+                h = wq.hops[l]
+                assert np.array_equal(np_of(mb.hops[l]["neighbors_eid"]), h.neighbors_eid[lo:hi])
+                assert np.array_equal(np_of(mb.hops[l]["neighbors_local"]), inv[off: off + hi - lo])
+                off += hi - lo
+                assert np.array_equal(np_of(mb.hops[l]["root_start_ptr"]), h.root_start_ptr[seg[l][b]: seg[l][b + 1] + 1] - lo)
+                assert np.array_equal(np_of(mb.edge_data[l]["f"]), efeat[h.neighbors_eid[lo:hi]])
+                y = oracle.time_encode(h.neighbors_dt[lo:hi], w, bias)
+                assert hi == lo or np.abs(np_of(mb.time_feat[l]) - y).max() <= 1e-6
+            blocks = mb.blocks()
+            assert [bk.num_edges() for bk in blocks] == mb.E[::-1]
+            assert blocks[0].num_dst_nodes() == mb.S[0] + mb.E[0]
+    with pytest.raises(ValueError):
+        pipe.run(stack(0)[:, :5], stack(2)[:, :5], stack(3), stack(4))
+
+
+@pytest.mark.parametrize("prefetch,ahead", [(2, 4), (3, 7)])
+def test_event_batch_loader_sampling_ahead(oracle, hot, prefetch, ahead):
+    """The loader with `sample_ahead` batches per pass: every yielded batch equals the oracle's most-recent sample
+    of its own events and negatives (the most-recent strategy does not depend on how batches are grouped)."""
+    from starrygl_amd.data import EventBatchLoader
+    from starrygl_amd.lib.libstarrygl_comm import from_edge_index
+    n, m, B, NEG = 2500, 50_000, 200, 150
+    src, dst, ts, eid = synth.graph_stream(n, m, 1.15, 30_000, 31)
+    order = np.argsort(ts, kind="stable")
+    src, dst, ts, eid = src[order], dst[order], ts[order], eid[order]
+    hg = host_graph(oracle, n, src, dst, ts, eid)
+    g = from_edge_index(n, 1, *(torch.from_numpy(x) for x in (src, dst, ts, eid)))
+    feat = np.random.default_rng(2).standard_normal((n, 100)).astype(np.float32)
+    lo_ev = 44_000                                   # 6000 events = 30 batches: groups of 4 or 7, the last one short
+    loader = EventBatchLoader(g, src[lo_ev:], dst[lo_ev:], ts[lo_ev:], B, NEG, 2, 5, "recent",
+                              node_tables={"x": hot.cache(400, to_dev(hot, feat, "f32"))}, prefetch=prefetch, sample_ahead=ahead)
+    for p in loader.pool.pipes:
+        p.view("x", torch.float32)
+    seen = 0
+    for i, mb in enumerate(loader):
+        lo = lo_ev + i * B
+        roots = np.concatenate([src[lo: lo + B], dst[lo: lo + B]])
+        root_ts = np.concatenate([ts[lo: lo + B], ts[lo: lo + B]])
+        assert np.array_equal(np_of(mb.slot_node)[: 2 * B], roots)
+        neg, neg_ts = np_of(mb.slot_node)[2 * B:], np_of(mb.slot_ts)[2 * B:]
+        assert np.array_equal(neg_ts, np.resize(ts[lo: lo + B], NEG))
+        want = oracle.sample_khop(hg, roots, np.arange(2 * B + 1, dtype=np.int64), root_ts, neg, neg_ts, 2, oracle.params("recent", 5))
+        assert mb.E == [h.E for h in want.hops]
+        _, uniq, _ = oracle.unique_compact([want.slot_node0] + [h.neighbors for h in want.hops], _abi.UNIQUE_SORTED, None, True)
+        assert np.array_equal(np_of(mb.nid_mapper), uniq) and np.array_equal(np_of(mb.node_data["x"]), feat[uniq])
+        for l, h in enumerate(want.hops):
+            assert np.array_equal(np_of(mb.hops[l]["neighbors_eid"]), h.neighbors_eid)
+        seen += 1
+    assert seen == len(loader) == 30
