@@ -138,10 +138,12 @@ int32_t sgl_tcsr_validate(const sgl_tcsr* g, void* workspace,
 #define SGL_SAMPLE_UNIFORM 1 /* "uniform" : k distinct window edges, uniform  */
 
 /* Largest fanout the uniform strategy accepts (a slot's picks are kept in the
- * registers of one wavefront up to 64, in its block's LDS beyond).  The recent
- * strategy has no limit; the reference has none for either
- * (uniform_sample_single_hop_kernel, sample.cu.hpp:783-827). */
+ * LDS of its block).  The most-recent strategy copies runs: its limit is what
+ * the 32-bit edge offsets inside a block's chunk of 512 slots can hold.  The
+ * reference has no limit for either (uniform_sample_single_hop_kernel,
+ * sample.cu.hpp:783-827); SGL_ENOTSUP beyond. */
 #define SGL_UNIFORM_MAX_FANOUT 1024
+#define SGL_RECENT_MAX_FANOUT  (1 << 21)
 
 /* Arguments of Graph::sample_src_in_chunks_khop (sample.cu.hpp:1532-1534,
  * export.cu:194-201).  Candidate window of a slot (v, t):

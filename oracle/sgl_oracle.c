@@ -309,6 +309,8 @@ static int32_t hop_impl(const sgl_tcsr* g, const int64_t* slot_node,
     if (p->fanout < 0) return fail(SGL_EINVAL, "sample_hop: fanout < 0");
     if (p->type == SGL_SAMPLE_UNIFORM && p->fanout > SGL_UNIFORM_MAX_FANOUT)
         return fail(SGL_ENOTSUP, "uniform fanout > SGL_UNIFORM_MAX_FANOUT");
+    if (p->type == SGL_SAMPLE_RECENT && p->fanout > SGL_RECENT_MAX_FANOUT)
+        return fail(SGL_ENOTSUP, "recent fanout > SGL_RECENT_MAX_FANOUT");
     int64_t S = S_dev ? *S_dev : S_max;
     if (S > S_max || S > out->capacity_slots) return fail(SGL_ENOMEM, "sample_hop: slots > capacity");
     if (out->capacity_edges < out->capacity_slots * (int64_t)p->fanout)

@@ -758,6 +758,7 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
 // (slots of deeper hops hold two edges on average on a power-law graph: a group of 8 lanes per slot left six idle),
 // and the stores of a block-iteration are one contiguous piece per output array.
 constexpr int FLAT_SLOTS = 2 * BLOCK;
+static_assert((int64_t)FLAT_SLOTS * SGL_RECENT_MAX_FANOUT <= INT32_MAX, "a chunk's edge offsets are 32-bit");
 __global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
     __shared__ int64_t s_red[NWAVE];
     __shared__ int32_t s_redb[NWAVE];
@@ -1218,6 +1219,9 @@ int32_t check_params(const sgl_sample_params* p) {
         return fail(SGL_EINVAL, "sample: bad mark_universe");
     if (p->type == SGL_SAMPLE_UNIFORM && p->fanout > SGL_UNIFORM_MAX_FANOUT)
         return fail(SGL_ENOTSUP, "uniform fanout %d > %d", p->fanout, SGL_UNIFORM_MAX_FANOUT);
+    // (fill_flat_kernel keeps the edge offsets of a chunk of FLAT_SLOTS slots in 32 bits)
+    if (p->type == SGL_SAMPLE_RECENT && p->fanout > SGL_RECENT_MAX_FANOUT)
+        return fail(SGL_ENOTSUP, "recent fanout %d > %d", p->fanout, SGL_RECENT_MAX_FANOUT);
     return SGL_OK;
 }
 

@@ -33,7 +33,8 @@ struct TEArgs {
     int32_t rpb;
 };
 
-// cos of an fp32 argument, accurate to < 1 ulp of the fp32 result for every
+// cos of an fp32 argument with an absolute error of at most 1.2e-7 (one ulp at 1.0; near the zeros of the
+// cosine, where the result is small, that is many ulps of the result) for every
 // magnitude the path produces (|a| up to 2^40 and beyond): the argument is reduced
 // in double precision by multiples of pi (two-constant Cody-Waite, exact through
 // FMA) to r in [-pi/2, pi/2]; then cos(r) = 1 - 2 sin^2(r/2) with one odd

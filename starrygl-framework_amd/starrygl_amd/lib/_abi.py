@@ -10,6 +10,7 @@ ABI_VERSION = 7
 SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
 UNIFORM_MAX_FANOUT = 1024
+RECENT_MAX_FANOUT = 1 << 21
 STATIC_HOP_MAX_SLOTS = 65536
 BATCH_MAX = 64
 UNIQUE_SORTED, UNIQUE_GROUPED, UNIQUE_PREMARKED, UNIQUE_MULTI_LAUNCH = 0, 1, 0x100, 0x200

@@ -152,7 +152,7 @@ def check_unique_total(u_total):
     an earlier tile (bounded wait): the result is void and the remap state has to be re-initialised."""
     if u_total == (1 << 63) - 1:
         raise RuntimeError("unique_compact: the result is void (a numbering pass gave up waiting, or a hashed state's "
-                           "capacity was exceeded); re-initialise the remap state")
+                           "capacity was exceeded); re-initialise the remap state (HotPath.remap_reinit)")
 
 
 class HotPath:
@@ -415,7 +415,8 @@ class HotPath:
     def sample_khop_multi(self, g, roots, ts_ptr, root_ts, neg_roots, neg_ts, layers, params, outs):
         """Several k-hop calls (params[q] -> outs[q], buffers of khop_buffers) over the same roots
         in one library call; a most-recent and a uniform 2-hop call share one launch.  The results
-        are not finalized; they share the hop-0 slot arrays of outs[0]."""
+        are not finalized; they share the hop-0 slot arrays of outs[0].  The inputs must stay unchanged
+        until the results have been finalized (a poisoned call is re-issued from them, see `recover` below)."""
         self._chk("i64", roots=roots, ts_ptr=ts_ptr, root_ts=root_ts, neg_roots=neg_roots, neg_ts=neg_ts)
         be, Q = self.be, len(params)
         R, S_pos, N_neg = int(roots.shape[0]), int(root_ts.shape[0]), int(neg_roots.shape[0])
@@ -432,13 +433,31 @@ class HotPath:
         if getattr(head, "ws_multi", None) is None or be.nbytes(head.ws_multi) < need:
             head.ws_multi = be.empty(max(need, 256), "u8")
         structs = (HopOut * max(Q * layers, 1))(*[o.struct for res in outs for o in res.hops])
-        pa = (_abi.SampleParams * max(Q, 1))(*params)
-        self._ck(self.lib.sample_khop_multi(C.byref(g.view), R, be.ptr(roots), be.ptr(ts_ptr), S_pos,
-                                            be.ptr(root_ts), N_neg, be.ptr(neg_roots), be.ptr(neg_ts),
-                                            layers, Q, pa, be.ptr(head.slot_node0), be.ptr(head.slot_ts0),
-                                            structs, be.ptr(head.ws_multi), be.nbytes(head.ws_multi), be.stream()))
+
+        def launch(ps):
+            pa = (_abi.SampleParams * max(Q, 1))(*ps)
+            self._ck(self.lib.sample_khop_multi(C.byref(g.view), R, be.ptr(roots), be.ptr(ts_ptr), S_pos,
+                                                be.ptr(root_ts), N_neg, be.ptr(neg_roots), be.ptr(neg_ts),
+                                                layers, Q, pa, be.ptr(head.slot_node0), be.ptr(head.slot_ts0),
+                                                structs, be.ptr(head.ws_multi), be.nbytes(head.ws_multi), be.stream()))
+
+        launch(params)
+
+        # Should a block of the shared single launch have given up its bounded wait, reading any of the results
+        # re-issues the WHOLE call once through the launch-per-hop route (a pair shares one kernel: both queries are
+        # void), after initialising the remap states that the queries were recording ids in.  The re-issue reads the
+        # input arrays again: they must hold this call's batch until the results have been finalized.
+        def recover():
+            for res in outs:
+                res._recover = None
+            for p in params:
+                self._reinit_marked(p)
+            launch([self.multi_launch(p) for p in params])
+
         for res in outs:
             res.slot_node0, res.slot_ts0, res.S0_live = head.slot_node0, head.slot_ts0, S0
+            res._recover = recover
+            res.final = False
         return outs
 
     # ---------------------------------------------- several batches per call
@@ -537,6 +556,20 @@ class HotPath:
         st = self.be.empty(max(nbytes, 8), "u8")
         self._ck(self.lib.remap_init(self.be.ptr(st), nbytes, universe, self.be.stream()))
         return RemapState(st, universe)
+
+    def remap_reinit(self, state):
+        """Initialise a remap state again in place (dense, hashed or batched): what a caller does after a call on
+        it reported a void result - a numbering pass that gave up its bounded wait, or a hashed state whose epoch
+        outgrew its capacity (that flag is sticky: every later call on the state reports it until this)."""
+        be = self.be
+        if isinstance(state, HashedRemapState):
+            self._ck(self.lib.remap_hashed_init(be.ptr(state.buf), be.nbytes(state.buf), state.universe, be.stream()))
+        elif getattr(state, "B", None) is not None:
+            self._ck(self.lib.remap_batched_init(be.ptr(state.buf), be.nbytes(state.buf), state.universe, state.B, be.stream()))
+        else:
+            self._ck(self.lib.remap_init(be.ptr(state.buf), be.nbytes(state.buf), state.universe, be.stream()))
+        state.count_bound = 0
+        return state
 
     def remap_hashed_state(self, capacity):
         """Persistent hash-set remap state for arbitrary non-negative ids: `capacity` is the largest

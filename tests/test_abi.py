@@ -39,6 +39,10 @@ def test_abi_version_and_host_side_errors():
     assert lib.sample_hop(None, None, None, 0, None, C.byref(p), None, None, 0, None) == _abi.SGL_EINVAL
     p.type, p.fanout = _abi.SAMPLE_UNIFORM, _abi.UNIFORM_MAX_FANOUT + 1
     assert lib.sample_hop(C.byref(g), None, None, 0, None, C.byref(p), None, None, 0, None) == _abi.SGL_ENOTSUP
+    p.type, p.fanout = _abi.SAMPLE_RECENT, _abi.RECENT_MAX_FANOUT + 1     # beyond what a chunk's 32-bit edge offsets hold
+    assert lib.sample_hop(C.byref(g), None, None, 0, None, C.byref(p), None, None, 0, None) == _abi.SGL_ENOTSUP
+    p.fanout = _abi.RECENT_MAX_FANOUT
+    assert lib.sample_hop(C.byref(g), None, None, 0, None, C.byref(p), None, None, 0, None) == _abi.SGL_EINVAL   # (out is NULL)
     c = _abi.Cache(10, 6, -1, None, 0, None, 8, 10, None, None, None)
     assert lib.gather(C.byref(c), 8, 1, None, 8, None, None, None) == _abi.SGL_EINVAL   # row_bytes % 4
     assert lib.time_encode(8, 5, 1, None, 8, 8, 4, 8, None) == _abi.SGL_EINVAL           # bad dtype

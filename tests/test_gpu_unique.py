@@ -212,8 +212,17 @@ def test_hashed_state_reports_an_outgrown_capacity(hot):
         hot.unique_compact([to_dev(hot, np.arange(200, dtype=np.int64) * 7 + 1)], _abi.UNIQUE_SORTED, sh, False)
     with pytest.raises(RuntimeError, match="void"):
         hot.unique_compact([a], _abi.UNIQUE_SORTED, sh, True)
-    # a fresh state works again
+    with pytest.raises(RuntimeError, match="remap_reinit"):      # the message names the way out
+        hot.unique_compact([a], _abi.UNIQUE_SORTED, sh, True)
+    # the same state, initialised again in place, works again; so does a fresh one
+    lh, uh, (th, _) = hot.unique_compact([a], _abi.UNIQUE_SORTED, hot.remap_reinit(sh), True)
+    assert th == 900 and np.array_equal(np_of(lh[0]), np.arange(900))
     lh, uh, (th, _) = hot.unique_compact([a], _abi.UNIQUE_SORTED, hot.remap_hashed_state(1000), True)
+    assert th == 900 and np.array_equal(np_of(lh[0]), np.arange(900))
+    # remap_reinit picks the initialiser by the kind of state
+    d = hot.remap_state(5000)
+    hot.unique_compact([a], _abi.UNIQUE_SORTED, d, True)
+    lh, uh, (th, _) = hot.unique_compact([a], _abi.UNIQUE_SORTED, hot.remap_reinit(d), False)
     assert th == 900 and np.array_equal(np_of(lh[0]), np.arange(900))
 
 

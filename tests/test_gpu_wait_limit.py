@@ -133,3 +133,47 @@ def test_pipeline_batch_is_reissued_after_a_give_up(oracle, hot):
     assert np.array_equal(np_of(mb.nid_mapper), uniq)
     if not recovered:
         pytest.skip("no block ever found a descriptor missing: the error path was not reached")
+
+
+def test_pair_call_gives_up_cleanly_and_the_whole_call_is_reissued(oracle, hot):
+    """The most-recent + uniform pair in one launch (sgl_sample_khop_multi) under a wait limit of one poll: whichever
+    query was poisoned, finalizing re-issues the whole call with this call's inputs and parameters - also when the
+    same buffers served another call before - and re-initialises the remap state the recent query marks ids in."""
+    _, g, batch = _hub_graph(oracle, hot)
+    dg = mirror_graph(hot, g)
+    args = [to_dev(hot, x) for x in batch]
+    S0 = batch[0].shape[0]
+    state = hot.remap_state(g.n)
+    p_rec, p_uni = hot.marking(hot.params("recent", 10), state), hot.params("uniform", 10, seed=4)
+    want = {st: oracle.sample_khop(g, *batch, 2, oracle.params(st, 10, seed=4)) for st in ("recent", "uniform")}
+    ids = [want["recent"].slot_node0] + [h.neighbors for h in want["recent"].hops]
+    want_u, want_inv = np.unique(np.concatenate(ids), return_inverse=True)
+    # an earlier, different call on the same buffers leaves its own recovery closure behind
+    other = [to_dev(hot, x) for x in (batch[0][::-1].copy(), batch[1], batch[2], batch[3], batch[4])]
+    hot.set_wait_limit(1)
+    poisoned, before = 0, hot.recoveries
+    try:
+        for _ in range(10):
+            outs = [hot.khop_buffers(S0, 2, 10) for _ in range(2)]
+            hot.sample_khop(dg, *other, 2, hot.params("recent", 10), finalize=False, out=outs[0])
+            hot.sample_khop_multi(dg, *args, 2, [p_rec, p_uni], outs)
+            bad = [int(np_of(o.counts)[2]) == INT64_MAX for o in outs]
+            poisoned += any(bad)
+            for o, st in zip(outs, ("recent", "uniform")):
+                o.finalize()
+                for l in range(2):
+                    assert_hop_equal(o.hops[l], want[st].hops[l], tag=f"{st} hop{l}, wait limit 1, poisoned {bad}")
+            # the marks of the (possibly re-issued) recent query feed the unique stage (whose own numbering pass waits
+            # too: it runs under the default limit)
+            kr = outs[0]
+            hot.set_wait_limit(0)
+            local, uniq, (total, _) = hot.unique_compact([kr.slot_node0] + [h.neighbors for h in kr.hops], _abi.UNIQUE_SORTED,
+                                                         state, True, premarked=True)
+            hot.set_wait_limit(1)
+            assert total == want_u.size and np.array_equal(np_of(uniq), want_u)
+            assert np.array_equal(np.concatenate([np_of(a) for a in local]), want_inv)
+        assert hot.recoveries - before >= (1 if poisoned else 0)
+    finally:
+        hot.set_wait_limit(0)
+    if not poisoned:
+        pytest.skip("no block ever found a descriptor missing: the error path was not reached")
