@@ -531,6 +531,28 @@ typedef struct sgl_gather_seg {
 int32_t sgl_gather_multi(int32_t num_segments, const sgl_gather_seg* segs,
                          void* stream);
 
+/* sgl_gather with every distinct cold row crossing PCIe once.  The requests of
+ * a batch repeat rows (configs of 40 % duplicates and more); sgl_gather reads a
+ * cold row from pinned host memory once per REQUEST.  Here the call first
+ * numbers the distinct cold rows it asks for (the LDS-staged hash set of
+ * sgl_unique_compact), fetches each of them once into `staging` (HBM,
+ * [staging_rows, row_bytes]; and its time into staging_ts when the cache has
+ * ts_cold and out_ts is wanted), overlapped with the gather of the hot rows,
+ * and then serves every request of a cold row from there.  This is the plan of
+ * the reference's per-shard selected-index lists (ShardTensor::operator[],
+ * feature.cu.hpp:346-392) and of DistNodeState.prefetch (NodeState.py:77-82),
+ * which index the host table once per request.  Results equal sgl_gather's.
+ * Distinct cold rows beyond staging_rows are read in place, once per request.
+ * stats (optional device int64[4]) += {hot requests, cold requests, absent,
+ * distinct cold rows}.  Rows, tables, out and staging must be 16-byte aligned /
+ * sized (SGL_ENOTSUP otherwise: use sgl_gather). */
+size_t  sgl_gather_dedup_workspace_bytes(int64_t N_max);
+int32_t sgl_gather_dedup(const sgl_cache* c, const int64_t* ids, int64_t N_max,
+                         const int64_t* N_dev, void* out, int64_t* out_ts,
+                         int64_t* stats, void* staging, int64_t* staging_ts,
+                         int64_t staging_rows, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
 /* Scatter rows back (replaces DistNodeState.update, NodeState.py:46-61):
  * ids that are not resident are skipped.  Duplicate ids: the highest i wins
  * is NOT guaranteed; callers pass unique ids (as the reference's callers do). */

@@ -949,6 +949,32 @@ int32_t sglo_gather(const sgl_cache* c, const int64_t* ids, int64_t N_max,
     return SGL_OK;
 }
 
+/* The gather with each distinct cold row fetched once: by definition the rows sglo_gather yields; the fourth
+ * statistic counts the distinct local rows of the cold tier among the requests (np.unique of their locs). */
+size_t sglo_gather_dedup_workspace_bytes(int64_t N_max) { (void)N_max; return 0; }
+
+int32_t sglo_gather_dedup(const sgl_cache* c, const int64_t* ids, int64_t N_max, const int64_t* N_dev,
+                          void* out, int64_t* out_ts, int64_t* stats, void* staging, int64_t* staging_ts,
+                          int64_t staging_rows, void* ws, size_t ws_bytes, void* stream) {
+    (void)staging; (void)staging_ts; (void)staging_rows; (void)ws; (void)ws_bytes;
+    int32_t rc = sglo_gather(c, ids, N_max, N_dev, out, out_ts, stats, stream);
+    if (rc != SGL_OK || !stats) return rc;
+    int64_t N = N_dev ? *N_dev : N_max;
+    int64_t* locs = (int64_t*)malloc((size_t)(N + 1) * sizeof(int64_t));
+    if (!locs) return fail(SGL_ENOMEM, "malloc");
+    int64_t nc = 0;
+    for (int64_t i = 0; i < N; ++i) {
+        int64_t loc = cache_loc(c, ids[i]);
+        if (loc >= 0 && c->hot_slot && c->hot_slot[loc] < 0) locs[nc++] = loc;
+    }
+    qsort(locs, (size_t)nc, sizeof(int64_t), i64_cmp);
+    int64_t distinct = 0;
+    for (int64_t i = 0; i < nc; ++i) if (i == 0 || locs[i] != locs[i - 1]) distinct++;
+    stats[3] += distinct;
+    free(locs);
+    return SGL_OK;
+}
+
 /* Reference: DistNodeState.update (NodeState.py:46-61): loc = to_local(gids),
  * rows with loc >= 0 are overwritten, ts likewise. */
 int32_t sglo_scatter_update(const sgl_cache* c, void* hot_rw, void* cold_rw,

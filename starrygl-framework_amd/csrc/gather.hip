@@ -14,6 +14,14 @@
 #include "common.hpp"
 
 namespace sgl {
+
+// the hash-set unique of unique_hash.hip (numbers the distinct cold rows a call asks for)
+size_t hash_unique_workspace_bytes(int32_t G, const int64_t* len_max);
+int32_t hash_unique_compact(int32_t mode, int32_t G, const int64_t* const* ids, const int64_t* len_max,
+                            const int64_t* const* len_dev, int64_t* const* local_out,
+                            int64_t* unique_out, int64_t unique_capacity, int64_t* U_dev, void* ws,
+                            size_t ws_bytes, hipStream_t st);
+
 namespace {
 
 constexpr int BLOCK = 256;
@@ -202,6 +210,173 @@ __global__ __launch_bounds__(BLOCK) void gather_multi_kernel(MultiArgs m) {
                 }
             }
         }
+    }
+}
+
+// ---- gather with the cold tier fetched once per distinct row -------------------------------------------
+// Requests of a batch repeat rows; a cold row crosses PCIe once per REQUEST in the kernels above.  Here:
+//   classify : key[i] = local row of request i when that row is cold, -1 otherwise;
+//   (the hash-set unique numbers the distinct keys: slot[i] = place of request i's row in the staging buffer)
+//   phase A  : one launch, two segments walked by all blocks in turn - the distinct cold rows from pinned host
+//              memory into the HBM staging buffer (PCIe bound, few tiles), then every request whose row is hot
+//              (HBM bound; blocks that have finished their staging tiles start on these while the others still
+//              wait for the link) and zero rows for absent ids;
+//   phase B  : the requests of cold rows, served from the staging buffer (HBM to HBM).
+struct DedupArgs {
+    sgl_cache c;
+    const int64_t* ids;
+    int64_t N_max;
+    const int64_t* N_dev;
+    char* out;
+    int64_t* out_ts;
+    int64_t* stats;         // [4] or nullptr: hot requests, cold requests, absent, distinct cold rows
+    int64_t* key;           // [N_max]
+    const int64_t* slot;    // [N_max] written by the unique
+    const int64_t* uniq;    // [<= N_max] distinct cold rows
+    const int64_t* U_dev;   // their number
+    char* staging;          // [staging_rows, row_bytes] HBM
+    int64_t* staging_ts;    // [staging_rows] or nullptr
+    int64_t staging_rows;
+    int32_t rpb, cpr;
+};
+
+// where the local row `loc` of the cold tier lives, and its time
+__device__ __forceinline__ const char* cold_row(const sgl_cache& c, int64_t loc, int64_t* ts_out) {
+    *ts_out = c.ts_cold != nullptr ? *reinterpret_cast<const int64_t*>(reinterpret_cast<const char*>(c.ts_cold) + loc * ts_cold_stride(c)) : 0;
+    return static_cast<const char*>(c.cold) + loc * cold_stride(c);
+}
+
+__global__ __launch_bounds__(BLOCK) void dedup_classify_kernel(DedupArgs a) {
+    __shared__ int32_t s_tier[3];
+    if (threadIdx.x < 3) s_tier[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t N = live_count(a.N_dev, a.N_max);
+    for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < N; i += (int64_t)gridDim.x * BLOCK) {
+        const int64_t id = a.ids[i];
+        int64_t key = -1;
+        int tier = 2;
+        if (id >= 0) {
+            int64_t loc = id & a.c.id_mask;
+            bool ok = true;
+            if (a.c.g2l != nullptr) {
+                ok = loc >= 0 && loc < a.c.g2l_len;
+                if (ok) loc = a.c.g2l[loc];
+            }
+            if (ok && loc >= 0 && loc < a.c.rows) {
+                const bool cold = a.c.hot_slot != nullptr && a.c.hot_slot[loc] < 0;
+                tier = cold ? 1 : 0;
+                if (cold) key = loc;
+            }
+        }
+        a.key[i] = key;
+        if (a.stats != nullptr) atomicAdd(&s_tier[tier], 1);
+    }
+    if (a.stats == nullptr) return;
+    __syncthreads();
+    if (threadIdx.x < 3 && s_tier[threadIdx.x] != 0)
+        atomicAdd(reinterpret_cast<unsigned long long*>(a.stats + threadIdx.x), (unsigned long long)s_tier[threadIdx.x]);
+}
+
+// the flat, coalesced copy of one tile whose source rows are parked in s_src (nullptr: zeros, SKIP: leave the row alone)
+__device__ __forceinline__ void copy_tile(const char* const* s_src, char* out_tile, int32_t rows, int32_t cpr, float inv_cpr, bool stream_out) {
+    const char* const SKIP = reinterpret_cast<const char*>(uintptr_t(1));
+    const int32_t total = rows * cpr;
+    u32x4* __restrict__ dst = reinterpret_cast<u32x4*>(out_tile);
+    for (int32_t base = 0; base < total; base += BLOCK * UNROLL) {
+        u32x4 val[UNROLL];
+        bool on[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int32_t lc = base + u * BLOCK + threadIdx.x;
+            u32x4 v = {};
+            on[u] = false;
+            if (lc < total) {
+                const int32_t r = row_of_chunk(lc, cpr, inv_cpr);
+                const char* src = s_src[r];
+                on[u] = src != SKIP;
+                if (src != nullptr && src != SKIP) v = reinterpret_cast<const u32x4*>(src)[lc - r * cpr];
+            }
+            val[u] = v;
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int32_t lc = base + u * BLOCK + threadIdx.x;
+            if (on[u]) {
+                if (stream_out) __builtin_nontemporal_store(val[u], dst + lc);
+                else dst[lc] = val[u];
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void dedup_phase_a_kernel(DedupArgs a) {
+    extern __shared__ const char* s_src[];
+    const char* const SKIP = reinterpret_cast<const char*>(uintptr_t(1));
+    const int32_t cpr = a.cpr;
+    const float inv_cpr = 1.0f / (float)cpr;
+    // segment 1: distinct cold rows -> staging (those that fit; the others are read in place by phase B)
+    int64_t U = a.U_dev[0];
+    if (a.stats != nullptr && blockIdx.x == 0 && threadIdx.x == 0) a.stats[3] += U;
+    U = U < a.staging_rows ? U : a.staging_rows;
+    for (int64_t row0 = (int64_t)blockIdx.x * a.rpb; row0 < U; row0 += (int64_t)gridDim.x * a.rpb) {
+        const int32_t rows = (int32_t)((U - row0) < a.rpb ? (U - row0) : a.rpb);
+        __syncthreads();
+        for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
+            int64_t ts;
+            s_src[r] = cold_row(a.c, a.uniq[row0 + r], &ts);
+            if (a.staging_ts != nullptr) a.staging_ts[row0 + r] = ts;
+        }
+        __syncthreads();
+        copy_tile(s_src, a.staging + row0 * a.c.row_bytes, rows, cpr, inv_cpr, false);
+    }
+    // segment 2: the requests of hot rows (and zero rows for absent ids)
+    const int64_t N = live_count(a.N_dev, a.N_max);
+    for (int64_t row0 = (int64_t)blockIdx.x * a.rpb; row0 < N; row0 += (int64_t)gridDim.x * a.rpb) {
+        const int32_t rows = (int32_t)((N - row0) < a.rpb ? (N - row0) : a.rpb);
+        __syncthreads();
+        for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
+            if (a.key[row0 + r] >= 0) {
+                s_src[r] = SKIP;
+            } else {
+                int64_t ts;
+                int tier;
+                s_src[r] = resolve(a.c, a.ids[row0 + r], &ts, &tier);
+                if (a.out_ts != nullptr) a.out_ts[row0 + r] = ts;
+            }
+        }
+        __syncthreads();
+        copy_tile(s_src, a.out + row0 * a.c.row_bytes, rows, cpr, inv_cpr, true);
+    }
+}
+
+__global__ __launch_bounds__(BLOCK) void dedup_phase_b_kernel(DedupArgs a) {
+    extern __shared__ const char* s_src[];
+    const char* const SKIP = reinterpret_cast<const char*>(uintptr_t(1));
+    const int32_t cpr = a.cpr;
+    const float inv_cpr = 1.0f / (float)cpr;
+    const int64_t N = live_count(a.N_dev, a.N_max);
+    for (int64_t row0 = (int64_t)blockIdx.x * a.rpb; row0 < N; row0 += (int64_t)gridDim.x * a.rpb) {
+        const int32_t rows = (int32_t)((N - row0) < a.rpb ? (N - row0) : a.rpb);
+        __syncthreads();
+        int any = 0;
+        for (int32_t r = threadIdx.x; r < rows; r += BLOCK) {
+            const int64_t key = a.key[row0 + r];
+            const char* src = SKIP;
+            if (key >= 0) {
+                const int64_t sl = a.slot[row0 + r];
+                int64_t ts;
+                if (sl >= 0 && sl < a.staging_rows) {
+                    src = a.staging + sl * a.c.row_bytes;
+                    ts = a.staging_ts != nullptr ? a.staging_ts[sl] : 0;
+                } else {
+                    src = cold_row(a.c, key, &ts);       // (a staging buffer smaller than the call's distinct cold rows)
+                }
+                if (a.out_ts != nullptr) a.out_ts[row0 + r] = ts;
+                any = 1;
+            }
+            s_src[r] = src;
+        }
+        if (__syncthreads_or(any)) copy_tile(s_src, a.out + row0 * a.c.row_bytes, rows, cpr, inv_cpr, true);
     }
 }
 
@@ -396,6 +571,64 @@ extern "C" int32_t sgl_scatter_update(const sgl_cache* c, void* hot_rw, void* co
         case 8: hipLaunchKernelGGL(scatter_kernel<u32x2>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
         default: hipLaunchKernelGGL(scatter_kernel<uint32_t>, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a); break;
     }
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
+}
+
+extern "C" size_t sgl_gather_dedup_workspace_bytes(int64_t N_max) {
+    if (N_max < 0) N_max = 0;
+    const int64_t lens[1] = {N_max};
+    return 3 * align_up((size_t)(N_max + 1) * 8) + align_up(16) + hash_unique_workspace_bytes(1, lens) + 1024;
+}
+
+extern "C" int32_t sgl_gather_dedup(const sgl_cache* c, const int64_t* ids, int64_t N_max, const int64_t* N_dev,
+                                    void* out, int64_t* out_ts, int64_t* stats, void* staging, int64_t* staging_ts,
+                                    int64_t staging_rows, void* ws, size_t ws_bytes, void* stream) {
+    int32_t rc;
+    if ((rc = check_cache(c)) != SGL_OK) return rc;
+    if (N_max < 0 || staging_rows < 0) return fail(SGL_EINVAL, "gather_dedup: negative size");
+    if (N_max == 0) return SGL_OK;
+    if (!ids || !out) return fail(SGL_EINVAL, "gather_dedup: ids/out is NULL");
+    if (staging_rows > 0 && !staging) return fail(SGL_EINVAL, "gather_dedup: staging is NULL");
+    if (pick_vec(c->row_bytes, cold_stride(*c), {c->hot, c->cold, out, staging}) != 16)
+        return fail(SGL_ENOTSUP, "gather_dedup: rows and tables must be 16-byte aligned / sized (use sgl_gather)");
+    if (!ws || ws_bytes < sgl_gather_dedup_workspace_bytes(N_max))
+        return fail(SGL_ENOMEM, "gather_dedup: workspace %zu < %zu bytes", ws_bytes, sgl_gather_dedup_workspace_bytes(N_max));
+    hipStream_t st = as_stream(stream);
+    Arena ar(ws, ws_bytes);
+    DedupArgs a;
+    a.c = *c; a.ids = ids; a.N_max = N_max; a.N_dev = N_dev;
+    a.out = static_cast<char*>(out); a.out_ts = out_ts; a.stats = stats;
+    a.key = ar.take<int64_t>(N_max + 1);
+    int64_t* slot = ar.take<int64_t>(N_max + 1);
+    int64_t* uniq = ar.take<int64_t>(N_max + 1);
+    int64_t* U_dev = ar.take<int64_t>(2);
+    a.slot = slot; a.uniq = uniq; a.U_dev = U_dev;
+    a.staging = static_cast<char*>(staging); a.staging_ts = (c->ts_cold != nullptr) ? staging_ts : nullptr;
+    a.staging_rows = (c->ts_cold != nullptr && out_ts != nullptr && !staging_ts) ? 0 : staging_rows;
+    a.cpr = (int32_t)(c->row_bytes / 16);
+    int64_t rpb = (int64_t)BLOCK * UNROLL / a.cpr;
+    rpb = rpb < 1 ? 1 : (rpb > 1024 ? 1024 : rpb);
+    a.rpb = (int32_t)rpb;
+    const size_t used = align_up(ar.used);
+    if (!ar.ok() || used > ws_bytes) return fail(SGL_ENOMEM, "gather_dedup: workspace too small");
+    int64_t cb = ceil_div<int64_t>(N_max, BLOCK);
+    if (cb > 2048) cb = 2048;
+    hipLaunchKernelGGL(dedup_classify_kernel, dim3((unsigned)cb), dim3(BLOCK), 0, st, a);
+    SGL_LAUNCH_CHECK();
+    const int64_t* kp[1] = {a.key};
+    int64_t* sp[1] = {slot};
+    const int64_t lens[1] = {N_max};
+    const int64_t* ld[1] = {N_dev};
+    rc = hash_unique_compact(SGL_UNIQUE_SORTED, 1, kp, lens, ld, sp, uniq, N_max, U_dev, static_cast<char*>(ws) + used,
+                             ws_bytes - used, st);
+    if (rc != SGL_OK) return rc;
+    int64_t blocks = ceil_div<int64_t>(N_max, rpb);
+    if (blocks > MAX_GRID) blocks = MAX_GRID;
+    const size_t shmem = (size_t)rpb * sizeof(char*);
+    hipLaunchKernelGGL(dedup_phase_a_kernel, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a);
+    SGL_LAUNCH_CHECK();
+    hipLaunchKernelGGL(dedup_phase_b_kernel, dim3((unsigned)blocks), dim3(BLOCK), shmem, st, a);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
 }

@@ -110,6 +110,8 @@ PROTOTYPES = {
     "unique_compact_batched": (i32, [vp, i64, i32, i32, P(vp), P(i64), P(vp), P(vp), vp, i64, vp, vp, sz, vp]),
     "gather": (i32, [P(Cache), vp, i64, vp, vp, vp, vp, vp]),
     "gather_multi": (i32, [i32, P(GatherSeg), vp]),
+    "gather_dedup_workspace_bytes": (sz, [i64]),
+    "gather_dedup": (i32, [P(Cache), vp, i64, vp, vp, vp, vp, vp, vp, i64, vp, sz, vp]),
     "scatter_update": (i32, [P(Cache), vp, vp, vp, vp, vp, i64, vp, vp, vp]),
     "chunk_index_workspace_bytes": (sz, [i64]),
     "chunk_index_build": (i32, [i64, i64, vp, vp, vp, vp, sz, vp]),

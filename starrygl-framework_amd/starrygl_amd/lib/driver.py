@@ -692,6 +692,19 @@ class HotPath:
                                  be.ptr(out), be.ptr(out_ts), be.ptr(stats), be.stream()))
         return out
 
+    def gather_dedup(self, cache, ids, out, staging, out_ts=None, staging_ts=None, stats=None, N_dev=None, workspace=None):
+        """`gather` with every distinct cold row of the call read from pinned host memory once (into `staging`, an
+        HBM buffer of [rows, row_bytes]; `staging_ts` int64[rows] when times are gathered too) and the requests of
+        cold rows served from there.  stats: optional int64[4] += {hot, cold requests, absent, distinct cold rows}."""
+        self._chk("i64", ids=ids, out_ts=out_ts, stats=stats, N_dev=N_dev, staging_ts=staging_ts)
+        be, N = self.be, int(ids.shape[0])
+        need = int(self.lib.gather_dedup_workspace_bytes(N))
+        ws, wsb = (workspace, be.nbytes(workspace)) if workspace is not None else self._workspace(need)
+        self._ck(self.lib.gather_dedup(C.byref(cache), be.ptr(ids), N, be.ptr(N_dev), be.ptr(out), be.ptr(out_ts),
+                                       be.ptr(stats), be.ptr(staging), be.ptr(staging_ts),
+                                       0 if staging is None else int(staging.shape[0]), be.ptr(ws), wsb, be.stream()))
+        return out
+
     def gather_plan(self, segments):
         """Pre-marshalled argument block for `gather_multi`: segments is a list of
         (cache, ids, out, out_ts or None, N_dev or None)."""

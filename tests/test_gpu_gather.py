@@ -251,3 +251,48 @@ def test_gather_multi_large_output(hot):
         ids_e = ids_e.flip(0).contiguous()
         plan = hot.gather_plan([(hot.cache(400, t_node), ids_n, out_n, None, live_n),
                                 (hot.cache(688, t_edge), ids_e, out_e, None, None)])
+
+
+@pytest.mark.parametrize("dim,dtype,hot_frac,dup", [(128, np.uint16, 0.1, 8), (100, np.float32, 0.3, 3), (172, np.float32, 0.0, 20),
+                                                    (128, np.uint16, 1.0, 4), (4, np.float32, 0.5, 2)])
+def test_gather_dedup_matches_numpy(oracle, hot, dim, dtype, hot_frac, dup):
+    """The gather that fetches every distinct cold row once: same rows, times and (first three) statistics as the
+    plain gather, the fourth statistic = np.unique of the cold requests' rows; with a staging buffer that holds all
+    distinct cold rows, one that holds a part of them, and none at all; live count on the device; absent ids."""
+    rows, N = 30_000, 60_000
+    full, h, c, slot = _tables(rows, dim, dtype, hot_frac, dim + dup)
+    rng = np.random.default_rng(dup)
+    ids = rng.integers(0, rows // dup, N).astype(np.int64) * dup          # every row asked for ~dup times
+    ids[::53] = -1
+    ids[::59] = rows + 7
+    ts_full = rng.integers(0, 10**9, rows).astype(np.int64)
+    ts_hot = np.zeros(max(h.shape[0], 1), dtype=np.int64)
+    ts_hot[slot[slot >= 0]] = ts_full[slot >= 0]
+    cache, keep = _dev_cache(hot, full, h, c, slot, ts_hot=to_dev(hot, ts_hot), ts_cold=torch.from_numpy(ts_full).pin_memory())
+    ok = (ids >= 0) & (ids < rows)
+    want = np.zeros((N, dim), dtype=full.dtype)
+    want[ok] = full[ids[ok]]
+    want_ts = np.zeros(N, dtype=np.int64)
+    want_ts[ok] = ts_full[ids[ok]]
+    cold_req = ok & (slot[np.clip(ids, 0, rows - 1)] < 0)
+    distinct = int(np.unique(ids[cold_req]).size)
+    tdt = torch.from_numpy(full[:1]).dtype
+    for stage_rows, live in ((distinct + 5, N), (max(distinct // 3, 1), N), (0, N), (distinct + 5, N // 2)):
+        out = torch.full((N, dim), 7, dtype=tdt, device=hot.be.device)
+        out_ts = hot.be.zeros(N)
+        stats = hot.be.zeros(4)
+        staging = torch.empty((stage_rows, dim), dtype=tdt, device=hot.be.device) if stage_rows else None
+        staging_ts = hot.be.empty(stage_rows) if stage_rows else None
+        n_dev = to_dev(hot, np.array([live], dtype=np.int64))
+        hot.gather_dedup(cache, to_dev(hot, ids), out, staging, out_ts=out_ts, staging_ts=staging_ts, stats=stats, N_dev=n_dev)
+        assert np.array_equal(np_of(out)[:live].view(np.uint8), want[:live].view(np.uint8)), (stage_rows, live)
+        assert np.array_equal(np_of(out_ts)[:live], want_ts[:live])
+        assert (np_of(out)[live:] == 7).all()        # rows beyond the live count stay untouched
+        n_hot = int((ok & ~cold_req)[:live].sum())
+        assert np_of(stats).tolist() == [n_hot, int(cold_req[:live].sum()), int((~ok)[:live].sum()),
+                                         int(np.unique(ids[:live][cold_req[:live]]).size)]
+    # the oracle's fourth statistic is pinned by np.unique as well
+    oc = oracle.cache(full.shape[1] * full.dtype.itemsize, h, rows=rows, cold=c, hot_slot=slot)
+    o_out, o_stats = np.empty((N, dim), dtype=full.dtype), np.zeros(4, dtype=np.int64)
+    oracle.gather_dedup(oc, ids, o_out, None, stats=o_stats)
+    assert np.array_equal(o_out.view(np.uint8), want.view(np.uint8)) and o_stats[3] == distinct
