@@ -175,6 +175,17 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     c_mem = hot.cache(400, mem_hot, rows=n, cold=mem_cold, hot_slot=slot, ts_hot=ts_hot, ts_cold=ts_cold)
     c_mem_packed = hot.cache(400, mem_hot, rows=n, cold=mem_cold_packed, hot_slot=slot, ts_hot=ts_hot, ts_cold=ts_cold_packed)
     c_nf = hot.cache(400, nf_hot, rows=n, cold=nf_cold, hot_slot=slot)
+    # What the step uses: ONE record per node in either tier - memory row, feature row and (host tier) the time
+    # of the last update side by side - so that a remote node costs the 7 lines of one 896-byte record instead of the
+    # 4 + 4 lines of two 400-byte rows in tables of their own.  The step gathers [U, 200] rows (memory | features,
+    # column views for the consumer); the memory update writes through a 400-byte view of the same storage.
+    node_hot = torch.cat([mem_hot, nf_hot], dim=1).contiguous()
+    node_cold, ts_cold_rec, _rec2 = hot.interleaved_cold(n, 200)
+    node_cold[:, :100].copy_(mem_cold_packed)
+    node_cold[:, 100:].copy_(nf_cold)
+    ts_cold_rec.copy_(ts_cold_packed)
+    c_node = hot.cache(800, node_hot, rows=n, cold=node_cold, hot_slot=slot, ts_hot=ts_hot, ts_cold=ts_cold_rec)
+    c_mem_view = hot.cache(400, node_hot[:, :100], rows=n, cold=node_cold[:, :100], hot_slot=slot, ts_hot=ts_hot, ts_cold=ts_cold_rec)
     del mem, nfeat
     efeat = torch.empty((m, 172), device=dev)
     for lo in range(0, m, 1 << 22):
@@ -205,9 +216,11 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
         P.state = hot.remap_state(n)
         P.local = [hot.be.empty(S0), hot.be.empty(S0 * k)]
         P.ubuf, P.U = hot.be.empty(S0 + S0 * k), hot.be.zeros(2)
-        P.o_mem = torch.empty((S0 + S0 * k, 100), device=dev)
+        P.o_node = torch.empty((S0 + S0 * k, 200), device=dev)       # memory | features of every unique node
+        P.o_mem, P.o_nf = P.o_node[:, :100], P.o_node[:, 100:]
         P.o_ts = hot.be.empty(S0 + S0 * k)
-        P.o_nf = torch.empty((S0 + S0 * k, 100), device=dev)
+        P.o_mem2 = torch.empty((S0 + S0 * k, 100), device=dev)       # (outputs of the two-table layout, for the comparison)
+        P.o_nf2 = torch.empty((S0 + S0 * k, 100), device=dev)
         P.o_ef = torch.empty((S0 * k, 172), device=dev)
         P.o_te = torch.empty((S0 * k, 100), device=dev)
         P.s_all = torch.empty_like(packed[0])
@@ -216,7 +229,7 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
         P.p = hot.marking(hot.with_root_hint(p, P.s_in[4]), P.state)
         P.E = P.kr.hops[0].counts[1:2]
         P.acc = torch.zeros(2, dtype=torch.int64, device=dev)
-        P.plan = hot.gather_plan([(c_mem, P.ubuf, P.o_mem, P.o_ts, P.U[0:1]), (c_nf, P.ubuf, P.o_nf, None, P.U[0:1]),
+        P.plan = hot.gather_plan([(c_node, P.ubuf, P.o_node, P.o_ts, P.U[0:1]),
                                   (c_ef, P.kr.hops[0].neighbors_eid, P.o_ef, None, P.E)])
 
         def body():
@@ -261,7 +274,11 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     wall, (e_tot, u_tot) = timed(len(pipes))
     P0 = pipes[0]
     kr, ubuf, U, E, plan, s_in = P0.kr, P0.ubuf, P0.U, P0.E, P0.plan, P0.s_in
-    o_mem, o_ts, o_ef, o_te, o_nf = P0.o_mem, P0.o_ts, P0.o_ef, P0.o_te, P0.o_nf
+    o_mem, o_ts, o_ef, o_te, o_nf = P0.o_mem2, P0.o_ts, P0.o_ef, P0.o_te, P0.o_nf2
+    # the step's rows against the generating tables: memory | features of every unique node, and their times
+    assert torch.equal(P0.o_node[:int(U[0].item()), :100].contiguous().cpu(), mem_cold_packed[ubuf[:int(U[0].item())].cpu()])
+    assert torch.equal(P0.o_node[:int(U[0].item()), 100:].contiguous().cpu(), nf_cold[ubuf[:int(U[0].item())].cpu()])
+    assert torch.equal(o_ts[:int(U[0].item())].cpu(), ts_cold_packed[ubuf[:int(U[0].item())].cpu()])
     with torch.cuda.stream(streams[0]):
         P0.s_all.copy_(packed[0]); P0.body()
     torch.cuda.synchronize()
@@ -278,17 +295,22 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     ms = _time_launches(torch, lambda: hot.gather(c_mem, ubuf, o_mem, out_ts=o_ts, N_dev=U[0:1]))
     res["gather_memory_30pct_host"] = {"ms": round(ms, 4), "rows": u1, "GBps": round(u1 * (8 + 4 + 800 + 16) / ms / 1e6, 1)}
     ms = _time_launches(torch, lambda: hot.gather_multi(plan))
-    res["gather_all_three_one_launch"] = {"ms": round(ms, 4), "GBps": round((u1 * (2 * 812 + 16) + e1 * 1384) / ms / 1e6, 1)}
+    res["gather_all_three_one_launch"] = {"ms": round(ms, 4), "GBps": round((u1 * (2 * 812 + 16) + e1 * 1384) / ms / 1e6, 1),
+                                          "layout": "one record per node: memory row | feature row | last update (896 bytes on the host)"}
+    plan_two = hot.gather_plan([(c_mem, ubuf, o_mem, o_ts, U[0:1]), (c_nf, ubuf, o_nf, None, U[0:1]),
+                                (c_ef, kr.hops[0].neighbors_eid, o_ef, None, E)])
+    ms_two = _time_launches(torch, lambda: hot.gather_multi(plan_two))
     plan_packed = hot.gather_plan([(c_mem_packed, ubuf, o_mem, o_ts, U[0:1]), (c_nf, ubuf, o_nf, None, U[0:1]),
                                    (c_ef, kr.hops[0].neighbors_eid, o_ef, None, E)])
     ms_packed = _time_launches(torch, lambda: hot.gather_multi(plan_packed))
-    # the launch is bound by the rows that cross PCIe: memory rows (400 B + 8 B last update) and node rows (400 B) of the
-    # unique nodes whose owner is remote.  Host memory is read in 128-byte lines: a 400-byte row at a 16-byte-aligned
-    # offset always spans 4 of them (512 B); a time in a table of its own costs another one, in the row's record none.
+    # the launch is bound by the rows that cross PCIe: memory row (400 B), last update (8 B) and feature row (400 B) of the
+    # unique nodes whose owner is remote.  Host memory is read in 128-byte lines: the 808 bytes of a node's record span 7
+    # of them; two 400-byte rows in tables of their own span 4 each, a time in a third table costs another one.
     st3 = hot.be.zeros(3)
     hot.gather(c_mem, ubuf, o_mem, out_ts=o_ts, N_dev=U[0:1], stats=st3)
     n_cold = int(st3[1].item())
-    cold_alg, cold_lines, cold_lines_packed = n_cold * (400 + 8 + 400), n_cold * (512 + 512), n_cold * (512 + 128 + 512)
+    cold_alg = n_cold * (400 + 8 + 400)
+    cold_lines, cold_lines_two, cold_lines_packed = n_cold * 896, n_cold * (512 + 512), n_cold * (512 + 128 + 512)
     probe = torch.empty(cold_alg, dtype=torch.uint8, device=dev)
     src_h = mem_cold_packed.view(torch.uint8).reshape(-1)[:cold_alg]
     ms_cp = _time_launches(torch, lambda: probe.copy_(src_h, non_blocking=True), reps=5)
@@ -298,6 +320,10 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
         "memcpy_h2d_same_bytes_GBps": round(cold_alg / ms_cp / 1e6, 2),
         "cold_rate_over_memcpy": round(ms_cp / ms, 3), "line_rate_over_memcpy": round(cold_lines / cold_alg * ms_cp / ms, 3),
         "ceiling_of_cold_rate_over_memcpy": round(cold_alg / cold_lines, 3),
+        "memory_and_features_in_two_tables": {"ms": round(ms_two, 4), "cold_GBps": round(cold_alg / ms_two / 1e6, 2),
+                                              "cold_rate_over_memcpy": round(ms_cp / ms_two, 3),
+                                              "line_rate_over_memcpy": round(cold_lines_two / cold_alg * ms_cp / ms_two, 3),
+                                              "note": "memory rows with their times in 512-byte records, feature rows in a table of their own"},
         "times_in_a_table_of_their_own": {"ms": round(ms_packed, 4), "cold_GBps": round(cold_alg / ms_packed / 1e6, 2),
                                           "cold_rate_over_memcpy": round(ms_cp / ms_packed, 3),
                                           "line_rate_over_memcpy": round(cold_lines_packed / cold_alg * ms_cp / ms_packed, 3)}})
@@ -331,7 +357,10 @@ def workload_tgn_step(hot, torch, np, synth, _abi, n=2_500_000, m=60_000_000, B=
     vals = torch.randn((u_n, 100), device=dev, generator=gen)
     ms_red = _time_launches(torch, lambda: hot.segment_max_ts(loc_[0], ends_ts, u_n))
     new_ts, _ = hot.segment_max_ts(loc_[0], ends_ts, u_n)
-    ms_upd = _time_launches(torch, lambda: hot.scatter_update(c_mem, mem_hot, mem_cold, ts_hot, ts_cold, uniq_, vals, new_ts))
+    ms_upd = _time_launches(torch, lambda: hot.scatter_update(c_mem_view, node_hot[:, :100], node_cold[:, :100], ts_hot, ts_cold_rec, uniq_, vals, new_ts))
+    hot.gather(c_node, uniq_, P0.o_node[:u_n], out_ts=o_ts[:u_n])        # read back through the step's cache: the memory half is new, the feature half untouched
+    assert torch.equal(P0.o_node[:u_n, :100], vals) and torch.equal(o_ts[:u_n], new_ts)
+    assert torch.equal(P0.o_node[:u_n, 100:].contiguous().cpu(), nf_cold[uniq_.cpu()])
     res["memory_update"] = {"nodes": int(u_n), "latest_event_per_node_ms": round(ms_red, 4), "scatter_update_ms": round(ms_upd, 4),
                             "GBps": round(u_n * (8 + 4 + 400 + 400 + 16) / ms_upd / 1e6, 1)}
     return res

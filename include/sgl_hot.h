@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define SGL_ABI_VERSION 7
+#define SGL_ABI_VERSION 8
 
 /* ------------------------------------------------------------------ status */
 #define SGL_OK        0
@@ -504,6 +504,10 @@ typedef struct sgl_cache {
                                     * multiple of 4, >= row_bytes)                       */
     int64_t        ts_cold_stride; /* bytes from one ts_cold entry to the next; 0 = 8 (a
                                     * multiple of 8)                                     */
+    int64_t        hot_stride;     /* bytes from one hot row to the next; 0 = row_bytes (a
+                                    * multiple of 4, >= row_bytes): a view of some columns of
+                                    * wider HBM rows, e.g. the memory part of rows that hold a
+                                    * node's memory and its features side by side          */
 } sgl_cache;
 
 /* out[i, :] = row(ids[i]); out_ts[i] = its last-update time when out_ts and the

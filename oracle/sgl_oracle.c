@@ -897,6 +897,7 @@ int32_t sglo_unique_compact_batched(void* state, int64_t universe, int32_t B, in
 
 /* cold rows and their times may sit at a stride of their own (0 = packed) */
 static int64_t cold_stride(const sgl_cache* c) { return c->cold_stride ? c->cold_stride : c->row_bytes; }
+static int64_t hot_stride(const sgl_cache* c) { return c->hot_stride ? c->hot_stride : c->row_bytes; }
 static int64_t* cold_ts_at(const sgl_cache* c, const int64_t* base, int64_t loc) {
     return (int64_t*)((char*)base + loc * (c->ts_cold_stride ? c->ts_cold_stride : 8));
 }
@@ -936,7 +937,7 @@ int32_t sglo_gather(const sgl_cache* c, const int64_t* ids, int64_t N_max,
         }
         int64_t slot = c->hot_slot ? (int64_t)c->hot_slot[loc] : loc;
         if (slot >= 0) {
-            memcpy(dst, (const char*)c->hot + slot * c->row_bytes, (size_t)c->row_bytes);
+            memcpy(dst, (const char*)c->hot + slot * hot_stride(c), (size_t)c->row_bytes);
             if (out_ts) out_ts[i] = c->ts_hot ? c->ts_hot[slot] : 0;
             hit++;
         } else {
@@ -989,7 +990,7 @@ int32_t sglo_scatter_update(const sgl_cache* c, void* hot_rw, void* cold_rw,
         int64_t slot = c->hot_slot ? (int64_t)c->hot_slot[loc] : loc;
         const char* srcp = (const char*)values + i * c->row_bytes;
         if (slot >= 0) {
-            memcpy((char*)hot_rw + slot * c->row_bytes, srcp, (size_t)c->row_bytes);
+            memcpy((char*)hot_rw + slot * hot_stride(c), srcp, (size_t)c->row_bytes);
             if (ts && ts_hot_rw) ts_hot_rw[slot] = ts[i];
         } else {
             memcpy((char*)cold_rw + loc * cold_stride(c), srcp, (size_t)c->row_bytes);

@@ -50,6 +50,7 @@ struct GatherArgs {
 
 __host__ __device__ __forceinline__ int64_t cold_stride(const sgl_cache& c) { return c.cold_stride ? c.cold_stride : c.row_bytes; }
 __host__ __device__ __forceinline__ int64_t ts_cold_stride(const sgl_cache& c) { return c.ts_cold_stride ? c.ts_cold_stride : 8; }
+__host__ __device__ __forceinline__ int64_t hot_stride(const sgl_cache& c) { return c.hot_stride ? c.hot_stride : c.row_bytes; }
 
 // lc / cpr for a chunk index inside a block's tile (lc < 2^22: a tile holds at most 1024 rows of at most 1024
 // chunks, or one row of at most 65536): one multiply and a fix-up in place of an integer division per chunk.
@@ -77,7 +78,7 @@ __device__ __forceinline__ const char* resolve(const sgl_cache& c, int64_t id, i
     if (slot >= 0) {
         *tier = 0;
         if (c.ts_hot != nullptr) *ts_out = c.ts_hot[slot];
-        return static_cast<const char*>(c.hot) + slot * c.row_bytes;
+        return static_cast<const char*>(c.hot) + slot * hot_stride(c);
     }
     *tier = 1;
     if (c.ts_cold != nullptr)
@@ -405,8 +406,8 @@ __global__ __launch_bounds__(BLOCK) void scatter_kernel(ScatterArgs a) {
             const char* p = resolve(a.c, a.ids[row0 + r], &ts_unused, &tier);
             char* d = nullptr;
             if (tier == 0) {
-                const int64_t slot = (p - static_cast<const char*>(a.c.hot)) / a.c.row_bytes;
-                d = a.hot_rw + slot * a.c.row_bytes;
+                const int64_t slot = (p - static_cast<const char*>(a.c.hot)) / hot_stride(a.c);
+                d = a.hot_rw + slot * hot_stride(a.c);
                 if (a.ts != nullptr && a.ts_hot_rw != nullptr) a.ts_hot_rw[slot] = a.ts[row0 + r];
             } else if (tier == 1) {
                 const int64_t loc = (p - static_cast<const char*>(a.c.cold)) / cold_stride(a.c);
@@ -446,15 +447,17 @@ int32_t check_cache(const sgl_cache* c) {
         return fail(SGL_EINVAL, "cache: hot_slot given but cold table is NULL");
     if (c->cold_stride != 0 && (c->cold_stride < c->row_bytes || c->cold_stride % 4 != 0))
         return fail(SGL_EINVAL, "cache: cold_stride %lld must be 0 or a multiple of 4 >= row_bytes", (long long)c->cold_stride);
+    if (c->hot_stride != 0 && (c->hot_stride < c->row_bytes || c->hot_stride % 4 != 0))
+        return fail(SGL_EINVAL, "cache: hot_stride %lld must be 0 or a multiple of 4 >= row_bytes", (long long)c->hot_stride);
     if (c->ts_cold_stride != 0 && (c->ts_cold_stride < 8 || c->ts_cold_stride % 8 != 0))
         return fail(SGL_EINVAL, "cache: ts_cold_stride %lld must be 0 or a multiple of 8", (long long)c->ts_cold_stride);
     return SGL_OK;
 }
 
 // widest chunk every involved address / the row size allows
-int pick_vec(int64_t row_bytes, int64_t cold_stride_bytes, std::initializer_list<const void*> ptrs) {
-    int v = 16;
-    if (row_bytes % 16 || cold_stride_bytes % 16) v = (row_bytes % 8 || cold_stride_bytes % 8) ? 4 : 8;
+int pick_vec(int64_t row_bytes, int64_t stride_bytes, std::initializer_list<const void*> ptrs) {
+    int v = 16;      // (stride_bytes: the cold and the hot row stride OR-ed together - a common divisor test)
+    if (row_bytes % 16 || stride_bytes % 16) v = (row_bytes % 8 || stride_bytes % 8) ? 4 : 8;
     for (const void* p : ptrs) {
         if (!p) continue;
         while (v > 4 && !aligned(p, v)) v >>= 1;
@@ -475,7 +478,7 @@ extern "C" int32_t sgl_gather(const sgl_cache* c, const int64_t* ids, int64_t N_
     if (N_max < 0) return fail(SGL_EINVAL, "gather: N_max < 0");
     if (N_max == 0) return SGL_OK;
     if (!ids || !out) return fail(SGL_EINVAL, "gather: ids/out is NULL");
-    const int vec = pick_vec(c->row_bytes, cold_stride(*c), {c->hot, c->cold, out});
+    const int vec = pick_vec(c->row_bytes, cold_stride(*c) | hot_stride(*c), {c->hot, c->cold, out});
     GatherArgs a;
     a.c = *c; a.ids = ids; a.N_max = N_max; a.N_dev = N_dev;
     a.out = static_cast<char*>(out); a.out_ts = out_ts; a.stats = stats;
@@ -520,7 +523,7 @@ extern "C" int32_t sgl_gather_multi(int32_t T, const sgl_gather_seg* segs, void*
         if (g.N_max < 0) return fail(SGL_EINVAL, "gather_multi: N_max < 0");
         if (g.N_max == 0) continue;
         if (!g.ids || !g.out) return fail(SGL_EINVAL, "gather_multi: ids/out is NULL");
-        if (pick_vec(g.cache->row_bytes, cold_stride(*g.cache), {g.cache->hot, g.cache->cold, g.out}) != 16)
+        if (pick_vec(g.cache->row_bytes, cold_stride(*g.cache) | hot_stride(*g.cache), {g.cache->hot, g.cache->cold, g.out}) != 16)
             return fail(SGL_ENOTSUP, "gather_multi: segment %d is not 16-byte aligned / sized", t);
         MultiSeg& a = m.seg[m.T++];
         a.c = *g.cache; a.ids = g.ids; a.N_max = g.N_max; a.N_dev = g.N_dev;
@@ -553,7 +556,7 @@ extern "C" int32_t sgl_scatter_update(const sgl_cache* c, void* hot_rw, void* co
     if (!ids || !values) return fail(SGL_EINVAL, "scatter_update: ids/values is NULL");
     if (c->hot != nullptr && hot_rw == nullptr) return fail(SGL_EINVAL, "scatter_update: hot_rw is NULL");
     if (c->hot_slot != nullptr && cold_rw == nullptr) return fail(SGL_EINVAL, "scatter_update: cold_rw is NULL");
-    const int vec = pick_vec(c->row_bytes, cold_stride(*c), {hot_rw, cold_rw, values});
+    const int vec = pick_vec(c->row_bytes, cold_stride(*c) | hot_stride(*c), {hot_rw, cold_rw, values});
     ScatterArgs a;
     a.c = *c; a.hot_rw = static_cast<char*>(hot_rw); a.cold_rw = static_cast<char*>(cold_rw);
     a.ts_hot_rw = ts_hot_rw; a.ts_cold_rw = ts_cold_rw; a.ids = ids; a.N = N;
@@ -590,7 +593,7 @@ extern "C" int32_t sgl_gather_dedup(const sgl_cache* c, const int64_t* ids, int6
     if (N_max == 0) return SGL_OK;
     if (!ids || !out) return fail(SGL_EINVAL, "gather_dedup: ids/out is NULL");
     if (staging_rows > 0 && !staging) return fail(SGL_EINVAL, "gather_dedup: staging is NULL");
-    if (pick_vec(c->row_bytes, cold_stride(*c), {c->hot, c->cold, out, staging}) != 16)
+    if (pick_vec(c->row_bytes, cold_stride(*c) | hot_stride(*c), {c->hot, c->cold, out, staging}) != 16)
         return fail(SGL_ENOTSUP, "gather_dedup: rows and tables must be 16-byte aligned / sized (use sgl_gather)");
     if (!ws || ws_bytes < sgl_gather_dedup_workspace_bytes(N_max))
         return fail(SGL_ENOMEM, "gather_dedup: workspace %zu < %zu bytes", ws_bytes, sgl_gather_dedup_workspace_bytes(N_max));

@@ -5,7 +5,7 @@ header declares.  The product library exports them as ``sgl_*``.
 """
 import ctypes as C
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 SGL_OK, SGL_EINVAL, SGL_ERANGE, SGL_ENOTSUP, SGL_EHIP, SGL_ENOMEM = 0, -1, -2, -3, -4, -5
 SAMPLE_RECENT, SAMPLE_UNIFORM = 0, 1
@@ -46,7 +46,7 @@ class Cache(C.Structure):
     _fields_ = [("rows", i64), ("row_bytes", i64), ("id_mask", i64),
                 ("g2l", vp), ("g2l_len", i64), ("hot_slot", vp),
                 ("hot", vp), ("hot_rows", i64), ("cold", vp),
-                ("ts_hot", vp), ("ts_cold", vp), ("cold_stride", i64), ("ts_cold_stride", i64)]
+                ("ts_hot", vp), ("ts_cold", vp), ("cold_stride", i64), ("ts_cold_stride", i64), ("hot_stride", i64)]
 
 
 class GatherSeg(C.Structure):

@@ -639,15 +639,16 @@ class HotPath:
     # ------------------------------------------------------------- gather
     def cache(self, row_bytes, hot, rows=None, cold=None, hot_slot=None, g2l=None,
               id_mask=-1, ts_hot=None, ts_cold=None):
-        """`cold` may be a row-strided view ([rows, width] with unit stride inside a row) and `ts_cold`
+        """`cold` and `hot` may be row-strided views ([rows, width] with unit stride inside a row) and `ts_cold`
         a strided 1-D view: their strides travel in the struct, so a cold tier that keeps a row and its
-        time in one record (see `interleaved_cold`) is read in place."""
+        time in one record (see `interleaved_cold`) is read in place, and a cache over some columns of wider
+        rows (the memory part of rows holding memory and features side by side) needs no copy."""
         be = self.be
         hot_rows = 0 if hot is None else int(hot.shape[0])
         if rows is None:
             rows = int(cold.shape[0]) if cold is not None else hot_rows
-        cold_stride = ts_cold_stride = 0
-        cold_ptr, ts_cold_ptr = None, None
+        cold_stride = ts_cold_stride = hot_stride = 0
+        cold_ptr, ts_cold_ptr, hot_ptr = None, None, None
         if cold is not None:
             st = _byte_strides(cold)
             if len(st) == 2 and cold.shape[0] > 1 and st[0] != cold.shape[1] * st[1]:
@@ -655,14 +656,21 @@ class HotPath:
                     raise ValueError("cache: the cold table must have unit stride inside a row")
                 cold_stride = int(st[0])
             cold_ptr = _address(cold)
+        if hot is not None:       # (a column slice of wider HBM rows: the row stride travels in the struct)
+            st = _byte_strides(hot)
+            if len(st) == 2 and hot.shape[0] > 1 and st[0] != hot.shape[1] * st[1]:
+                if st[1] != _itemsize(hot):
+                    raise ValueError("cache: the hot table must have unit stride inside a row")
+                hot_stride = int(st[0])
+            hot_ptr = _address(hot)
         if ts_cold is not None:
             st = _byte_strides(ts_cold)
             if len(st) == 1 and ts_cold.shape[0] > 1 and st[0] != _itemsize(ts_cold):
                 ts_cold_stride = int(st[0])
             ts_cold_ptr = _address(ts_cold)
         c = Cache(int(rows), int(row_bytes), int(id_mask), be.ptr(g2l),
-                  0 if g2l is None else int(g2l.shape[0]), be.ptr(hot_slot), be.ptr(hot),
-                  hot_rows, cold_ptr, be.ptr(ts_hot), ts_cold_ptr, cold_stride, ts_cold_stride)
+                  0 if g2l is None else int(g2l.shape[0]), be.ptr(hot_slot), hot_ptr,
+                  hot_rows, cold_ptr, be.ptr(ts_hot), ts_cold_ptr, cold_stride, ts_cold_stride, hot_stride)
         c._keep = (hot, cold, hot_slot, g2l, ts_hot, ts_cold)  # keep the arrays alive
         return c
 

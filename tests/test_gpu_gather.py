@@ -296,3 +296,47 @@ def test_gather_dedup_matches_numpy(oracle, hot, dim, dtype, hot_frac, dup):
     o_out, o_stats = np.empty((N, dim), dtype=full.dtype), np.zeros(4, dtype=np.int64)
     oracle.gather_dedup(oc, ids, o_out, None, stats=o_stats)
     assert np.array_equal(o_out.view(np.uint8), want.view(np.uint8)) and o_stats[3] == distinct
+
+
+def test_column_views_of_wider_rows_in_both_tiers(oracle, hot):
+    """One record per node in either tier - memory | features (| time, host tier) - gathered whole through one
+    cache, and its memory half read and updated through a second cache that is a column view of the same storage
+    (row strides travel in sgl_cache: hot_stride, cold_stride, ts_cold_stride).  Against numpy and the oracle."""
+    rows, N = 6000, 20_000
+    rng = np.random.default_rng(12)
+    mem, nf = rng.standard_normal((rows, 100)).astype(np.float32), rng.standard_normal((rows, 100)).astype(np.float32)
+    ts_full = rng.integers(0, 10**9, rows).astype(np.int64)
+    hot_ids = rng.permutation(rows)[: rows * 7 // 10]
+    slot = np.full(rows, -1, np.int32); slot[hot_ids] = np.arange(hot_ids.size, dtype=np.int32)
+    dev = hot.be.device
+    node_hot = torch.from_numpy(np.concatenate([mem[hot_ids], nf[hot_ids]], axis=1)).to(dev)
+    ts_hot = to_dev(hot, ts_full[hot_ids])
+    node_cold, ts_cold, rec = hot.interleaved_cold(rows, 200)
+    assert rec.shape[1] == 896                              # 800 bytes of rows + 8 of time in seven 128-byte lines
+    node_cold.copy_(torch.from_numpy(np.concatenate([mem, nf], axis=1))); ts_cold.copy_(torch.from_numpy(ts_full))
+    d_slot = to_dev(hot, slot, "i32")
+    c_node = hot.cache(800, node_hot, rows=rows, cold=node_cold, hot_slot=d_slot, ts_hot=ts_hot, ts_cold=ts_cold)
+    c_mem = hot.cache(400, node_hot[:, :100], rows=rows, cold=node_cold[:, :100], hot_slot=d_slot, ts_hot=ts_hot, ts_cold=ts_cold)
+    c_nf = hot.cache(400, node_hot[:, 100:], rows=rows, cold=node_cold[:, 100:], hot_slot=d_slot)
+    assert c_mem.hot_stride == 800 and c_mem.cold_stride == 896 and c_node.hot_stride == 0
+    ids = rng.integers(0, rows, N).astype(np.int64)
+    d_ids = to_dev(hot, ids)
+    out, out_ts = torch.empty((N, 200), device=dev), hot.be.empty(N)
+    hot.gather(c_node, d_ids, out, out_ts=out_ts)
+    assert np.array_equal(np_of(out), np.concatenate([mem[ids], nf[ids]], axis=1)) and np.array_equal(np_of(out_ts), ts_full[ids])
+    o_m, o_f = torch.empty((N, 100), device=dev), torch.empty((N, 100), device=dev)
+    hot.gather_multi(hot.gather_plan([(c_mem, d_ids, o_m, out_ts, None), (c_nf, d_ids, o_f, None, None)]))
+    assert np.array_equal(np_of(o_m), mem[ids]) and np.array_equal(np_of(o_f), nf[ids]) and np.array_equal(np_of(out_ts), ts_full[ids])
+    # memory update through the view: the feature half and the rows of other nodes stay as they are
+    upd = np.unique(rng.integers(0, rows, 900)).astype(np.int64)
+    vals, new_ts = rng.standard_normal((upd.size, 100)).astype(np.float32), rng.integers(0, 10**9, upd.size).astype(np.int64)
+    hot.scatter_update(c_mem, node_hot[:, :100], node_cold[:, :100], ts_hot, ts_cold, to_dev(hot, upd), to_dev(hot, vals, "f32"), to_dev(hot, new_ts))
+    mem2, ts2 = mem.copy(), ts_full.copy()
+    mem2[upd], ts2[upd] = vals, new_ts
+    hot.gather(c_node, d_ids, out, out_ts=out_ts)
+    assert np.array_equal(np_of(out), np.concatenate([mem2[ids], nf[ids]], axis=1)) and np.array_equal(np_of(out_ts), ts2[ids])
+    # the oracle reads the same views on the host
+    oc = oracle.cache(400, np_of(node_hot)[:, :100], rows=rows, cold=node_cold.numpy()[:, :100], hot_slot=slot)
+    o_out = np.empty((N, 100), dtype=np.float32)
+    oracle.gather(oc, ids, o_out)
+    assert np.array_equal(o_out, mem2[ids])
