@@ -921,9 +921,11 @@ __global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
 // of every such slot, one (slot, draw) pair per lane - the generator is most of the cost, and with a group of lanes
 // per slot the lanes of slots that do not draw (most slots of a deeper hop hold a handful of edges) idle through it
 // - then a group of KP lanes turns a slot's draws into its ascending picks in place: rank = number of smaller draws;
-// only when two draws of the slot are equal does one lane replay Floyd's construction (step j keeps its draw
-// unless an earlier step holds that value, then it takes len - k + j).  Picks are kept as 32-bit offsets into the
-// window; a window of 2^32 edges or more (no row of a graph this library can hold today) is picked lane by lane.
+// only in wavefronts where two draws of a slot are equal do the groups replay Floyd's construction first, stepping
+// together (step j keeps its draw unless an earlier step holds that value, then it takes len - k + j; with 20 picks
+// from windows of a few hundred edges most slots see such a pair, and one lane replaying it alone took three times
+// as long as the whole rest of the hop).  Picks are kept as 32-bit offsets into the window; a window of 2^32 edges or
+// more (no row of a graph this library can hold today) is picked by one lane into the slot's own output stretch.
 // The k picks of one slot whose window has 2^32 edges or more, by one lane, into `row` (global memory: the slot's
 // own k entries of an output array, which the copy that follows overwrites): Floyd's construction and an insertion
 // sort, or the draws in their order when drawing with replacement.
@@ -1088,47 +1090,48 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
                 // ascending picks in place, a group of KP lanes per drawing slot (all inside one wavefront, whose LDS
                 // accesses are served in program order: the group reads its row, then writes it)
                 const int lig = threadIdx.x % KP;
+                const int gsh = wlane / KP * KP;
+                // rank of `v` among the k values of row `di` (how many are smaller), and how many equal it
+                auto count = [&](int32_t di, uint32_t v, int32_t* smaller, int32_t* equal) {
+                    int32_t r = 0, e = 0;
+                    for (int32_t q = 0; q < k; q += 4) {
+                        const uint4 o = *reinterpret_cast<const uint4*>(&s_pick[di * KP + q]);
+                        r += (o.x < v ? 1 : 0) + ((q + 1 < k && o.y < v) ? 1 : 0) + ((q + 2 < k && o.z < v) ? 1 : 0) +
+                             ((q + 3 < k && o.w < v) ? 1 : 0);
+                        e += (o.x == v ? 1 : 0) + ((q + 1 < k && o.y == v) ? 1 : 0) + ((q + 2 < k && o.z == v) ? 1 : 0) +
+                             ((q + 3 < k && o.w == v) ? 1 : 0);
+                    }
+                    *smaller = r;
+                    *equal = e;
+                };
+                auto wave_sync = [] {          // orders this wavefront's LDS accesses before and after
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                };
                 for (int32_t di0 = 0; di0 < nd; di0 += BLOCK / KP) {           // block-uniform trip count
                     const int32_t di = di0 + (int)threadIdx.x / KP;
                     const bool on = di < nd && s_dl[di < nd ? di : 0] >= 0;
-                    const uint32_t mine = (on && lig < k) ? s_pick[di * KP + lig] : 0xFFFFFFFFu;
+                    const bool mine_on = on && lig < k;
+                    uint32_t m = mine_on ? s_pick[di * KP + lig] : 0xFFFFFFFFu;
                     int32_t r = 0, e = 0;
-                    if (on) {
-                        for (int32_t q = 0; q < k; q += 4) {
-                            const uint4 o = *reinterpret_cast<const uint4*>(&s_pick[di * KP + q]);
-                            r += (o.x < mine ? 1 : 0) + ((q + 1 < k && o.y < mine) ? 1 : 0) + ((q + 2 < k && o.z < mine) ? 1 : 0) +
-                                 ((q + 3 < k && o.w < mine) ? 1 : 0);
-                            e += (o.x == mine ? 1 : 0) + ((q + 1 < k && o.y == mine) ? 1 : 0) + ((q + 2 < k && o.z == mine) ? 1 : 0) +
-                                 ((q + 3 < k && o.w == mine) ? 1 : 0);
+                    if (on) count(di, m, &r, &e);
+                    if (__any(mine_on && e > 1)) {
+                        // two equal draws somewhere in the wavefront: Floyd's construction, the groups stepping together -
+                        // step j keeps its draw unless an earlier step holds that value, then it takes len - k + j
+                        const int64_t len = on ? s_len[s_dl[di]] : 0;
+                        for (int32_t jj = 1; jj < k; ++jj) {
+                            const uint32_t cand = (uint32_t)__shfl((int)m, gsh + jj);
+                            const bool hit = group_ballot<KP>(mine_on && lig < jj && m == cand, gsh) != 0;
+                            if (mine_on && lig == jj && hit) m = (uint32_t)(len - k + jj);
                         }
+                        wave_sync();
+                        if (mine_on) s_pick[di * KP + lig] = m;
+                        wave_sync();
+                        if (on) count(di, m, &r, &e);
                     }
-                    const bool clash = on && lig < k && e > 1;
-                    const uint64_t cm = __ballot(clash);
-                    const int gsh = wlane / KP * KP;
-                    const bool gclash = ((cm >> gsh) & ((1ull << KP) - 1ull)) != 0;
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                    __builtin_amdgcn_wave_barrier();
-                    if (on && !gclash && lig < k) s_pick[di * KP + r] = mine;
-                    if (on && gclash && lig == 0) {
-                        // two equal draws: Floyd's construction step by step, then an insertion sort, by one lane
-                        const int64_t len = s_len[s_dl[di]];
-                        uint32_t* row = &s_pick[di * KP];
-                        for (int32_t j = 1; j < k; ++j) {
-                            const uint32_t cand = row[j];
-                            bool dup = false;
-                            for (int32_t i = 0; i < j; ++i) dup |= row[i] == cand;
-                            if (dup) row[j] = (uint32_t)(len - k + j);
-                        }
-                        for (int32_t x = 1; x < k; ++x) {
-                            const uint32_t v = row[x];
-                            int32_t y = x - 1;
-                            while (y >= 0 && row[y] > v) {
-                                row[y + 1] = row[y];
-                                --y;
-                            }
-                            row[y + 1] = v;
-                        }
-                    }
+                    wave_sync();
+                    if (mine_on) s_pick[di * KP + r] = m;      // (all distinct now: the rank is the place)
                 }
             }
             __syncthreads();
@@ -1266,7 +1269,7 @@ HopKernel fill_fn(int G, bool uniform) {
     if (uniform) {
         switch (G) {
             case 16: return fill_uniform_flat_kernel<16, 256, 2>;
-            case 32: return fill_uniform_flat_kernel<32, 256, 2>;
+            case 32: return fill_uniform_flat_kernel<32, 256, 4>;
             default: return fill_kernel<64>;      // fanouts beyond 32: a wavefront per slot
         }
     }
