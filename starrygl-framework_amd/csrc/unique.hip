@@ -177,30 +177,60 @@ __global__ __launch_bounds__(BLOCK) void reduce_kernel(State s, int64_t* tile_su
     }
 }
 
-// exclusive scan of `nt` tile sums in place (only used beyond FUSED_SCAN_MAX tiles)
+// exclusive scan of `nt` tile sums in place (+ the grand total at [nt]), by one block, in pieces of SCAN_PIECE
+// sums: coalesced loads into LDS (a block that reads 8 consecutive sums per thread straight from memory issues
+// strided 64-byte reads, which one CU serves slowly), thread t then owns the 8 consecutive sums of its stretch, one
+// round of shuffles per wavefront scans the stretch totals, and the offsets leave through LDS, coalesced again.
+constexpr int SCAN_PER = 8;
+constexpr int SCAN_PIECE = SCAN_BLOCK * SCAN_PER;
 __global__ __launch_bounds__(SCAN_BLOCK) void scan_tiles_kernel(int64_t* tile_sum, int64_t nt) {
-    __shared__ int64_t s_part[SCAN_BLOCK];
-    const int64_t per = ceil_div<int64_t>(nt, SCAN_BLOCK);
-    const int64_t b0 = (int64_t)threadIdx.x * per;
-    const int64_t b1 = b0 + per < nt ? b0 + per : nt;
-    int64_t sum = 0;
-    for (int64_t b = b0; b < b1; ++b) sum += tile_sum[b];
-    s_part[threadIdx.x] = sum;
-    __syncthreads();
-    for (int d = 1; d < SCAN_BLOCK; d <<= 1) {
-        int64_t x = 0;
-        if ((int)threadIdx.x >= d) x = s_part[threadIdx.x - d];
+    constexpr int NW = SCAN_BLOCK / WAVE;
+    __shared__ int64_t s_v[SCAN_PIECE + SCAN_PIECE / 32];      // (a pad word per 32: the stretches start in different banks)
+    __shared__ int64_t s_w[NW];
+    const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
+    auto at = [](int i) { return i + (i >> 5); };
+    int64_t base = 0;
+    for (int64_t p0 = 0; p0 < nt; p0 += SCAN_PIECE) {          // block-uniform
         __syncthreads();
-        s_part[threadIdx.x] += x;
+#pragma unroll
+        for (int q = 0; q < SCAN_PER; ++q) {
+            const int i = q * SCAN_BLOCK + threadIdx.x;
+            s_v[at(i)] = p0 + i < nt ? tile_sum[p0 + i] : 0;
+        }
         __syncthreads();
+        int64_t v[SCAN_PER], sum = 0;
+#pragma unroll
+        for (int q = 0; q < SCAN_PER; ++q) {
+            v[q] = s_v[at(threadIdx.x * SCAN_PER + q)];
+            sum += v[q];
+        }
+        int64_t inc = sum;
+        for (int d = 1; d < WAVE; d <<= 1) {
+            const int64_t y = shfl_i64(inc, lane >= d ? lane - d : lane);
+            if (lane >= d) inc += y;
+        }
+        if (lane == WAVE - 1) s_w[wid] = inc;
+        __syncthreads();
+        int64_t run = base + inc - sum, total = 0;
+#pragma unroll
+        for (int q = 0; q < NW; ++q) {
+            if (q < wid) run += s_w[q];
+            total += s_w[q];
+        }
+#pragma unroll
+        for (int q = 0; q < SCAN_PER; ++q) {
+            s_v[at(threadIdx.x * SCAN_PER + q)] = run;
+            run += v[q];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < SCAN_PER; ++q) {
+            const int i = q * SCAN_BLOCK + threadIdx.x;
+            if (p0 + i < nt) tile_sum[p0 + i] = s_v[at(i)];
+        }
+        base += total;
     }
-    int64_t run = s_part[threadIdx.x] - sum;
-    for (int64_t b = b0; b < b1; ++b) {
-        const int64_t x = tile_sum[b];
-        tile_sum[b] = run;
-        run += x;
-    }
-    if (threadIdx.x == SCAN_BLOCK - 1) tile_sum[nt] = s_part[SCAN_BLOCK - 1];  // grand total
+    if (threadIdx.x == 0) tile_sum[nt] = base;
 }
 
 // Numbers the set bits in ascending id order.

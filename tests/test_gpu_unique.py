@@ -220,7 +220,7 @@ def test_hashed_state_reports_an_outgrown_capacity(hot):
     lh, uh, (th, _) = hot.unique_compact([a], _abi.UNIQUE_SORTED, hot.remap_hashed_state(1000), True)
     assert th == 900 and np.array_equal(np_of(lh[0]), np.arange(900))
     # remap_reinit picks the initialiser by the kind of state
-    d = hot.remap_state(5000)
+    d = hot.remap_state(7000)
     hot.unique_compact([a], _abi.UNIQUE_SORTED, d, True)
     lh, uh, (th, _) = hot.unique_compact([a], _abi.UNIQUE_SORTED, hot.remap_reinit(d), False)
     assert th == 900 and np.array_equal(np_of(lh[0]), np.arange(900))
