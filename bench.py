@@ -6,15 +6,20 @@ synthetic power-law graph: 2-hop most-recent 10x10 sampling, unique/compaction
 of the sampled node ids, node + edge feature gather, and 2-hop uniform 10x10
 sampling.  All inputs (graph, features, batches) are resident in HBM before the
 timed region starts; nothing inside the region synchronises with the host.
-The K timed steps are dealt in turn to a few independent pipelines (own
-buffers, HIP graph and stream each), so a few batches are in flight together
-as under a loader with a prefetch queue; `one_batch_in_flight` is the same K
-steps one after the other.
+
+The K timed steps run as a loader that samples ahead runs them: in groups of
+`--batches-per-call` mini-batches per pass of the library calls (one batched
+sampler call for both strategies, one batched unique with a local-id space per
+batch, one gather launch over all the group's rows), every batch keeping its
+own segment of every output; the groups are dealt in turn to a few independent
+pipelines (own buffers, HIP graph and stream each).  The same K steps with one
+set of library calls per batch (`per_batch_calls`, `one_batch_in_flight`) are
+reported beside the headline.
 
 Prints ONE JSON line: whole-step sampled edges/s as `value`, per-stage figures
-under `stages`, the HBM roofline of the dominant kernel (the step's gather
-launch) under `roofline`, and the CPU oracle sampler timed on the host cores
-under `cpu_baseline`.
+under `stages` / `stages_of_a_batched_pass`, the HBM roofline of the dominant
+kernel (the gather launch) under `roofline`, and the CPU oracle sampler timed
+on the host cores under `cpu_baseline`.
 """
 import argparse
 import json
@@ -37,7 +42,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes moved per algorithmic byte by the step's gather launch (node rows + hop-1 + hop-2 edge rows),
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (summary and commands:
 # profiles/gather_multi_kernel_configs1_hbm_traffic.md)
-MEASURED_HBM_PER_ALGORITHMIC_BYTE = {"read": 0.984, "write": 1.015}
+MEASURED_HBM_PER_ALGORITHMIC_BYTE = {"read": 1.027, "write": 1.015}
 
 
 def log(*a):
@@ -1210,6 +1215,7 @@ def main():
         # group's ids, each between a HIP event pair of its own on the stream it is launched on (the pair adds ~4 us
         # to a launch of several hundred)
         NR = 6
+        rl_each = []
         P = make_group_pipeline(pipe_streams[0], use_root_hint)
         torch.cuda.set_stream(P.stream)
         evp = []
@@ -1220,7 +1226,8 @@ def main():
             e0_.record(); P.stage_fns["gathers"](); e1_.record()
             if i > 0:       # (the first launch warms up)
                 evp.append((e0_, e1_))
-                rl_rows += np.array([int(P.uoff[BPC].item()), int(P.kb.counts[1].item()), int(P.kb.counts[4].item())])
+                rl_each.append([int(P.uoff[BPC].item()), int(P.kb.counts[1].item()), int(P.kb.counts[4].item())])
+                rl_rows += np.array(rl_each[-1])
         torch.cuda.synchronize()
         torch.cuda.set_stream(main_stream)
         dom_ms = float(np.mean([a_.elapsed_time(b_) for a_, b_ in evp]))
@@ -1268,6 +1275,8 @@ def main():
                 "avg_launch_ms": round(dom_ms, 5), "launches_timed": NR,
                 "algorithmic_bytes_per_launch": int(dom_bytes),
                 "mean_rows_per_launch": {"node": rl_rows[0], "edge_hop1": rl_rows[1], "edge_hop2": rl_rows[2]}}
+    if grouped:
+        roofline["rows_of_each_launch"] = rl_each      # [node, edge hop 1, edge hop 2] of the timed launches, in order
 
     # ---- CPU baseline: the oracle's 2-hop recent sampler on the host cores, same batches.  Every distinct
     # batch the CPU leg samples is compared with the GPU's result for that batch, array by array, bit-exact.

@@ -488,10 +488,13 @@ __global__ __launch_bounds__(BLOCK) void lookup_kernel(State s, Arrays a, int fo
 // universe rounded up to whole tiles of flag words, so that a tile belongs to one batch); array g's
 // elements [seg[g][b], seg[g][b+1]) belong to batch b.  Ascending numbering over the big universe is
 // batch-major and ascending inside a batch: batch b's local id = global rank - rank of the batch's first
-// tile.  Every call numbers afresh and looks up only ids it has numbered itself, so the table needs
-// neither epoch stamps nor clearing: 4 bytes per id, written by assign, read by lookup.
+// tile.  There is no id -> local id table: numbering leaves, per group of 64 ids, the 64 pending bits and the
+// batch-local rank of the group's first pending id (16 bytes per 64 ids: 256 KB for a million ids, which an L2
+// holds, where a 4-byte entry per id made every lookup a sector of its own out of a table that no L2 held), and
+// a lookup is that one 16-byte load and a popcount of the bits below the id's own.  Every call numbers afresh
+// and looks up only ids it has numbered itself, so nothing needs epoch stamps or clearing.
 constexpr int BATCH_MAX = SGL_BATCH_MAX;
-constexpr int64_t BATCH_STRIDE_ALIGN = (int64_t)TILE * 64;   // ids per tile of a bitmap state (a byte-flag tile holds TILE * 8)
+constexpr int64_t BATCH_STRIDE_ALIGN = (int64_t)TILE * 64;   // ids per tile: a thread of reduce / assign owns a group of 64
 
 struct Batched {
     int32_t B;
@@ -499,14 +502,19 @@ struct Batched {
     const int64_t* seg[MAXG];
 };
 
+struct alignas(16) RankWord {
+    uint64_t mask;      // pending bits of ids [64 w, 64 w + 64)
+    int64_t rank;       // batch-local rank of the first of them
+};
+
 struct BState {
-    uint32_t* table;    // [B * stride] local id inside the batch
+    RankWord* rank;     // [B * stride / 64]
     uint64_t* flags;    // pending flags: a byte per id (8 per word) or a bit per id
-    int64_t universe, words;
+    int64_t universe, words, groups;
     int32_t bytes;
 };
 
-// A flag byte per id up to 64M ids in all (B x the universe): a batch's marks are plain stores, and the two sweeps
+// A flag byte per id up to 64M ids in all (B x the universe): a batch's marks are plain stores, and the sweeps
 // over the flags cost less than atomics on a bitmap do (20 x 1M ids: 7.6 against 11.9 us per batch for the whole call).
 constexpr int64_t BATCHED_BYTE_FLAGS_MAX = 1ll << 26;
 inline bool batched_byte_flags(int64_t big) { return big <= BATCHED_BYTE_FLAGS_MAX; }
@@ -517,25 +525,16 @@ BState carve_batched(void* state, int64_t universe, int32_t B) {
     char* p = static_cast<char*>(state);
     s.universe = (int64_t)B * batch_stride(universe);
     s.bytes = batched_byte_flags(s.universe) ? 1 : 0;
-    s.words = ceil_div<int64_t>(s.universe, s.bytes ? 8 : 64);
-    s.flags = reinterpret_cast<uint64_t*>(p + HEADER_BYTES);
-    s.table = reinterpret_cast<uint32_t*>(s.flags + s.words);
+    s.words = s.universe / (s.bytes ? 8 : 64);
+    s.groups = s.universe / 64;
+    s.rank = reinterpret_cast<RankWord*>(p + HEADER_BYTES);                 // HEADER_BYTES is a multiple of 16
+    s.flags = reinterpret_cast<uint64_t*>(s.rank + s.groups);
     return s;
 }
 
 __global__ void init_batched_kernel(BState s) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < s.words; i += stride) s.flags[i] = 0;
-}
-
-// batch of element i of an array whose batch offsets are seg[0..B] (in LDS): the last b with seg[b] <= i
-__device__ __forceinline__ int batch_of(const int64_t* seg, int B, int64_t i) {
-    int lo = 0, hi = B;     // seg[lo] <= i < seg[hi] for a live element
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (seg[mid] <= i) lo = mid; else hi = mid;
-    }
-    return lo;
 }
 
 __device__ __forceinline__ void stage_segs(const Batched& bt, int G, int64_t (*s_seg)[BATCH_MAX + 1]) {
@@ -548,51 +547,133 @@ __device__ __forceinline__ void stage_segs(const Batched& bt, int G, int64_t (*s
 
 // LOOKUP == false: sets the flag of every id (a new numbering per call: no table read);
 // LOOKUP == true : rewrites every array through the table.
+//
+// Which block walks which batch follows the chip: workgroups go to the 8 XCDs in turn (block i runs on XCD i % 8) and
+// every XCD has an L2 of its own, so all blocks of one XCD work on the same batch at the same time (batch b belongs to
+// the blocks of class b % V; V = 8 from eight batches on, the largest power of two <= B below).  A batch's flags (1 MB
+// for a million ids) and its slice of the table (4 MB) then stay in one L2 while the batch is walked: with every block
+// striding over all batches the lookup walk of 16 batches fetched a 64-byte sector per element (240 MB for 19 MB of
+// ids) and the marking walk wrote one per flag byte.  Only the speed depends on that placement, the result does not.
+constexpr int XCDS = 8;
+constexpr int WALK_ILP = 4;
+constexpr int WALK_SEGS = (BATCH_MAX / XCDS) * MAXG;        // (batch, array) pieces one class of blocks can own
+static_assert(BATCH_MAX % XCDS == 0 && WALK_SEGS <= WAVE && MAXG <= XCDS, "the pieces of a class are listed by one wavefront");
+
 template <bool LOOKUP>
 __global__ __launch_bounds__(BLOCK) void walk_batched_kernel(BState s, Arrays a, Batched bt) {
     __shared__ int64_t s_seg[MAXG][BATCH_MAX + 1];
+    __shared__ int64_t s_pref[WALK_SEGS + 1], s_lo[WALK_SEGS], s_base[WALK_SEGS];
+    __shared__ const int64_t* s_ids[WALK_SEGS];
+    __shared__ int64_t* s_out[WALK_SEGS];
     stage_segs(bt, a.G, s_seg);
-    int64_t len[MAXG], max_len = 0;
-#pragma unroll
-    for (int g = 0; g < MAXG; ++g) {
-        len[g] = 0;
-        if (g < a.G) {
-            const int64_t l = s_seg[g][bt.B];
-            len[g] = l < 0 ? 0 : (l > a.len_max[g] ? a.len_max[g] : l);
+    int V = XCDS;
+    while (V > bt.B) V >>= 1;                                   // classes of blocks (a power of two, >= 1)
+    const int x = blockIdx.x % XCDS;
+    const int cls = x % V;
+    // this block's place among the blocks of its class, and how many those are (the grid is a multiple of XCDS)
+    const int64_t worker = (int64_t)(blockIdx.x / XCDS) * (XCDS / V) + x / V;
+    const int64_t step = (int64_t)(gridDim.x / XCDS) * (XCDS / V) * BLOCK;
+    // The class's pieces - array g's elements of batch b, for every batch of the class - laid end to end as one
+    // index range, so that every lane has an element whatever the pieces' sizes are (a batch's root list is a
+    // twentieth of its hop-2 list).  Piece e = (e / MAXG)-th batch of the class, array e % MAXG.
+    if (threadIdx.x < WAVE) {
+        const int e = threadIdx.x;
+        const int g = e % MAXG, b = cls + (e / MAXG) * V;
+        int64_t lo = 0, n = 0;
+        if (e < WALK_SEGS && g < a.G && b < bt.B) {
+            int64_t top = s_seg[g][bt.B];
+            top = top < 0 ? 0 : (top > a.len_max[g] ? a.len_max[g] : top);
+            lo = s_seg[g][b];
+            int64_t hi = s_seg[g][b + 1];
+            lo = lo < 0 ? 0 : lo;
+            hi = hi > top ? top : hi;
+            n = hi > lo ? hi - lo : 0;
         }
-        max_len = len[g] > max_len ? len[g] : max_len;
+        int64_t inc = n;
+        for (int d = 1; d < WAVE; d <<= 1) {
+            const int64_t y = __shfl_up(inc, d);
+            if (e >= d) inc += y;
+        }
+        if (e < WALK_SEGS) {
+            s_pref[e] = inc - n;
+            s_lo[e] = lo;
+            s_base[e] = (int64_t)b * bt.stride;
+            s_ids[e] = g < a.G ? a.ids[g] : nullptr;
+            s_out[e] = g < a.G ? a.out[g] : nullptr;
+        }
+        if (e == WALK_SEGS - 1) s_pref[WALK_SEGS] = inc;
     }
-    for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < max_len; i += (int64_t)gridDim.x * BLOCK) {
-        int64_t id[MAXG];
-        int64_t at[MAXG];
+    __syncthreads();
+    const int64_t total = s_pref[WALK_SEGS];
+    for (int64_t j0 = worker * BLOCK + threadIdx.x; j0 < total; j0 += step * WALK_ILP) {
+        int64_t id[WALK_ILP], at[WALK_ILP];
+        int64_t* dst[WALK_ILP];
 #pragma unroll
-        for (int g = 0; g < MAXG; ++g) {
-            id[g] = -1;
-            at[g] = 0;
-            if (g < a.G && i < len[g]) {
-                id[g] = a.ids[g][i];       // ids may alias out
-                at[g] = id[g] + (int64_t)batch_of(s_seg[g], bt.B, i) * bt.stride;
+        for (int u = 0; u < WALK_ILP; ++u) {
+            const int64_t j = j0 + u * step;
+            id[u] = -1;
+            at[u] = 0;
+            dst[u] = nullptr;
+            if (j < total) {
+                int e = 0;                                  // the last piece that starts at or before j
+#pragma unroll
+                for (int h = WALK_SEGS / 2; h > 0; h >>= 1)
+                    if (s_pref[e + h] <= j) e += h;
+                const int64_t i = s_lo[e] + (j - s_pref[e]);
+                id[u] = s_ids[e][i];                        // ids may alias out: every element is read before it is written
+                at[u] = s_base[e] + id[u];
+                dst[u] = s_out[e] + i;
             }
         }
         if constexpr (LOOKUP) {
-            uint32_t e[MAXG];
+            RankWord v[WALK_ILP];
 #pragma unroll
-            for (int g = 0; g < MAXG; ++g) e[g] = (id[g] >= 0 && id[g] < bt.universe) ? s.table[at[g]] : 0u;
+            for (int u = 0; u < WALK_ILP; ++u) v[u] = (id[u] >= 0 && id[u] < bt.universe) ? s.rank[at[u] >> 6] : RankWord{0ull, -1};
 #pragma unroll
-            for (int g = 0; g < MAXG; ++g)
-                if (g < a.G && i < len[g]) a.out[g][i] = (id[g] >= 0 && id[g] < bt.universe) ? (int64_t)e[g] : -1;
+            for (int u = 0; u < WALK_ILP; ++u)
+                if (dst[u])
+                    *dst[u] = (id[u] >= 0 && id[u] < bt.universe)
+                                  ? v[u].rank + __popcll(v[u].mask & ((1ull << (at[u] & 63)) - 1ull)) : -1;
         } else {
 #pragma unroll
-            for (int g = 0; g < MAXG; ++g)
-                if (id[g] >= 0 && id[g] < bt.universe) remap_set_pending(s.flags, s.bytes, at[g]);
+            for (int u = 0; u < WALK_ILP; ++u)
+                if (id[u] >= 0 && id[u] < bt.universe) remap_set_pending(s.flags, s.bytes, at[u]);
         }
     }
 }
 
+// the eight flag bytes (0 or 1 each) of a word as eight bits, byte i -> bit i
+__device__ __forceinline__ uint64_t pack_flag_bytes(uint64_t w) {
+    return (((w << 7) & 0x8080808080808080ull) * 0x0002040810204081ull) >> 56;
+}
+
+// Thread w owns ids [64 w, 64 w + 64): it turns their flags into the group's 64 pending bits (left in rank[w].mask),
+// clears the flags for the next call and counts; a block's count is its tile's sum.
 __global__ __launch_bounds__(BLOCK) void reduce_batched_kernel(BState s, int64_t* tile_sum) {
     __shared__ int32_t s_w[BLOCK / WAVE];
     const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
-    int32_t c = (w < s.words) ? __popcll(s.flags[w]) : 0;
+    uint64_t mask = 0;
+    if (w < s.groups) {
+        if (s.bytes) {
+            const ulonglong2* f = reinterpret_cast<const ulonglong2*>(s.flags + w * 8);
+            ulonglong2 q[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) q[j] = f[j];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) mask |= (pack_flag_bytes(q[j].x) | (pack_flag_bytes(q[j].y) << 8)) << (16 * j);
+            if (mask) {
+                ulonglong2* fw = reinterpret_cast<ulonglong2*>(s.flags + w * 8);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (q[j].x | q[j].y) fw[j] = ulonglong2{0ull, 0ull};
+            }
+        } else {
+            mask = s.flags[w];
+            if (mask) s.flags[w] = 0;
+        }
+        s.rank[w].mask = mask;
+    }
+    int32_t c = __popcll(mask);
     for (int d = WAVE / 2; d > 0; d >>= 1) c += __shfl_down(c, d);
     if (threadIdx.x % WAVE == 0) s_w[threadIdx.x / WAVE] = c;
     __syncthreads();
@@ -603,7 +684,7 @@ __global__ __launch_bounds__(BLOCK) void reduce_batched_kernel(BState s, int64_t
     }
 }
 
-// Numbers the set flags (tile_sum holds the exclusive tile offsets, the total at [nt]): an id's local id is its
+// Numbers the pending ids (tile_sum holds the exclusive tile offsets, the total at [nt]): an id's local id is its
 // rank inside its batch, i.e. the global rank minus the offset of the batch's first tile; the first tile of
 // every batch records where the batch's list begins.
 __global__ __launch_bounds__(BLOCK) void assign_batched_kernel(BState s, const int64_t* tile_sum, int64_t nt, Batched bt,
@@ -611,7 +692,7 @@ __global__ __launch_bounds__(BLOCK) void assign_batched_kernel(BState s, const i
     __shared__ int32_t s_wave[BLOCK / WAVE];
     const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
     const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
-    uint64_t word = (w < s.words) ? s.flags[w] : 0ull;
+    uint64_t word = (w < s.groups) ? s.rank[w].mask : 0ull;
     const int32_t c = __popcll(word);
     int32_t inc = c;
     for (int d = 1; d < WAVE; d <<= 1) {
@@ -623,34 +704,28 @@ __global__ __launch_bounds__(BLOCK) void assign_batched_kernel(BState s, const i
     int32_t wave_off = 0;
     for (int q = 0; q < wid; ++q) wave_off += s_wave[q];
     const int64_t tile_off = tile_sum[blockIdx.x];
-    const int ipw = s.bytes ? 8 : 64;                       // ids per flag word
-    const int64_t tiles_per_batch = bt.stride / ((int64_t)TILE * ipw);
+    const int64_t tiles_per_batch = bt.stride / BATCH_STRIDE_ALIGN;
     const int64_t b = (int64_t)blockIdx.x / tiles_per_batch;        // the tile's batch (a stride is a whole number of tiles)
     const int64_t batch_off = tile_sum[b * tiles_per_batch];
     if (threadIdx.x == 0) {
         if ((int64_t)blockIdx.x == b * tiles_per_batch) U_off[b] = tile_off;
         if (blockIdx.x == nt - 1) U_off[bt.B] = tile_sum[nt];
     }
-    if (c == 0) return;
+    if (w >= s.groups) return;
     int64_t rank = tile_off + wave_off + (inc - c);
-    const int64_t id0 = w * ipw;
-    const int shift = s.bytes ? 3 : 0;
-    const int64_t base = b * bt.stride;
+    s.rank[w].rank = rank - batch_off;
+    const int64_t id0 = w * 64 - b * bt.stride;
     while (word) {
         const int bit = __ffsll((unsigned long long)word) - 1;
         word &= word - 1;
-        const int64_t id = id0 + (bit >> shift);
-        s.table[id] = (uint32_t)(rank - batch_off);
-        if (rank < unique_capacity) unique_out[rank] = id - base;
+        if (rank < unique_capacity) unique_out[rank] = id0 + bit;
         ++rank;
     }
-    s.flags[w] = 0;
 }
 
 size_t batched_workspace_bytes(int64_t universe, int32_t B) {
     const int64_t big = (int64_t)B * batch_stride(universe);
-    const int64_t words = ceil_div<int64_t>(big, batched_byte_flags(big) ? 8 : 64);
-    return align_up((size_t)(ceil_div<int64_t>(words, TILE) + 2) * 8) + 512;
+    return align_up((size_t)(big / BATCH_STRIDE_ALIGN + 2) * 8) + 512;
 }
 
 size_t dense_workspace_bytes(int64_t universe) {
@@ -828,8 +903,7 @@ extern "C" int32_t sgl_unique_compact(void* state, int64_t universe, int32_t res
 extern "C" size_t sgl_remap_batched_state_bytes(int64_t universe, int32_t B) {
     if (universe <= 0 || B < 1 || B > BATCH_MAX) return 0;
     const int64_t big = (int64_t)B * batch_stride(universe);
-    const int64_t words = ceil_div<int64_t>(big, batched_byte_flags(big) ? 8 : 64);
-    return HEADER_BYTES + (size_t)words * 8 + (size_t)big * 4 + 8;
+    return HEADER_BYTES + (size_t)(big / 64) * sizeof(RankWord) + (size_t)(big / (batched_byte_flags(big) ? 1 : 8)) + 16;
 }
 
 extern "C" int32_t sgl_remap_batched_init(void* state, size_t state_bytes, int64_t universe, int32_t B, void* stream) {
@@ -838,7 +912,7 @@ extern "C" int32_t sgl_remap_batched_init(void* state, size_t state_bytes, int64
     if ((int64_t)B * batch_stride(universe) > 0xFFFFFFFFll) return fail(SGL_ENOTSUP, "remap_batched_init: B * universe > 2^32");
     if (state_bytes < sgl_remap_batched_state_bytes(universe, B))
         return fail(SGL_ENOMEM, "remap_batched_init: state %zu < %zu bytes", state_bytes, sgl_remap_batched_state_bytes(universe, B));
-    if (reinterpret_cast<uintptr_t>(state) % 8) return fail(SGL_EINVAL, "remap_batched_init: state must be 8-byte aligned");
+    if (reinterpret_cast<uintptr_t>(state) % 16) return fail(SGL_EINVAL, "remap_batched_init: state must be 16-byte aligned");
     BState s = carve_batched(state, universe, B);
     int64_t blocks = ceil_div<int64_t>(s.words, 256);
     if (blocks > 65536) blocks = 65536;
@@ -864,6 +938,7 @@ extern "C" int32_t sgl_unique_compact_batched(void* state, int64_t universe, int
     if (G > MAXG) return fail(SGL_ENOTSUP, "unique_compact_batched: more than %d arrays", MAXG);
     if (unique_capacity < 0 || (unique_capacity > 0 && !unique_out))
         return fail(SGL_EINVAL, "unique_compact_batched: unique_out is NULL");
+    if (reinterpret_cast<uintptr_t>(state) % 16) return fail(SGL_EINVAL, "unique_compact_batched: state must be 16-byte aligned");
     if (!ws || ws_bytes < batched_workspace_bytes(universe, B))
         return fail(SGL_ENOMEM, "unique_compact_batched: workspace %zu < %zu bytes", ws_bytes, batched_workspace_bytes(universe, B));
     Arrays all;
@@ -888,10 +963,12 @@ extern "C" int32_t sgl_unique_compact_batched(void* state, int64_t universe, int
     hipStream_t st = as_stream(stream);
     BState s = carve_batched(state, universe, B);
     Arena ar(ws, ws_bytes);
-    const int64_t nt = ceil_div<int64_t>(s.words, TILE);
+    const int64_t nt = s.groups / TILE;
     int64_t* tile_sum = ar.take<int64_t>(nt + 2);
     if (!ar.ok()) return fail(SGL_ENOMEM, "unique_compact_batched: workspace too small");
-    int64_t mb = ceil_div<int64_t>(longest > 0 ? longest : 1, BLOCK);
+    // a whole number of blocks per XCD; the walk deals the batches to classes of blocks, so the grid follows the
+    // ids in all, not the longest array
+    int64_t mb = ceil_div<int64_t>(ceil_div<int64_t>(all.start[MAXG] > 0 ? all.start[MAXG] : 1, BLOCK * WALK_ILP), XCDS) * XCDS;
     if (mb > MAX_GRID) mb = MAX_GRID;
     if (longest > 0) {
         hipLaunchKernelGGL(walk_batched_kernel<false>, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, all, bt);
