@@ -965,9 +965,12 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
     __shared__ int64_t s_start[SLOTS], s_t[SLOTS], s_len[SLOTS];
     __shared__ int32_t s_dl[SLOTS];          // chunk-local index of the q-th drawing slot
     __shared__ int32_t s_didx[SLOTS];        // slot -> its place in s_dl, -1: copies its window, -2: window >= 2^32 edges
-    __shared__ __attribute__((aligned(16))) uint32_t s_pick[SLOTS * KP];
+    // a drawing slot's picks: rows of kp = fanout rounded up to 4 entries (16-byte rows), SLOTS rows, sized at the launch
+    // (uniform_flat_lds): with rows of KP entries a block of the fanout-20 kernel held 41 KB of LDS and three blocks shared a CU
+    extern __shared__ __attribute__((aligned(16))) uint32_t s_pick[];
     const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
     const int32_t k = a.k;
+    const int32_t kp = (k + 3) & ~3;
     const int64_t S = live_count(a.S_dev, a.S_max);
     int64_t first, run;
     block_run(S, a.align, &first, &run);
@@ -1080,7 +1083,7 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
                 if (j >= 0) {
                     const int64_t len = s_len[j];
                     const uint64_t bits = draw_bits(a.seed, a.hop, chunk0 + j, d);
-                    s_pick[di * KP + d] = (uint32_t)(a.replace ? bounded(bits, len) : bounded(bits, len - k + d + 1));
+                    s_pick[di * kp + d] = (uint32_t)(a.replace ? bounded(bits, len) : bounded(bits, len - k + d + 1));
                 }
             }
             // (windows of 2^32 edges or more: 64-bit picks, parked in the slot's own stretch of the output)
@@ -1096,7 +1099,7 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
                 auto count = [&](int32_t di, uint32_t v, int32_t* smaller, int32_t* equal) {
                     int32_t r = 0, e = 0;
                     for (int32_t q = 0; q < k; q += 4) {
-                        const uint4 o = *reinterpret_cast<const uint4*>(&s_pick[di * KP + q]);
+                        const uint4 o = *reinterpret_cast<const uint4*>(&s_pick[di * kp + q]);
                         r += (o.x < v ? 1 : 0) + ((q + 1 < k && o.y < v) ? 1 : 0) + ((q + 2 < k && o.z < v) ? 1 : 0) +
                              ((q + 3 < k && o.w < v) ? 1 : 0);
                         e += (o.x == v ? 1 : 0) + ((q + 1 < k && o.y == v) ? 1 : 0) + ((q + 2 < k && o.z == v) ? 1 : 0) +
@@ -1114,7 +1117,7 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
                     const int32_t di = di0 + (int)threadIdx.x / KP;
                     const bool on = di < nd && s_dl[di < nd ? di : 0] >= 0;
                     const bool mine_on = on && lig < k;
-                    uint32_t m = mine_on ? s_pick[di * KP + lig] : 0xFFFFFFFFu;
+                    uint32_t m = mine_on ? s_pick[di * kp + lig] : 0xFFFFFFFFu;
                     int32_t r = 0, e = 0;
                     if (on) count(di, m, &r, &e);
                     if (__any(mine_on && e > 1)) {
@@ -1127,12 +1130,12 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
                             if (mine_on && lig == jj && hit) m = (uint32_t)(len - k + jj);
                         }
                         wave_sync();
-                        if (mine_on) s_pick[di * KP + lig] = m;
+                        if (mine_on) s_pick[di * kp + lig] = m;
                         wave_sync();
                         if (on) count(di, m, &r, &e);
                     }
                     wave_sync();
-                    if (mine_on) s_pick[di * KP + r] = m;      // (all distinct now: the rank is the place)
+                    if (mine_on) s_pick[di * kp + r] = m;      // (all distinct now: the rank is the place)
                 }
             }
             __syncthreads();
@@ -1155,7 +1158,7 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
                     const int32_t j = x - s_off[lo], di = s_didx[lo];
                     int64_t sel = j;
                     if (di >= 0) {
-                        sel = (int64_t)s_pick[di * KP + j];
+                        sel = (int64_t)s_pick[di * kp + j];
                     } else if (di == -2) {
                         sel = a.nbr_dt[run_off + x];      // parked there by huge_window_picks (this lane overwrites it below)
                     }
@@ -1254,6 +1257,11 @@ int32_t check_out(const sgl_hop_out* o, int64_t S_max, int32_t k) {
 
 using HopKernel = void (*)(HopArgs);
 
+// dynamic LDS of fill_uniform_flat_kernel: UFLAT_SLOTS rows of the fanout rounded up to 4 picks
+constexpr int UFLAT_SLOTS = 256;
+inline size_t uniform_flat_lds(int32_t k) { return (size_t)UFLAT_SLOTS * ((k + 3) & ~3) * sizeof(uint32_t); }
+
+
 HopKernel count_fn(int G) {
     switch (G) {
         case 1: return count_lane_kernel;
@@ -1269,8 +1277,8 @@ HopKernel count_fn(int G) {
 HopKernel fill_fn(int G, bool uniform) {
     if (uniform) {
         switch (G) {
-            case 16: return fill_uniform_flat_kernel<16, 256, 2>;
-            case 32: return fill_uniform_flat_kernel<32, 256, 4>;
+            case 16: return fill_uniform_flat_kernel<16, UFLAT_SLOTS, 2>;
+            case 32: return fill_uniform_flat_kernel<32, UFLAT_SLOTS, 4>;
             default: return fill_kernel<64>;      // fanouts beyond 32: a wavefront per slot
         }
     }
@@ -1311,7 +1319,8 @@ int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf, bool do_count = tr
     }
     if (!do_fill) return SGL_OK;
     // a uniform fanout beyond one wavefront keeps a slot's picks in LDS (one wave per slot)
-    const size_t wide_lds = (a.type == SGL_SAMPLE_UNIFORM && a.k > WAVE) ? (size_t)NWAVE * a.k * sizeof(int64_t) : 0;
+    size_t wide_lds = (a.type == SGL_SAMPLE_UNIFORM && a.k > WAVE) ? (size_t)NWAVE * a.k * sizeof(int64_t) : 0;
+    if (a.type == SGL_SAMPLE_UNIFORM && Gf <= 32) wide_lds = uniform_flat_lds(a.k);
     hipLaunchKernelGGL(fill_fn(Gf, a.type == SGL_SAMPLE_UNIFORM), dim3((unsigned)blocks), dim3(BLOCK), wide_lds, st, a);
     SGL_LAUNCH_CHECK();
     return SGL_OK;
