@@ -91,10 +91,12 @@ def test_batched_sampler_refuses_marking_and_bad_sizes(hot, small):
         hot.sample_khop_batched(dg, node, t[:5], ptr, 2, [hot.params("recent", 3)])
 
 
-@pytest.mark.parametrize("universe,B", [(5000, 6), (16384, 4), (16385, 3), (1_000_000, 16), (3_000_000, 8), (70_000, 64), (9_000_000, 8)])
+@pytest.mark.parametrize("universe,B", [(5000, 6), (16384, 4), (16385, 3), (1_000_000, 16), (3_000_000, 8), (70_000, 64), (9_000_000, 8),
+                                        (2000, 1), (50_000, 7), (300, 9), (40_000, 33)])
 def test_batched_unique_parity(oracle, hot, universe, B):
-    """universes below, at and above one tile of flag words; states of up to 64M ids in all keep a flag byte per id,
-    8 x 9M runs on the bitmap"""
+    """universes below, at and above one tile of 16384 ids; states of up to 64M ids in all keep a flag byte per id,
+    8 x 9M runs on the bitmap; batch counts below, at and above the eight classes of blocks that share the batches out
+    (one class per XCD), also ones that do not divide evenly"""
     rng = np.random.default_rng(universe + B)
     hs, ds = oracle.remap_batched_state(universe, B), hot.remap_batched_state(universe, B)
     for trial in range(3):             # consecutive epochs on one state, the last call smaller
