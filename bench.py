@@ -42,7 +42,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes moved per algorithmic byte by the step's gather launch (node rows + hop-1 + hop-2 edge rows),
 # from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script (summary and commands:
 # profiles/gather_multi_kernel_configs1_hbm_traffic.md)
-MEASURED_HBM_PER_ALGORITHMIC_BYTE = {"read": 1.027, "write": 1.015}
+MEASURED_HBM_PER_ALGORITHMIC_BYTE = {"read": 0.985, "write": 1.014}
 
 
 def log(*a):
