@@ -170,12 +170,13 @@ __device__ __forceinline__ void mark_id(const HopArgs& a, int64_t id) {
 // Slots [first, first + run) belong to block b; run is a multiple of `spb`, itself a
 // multiple of the slots either kernel of the hop handles per block iteration, so that
 // iterations never straddle two blocks and both kernels see the same partition.
-__device__ __forceinline__ void block_run(int64_t S, int spb, int64_t* first, int64_t* run) {
-    int64_t r = ceil_div<int64_t>(S, (int64_t)gridDim.x);
+__device__ __forceinline__ void block_run(int64_t S, int spb, int64_t* first, int64_t* run, unsigned bid = blockIdx.x,
+                                          unsigned nblk = gridDim.x) {
+    int64_t r = ceil_div<int64_t>(S, (int64_t)nblk);
     r = ceil_div<int64_t>(r, spb) * spb;
     if (r < spb) r = spb;
     *run = r;
-    *first = (int64_t)blockIdx.x * r;
+    *first = (int64_t)bid * r;
 }
 
 // (node, t) of slot s
@@ -332,13 +333,13 @@ __device__ __forceinline__ int64_t lane_lower_bound(const int64_t* __restrict__ 
 // slots per lane with their searches stepping together were measured slower: 116 and 122 us against 114 us per
 // 192 000-root two-hop call at two and four slots per lane; so was ending every bisection at 16 entries that are
 // loaded side by side and counted, 124 us: more loads cost more than fewer dependent rounds save.)
-__global__ __launch_bounds__(BLOCK) void count_lane_kernel(HopArgs a) {
+__device__ __forceinline__ void count_lane_body(const HopArgs& a, unsigned bid, unsigned nblk) {
     __shared__ int32_t s_cnt[NWAVE];
     __shared__ int32_t s_bad[NWAVE];
     const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
     const int64_t S = live_count(a.S_dev, a.S_max);
     int64_t first, run;
-    block_run(S, a.align, &first, &run);
+    block_run(S, a.align, &first, &run, bid, nblk);
     const int64_t end = first + run < S ? first + run : S;
     const int64_t eq = a.equal_root_time ? 1 : 0;
     int32_t sum = 0, nbad = 0;
@@ -385,9 +386,21 @@ __global__ __launch_bounds__(BLOCK) void count_lane_kernel(HopArgs a) {
             tot += s_cnt[i];
             totb += s_bad[i];
         }
-        a.block_sum[blockIdx.x] = tot;
-        a.block_bad[blockIdx.x] = totb;
+        a.block_sum[bid] = tot;
+        a.block_bad[bid] = totb;
     }
+}
+
+__global__ __launch_bounds__(BLOCK) void count_lane_kernel(HopArgs a) { count_lane_body(a, blockIdx.x, gridDim.x); }
+
+// Two hops' kernels in one launch (the same hop of two queries over grids of the same size: a most-recent and a
+// uniform query of a batched call): the blocks of the two take turns in the grid, so that both kinds are spread over
+// all CUs and run beside each other - each of these kernels alone leaves a chip of 256 CUs waiting on its dependent
+// loads, and two launches one after the other pay two ramps and two tails.
+__global__ __launch_bounds__(BLOCK) void count_lane_dual_kernel(HopArgs a, HopArgs b) {
+    const unsigned bid = blockIdx.x >> 1, nblk = gridDim.x >> 1;
+    if (blockIdx.x & 1) count_lane_body(b, bid, nblk);
+    else count_lane_body(a, bid, nblk);
 }
 
 // Prefix of the block sums at a granularity of CHUNK blocks, by one block (only
@@ -397,7 +410,7 @@ __global__ __launch_bounds__(BLOCK) void count_lane_kernel(HopArgs a) {
 // fill block adds the < CHUNK sums of its own chunk (one cache line) itself.
 // Publishes the counts and the terminating pointer entries.
 constexpr int CHUNK = MAX_BLOCKS / SCAN_BLOCK;
-__global__ __launch_bounds__(SCAN_BLOCK) void scan_kernel(HopArgs a, int nb) {
+__device__ __forceinline__ void scan_body(const HopArgs& a, int nb) {
     constexpr int NW = SCAN_BLOCK / WAVE;
     __shared__ int32_t s_v[MAX_BLOCKS];
     __shared__ int64_t s_w[NW];
@@ -440,6 +453,11 @@ __global__ __launch_bounds__(SCAN_BLOCK) void scan_kernel(HopArgs a, int nb) {
         a.root_start_ptr[S] = total;
         a.root_end_ptr[S] = total;
     }
+}
+__global__ __launch_bounds__(SCAN_BLOCK) void scan_kernel(HopArgs a, int nb) { scan_body(a, nb); }
+__global__ __launch_bounds__(SCAN_BLOCK) void scan_dual_kernel(HopArgs a, HopArgs b, int nb) {     // two blocks
+    if (blockIdx.x) scan_body(b, nb);
+    else scan_body(a, nb);
 }
 
 // Philox4x32-10, counter (draw, slot_lo, slot_hi, hop), key (seed_lo, seed_hi);
@@ -760,12 +778,20 @@ __global__ __launch_bounds__(BLOCK) void fill_kernel(HopArgs a) {
 // and the stores of a block-iteration are one contiguous piece per output array.
 constexpr int FLAT_SLOTS = 2 * BLOCK;
 static_assert((int64_t)FLAT_SLOTS * SGL_RECENT_MAX_FANOUT <= INT32_MAX, "a chunk's edge offsets are 32-bit");
-__global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
-    __shared__ int64_t s_red[NWAVE];
-    __shared__ int32_t s_redb[NWAVE];
-    __shared__ int32_t s_w[NWAVE];
-    __shared__ int32_t s_off[FLAT_SLOTS + 1];
-    __shared__ int64_t s_start[FLAT_SLOTS], s_t[FLAT_SLOTS];
+struct FlatLds {      // the LDS of one block of the most-recent copy
+    int64_t red[NWAVE];
+    int64_t start[FLAT_SLOTS], t[FLAT_SLOTS];
+    int32_t redb[NWAVE];
+    int32_t w[NWAVE];
+    int32_t off[FLAT_SLOTS + 1];
+};
+__device__ __forceinline__ void fill_flat_body(const HopArgs& a, unsigned bid, unsigned nblk, FlatLds& lds) {
+    int64_t* const s_red = lds.red;
+    int32_t* const s_redb = lds.redb;
+    int32_t* const s_w = lds.w;
+    int32_t* const s_off = lds.off;
+    int64_t* const s_start = lds.start;
+    int64_t* const s_t = lds.t;
     const int wlane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
     const int32_t k = a.k;
     // Runs of up to 16 edges come from the graph's interleaved records when it has them: a run then lies in one
@@ -774,7 +800,7 @@ __global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
     const bool use_rec = a.rec != nullptr && k <= 16;
     const int64_t S = live_count(a.S_dev, a.S_max);
     int64_t first, run;
-    block_run(S, a.align, &first, &run);
+    block_run(S, a.align, &first, &run, bid, nblk);
     const int64_t run_end = first + run < S ? first + run : S;
     // the first chunk's slots (two consecutive ones per thread): loaded beside the block's offset
     constexpr int SPT = FLAT_SLOTS / BLOCK;      // consecutive slots per thread
@@ -795,16 +821,16 @@ __global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
     int64_t run_off = 0;
     if (a.scanned) {
         constexpr int CH = MAX_BLOCKS / SCAN_BLOCK;
-        const int c0 = (int)blockIdx.x / CH * CH;
-        run_off = a.chunk_off[blockIdx.x / CH];
+        const int c0 = (int)bid / CH * CH;
+        run_off = a.chunk_off[bid / CH];
 #pragma unroll
         for (int q = 0; q < CH - 1; ++q)
-            if (c0 + q < (int)blockIdx.x) run_off += a.block_sum[c0 + q];
+            if (c0 + q < (int)bid) run_off += a.block_sum[c0 + q];
     } else {
         int64_t part = 0;
         int32_t partb = 0;
-        const bool last = blockIdx.x == gridDim.x - 1;
-        for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += BLOCK) {
+        const bool last = bid == nblk - 1;
+        for (int64_t b = threadIdx.x; b < (int64_t)bid; b += BLOCK) {
             part += a.block_sum[b];
             if (last) partb += a.block_bad[b];
         }
@@ -824,10 +850,10 @@ __global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
             bad_total += s_redb[q];
         }
         if (last && threadIdx.x == 0) {
-            const int64_t E = run_off + a.block_sum[blockIdx.x];
+            const int64_t E = run_off + a.block_sum[bid];
             a.counts[0] = S;
             a.counts[1] = E;
-            a.counts[2] = bad_total + a.block_bad[blockIdx.x];
+            a.counts[2] = bad_total + a.block_bad[bid];
             a.root_start_ptr[S] = E;
             a.root_end_ptr[S] = E;
         }
@@ -915,6 +941,10 @@ __global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
         run_off += total;
     }
 }
+__global__ __launch_bounds__(BLOCK) void fill_flat_kernel(HopArgs a) {
+    __shared__ FlatLds lds;
+    fill_flat_body(a, blockIdx.x, gridDim.x, lds);
+}
 
 // Uniform picks with a lane per PICK.  As fill_flat_kernel a block takes its run in chunks of SLOTS slots and walks
 // the chunk's output edges flat; what differs is where an edge comes from.  A slot whose window holds at most k edges
@@ -954,17 +984,29 @@ __device__ __forceinline__ void huge_window_picks(const HopArgs& a, int64_t slot
     }
 }
 
+template <int SLOTS>
+struct UniformFlatLds {      // the static LDS of one block of the uniform picks (the picks themselves are dynamic LDS)
+    int64_t red[NWAVE];
+    int64_t start[SLOTS], t[SLOTS], len[SLOTS];
+    int32_t redb[NWAVE];
+    int32_t w[NWAVE];
+    int32_t off[SLOTS + 1];
+    int32_t dl[SLOTS];
+    int32_t didx[SLOTS];
+};
 template <int KP, int SLOTS, int ROUNDS>
-__global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
+__device__ __forceinline__ void fill_uniform_flat_body(const HopArgs& a, unsigned bid, unsigned nblk, UniformFlatLds<SLOTS>& lds) {
     static_assert(SLOTS % BLOCK == 0 && BLOCK % KP == 0 && KP % 4 == 0 && KP < WAVE, "chunk layout");
     constexpr int SPT = SLOTS / BLOCK;
-    __shared__ int64_t s_red[NWAVE];
-    __shared__ int32_t s_redb[NWAVE];
-    __shared__ int32_t s_w[NWAVE];
-    __shared__ int32_t s_off[SLOTS + 1];
-    __shared__ int64_t s_start[SLOTS], s_t[SLOTS], s_len[SLOTS];
-    __shared__ int32_t s_dl[SLOTS];          // chunk-local index of the q-th drawing slot
-    __shared__ int32_t s_didx[SLOTS];        // slot -> its place in s_dl, -1: copies its window, -2: window >= 2^32 edges
+    int64_t* const s_red = lds.red;
+    int32_t* const s_redb = lds.redb;
+    int32_t* const s_w = lds.w;
+    int32_t* const s_off = lds.off;
+    int64_t* const s_start = lds.start;
+    int64_t* const s_t = lds.t;
+    int64_t* const s_len = lds.len;
+    int32_t* const s_dl = lds.dl;            // chunk-local index of the q-th drawing slot
+    int32_t* const s_didx = lds.didx;        // slot -> its place in s_dl, -1: copies its window, -2: window >= 2^32 edges
     // a drawing slot's picks: rows of kp = fanout rounded up to 4 entries (16-byte rows), SLOTS rows, sized at the launch
     // (uniform_flat_lds): with rows of KP entries a block of the fanout-20 kernel held 41 KB of LDS and three blocks shared a CU
     extern __shared__ __attribute__((aligned(16))) uint32_t s_pick[];
@@ -973,7 +1015,7 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
     const int32_t kp = (k + 3) & ~3;
     const int64_t S = live_count(a.S_dev, a.S_max);
     int64_t first, run;
-    block_run(S, a.align, &first, &run);
+    block_run(S, a.align, &first, &run, bid, nblk);
     const int64_t run_end = first + run < S ? first + run : S;
     int64_t st[SPT], ln[SPT], tt[SPT];
     auto load_slots = [&](int64_t chunk0) {
@@ -992,16 +1034,16 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
     int64_t run_off = 0;
     if (a.scanned) {
         constexpr int CH = MAX_BLOCKS / SCAN_BLOCK;
-        const int c0 = (int)blockIdx.x / CH * CH;
-        run_off = a.chunk_off[blockIdx.x / CH];
+        const int c0 = (int)bid / CH * CH;
+        run_off = a.chunk_off[bid / CH];
 #pragma unroll
         for (int q = 0; q < CH - 1; ++q)
-            if (c0 + q < (int)blockIdx.x) run_off += a.block_sum[c0 + q];
+            if (c0 + q < (int)bid) run_off += a.block_sum[c0 + q];
     } else {
         int64_t part = 0;
         int32_t partb = 0;
-        const bool last = blockIdx.x == gridDim.x - 1;
-        for (int64_t b = threadIdx.x; b < (int64_t)blockIdx.x; b += BLOCK) {
+        const bool last = bid == nblk - 1;
+        for (int64_t b = threadIdx.x; b < (int64_t)bid; b += BLOCK) {
             part += a.block_sum[b];
             if (last) partb += a.block_bad[b];
         }
@@ -1021,10 +1063,10 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
             bad_total += s_redb[q];
         }
         if (last && threadIdx.x == 0) {
-            const int64_t E = run_off + a.block_sum[blockIdx.x];
+            const int64_t E = run_off + a.block_sum[bid];
             a.counts[0] = S;
             a.counts[1] = E;
-            a.counts[2] = bad_total + a.block_bad[blockIdx.x];
+            a.counts[2] = bad_total + a.block_bad[bid];
             a.root_start_ptr[S] = E;
             a.root_end_ptr[S] = E;
         }
@@ -1182,6 +1224,23 @@ __global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
         }
         run_off += total;
     }
+}
+template <int KP, int SLOTS, int ROUNDS>
+__global__ __launch_bounds__(BLOCK) void fill_uniform_flat_kernel(HopArgs a) {
+    __shared__ UniformFlatLds<SLOTS> lds;
+    fill_uniform_flat_body<KP, SLOTS, ROUNDS>(a, blockIdx.x, gridDim.x, lds);
+}
+// A most-recent and a uniform fill of the same hop over grids of the same size in one launch (see count_lane_dual_kernel):
+// even blocks copy windows for `r`, odd blocks pick for `u`.
+template <int KP, int SLOTS, int ROUNDS>
+__global__ __launch_bounds__(BLOCK) void fill_dual_kernel(HopArgs r, HopArgs u) {
+    __shared__ union {       // a block runs one of the two
+        FlatLds r;
+        UniformFlatLds<SLOTS> u;
+    } lds;
+    const unsigned bid = blockIdx.x >> 1, nblk = gridDim.x >> 1;
+    if (blockIdx.x & 1) fill_uniform_flat_body<KP, SLOTS, ROUNDS>(u, bid, nblk, lds.u);
+    else fill_flat_body(r, bid, nblk, lds.r);
 }
 
 // Lanes per slot of the uniform strategy's draws (fanout <= G: one lane per draw).  The most-recent strategy
@@ -1802,10 +1861,15 @@ struct RootSpec {  // hop-0 slot source of the k-hop driver
     int64_t *slot_node_out, *slot_ts_out;
 };
 
-int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot_ts, const RootSpec* derive,
-                int64_t S_max, const int64_t* S_dev, const sgl_sample_params* p, const sgl_hop_out* out, void* ws,
-                size_t ws_bytes, hipStream_t st, const int64_t* slot_hint = nullptr, int64_t* hint_out = nullptr,
-                bool hint_optional = false, bool do_count = true) {
+// The kernel arguments of one hop (its scratch carved out of `ws`), and the lanes per slot its two halves use.
+struct PreparedHop {
+    HopArgs a;
+    int Gc, Gf;
+};
+
+int32_t prepare_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot_ts, const RootSpec* derive,
+                    int64_t S_max, const int64_t* S_dev, const sgl_sample_params* p, const sgl_hop_out* out, void* ws,
+                    size_t ws_bytes, const int64_t* slot_hint, int64_t* hint_out, bool hint_optional, PreparedHop* ph) {
     if (!derive && S_max > 0 && (!slot_node || !slot_ts)) return fail(SGL_EINVAL, "sample: slot array is NULL");
     if (ws_bytes < hop_workspace_bytes(S_max) || !ws)
         return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, hop_workspace_bytes(S_max));
@@ -1836,8 +1900,62 @@ int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot
     a.root_start_ptr = out->root_start_ptr; a.root_end_ptr = out->root_end_ptr;
     a.nbr = out->neighbors; a.nbr_ts = out->neighbors_ts; a.nbr_eid = out->neighbors_eid;
     a.nbr_dt = out->neighbors_dt; a.counts = out->counts;
-    const int Gf = pick_group(p, S_max);
-    return launch_hop(a, st, pick_search_group(Gf, S_max), Gf, do_count, true);
+    ph->a = a;
+    ph->Gf = pick_group(p, S_max);
+    ph->Gc = pick_search_group(ph->Gf, S_max);
+    return SGL_OK;
+}
+
+int32_t run_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* slot_ts, const RootSpec* derive,
+                int64_t S_max, const int64_t* S_dev, const sgl_sample_params* p, const sgl_hop_out* out, void* ws,
+                size_t ws_bytes, hipStream_t st, const int64_t* slot_hint = nullptr, int64_t* hint_out = nullptr,
+                bool hint_optional = false, bool do_count = true) {
+    PreparedHop ph;
+    const int32_t rc = prepare_hop(g, slot_node, slot_ts, derive, S_max, S_dev, p, out, ws, ws_bytes, slot_hint, hint_out,
+                                   hint_optional, &ph);
+    if (rc != SGL_OK) return rc;
+    return launch_hop(ph.a, st, ph.Gc, ph.Gf, do_count, true);
+}
+
+// The same hop of a most-recent query `r` and a uniform query `u` whose grids are the same, in launches that run
+// the two side by side: one counting launch (or only the fill when the two share the counting pass: `u` then reads
+// r's window arrays), one scan launch of two blocks, one fill launch.  false: the pair does not fit (the caller
+// launches the hops one after the other).
+bool dual_hop_fits(const PreparedHop& r, const PreparedHop& u) {
+    if (r.a.type != SGL_SAMPLE_RECENT || u.a.type != SGL_SAMPLE_UNIFORM) return false;
+    if (r.a.S_max != u.a.S_max || r.Gc != 1 || u.Gc != 1 || (u.Gf != 16 && u.Gf != 32)) return false;
+    const HopGrid gr = hop_grid(r.a.S_max, r.Gc, r.Gf), gu = hop_grid(u.a.S_max, u.Gc, u.Gf);
+    if (gr.align != gu.align || gr.blocks != gu.blocks) return false;
+    const int64_t run = ceil_div<int64_t>(ceil_div<int64_t>(r.a.S_max > 0 ? r.a.S_max : 1, gr.blocks), gr.align) * gr.align;
+    const int32_t kmax = r.a.k > u.a.k ? r.a.k : u.a.k;
+    return !(kmax > 0 && run > (int64_t)INT32_MAX / kmax);
+}
+
+int32_t launch_dual_hop(PreparedHop r, PreparedHop u, hipStream_t st, bool shared_count) {
+    const HopGrid hg = hop_grid(r.a.S_max, r.Gc, r.Gf);
+    r.a.align = u.a.align = hg.align;
+    const unsigned blocks = (unsigned)hg.blocks;
+    r.a.scanned = u.a.scanned = hg.blocks > FUSED_PREFIX_MAX ? 1 : 0;
+    if (shared_count) {
+        hipLaunchKernelGGL(count_lane_kernel, dim3(blocks), dim3(BLOCK), 0, st, r.a);
+        SGL_LAUNCH_CHECK();
+        if (r.a.scanned) {
+            hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, r.a, (int)blocks);
+            SGL_LAUNCH_CHECK();
+        }
+    } else {
+        hipLaunchKernelGGL(count_lane_dual_kernel, dim3(2 * blocks), dim3(BLOCK), 0, st, r.a, u.a);
+        SGL_LAUNCH_CHECK();
+        if (r.a.scanned) {
+            hipLaunchKernelGGL(scan_dual_kernel, dim3(2), dim3(SCAN_BLOCK), 0, st, r.a, u.a, (int)blocks);
+            SGL_LAUNCH_CHECK();
+        }
+    }
+    const size_t lds = uniform_flat_lds(u.a.k);
+    if (u.Gf == 16) hipLaunchKernelGGL((fill_dual_kernel<16, UFLAT_SLOTS, 2>), dim3(2 * blocks), dim3(BLOCK), lds, st, r.a, u.a);
+    else hipLaunchKernelGGL((fill_dual_kernel<32, UFLAT_SLOTS, 4>), dim3(2 * blocks), dim3(BLOCK), lds, st, r.a, u.a);
+    SGL_LAUNCH_CHECK();
+    return SGL_OK;
 }
 
 
@@ -2189,6 +2307,8 @@ extern "C" int32_t sgl_sample_khop_batched(const sgl_tcsr* g, int32_t B, const i
     }
     const int Gf0 = pick_group(&p[0], S_max);
     const HopGrid grid0 = hop_grid(S_max, pick_search_group(Gf0, S_max), Gf0);
+    PreparedHop ph[SEG_MAX_CHAINS];
+    bool shares[SEG_MAX_CHAINS];
     for (int32_t l = 0; l < layers; ++l) {
         for (int32_t q = 0; q < Q; ++q) {
             const sgl_sample_params* pq = &p[q];
@@ -2217,10 +2337,20 @@ extern "C" int32_t sgl_sample_khop_batched(const sgl_tcsr* g, int32_t B, const i
                         (pq->equal_root_time != 0) == (p[0].equal_root_time != 0) && gq.align == grid0.align &&
                         gq.blocks == grid0.blocks;      // (a hop's scratch is carved by its own slot count: same places)
             }
-            rc = run_hop(g, sn[q], stt[q], nullptr, s_max, S_dev[q], &pl, &oq[l], share ? static_cast<char*>(ws) : wq,
-                         carry ? hop_ws : per, st, hint_in, (carry && l + 1 < layers) ? carry_buf[l & 1] : nullptr, l == 0, !share);
+            shares[q] = share;
+            rc = prepare_hop(g, sn[q], stt[q], nullptr, s_max, S_dev[q], &pl, &oq[l], share ? static_cast<char*>(ws) : wq,
+                             carry ? hop_ws : per, hint_in, (carry && l + 1 < layers) ? carry_buf[l & 1] : nullptr, l == 0, &ph[q]);
             if (rc != SGL_OK) return rc;
-            if (share && grid0.blocks > FUSED_PREFIX_MAX) {   // the scan launch of query 0 published that query's counts only
+        }
+        // a most-recent query followed by a uniform one over grids of the same size: their kernels of this hop side by side
+        const bool dual = Q == 2 && dual_hop_fits(ph[0], ph[1]);
+        if (dual) {
+            if ((rc = launch_dual_hop(ph[0], ph[1], st, shares[1])) != SGL_OK) return rc;
+        }
+        for (int32_t q = 0; q < Q; ++q) {
+            const sgl_hop_out* oq = outs + (size_t)q * layers;
+            if (!dual && (rc = launch_hop(ph[q].a, st, ph[q].Gc, ph[q].Gf, !shares[q], true)) != SGL_OK) return rc;
+            if (shares[q] && grid0.blocks > FUSED_PREFIX_MAX) {   // the scan launch of query 0 published that query's counts only
                 hipLaunchKernelGGL(share_counts_kernel, dim3(1), dim3(1), 0, st, outs[0].counts, oq[0].counts,
                                    oq[0].root_start_ptr, oq[0].root_end_ptr, oq[0].capacity_slots);
                 SGL_LAUNCH_CHECK();
