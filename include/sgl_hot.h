@@ -448,6 +448,9 @@ int32_t sgl_unique_compact_hashed(void* state, int64_t capacity, int32_t reset,
  * starts a new epoch, Remapper with op 'r', sample.cu.hpp:1825-1852; np.unique
  * per batch in prepare_sample.py:205-213).  The state spans B copies of the
  * universe [0, universe) (B <= SGL_BATCH_MAX); every call starts a new epoch.
+ * The caller allocates sgl_remap_batched_state_bytes(universe, B) device bytes,
+ * 16-byte aligned (about 1.25 bytes per id of B x universe up to 2^26 ids in
+ * all, 0.4 beyond), and calls sgl_remap_batched_init once.
  *   ids[g] / local_out[g]  G arrays of len_max[g] entries holding all batches;
  *   seg[g]     device int64[B+1]: elements [seg[g][b], seg[g][b+1]) of array g
  *              belong to batch b (seg[g][B] = live length <= len_max[g]) -
