@@ -80,6 +80,38 @@ def test_batched_sampler_window_flags(oracle, hot, small, kw, layers):
     run_both(oracle, hot, g, dg, node, t, ptr, layers, kws, hint=hint)
 
 
+@pytest.mark.parametrize("case", range(6))
+def test_batched_pair_side_by_side_sweep(oracle, hot, small, case):
+    """Calls of 131072 slots and more take the lane-per-slot kernels, and a most-recent query followed by a uniform
+    one with the same fanout runs its kernels of a hop side by side in one launch: random batch sizes (empty ones
+    among them), hops, fanouts (16-lane and 32-lane groups), window rules, hints and index on or off."""
+    (src, dst, ts), g, _ = small
+    rng = np.random.default_rng(900 + case)
+    dg = mirror_graph(hot, g)
+    with_index = bool(case & 1)
+    if with_index:
+        hot.build_hop_hint(dg)
+    if case & 2:
+        hot.build_records(dg)
+    B = int(rng.integers(1, 12))
+    sizes = rng.multinomial(140_000 + int(rng.integers(0, 20_000)), rng.dirichlet(np.ones(B))).astype(np.int64)
+    if B > 2:
+        sizes[int(rng.integers(0, B))] = 0
+    node = rng.integers(0, g.n, int(sizes.sum())).astype(np.int64)
+    t = rng.integers(0, int(ts.max()) + 2, node.size).astype(np.int64)
+    ptr = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+    hint = oracle.window_end(g, node, t)
+    hint[rng.random(hint.size) < 0.5] = -1
+    layers = [2, 1, 3, 2, 2, 2][case]
+    fan = [5, 10, 3, 20, 7, 16][case]
+    extra = [dict(), dict(allowed_offset=40_000), dict(), dict(), dict(keep_root_time=True), dict(replace=True)][case]
+    kws = [dict(sample_type="recent", fanout=fan, **{k: v for k, v in extra.items() if k == "allowed_offset"}),
+           dict(sample_type="uniform", fanout=fan, seed=11 + case, **extra)]
+    if case == 4:           # a pair whose fanouts differ runs its hops one after the other
+        kws[0]["fanout"] = 4
+    run_both(oracle, hot, g, dg, node, t, ptr, layers, kws, hint=hint if with_index else None)
+
+
 def test_batched_sampler_refuses_marking_and_bad_sizes(hot, small):
     _, g, dg = small
     node, t = to_dev(hot, np.arange(10)), to_dev(hot, np.arange(10))
