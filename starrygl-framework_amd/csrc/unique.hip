@@ -649,9 +649,24 @@ __device__ __forceinline__ uint64_t pack_flag_bytes(uint64_t w) {
 
 // Thread w owns ids [64 w, 64 w + 64): it turns their flags into the group's 64 pending bits (left in rank[w].mask),
 // clears the flags for the next call and counts; a block's count is its tile's sum.
-__global__ __launch_bounds__(BLOCK) void reduce_batched_kernel(BState s, int64_t* tile_sum) {
+// A batch none of whose arrays holds an element in this call (a group of batches with fewer live ones than the state
+// has room for): its flags are all clear and nobody will look its ids up, so reduce and assign leave its tiles alone
+// (both ask the same question, so a tile's pending bits are read by assign only when reduce wrote them in this call).
+__device__ __forceinline__ bool batch_live(const Batched& bt, int G, int64_t b) {
+    bool live = false;
+#pragma unroll
+    for (int g = 0; g < MAXG; ++g)
+        if (g < G && bt.seg[g][b + 1] > bt.seg[g][b]) live = true;
+    return live;
+}
+
+__global__ __launch_bounds__(BLOCK) void reduce_batched_kernel(BState s, int64_t* tile_sum, Batched bt, int G) {
     __shared__ int32_t s_w[BLOCK / WAVE];
     const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
+    if (!batch_live(bt, G, (int64_t)blockIdx.x / (bt.stride / BATCH_STRIDE_ALIGN))) {      // block-uniform
+        if (threadIdx.x == 0) tile_sum[blockIdx.x] = 0;
+        return;
+    }
     uint64_t mask = 0;
     if (w < s.groups) {
         if (s.bytes) {
@@ -687,12 +702,13 @@ __global__ __launch_bounds__(BLOCK) void reduce_batched_kernel(BState s, int64_t
 // Numbers the pending ids (tile_sum holds the exclusive tile offsets, the total at [nt]): an id's local id is its
 // rank inside its batch, i.e. the global rank minus the offset of the batch's first tile; the first tile of
 // every batch records where the batch's list begins.
-__global__ __launch_bounds__(BLOCK) void assign_batched_kernel(BState s, const int64_t* tile_sum, int64_t nt, Batched bt,
+__global__ __launch_bounds__(BLOCK) void assign_batched_kernel(BState s, const int64_t* tile_sum, int64_t nt, Batched bt, int G,
                                                                int64_t* unique_out, int64_t unique_capacity, int64_t* U_off) {
     __shared__ int32_t s_wave[BLOCK / WAVE];
     const int lane = threadIdx.x % WAVE, wid = threadIdx.x / WAVE;
     const int64_t w = (int64_t)blockIdx.x * TILE + threadIdx.x;
-    uint64_t word = (w < s.groups) ? s.rank[w].mask : 0ull;
+    const bool live = batch_live(bt, G, (int64_t)blockIdx.x / (bt.stride / BATCH_STRIDE_ALIGN));       // block-uniform
+    uint64_t word = (live && w < s.groups) ? s.rank[w].mask : 0ull;
     const int32_t c = __popcll(word);
     int32_t inc = c;
     for (int d = 1; d < WAVE; d <<= 1) {
@@ -711,7 +727,7 @@ __global__ __launch_bounds__(BLOCK) void assign_batched_kernel(BState s, const i
         if ((int64_t)blockIdx.x == b * tiles_per_batch) U_off[b] = tile_off;
         if (blockIdx.x == nt - 1) U_off[bt.B] = tile_sum[nt];
     }
-    if (w >= s.groups) return;
+    if (!live || w >= s.groups) return;
     int64_t rank = tile_off + wave_off + (inc - c);
     s.rank[w].rank = rank - batch_off;
     const int64_t id0 = w * 64 - b * bt.stride;
@@ -974,11 +990,11 @@ extern "C" int32_t sgl_unique_compact_batched(void* state, int64_t universe, int
         hipLaunchKernelGGL(walk_batched_kernel<false>, dim3((unsigned)mb), dim3(BLOCK), 0, st, s, all, bt);
         SGL_LAUNCH_CHECK();
     }
-    hipLaunchKernelGGL(reduce_batched_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum);
+    hipLaunchKernelGGL(reduce_batched_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, bt, G);
     SGL_LAUNCH_CHECK();
     hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(SCAN_BLOCK), 0, st, tile_sum, nt);
     SGL_LAUNCH_CHECK();
-    hipLaunchKernelGGL(assign_batched_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, bt, unique_out,
+    hipLaunchKernelGGL(assign_batched_kernel, dim3((unsigned)nt), dim3(BLOCK), 0, st, s, tile_sum, nt, bt, G, unique_out,
                        unique_capacity, U_off);
     SGL_LAUNCH_CHECK();
     if (longest > 0) {
