@@ -25,7 +25,8 @@ class EventBatchLoader:
         pipelines that share one take turns).  sample_ahead: mini-batches per pass of the library calls; above 1
         the loader runs groups of that many consecutive batches through MiniBatchGroupPipeline objects (the
         batched sampler and unique: a batch of a group costs a fraction of a batch sampled alone), `prefetch`
-        then counts groups in flight (two are enough), and a yielded batch stays valid until all batches of its
+        then counts groups in flight (three keep the GPU busy while the host reads a finished group's counts; with two
+        the passes wait for the host), and a yielded batch stays valid until all batches of its
         group and of the `prefetch - 2` following groups have been yielded.  Remaining keywords go to the pipelines.
         Only full batches are produced (every buffer of a pipeline is planned for one batch shape)."""
         if not drop_last:
