@@ -878,6 +878,12 @@ def main():
             P.graph = torch.cuda.CUDAGraph()
             with graph_capture(P.graph, stream=stream):
                 step()
+            # (the runtime uploads a graph at its first launch: part of building the pipeline, as for the per-batch
+            # pipelines, whose graphs the warm-up steps launch)
+            P.graph.replay()
+            stream.synchronize()
+            P.acc.zero_()
+            stream.synchronize()
         # a last, shorter group: the trailing batches are empty (batch_ptr is read on the device)
         P.ptr_tail = {live: D(np.minimum(np.arange(B + 1), live).astype(np.int64) * S0) for live in {args.steps % B} - {0}}
 

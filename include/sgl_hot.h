@@ -85,7 +85,10 @@ typedef struct sgl_tcsr {
     const int64_t* hop_hint;/* [m]   device, or NULL            */
     /* Optional (NULL = absent) interleaved copy of the edge arrays, filled by
      * sgl_tcsr_records_build: rec[4*e .. 4*e+3] = {col[e], ts[e], eid[e],
-     * hop_hint[e] (-1 without the index)}, 32 bytes per edge.  The uniform
+     * x}, 32 bytes per edge; x = -1 without the index, else hop_hint[e] in bits
+     * 0..39 and, in bits 40..62, the length of the window that entry ends
+     * (hop_hint[e] - row_ptr[col[e]]) plus one, saturating at 2^23 - 1 (0 = not
+     * recorded): a slot of the next hop then knows its whole window.  The uniform
      * strategy picks edges scattered over a window: from the separate arrays
      * every pick costs one memory sector per array, from the records one per
      * pick.  Searches always run on `ts`; results do not depend on it. */

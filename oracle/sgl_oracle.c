@@ -181,14 +181,25 @@ int32_t sglo_tcsr_hop_hint_build(const sgl_tcsr* g, int64_t* hop_hint, void* str
 }
 
 /* The interleaved records are an accelerator of the kernels as well: the oracle samples from the
- * separate arrays and only restates the layout so that the built array can be checked. */
+ * separate arrays and only restates the layout so that the built array can be checked.  Fourth field: the
+ * edge's next-hop index entry p (bits 0..39) with the length of the window it ends, p - row_ptr[col[e]], as
+ * length + 1 in bits 40..62 (saturating at 2^23 - 1; 0 = not recorded: graphs beyond 2^40 edges, destinations
+ * outside [0, n)); -1 without the index. */
 int32_t sglo_tcsr_records_build(const sgl_tcsr* g, int64_t* rec, void* stream) {
     (void)stream;
     if (!g || g->n < 0 || g->m < 0) return fail(SGL_EINVAL, "tcsr_records_build: null");
-    if (g->m > 0 && (!g->col || !g->ts || !g->eid || !rec)) return fail(SGL_EINVAL, "tcsr_records_build: null array");
+    if (g->m > 0 && (!g->col || !g->ts || !g->eid || !rec || (g->hop_hint && !g->row_ptr)))
+        return fail(SGL_EINVAL, "tcsr_records_build: null array");
+    const int64_t pos_mask = (1ll << 40) - 1, sat = (1ll << 23) - 1;
     for (int64_t e = 0; e < g->m; ++e) {
         rec[4 * e] = g->col[e]; rec[4 * e + 1] = g->ts[e]; rec[4 * e + 2] = g->eid[e];
-        rec[4 * e + 3] = g->hop_hint ? g->hop_hint[e] : -1;
+        int64_t h = g->hop_hint ? g->hop_hint[e] : -1;
+        const int64_t v = g->col[e];
+        if (h >= 0 && g->m <= pos_mask && v >= 0 && v < g->n) {
+            const int64_t len = h - g->row_ptr[v];
+            if (len >= 0) h |= (len + 1 < sat ? len + 1 : sat) << 40;
+        }
+        rec[4 * e + 3] = h;
     }
     return SGL_OK;
 }

@@ -60,6 +60,27 @@ struct Arena {
 constexpr int32_t WAIT_LIMIT_DEFAULT = 1 << 20;
 int32_t wait_limit();
 
+// The fourth field of an interleaved edge record (sgl_tcsr_records_build) is the edge's next-hop index entry - the
+// position where the window of the slot (col[e], ts[e]) ends - with the LENGTH of that window in its upper bits:
+// bits 0..39 the position (graphs of up to 2^40 edges), bits 40..62 a field f: 0 = not recorded, 1..HINT_LEN_SAT-1 =
+// length + 1, HINT_LEN_SAT = longer than the field holds.  A slot of a deeper hop whose index entry came out of a
+// record then knows its whole window [position - length, position) without reading the row pointers of its node.
+// A plain index entry (from the hop_hint array, a caller's root hint) has f = 0; -1 stays -1.
+constexpr int HINT_POS_BITS = 40;
+constexpr int64_t HINT_POS_MASK = (1ll << HINT_POS_BITS) - 1;
+constexpr int64_t HINT_LEN_SAT = (1ll << 23) - 1;
+__host__ __device__ __forceinline__ int64_t hint_pos(int64_t h) { return h < 0 ? h : (h & HINT_POS_MASK); }
+// window length recorded in an entry, or -1
+__host__ __device__ __forceinline__ int64_t hint_len(int64_t h) {
+    if (h < 0) return -1;
+    const int64_t f = h >> HINT_POS_BITS;
+    return (f == 0 || f >= HINT_LEN_SAT) ? -1 : f - 1;
+}
+__host__ __device__ __forceinline__ int64_t hint_pack(int64_t pos, int64_t len) {
+    const int64_t f = len + 1 < HINT_LEN_SAT ? len + 1 : HINT_LEN_SAT;
+    return pos | (f << HINT_POS_BITS);
+}
+
 constexpr size_t REMAP_HEADER_BYTES = 256;
 constexpr int64_t REMAP_BYTE_FLAGS_MAX = 1ll << 24;
 inline bool remap_byte_flags(int64_t universe) { return universe <= REMAP_BYTE_FLAGS_MAX; }

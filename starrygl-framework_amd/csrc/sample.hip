@@ -43,7 +43,7 @@ constexpr int SCAN_BLOCK = 1024;
 
 struct HopArgs {
     // graph
-    int64_t n;
+    int64_t n, m;
     const int64_t* row_ptr;
     const int64_t* col;
     const int64_t* ts;
@@ -216,6 +216,7 @@ __device__ __forceinline__ int64_t root_hint_of(const HopArgs& a, int64_t s) {
 
 // A caller's window end, kept inside the row [rs, re]
 __device__ __forceinline__ int64_t clamp_to_row(int64_t h, int64_t rs, int64_t re) {
+    h = hint_pos(h);        // (an entry that came out of an edge record carries the window's length above the position)
     return h < rs ? rs : (h > re ? re : h);
 }
 
@@ -343,7 +344,20 @@ __device__ __forceinline__ void count_lane_body(const HopArgs& a, unsigned bid, 
     const int64_t end = first + run < S ? first + run : S;
     const int64_t eq = a.equal_root_time ? 1 : 0;
     int32_t sum = 0, nbad = 0;
+    // slots of a deeper hop whose index entries carry their windows' lengths (entries out of edge records): the
+    // window is [position - length, position), no row pointer and no slot is read
+    const bool whole = a.slot_hint != nullptr && !a.hint_optional && !a.derive && a.allowed_offset < 0;   // kernel arguments
     for (int64_t slot = first + threadIdx.x; slot < end; slot += BLOCK) {
+        if (whole) {
+            const int64_t h = a.slot_hint[slot];
+            const int64_t len = hint_len(h), pos = hint_pos(h);
+            if (len >= 0 && len <= pos && pos <= a.m) {
+                a.w_start[slot] = pos - len;
+                a.w_len[slot] = len;
+                sum += (int32_t)(len < a.k ? len : a.k);
+                continue;
+            }
+        }
         int64_t v, t;
         load_slot(a, slot, &v, &t);
         const int64_t rh = a.slot_hint != nullptr ? a.slot_hint[slot] : root_hint_of(a, slot);
@@ -1875,7 +1889,7 @@ int32_t prepare_hop(const sgl_tcsr* g, const int64_t* slot_node, const int64_t* 
         return fail(SGL_ENOMEM, "sample: workspace %zu < %zu bytes", ws_bytes, hop_workspace_bytes(S_max));
     Arena ar(ws, ws_bytes);
     HopArgs a{};
-    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint; a.rec = g->rec;
+    a.n = g->n; a.m = g->m; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint; a.rec = g->rec;
     a.slot_node = slot_node; a.slot_ts = slot_ts; a.S_max = S_max; a.S_dev = S_dev;
     a.slot_hint = slot_hint; a.hint_out = hint_out; a.hint_optional = hint_optional ? 1 : 0;
     a.root_hint = (derive && !p->equal_root_time) ? p->root_hint : nullptr;
@@ -1963,7 +1977,7 @@ Fused2Args fused2_args(const sgl_tcsr* g, const RootSpec* spec, int64_t S0, cons
                        const sgl_hop_out* outs, unsigned long long* desc) {
     Fused2Args f{};
     HopArgs& a = f.h;
-    a.n = g->n; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint; a.rec = g->rec;
+    a.n = g->n; a.m = g->m; a.row_ptr = g->row_ptr; a.col = g->col; a.ts = g->ts; a.eid = g->eid; a.hint = g->hop_hint; a.rec = g->rec;
     a.S_max = S0; a.derive = 1;
     a.root_hint = p->equal_root_time ? nullptr : p->root_hint;
     a.R = spec->R; a.S_pos = spec->S_pos; a.roots = spec->roots; a.ts_ptr = spec->ts_ptr;

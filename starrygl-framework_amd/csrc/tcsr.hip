@@ -351,7 +351,13 @@ __global__ __launch_bounds__(BLOCK) void records_kernel(sgl_tcsr g, int64_t* __r
         a.x = g.col[e];
         a.y = g.ts[e];
         b.x = g.eid[e];
-        b.y = g.hop_hint != nullptr ? g.hop_hint[e] : -1;
+        int64_t h = g.hop_hint != nullptr ? g.hop_hint[e] : -1;
+        // with the window's length (hint_pack): the entry lies in row col[e], whose start the row pointers give
+        if (h >= 0 && g.m <= HINT_POS_MASK && a.x >= 0 && a.x < g.n) {
+            const int64_t len = h - g.row_ptr[a.x];
+            if (len >= 0) h = hint_pack(h, len);
+        }
+        b.y = h;
         reinterpret_cast<longlong2*>(rec)[2 * e] = a;
         reinterpret_cast<longlong2*>(rec)[2 * e + 1] = b;
     }
@@ -362,7 +368,7 @@ __global__ __launch_bounds__(BLOCK) void records_kernel(sgl_tcsr g, int64_t* __r
 extern "C" int32_t sgl_tcsr_records_build(const sgl_tcsr* g, int64_t* rec, void* stream) {
     if (!g || g->n < 0 || g->m < 0) return fail(SGL_EINVAL, "tcsr_records_build: NULL graph");
     if (g->m == 0) return SGL_OK;
-    if (!g->col || !g->ts || !g->eid || !rec) return fail(SGL_EINVAL, "tcsr_records_build: NULL array");
+    if (!g->col || !g->ts || !g->eid || !rec || (g->hop_hint && !g->row_ptr)) return fail(SGL_EINVAL, "tcsr_records_build: NULL array");
     if (reinterpret_cast<uintptr_t>(rec) % 32 != 0) return fail(SGL_EINVAL, "tcsr_records_build: rec must be 32-byte aligned");
     int64_t blocks = ceil_div<int64_t>(g->m, BLOCK);
     if (blocks > (1 << 20)) blocks = 1 << 20;

@@ -419,7 +419,11 @@ def test_interleaved_records_give_the_same_samples(oracle, hot, index, layers, f
     hot.build_records(dg)
     rec = np_of(dg.rec).reshape(-1, 4)
     assert np.array_equal(rec[:, 0], g.col) and np.array_equal(rec[:, 1], g.ts) and np.array_equal(rec[:, 2], g.eid)
-    assert np.array_equal(rec[:, 3], np_of(dg.hop_hint) if index else np.full(g.m, -1))
+    if index:       # the index entry with the length of the window it ends (+ 1) above bit 40
+        hh = np_of(dg.hop_hint)
+        assert np.array_equal(rec[:, 3], hh | ((hh - g.row_ptr[g.col] + 1) << 40))
+    else:
+        assert np.array_equal(rec[:, 3], np.full(g.m, -1))
     rng = np.random.default_rng(5)
     roots = rng.integers(0, g.n, n_roots).astype(np.int64)
     root_ts = rng.integers(0, 400_000, n_roots).astype(np.int64)

@@ -398,8 +398,9 @@ def test_edge_records_are_the_four_arrays_side_by_side(oracle):
     g = host_graph(oracle, n, rng.integers(0, n, m), rng.integers(0, n, m), rng.integers(0, 100, m))
     oracle.build_records(g)
     assert np.array_equal(g.rec.reshape(-1, 4), np.stack([g.col, g.ts, g.eid, np.full(m, -1)], axis=1))
-    oracle.build_hop_hint(g)          # the records follow the index
-    assert np.array_equal(g.rec.reshape(-1, 4), np.stack([g.col, g.ts, g.eid, g.hop_hint], axis=1))
+    oracle.build_hop_hint(g)          # the records follow the index: entry in bits 0..39, length of the window it ends (+ 1) above
+    packed = g.hop_hint | ((g.hop_hint - g.row_ptr[g.col] + 1) << 40)
+    assert np.array_equal(g.rec.reshape(-1, 4), np.stack([g.col, g.ts, g.eid, packed], axis=1))
 
 
 def test_sample_window_is_brute_force(oracle):
