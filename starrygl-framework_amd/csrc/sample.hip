@@ -1550,6 +1550,12 @@ __device__ __forceinline__ void fused2_count(const Fused2Args& f, const int64_t 
             const Edge ed = load_picked_edge(a, pos);
             nbr = ed.col; ets = ed.ts; id = ed.eid;
             if (a.hint != nullptr) hint = ed.hint;
+        } else if (a.rec != nullptr) {
+            // the lane's one hop-1 edge out of the graph's records: one 32-byte access instead of a sector per array,
+            // and an index entry that carries the length of the hop-2 window
+            const Edge ed = load_picked_edge(a, pos);
+            nbr = ed.col; ets = ed.ts; id = ed.eid;
+            if (a.hint != nullptr) hint = ed.hint;
         } else {
             nbr = a.col[pos];
             ets = a.ts[pos];
@@ -1567,10 +1573,18 @@ __device__ __forceinline__ void fused2_count(const Fused2Args& f, const int64_t 
             // no search (strictly-before windows only; a uniform call that keeps the root's time asks
             // about another time and searches)
             const bool hinted = hint >= 0 && eq == 0 && t2 == ets;
-            const int64_t rs2 = a.row_ptr[nbr], re2 = a.row_ptr[nbr + 1];
-            const int64_t hi2 = hinted ? clamp_to_row(hint, rs2, re2) : lane_lower_bound(a.ts, rs2, re2, t2 + eq);
-            int64_t lo2 = rs2;
-            if (a.allowed_offset >= 0) lo2 = lane_lower_bound(a.ts, rs2, hi2, t2 - a.allowed_offset);
+            const int64_t hl = hinted ? hint_len(hint) : -1, hp = hint_pos(hint);
+            int64_t lo2, hi2;
+            if (hl >= 0 && hl <= hp && hp <= a.m && a.allowed_offset < 0) {
+                // the entry came out of an edge record and carries the window's length: no row pointer is read
+                hi2 = hp;
+                lo2 = hp - hl;
+            } else {
+                const int64_t rs2 = a.row_ptr[nbr], re2 = a.row_ptr[nbr + 1];
+                hi2 = hinted ? clamp_to_row(hint, rs2, re2) : lane_lower_bound(a.ts, rs2, re2, t2 + eq);
+                lo2 = rs2;
+                if (a.allowed_offset >= 0) lo2 = lane_lower_bound(a.ts, rs2, hi2, t2 - a.allowed_offset);
+            }
             len2 = hi2 - lo2;
             c2 = (int32_t)(len2 < k ? len2 : k);
             start2 = UNIFORM ? lo2 : hi2 - c2;
