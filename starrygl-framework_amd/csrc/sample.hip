@@ -1652,10 +1652,12 @@ __device__ __forceinline__ void fused2_write(const Fused2Args& f, const int64_t 
                 const int64_t st2 = shfl_i64(start2, gbase + j);
                 const int32_t cc = __shfl(c2, gbase + j);
                 if (j < c && lig < cc) {
-                    const int64_t e = st2 + lig;
-                    pre_ts[j] = a.ts[e];
-                    pre_col[j] = a.col[e];
-                    pre_eid[j] = a.eid[e];
+                    // (from the records when the graph has them: a hop-2 slot holds an edge or two, one memory sector
+                    // of records against one per array)
+                    const Edge ed = load_picked_edge(a, st2 + lig);
+                    pre_ts[j] = ed.ts;
+                    pre_col[j] = ed.col;
+                    pre_eid[j] = ed.eid;
                 }
             }
         }
@@ -1830,10 +1832,10 @@ __device__ __forceinline__ void fused2_write(const Fused2Args& f, const int64_t 
                     dst2[r] = ed.col;
                     id2[r] = ed.eid;
                 } else {
-                    const int64_t e = st2 + lig;
-                    ets2[r] = a.ts[e];
-                    dst2[r] = a.col[e];
-                    id2[r] = a.eid[e];
+                    const Edge ed = load_picked_edge(a, st2 + lig);
+                    ets2[r] = ed.ts;
+                    dst2[r] = ed.col;
+                    id2[r] = ed.eid;
                 }
             }
         }
