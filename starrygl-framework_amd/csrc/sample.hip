@@ -934,7 +934,8 @@ __device__ __forceinline__ void fill_flat_body(const HopArgs& a, unsigned bid, u
                         ets[r] = a.ts[e];
                         dst[r] = a.col[e];
                         id[r] = a.eid[e];
-                        if (a.hint_out != nullptr) hnt[r] = a.hint[e];
+                        // (the entry out of the records when the graph has them: it carries the next window's length)
+                        if (a.hint_out != nullptr) hnt[r] = a.rec != nullptr ? a.rec[4 * e + 3] : a.hint[e];
                     }
                 }
             }
