@@ -71,6 +71,8 @@ struct HopArgs {
     const int64_t* neg_ts;
     int64_t R, S_pos;
     int32_t derive;      // 1: slots come from roots/negatives
+    int32_t lean;        // 1: slots whose index entry carries the window's length keep their window in that entry only
+                         //    (count_lane_kernel does not write w_start / w_len for them, the flat fill kernels read the entry)
     int32_t scanned;     // 1: scan_kernel wrote chunk_off and published the counts
     int32_t align;       // a block's run of slots is a multiple of this (both kernels of a hop agree on it)
     int64_t* slot_node_out;
@@ -220,6 +222,26 @@ __device__ __forceinline__ int64_t clamp_to_row(int64_t h, int64_t rs, int64_t r
     return h < rs ? rs : (h > re ? re : h);
 }
 
+// Slots of a deeper hop whose index entries may carry their windows' lengths (entries out of edge records): for such
+// an entry the window is [position - length, position) and neither the slot nor a row pointer is read.
+__device__ __forceinline__ bool whole_window_hop(const HopArgs& a) {      // kernel arguments: uniform across the launch
+    return a.slot_hint != nullptr && !a.hint_optional && !a.derive && a.allowed_offset < 0 && !a.equal_root_time;
+}
+__device__ __forceinline__ bool whole_window(const HopArgs& a, int64_t h, int64_t* start, int64_t* len) {
+    const int64_t l = hint_len(h), pos = hint_pos(h);
+    if (l < 0 || l > pos || pos > a.m) return false;
+    *start = pos - l;
+    *len = l;
+    return true;
+}
+// (start, length) of slot's window for the fill kernels: out of the slot's entry in a lean hop, else what the counting
+// kernel stored
+__device__ __forceinline__ void slot_window(const HopArgs& a, int64_t slot, int64_t* start, int64_t* len) {
+    if (a.lean && whole_window_hop(a) && whole_window(a, a.slot_hint[slot], start, len)) return;
+    *start = a.w_start[slot];
+    *len = a.w_len[slot];
+}
+
 template <int G>
 __global__ __launch_bounds__(BLOCK) void count_kernel(HopArgs a) {
     constexpr int SPB = BLOCK / G;  // slots per block iteration
@@ -346,14 +368,15 @@ __device__ __forceinline__ void count_lane_body(const HopArgs& a, unsigned bid, 
     int32_t sum = 0, nbad = 0;
     // slots of a deeper hop whose index entries carry their windows' lengths (entries out of edge records): the
     // window is [position - length, position), no row pointer and no slot is read
-    const bool whole = a.slot_hint != nullptr && !a.hint_optional && !a.derive && a.allowed_offset < 0;   // kernel arguments
+    const bool whole = whole_window_hop(a);
     for (int64_t slot = first + threadIdx.x; slot < end; slot += BLOCK) {
         if (whole) {
-            const int64_t h = a.slot_hint[slot];
-            const int64_t len = hint_len(h), pos = hint_pos(h);
-            if (len >= 0 && len <= pos && pos <= a.m) {
-                a.w_start[slot] = pos - len;
-                a.w_len[slot] = len;
+            int64_t st, len;
+            if (whole_window(a, a.slot_hint[slot], &st, &len)) {
+                if (!a.lean) {
+                    a.w_start[slot] = st;
+                    a.w_len[slot] = len;
+                }
                 sum += (int32_t)(len < a.k ? len : a.k);
                 continue;
             }
@@ -825,8 +848,8 @@ __device__ __forceinline__ void fill_flat_body(const HopArgs& a, unsigned bid, u
             const int64_t slot = chunk0 + SPT * threadIdx.x + q;
             st[q] = ln[q] = tt[q] = 0;
             if (slot < run_end) {
-                ln[q] = a.w_len[slot];
-                st[q] = a.w_start[slot] + (ln[q] > k ? ln[q] - k : 0);       // the last min(len, k) edges of the window
+                slot_window(a, slot, &st[q], &ln[q]);
+                st[q] += ln[q] > k ? ln[q] - k : 0;       // the last min(len, k) edges of the window
                 tt[q] = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
             }
         }
@@ -1039,8 +1062,7 @@ __device__ __forceinline__ void fill_uniform_flat_body(const HopArgs& a, unsigne
             const int64_t slot = chunk0 + SPT * threadIdx.x + q;
             st[q] = ln[q] = tt[q] = 0;
             if (slot < run_end) {
-                st[q] = a.w_start[slot];
-                ln[q] = a.w_len[slot];
+                slot_window(a, slot, &st[q], &ln[q]);
                 tt[q] = a.derive ? a.slot_ts_out[slot] : a.slot_ts[slot];
             }
         }
@@ -1383,6 +1405,7 @@ int32_t launch_hop(HopArgs a, hipStream_t st, int Gc, int Gf, bool do_count = tr
     if (a.k > 0 && run > (int64_t)INT32_MAX / a.k)
         return fail(SGL_ENOTSUP, "sample: %lld slots x fanout %d exceed what a block counts in 32 bits", (long long)a.S_max, a.k);
     a.scanned = blocks > FUSED_PREFIX_MAX ? 1 : 0;
+    a.lean = (a.type == SGL_SAMPLE_UNIFORM && Gf > 32) ? 0 : 1;      // the flat fill kernels read a window through slot_window
     if (do_count) {
         hipLaunchKernelGGL(count_fn(Gc), dim3((unsigned)blocks), dim3(BLOCK), 0, st, a);
         SGL_LAUNCH_CHECK();
@@ -1967,6 +1990,7 @@ int32_t launch_dual_hop(PreparedHop r, PreparedHop u, hipStream_t st, bool share
     r.a.align = u.a.align = hg.align;
     const unsigned blocks = (unsigned)hg.blocks;
     r.a.scanned = u.a.scanned = hg.blocks > FUSED_PREFIX_MAX ? 1 : 0;
+    r.a.lean = u.a.lean = 1;
     if (shared_count) {
         hipLaunchKernelGGL(count_lane_kernel, dim3(blocks), dim3(BLOCK), 0, st, r.a);
         SGL_LAUNCH_CHECK();
