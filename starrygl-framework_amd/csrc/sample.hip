@@ -1384,6 +1384,7 @@ HopKernel fill_fn(int G, bool uniform) {
 // Gc lanes per slot search, Gf lanes per slot copy or draw.  do_count / do_fill: the two halves of a hop; a second
 // query over the same slots with the same window rule and fanout runs only the fill, on the first query's
 // window arrays and block sums (same grid and run alignment: hop_grid).
+constexpr int64_t LANE_MAX_BLOCKS = 2048;
 struct HopGrid {
     int32_t align;
     int64_t blocks;
@@ -1393,6 +1394,9 @@ HopGrid hop_grid(int64_t S_max, int Gc, int Gf) {
     hg.align = BLOCK / (Gc < Gf ? Gc : Gf);
     hg.blocks = ceil_div<int64_t>(S_max > 0 ? S_max : 1, hg.align);
     if (hg.blocks > MAX_BLOCKS) hg.blocks = MAX_BLOCKS;
+    // hops of the lane-per-slot kernels: eight blocks per CU, each walking its run in several trips (the two hop-2
+    // counting kernels of a 16-batch pass 17.7 -> 9.2 us, the fills 2-5 % shorter, against a block per 256 slots of capacity)
+    if (Gc == 1 && hg.blocks > LANE_MAX_BLOCKS) hg.blocks = LANE_MAX_BLOCKS;
     return hg;
 }
 
