@@ -1080,18 +1080,31 @@ def main():
                                   + ("are looked up by the loader before the timed region and travel with the batch"
                                      if not use_root_hint else "are searched inside the step")}
         # ---- one set of library calls per mini-batch, args.pipelines batches in flight (single-launch samplers)
-        pipes = [make_pipeline(st_, use_root_hint) for st_ in pipe_streams[: args.pipelines]]
-        wall_p, sub_p, tot_p = timed_region(lambda i, b: pipes[i % len(pipes)].run(b), [P_.acc for P_ in pipes])
-        del pipes
-        assert np.array_equal(tot_p[SAME], tot[SAME]), f"batched and per-batch passes disagree: {tot} {tot_p}"
-        per_batch_calls = {"ms_per_step": round(wall_p / K * 1e3, 4), "value": round(float(tot_p[:4].sum()) / wall_p, 1),
-                           "host_submit_ms_per_step": round(sub_p / K * 1e3, 4), "batches_in_flight": args.pipelines,
-                           "note": "the same K steps with one set of library calls per mini-batch (sgl_sample_khop_multi as one "
-                                   "launch, sgl_unique_compact on the sampler's marks, one gather launch), dealt to pipelines"}
-        wall1, _, tot1 = timed_region(plain_batch, [acc])
-        assert np.array_equal(tot1[SAME], tot[SAME]), "batched and plain pass disagree"
-        one_in_flight = {"ms_per_step": round(wall1 / K * 1e3, 4), "value": round(float(tot1[:4].sum()) / wall1, 1),
-                         "note": "one set of library calls per mini-batch, one batch at a time"}
+        # (These two comparison legs run the single-launch kernels, whose blocks wait - bounded - for the blocks before
+        # them; the library's callers re-issue a call that gave up, this loop does not.  A leg that saw a give-up, or
+        # whose counts differ from the headline's, is reported as an error in its place: the headline stands.)
+        try:
+            pipes = [make_pipeline(st_, use_root_hint) for st_ in pipe_streams[: args.pipelines]]
+            wall_p, sub_p, tot_p = timed_region(lambda i, b: pipes[i % len(pipes)].run(b), [P_.acc for P_ in pipes])
+            del pipes
+            if not np.array_equal(tot_p[SAME], tot[SAME]):
+                raise RuntimeError(f"batched and per-batch passes disagree: {tot.tolist()} {tot_p.tolist()}")
+            per_batch_calls = {"ms_per_step": round(wall_p / K * 1e3, 4), "value": round(float(tot_p[:4].sum()) / wall_p, 1),
+                               "host_submit_ms_per_step": round(sub_p / K * 1e3, 4), "batches_in_flight": args.pipelines,
+                               "note": "the same K steps with one set of library calls per mini-batch (sgl_sample_khop_multi as one "
+                                       "launch, sgl_unique_compact on the sampler's marks, one gather launch), dealt to pipelines"}
+        except RuntimeError as exc:
+            log(f"[bench] per-batch leg: {exc}")
+            per_batch_calls = {"error": str(exc)}
+        try:
+            wall1, _, tot1 = timed_region(plain_batch, [acc])
+            if not np.array_equal(tot1[SAME], tot[SAME]):
+                raise RuntimeError(f"batched and plain pass disagree: {tot.tolist()} {tot1.tolist()}")
+            one_in_flight = {"ms_per_step": round(wall1 / K * 1e3, 4), "value": round(float(tot1[:4].sum()) / wall1, 1),
+                             "note": "one set of library calls per mini-batch, one batch at a time"}
+        except RuntimeError as exc:
+            log(f"[bench] one-batch-at-a-time leg: {exc}")
+            one_in_flight = {"error": str(exc)}
     elif piped:
         # ---- the headline: K steps dealt in turn to the pipelines
         pipes = [make_pipeline(st_, use_root_hint) for st_ in pipe_streams[: args.pipelines]]
